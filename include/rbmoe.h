@@ -1,0 +1,206 @@
+/*
+ * rbmoe.h — C ABI of the MI355X (gfx950) mixture-of-experts layer.
+ *
+ * Drop-in boundary for the forward pass of RustingBrain's `MoeLayer`
+ * (reference src/moe.rs:203-341) and the two auxiliary losses.  The reference
+ * has no FFI seam for this layer; each entry point below names the reference
+ * interface it stands in for, so that a Rust `extern "C"` block can bind them
+ * one to one.  Plain pointers and sizes only.  Every function returns an
+ * `rbmoe_status`; none throws, aborts or falls back to a CPU path.
+ *
+ * Matrices are row-major and contiguous, exactly like the reference `Matrix`
+ * (src/matrix.rs:13-18).  A `Linear` weight is `[out_features, in_features]`
+ * (src/param.rs:620-633): router `[E, d]`, gate/up `[F, d]`, down `[d, F]`.
+ */
+#ifndef RBMOE_H
+#define RBMOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Mirrors the `NetworkError` variants that can leave this path
+ * (reference src/network.rs:19-83). */
+typedef enum rbmoe_status {
+    RBMOE_OK = 0,
+    RBMOE_INVALID_INPUT = 1,      /* NetworkError::InvalidInput{expected, actual}      */
+    RBMOE_INVALID_CONFIG = 2,     /* NetworkError::InvalidConfig(String)               */
+    RBMOE_DEVICE_ERROR = 3,       /* NetworkError::Cuda(String): a HIP call failed     */
+    RBMOE_BACKEND_UNAVAILABLE = 4,/* NetworkError::CudaFeatureDisabled: no usable GPU  */
+    RBMOE_MEMORY_BUDGET = 5,      /* NetworkError::CudaMemoryBudget{estimated, budget} */
+    RBMOE_OUT_OF_MEMORY = 6,      /* NetworkError::CudaOutOfMemory{requested, free}    */
+    RBMOE_UNSUPPORTED = 7,        /* NetworkError::UnsupportedCuda(String)             */
+    RBMOE_NULL_POINTER = 8        /* a required pointer argument was NULL              */
+} rbmoe_status;
+
+typedef enum rbmoe_dtype {
+    RBMOE_F32 = 0,
+    RBMOE_BF16 = 1,  /* raw 16-bit patterns, round-to-nearest-even from f32 */
+    RBMOE_I8 = 2     /* weights only: symmetric int8 + one f32 scale per output row */
+} rbmoe_dtype;
+
+/* Which weight of the layer; the order is the reference's parameter traversal
+ * (src/moe.rs:516-525 with src/ffn.rs:126-131). */
+typedef enum rbmoe_weight {
+    RBMOE_W_ROUTER = 0,       /* [E, d]              Router.projection  (src/moe.rs:91-100) */
+    RBMOE_W_GATE = 1,         /* [F, d]  per expert  SwiGlu.gate        (src/ffn.rs:19-23)  */
+    RBMOE_W_UP = 2,           /* [F, d]  per expert  SwiGlu.up                              */
+    RBMOE_W_DOWN = 3,         /* [d, F]  per expert  SwiGlu.down                            */
+    RBMOE_W_SHARED_GATE = 4,  /* [Fs, d]             MoeLayer.shared    (src/moe.rs:210)    */
+    RBMOE_W_SHARED_UP = 5,    /* [Fs, d]                                                    */
+    RBMOE_W_SHARED_DOWN = 6   /* [d, Fs]                                                    */
+} rbmoe_weight;
+
+/* `MoeConfig` (reference src/moe.rs:25-39) plus what a device layer must know
+ * up front.  `shared_d_ff` exists because the reference's `shared` field is
+ * public and may hold an expert of another width (src/moe.rs:210, used that way
+ * at src/moe.rs:841-843); 0 means "same as d_ff". */
+typedef struct rbmoe_config {
+    int32_t d_model;
+    int32_t num_experts;
+    int32_t experts_per_token;
+    int32_t d_ff;
+    int32_t shared_expert;         /* 0 / 1 */
+    int32_t shared_d_ff;           /* 0 = d_ff */
+    float aux_loss_weight;         /* DEFAULT_AUX_LOSS_WEIGHT = 0.01 (src/moe.rs:20)           */
+    float router_z_loss_weight;    /* DEFAULT_ROUTER_Z_LOSS_WEIGHT = 1e-3 (src/moe.rs:23)      */
+    int32_t weight_dtype;          /* rbmoe_dtype of the expert weights                        */
+    int32_t act_dtype;             /* rbmoe_dtype of x / out: RBMOE_F32 or RBMOE_BF16          */
+    int32_t max_tokens;            /* workspace is sized for this many rows; forward allocates nothing */
+} rbmoe_config;
+
+/* Routing tables of the last forward, the bit-exact comparands.
+ * Slot s = token * k + rank (rank 0 = highest probability), as the reference's
+ * `assignments` (src/moe.rs:142-145).  All pointers are optional (NULL = skip)
+ * and must be host memory. */
+typedef struct rbmoe_routing {
+    int32_t* expert_of;   /* [T*k]  expert per slot, -1 = UNROUTED (src/moe.rs:190-191) */
+    float* gate_of;       /* [T*k]  renormalised gate per slot                          */
+    int32_t* counts;      /* [E]    expert_tokens[e].len() (src/moe.rs:266-274)         */
+    int32_t* offsets;     /* [E+1]  exclusive prefix of counts                          */
+    int32_t* perm_slot;   /* [T*k]  expert_slots, experts concatenated; first offsets[E] valid  */
+    int32_t* perm_token;  /* [T*k]  expert_tokens, experts concatenated                 */
+    float* probabilities; /* [T*E]  MoeCache.probabilities (src/moe.rs:137-140)         */
+    float* log_sum_exp;   /* [T]    MoeCache.log_sum_exp   (src/moe.rs:141-142)         */
+} rbmoe_routing;
+
+typedef struct rbmoe_ctx rbmoe_ctx;
+typedef struct rbmoe_layer rbmoe_layer;
+
+/* MoeConfig::new (src/moe.rs:41-51): defaults for everything but the three
+ * arguments; dtypes default to f32, max_tokens to 0 (must be set). */
+int rbmoe_config_init(rbmoe_config* cfg, int32_t d_model, int32_t num_experts,
+                      int32_t experts_per_token, int32_t d_ff);
+
+/* MoeConfig::validate (src/moe.rs:68-86) plus dtype/limit checks.  Touches no
+ * GPU.  On failure writes a message (same wording as the reference where one
+ * exists) into `msg` if `msg_cap` > 0. */
+int rbmoe_validate(const rbmoe_config* cfg, char* msg, size_t msg_cap);
+
+/* TransformerConfig::parameter_counts restricted to one layer
+ * (src/transformer.rs:194-227; MoeLayer::num_parameters / active_parameters,
+ * src/moe.rs:527-545). */
+int rbmoe_parameter_counts(const rbmoe_config* cfg, uint64_t* total, uint64_t* active);
+
+/* Opens device `device` with a memory budget in MiB (0 = unlimited): the role of
+ * `CudaDevice::open` + `GpuContext` (src/param.rs:86-190,
+ * src/gpu_transformer.rs:45-76).  Fails closed with RBMOE_BACKEND_UNAVAILABLE
+ * when no GPU can be used. */
+int rbmoe_ctx_create(int32_t device, size_t budget_mib, rbmoe_ctx** out);
+void rbmoe_ctx_destroy(rbmoe_ctx* ctx);
+
+/* Use the caller's HIP stream (a `hipStream_t` passed as void*) instead of the
+ * context's own; NULL restores the context's own stream. */
+int rbmoe_ctx_set_stream(rbmoe_ctx* ctx, void* hip_stream);
+
+/* GpuContext::synchronize (src/gpu_transformer.rs:179-187). */
+int rbmoe_synchronize(rbmoe_ctx* ctx);
+
+/* Message of the last failure on this context (owned by the context). */
+const char* rbmoe_last_error(const rbmoe_ctx* ctx);
+/* Message of the last failure of a call that had no context to attach it to
+ * (thread-local). */
+const char* rbmoe_last_global_error(void);
+
+/* MoeLayer::new (src/moe.rs:215-231) + TransformerLm::to_cuda's upload of the
+ * layer (src/transformer.rs:1263-1296): validates, checks the budget BEFORE
+ * allocating (src/param.rs:172-189), allocates weights (zeroed) and workspace. */
+int rbmoe_layer_create(rbmoe_ctx* ctx, const rbmoe_config* cfg, rbmoe_layer** out);
+void rbmoe_layer_destroy(rbmoe_layer* layer);
+
+/* DeviceParam::new (src/gpu_transformer.rs:471-490): copies one weight matrix
+ * from HOST memory to the device (the caller keeps its buffer).  `dtype` is the
+ * dtype of `data`; f32 data is converted to the layer's weight dtype (bf16 by
+ * RNE; int8 by the checkpoint rule scale = absmax/127, q = round(w/scale),
+ * src/transformer.rs:512-519).  For RBMOE_I8 data, `scales` holds one f32 per
+ * row.  `expert` is ignored for the router and the shared expert. */
+int rbmoe_set_weight(rbmoe_layer* layer, int32_t which, int32_t expert, const void* data,
+                     int32_t dtype, const float* scales, int32_t rows, int32_t cols);
+
+/* MoeLayer::forward_train (src/moe.rs:243-341) on DEVICE pointers, enqueued on
+ * the context's stream; returns without synchronising.
+ *   x        [T, cols] act_dtype; cols must equal d_model (else InvalidInput)
+ *   valid    [T] bytes, 0 = padding row (Layout.valid, src/batch.rs:224-269), or NULL
+ *   router_bias [E] f32 added to the logits, or NULL (the reference router is
+ *            bias-free; this is a benchmark hook for skewed loads)
+ *   residual [T, d] act_dtype added to the result (the block's residual add,
+ *            src/transformer_block.rs:221-222), or NULL
+ *   out      [T, d] act_dtype
+ * Auxiliary losses and routing tables stay on the device until fetched. */
+int rbmoe_forward(rbmoe_layer* layer, const void* x, int32_t T, int32_t cols, const uint8_t* valid,
+                  const float* router_bias, const void* residual, void* out);
+
+/* Same on HOST pointers: copies in, runs, synchronises, copies out. */
+int rbmoe_forward_host(rbmoe_layer* layer, const void* x, int32_t T, int32_t cols,
+                       const uint8_t* valid, const float* router_bias, const void* residual,
+                       void* out);
+
+/* MoeCache::aux_loss / z_loss (src/moe.rs:158-172) of the last forward.
+ * Synchronises the stream. */
+int rbmoe_get_losses(rbmoe_layer* layer, float* aux_loss, float* z_loss);
+
+/* Routing tables of the last forward into host buffers.  Synchronises. */
+int rbmoe_get_routing(rbmoe_layer* layer, rbmoe_routing* routing);
+
+/* Expert hidden rows H [offsets[E], F] and expert output rows Y [offsets[E], d]
+ * of the last forward, in permuted order, converted to f32, into host buffers
+ * (either may be NULL) — the reference keeps both in MoeCache
+ * (src/moe.rs:150-152, src/ffn.rs:27-33).  Synchronises. */
+int rbmoe_get_expert_rows(rbmoe_layer* layer, float* hidden, float* expert_out);
+
+/* Per-stage timing of one forward with HIP events on the context's stream.
+ * `ms` receives RBMOE_NUM_STAGES durations in milliseconds.  Synchronises. */
+#define RBMOE_NUM_STAGES 8
+enum {
+    RBMOE_STAGE_ROUTER = 0,   /* logits + softmax + top-k + block histogram     */
+    RBMOE_STAGE_SCAN = 1,     /* prefix scan, tile table, auxiliary losses      */
+    RBMOE_STAGE_DISPATCH = 2, /* permutation + row gather                       */
+    RBMOE_STAGE_GATE_UP = 3,  /* grouped gate/up product + SwiGLU               */
+    RBMOE_STAGE_DOWN = 4,     /* grouped down product                           */
+    RBMOE_STAGE_SHARED = 5,   /* shared expert (both products)                  */
+    RBMOE_STAGE_COMBINE = 6,  /* gate-weighted combine (+ shared, + residual)   */
+    RBMOE_STAGE_TOTAL = 7
+};
+int rbmoe_forward_timed(rbmoe_layer* layer, const void* x, int32_t T, int32_t cols,
+                        const uint8_t* valid, const float* router_bias, const void* residual,
+                        void* out, float* ms);
+
+/* Name of the kernel variant the last forward used for the expert products
+ * ("mfma_bf16", "generic", ...), for reports.  Static storage. */
+const char* rbmoe_expert_kernel_name(const rbmoe_layer* layer);
+
+/* Device memory helpers for hosts without their own HIP binding. */
+int rbmoe_device_alloc(rbmoe_ctx* ctx, size_t bytes, void** out);
+int rbmoe_device_free(rbmoe_ctx* ctx, void* ptr);
+int rbmoe_copy_to_device(rbmoe_ctx* ctx, void* dst, const void* src, size_t bytes);
+int rbmoe_copy_to_host(rbmoe_ctx* ctx, void* dst, const void* src, size_t bytes);
+
+const char* rbmoe_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RBMOE_H */

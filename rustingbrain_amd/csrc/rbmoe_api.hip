@@ -1,0 +1,790 @@
+// C ABI of the gfx950 mixture-of-experts layer (see include/rbmoe.h).
+//
+// Host-side orchestration only: configuration checks, weight upload and
+// conversion, workspace, and the launch sequence of one forward pass
+//   router -> scan -> dispatch -> gate/up (+SwiGLU) -> down -> shared -> combine
+// which follows MoeLayer::forward_train (reference src/moe.rs:243-341) stage by
+// stage without any host round trip between the stages.  There is no CPU
+// fallback: without a usable GPU every device entry point fails.
+#include "../../include/rbmoe.h"
+
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "rbmoe_kernels.h"
+
+using namespace rbmoe;
+
+namespace {
+
+thread_local std::string g_global_error;
+
+size_t dtype_size(int dt) { return dt == RBMOE_F32 ? 4 : dt == RBMOE_BF16 ? 2 : 1; }
+
+uint16_t host_f32_to_bf16(float f) {
+    uint32_t b;
+    std::memcpy(&b, &f, 4);
+    if ((b & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((b >> 16) | 0x0040u);
+    b += 0x7fffu + ((b >> 16) & 1u);
+    return (uint16_t)(b >> 16);
+}
+float host_bf16_to_f32(uint16_t h) {
+    uint32_t b = (uint32_t)h << 16;
+    float f;
+    std::memcpy(&f, &b, 4);
+    return f;
+}
+
+std::string config_problem(const rbmoe_config* c) {
+    char buf[256];
+    // The first three are MoeConfig::validate (reference src/moe.rs:68-86), same wording.
+    if (c->num_experts <= 0) return "a MoE layer needs at least one expert";
+    if (c->experts_per_token <= 0 || c->experts_per_token > c->num_experts) {
+        std::snprintf(buf, sizeof buf, "experts_per_token must be between 1 and num_experts (%d), got %d",
+                      c->num_experts, c->experts_per_token);
+        return buf;
+    }
+    if (c->d_ff <= 0) return "expert d_ff must be non-zero";
+    if (c->d_model <= 0) return "d_model must be non-zero";
+    if (c->shared_d_ff < 0) return "shared_d_ff must not be negative";
+    if (c->weight_dtype != RBMOE_F32 && c->weight_dtype != RBMOE_BF16 && c->weight_dtype != RBMOE_I8)
+        return "weight_dtype must be f32, bf16 or int8";
+    if (c->act_dtype != RBMOE_F32 && c->act_dtype != RBMOE_BF16) return "act_dtype must be f32 or bf16";
+    if (c->max_tokens < 0) return "max_tokens must not be negative";
+    return "";
+}
+
+std::string limit_problem(const rbmoe_config* c) {
+    char buf[256];
+    if (c->num_experts > kMaxExperts) {
+        std::snprintf(buf, sizeof buf, "more than %d experts (got %d)", kMaxExperts, c->num_experts);
+        return buf;
+    }
+    if (c->experts_per_token > kMaxTopK) {
+        std::snprintf(buf, sizeof buf, "experts_per_token above %d (got %d)", kMaxTopK, c->experts_per_token);
+        return buf;
+    }
+    if ((int64_t)c->max_tokens * c->experts_per_token > (int64_t)1 << 28) return "max_tokens * experts_per_token above 2^28";
+    return "";
+}
+
+}  // namespace
+
+struct rbmoe_ctx {
+    int device = 0;
+    hipStream_t own_stream = nullptr;
+    hipStream_t stream = nullptr;
+    size_t budget_bytes = 0;
+    size_t allocated = 0;
+    std::string last_error;
+};
+
+namespace {
+
+struct Buf {
+    void* p = nullptr;
+    size_t bytes = 0;
+};
+
+int fail(rbmoe_ctx* ctx, int code, const std::string& msg) {
+    if (ctx) ctx->last_error = msg;
+    g_global_error = msg;
+    return code;
+}
+
+int hip_fail(rbmoe_ctx* ctx, hipError_t e, const char* what) {
+    std::string msg = std::string(what) + ": " + hipGetErrorString(e);
+    if (e == hipErrorOutOfMemory) return fail(ctx, RBMOE_OUT_OF_MEMORY, msg);
+    return fail(ctx, RBMOE_DEVICE_ERROR, msg);
+}
+
+#define HIP_TRY(ctx, expr)                                         \
+    do {                                                           \
+        hipError_t _e = (expr);                                    \
+        if (_e != hipSuccess) return hip_fail((ctx), _e, #expr);   \
+    } while (0)
+
+}  // namespace
+
+struct rbmoe_layer {
+    rbmoe_ctx* ctx = nullptr;
+    rbmoe_config cfg{};
+    int Fs = 0;       // shared expert width
+    int max_T = 0;
+    int max_S = 0;
+    int max_nb = 0;
+    int max_tiles = 0;
+    bool force_generic = false;
+    const char* kernel_name = "none";
+    int last_T = -1;
+
+    // weights
+    Buf router;            // f32 [E, d]
+    Buf wgu, wd;           // [E, 2F, d], [E, d, F] weight dtype
+    Buf sgu, sd;           // int8 scales [E, 2F], [E, d]
+    Buf swgu, swd;         // shared [2Fs, d], [d, Fs]
+    Buf ssgu, ssd;         // shared scales
+    // workspace
+    Buf P, lse, expert_of, gate_of, rank_in_block, blockcnt, blockbase, partial;
+    Buf counts, offsets, tile_expert, tile_row0, tile_rows, ntiles, losses, mass;
+    Buf perm_slot, perm_token, inv_pos;
+    Buf xg, h, y, hs, ys;
+    // staging for the host entry point
+    Buf st_x, st_out, st_valid, st_bias, st_res;
+    std::vector<Buf*> all;
+    hipEvent_t ev[RBMOE_NUM_STAGES + 1] = {};
+    bool have_events = false;
+};
+
+namespace {
+
+struct Plan {
+    std::vector<std::pair<Buf*, size_t>> items;
+    size_t total = 0;
+    void add(Buf* b, size_t bytes) {
+        bytes = (bytes + 255) & ~(size_t)255;
+        if (bytes == 0) bytes = 256;
+        items.push_back({b, bytes});
+        total += bytes;
+    }
+};
+
+Plan make_plan(rbmoe_layer* L) {
+    const rbmoe_config& c = L->cfg;
+    const size_t E = c.num_experts, d = c.d_model, F = c.d_ff, k = c.experts_per_token;
+    const size_t Fs = L->Fs, T = L->max_T, S = L->max_S, nb = L->max_nb;
+    const size_t ws = dtype_size(c.weight_dtype), as = dtype_size(c.act_dtype);
+    Plan p;
+    p.add(&L->router, E * d * 4);
+    p.add(&L->wgu, E * 2 * F * d * ws);
+    p.add(&L->wd, E * d * F * ws);
+    if (c.weight_dtype == RBMOE_I8) {
+        p.add(&L->sgu, E * 2 * F * 4);
+        p.add(&L->sd, E * d * 4);
+    }
+    if (c.shared_expert) {
+        p.add(&L->swgu, 2 * Fs * d * ws);
+        p.add(&L->swd, d * Fs * ws);
+        if (c.weight_dtype == RBMOE_I8) {
+            p.add(&L->ssgu, 2 * Fs * 4);
+            p.add(&L->ssd, d * 4);
+        }
+        p.add(&L->hs, T * Fs * as);
+        p.add(&L->ys, T * d * as);
+    }
+    p.add(&L->P, T * E * 4);
+    p.add(&L->lse, T * 4);
+    p.add(&L->expert_of, S * 4);
+    p.add(&L->gate_of, S * 4);
+    p.add(&L->rank_in_block, S * 4);
+    p.add(&L->blockcnt, nb * E * 4);
+    p.add(&L->blockbase, nb * E * 4);
+    p.add(&L->partial, nb * (E + 1) * 4);
+    p.add(&L->counts, E * 4);
+    p.add(&L->offsets, (E + 1) * 4);
+    p.add(&L->tile_expert, (size_t)L->max_tiles * 4);
+    p.add(&L->tile_row0, (size_t)L->max_tiles * 4);
+    p.add(&L->tile_rows, (size_t)L->max_tiles * 4);
+    p.add(&L->ntiles, 4);
+    p.add(&L->losses, 8);
+    p.add(&L->mass, (E + 1) * 4);
+    p.add(&L->perm_slot, S * 4);
+    p.add(&L->perm_token, S * 4);
+    p.add(&L->inv_pos, S * 4);
+    p.add(&L->xg, S * d * as);
+    p.add(&L->h, S * F * as);
+    p.add(&L->y, S * d * as);
+    p.add(&L->st_x, T * d * as);
+    p.add(&L->st_out, T * d * as);
+    p.add(&L->st_res, T * d * as);
+    p.add(&L->st_valid, T);
+    p.add(&L->st_bias, E * 4);
+    (void)k;
+    return p;
+}
+
+void free_layer_buffers(rbmoe_layer* L) {
+    for (Buf* b : L->all) {
+        if (b->p) {
+            (void)hipFree(b->p);
+            if (L->ctx && L->ctx->allocated >= b->bytes) L->ctx->allocated -= b->bytes;
+            b->p = nullptr;
+            b->bytes = 0;
+        }
+    }
+    L->all.clear();
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* rbmoe_version(void) { return "rbmoe 0.1 (gfx950)"; }
+
+const char* rbmoe_last_global_error(void) { return g_global_error.c_str(); }
+
+int rbmoe_config_init(rbmoe_config* cfg, int32_t d_model, int32_t num_experts, int32_t experts_per_token,
+                      int32_t d_ff) {
+    if (!cfg) return fail(nullptr, RBMOE_NULL_POINTER, "cfg is NULL");
+    std::memset(cfg, 0, sizeof *cfg);
+    cfg->d_model = d_model;
+    cfg->num_experts = num_experts;
+    cfg->experts_per_token = experts_per_token;
+    cfg->d_ff = d_ff;
+    cfg->shared_expert = 0;
+    cfg->shared_d_ff = 0;
+    cfg->aux_loss_weight = 0.01f;
+    cfg->router_z_loss_weight = 1e-3f;
+    cfg->weight_dtype = RBMOE_F32;
+    cfg->act_dtype = RBMOE_F32;
+    cfg->max_tokens = 0;
+    return RBMOE_OK;
+}
+
+int rbmoe_validate(const rbmoe_config* cfg, char* msg, size_t msg_cap) {
+    if (!cfg) return fail(nullptr, RBMOE_NULL_POINTER, "cfg is NULL");
+    std::string problem = config_problem(cfg);
+    int code = RBMOE_INVALID_CONFIG;
+    if (problem.empty()) {
+        problem = limit_problem(cfg);
+        code = RBMOE_UNSUPPORTED;
+    }
+    if (msg && msg_cap > 0) {
+        std::snprintf(msg, msg_cap, "%s", problem.c_str());
+    }
+    if (problem.empty()) return RBMOE_OK;
+    return fail(nullptr, code, problem);
+}
+
+int rbmoe_parameter_counts(const rbmoe_config* cfg, uint64_t* total, uint64_t* active) {
+    if (!cfg) return fail(nullptr, RBMOE_NULL_POINTER, "cfg is NULL");
+    const uint64_t d = cfg->d_model, E = cfg->num_experts, k = cfg->experts_per_token, F = cfg->d_ff;
+    const uint64_t Fs = cfg->shared_d_ff > 0 ? cfg->shared_d_ff : cfg->d_ff;
+    const uint64_t expert = 3 * d * F;
+    const uint64_t shared = cfg->shared_expert ? 3 * d * Fs : 0;
+    const uint64_t router = E * d;
+    if (total) *total = router + E * expert + shared;
+    if (active) *active = router + k * expert + shared;
+    return RBMOE_OK;
+}
+
+int rbmoe_ctx_create(int32_t device, size_t budget_mib, rbmoe_ctx** out) {
+    if (!out) return fail(nullptr, RBMOE_NULL_POINTER, "out is NULL");
+    *out = nullptr;
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0) {
+        (void)hipGetLastError();
+        return fail(nullptr, RBMOE_BACKEND_UNAVAILABLE,
+                    std::string("no usable HIP device: ") + (e != hipSuccess ? hipGetErrorString(e) : "device count is 0"));
+    }
+    if (device < 0 || device >= n) return fail(nullptr, RBMOE_INVALID_CONFIG, "device index out of range");
+    hipDeviceProp_t prop;
+    HIP_TRY(nullptr, hipGetDeviceProperties(&prop, device));
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(nullptr, RBMOE_UNSUPPORTED, std::string("kernels are built for gfx950, device is ") + prop.gcnArchName);
+    HIP_TRY(nullptr, hipSetDevice(device));
+    rbmoe_ctx* ctx = new rbmoe_ctx();
+    ctx->device = device;
+    ctx->budget_bytes = budget_mib << 20;
+    hipError_t se = hipStreamCreateWithFlags(&ctx->own_stream, hipStreamNonBlocking);
+    if (se != hipSuccess) {
+        delete ctx;
+        return hip_fail(nullptr, se, "hipStreamCreateWithFlags");
+    }
+    ctx->stream = ctx->own_stream;
+    *out = ctx;
+    return RBMOE_OK;
+}
+
+void rbmoe_ctx_destroy(rbmoe_ctx* ctx) {
+    if (!ctx) return;
+    if (ctx->own_stream) {
+        (void)hipStreamSynchronize(ctx->own_stream);
+        (void)hipStreamDestroy(ctx->own_stream);
+    }
+    delete ctx;
+}
+
+int rbmoe_ctx_set_stream(rbmoe_ctx* ctx, void* hip_stream) {
+    if (!ctx) return fail(nullptr, RBMOE_NULL_POINTER, "ctx is NULL");
+    ctx->stream = hip_stream ? static_cast<hipStream_t>(hip_stream) : ctx->own_stream;
+    return RBMOE_OK;
+}
+
+int rbmoe_synchronize(rbmoe_ctx* ctx) {
+    if (!ctx) return fail(nullptr, RBMOE_NULL_POINTER, "ctx is NULL");
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return RBMOE_OK;
+}
+
+const char* rbmoe_last_error(const rbmoe_ctx* ctx) { return ctx ? ctx->last_error.c_str() : g_global_error.c_str(); }
+
+int rbmoe_layer_create(rbmoe_ctx* ctx, const rbmoe_config* cfg, rbmoe_layer** out) {
+    if (!ctx || !cfg || !out) return fail(ctx, RBMOE_NULL_POINTER, "ctx, cfg or out is NULL");
+    *out = nullptr;
+    std::string problem = config_problem(cfg);
+    if (!problem.empty()) return fail(ctx, RBMOE_INVALID_CONFIG, problem);
+    problem = limit_problem(cfg);
+    if (!problem.empty()) return fail(ctx, RBMOE_UNSUPPORTED, problem);
+    if (cfg->max_tokens <= 0) return fail(ctx, RBMOE_INVALID_CONFIG, "max_tokens must be positive");
+    if (router_lds_bytes(cfg->num_experts, cfg->experts_per_token) > 64 * 1024)
+        return fail(ctx, RBMOE_UNSUPPORTED, "router tile does not fit in LDS for this expert count and top-k");
+
+    rbmoe_layer* L = new rbmoe_layer();
+    L->ctx = ctx;
+    L->cfg = *cfg;
+    L->Fs = cfg->shared_d_ff > 0 ? cfg->shared_d_ff : cfg->d_ff;
+    L->cfg.shared_d_ff = L->Fs;
+    L->max_T = cfg->max_tokens;
+    L->max_S = cfg->max_tokens * cfg->experts_per_token;
+    L->max_nb = (cfg->max_tokens + kRouterTokens - 1) / kRouterTokens;
+    L->max_tiles = L->max_S / kGenericTileM + cfg->num_experts + 1;
+    const char* fg = std::getenv("RBMOE_FORCE_GENERIC");
+    L->force_generic = fg && fg[0] == '1';
+
+    Plan plan = make_plan(L);
+    // Refuse before allocating anything, as the reference's budget check does
+    // (src/param.rs:172-189).
+    if (ctx->budget_bytes && ctx->allocated + plan.total > ctx->budget_bytes) {
+        char buf[200];
+        std::snprintf(buf, sizeof buf, "memory budget exceeded: estimated %zu MiB exceeds budget %zu MiB",
+                      (ctx->allocated + plan.total + (1 << 20) - 1) >> 20, ctx->budget_bytes >> 20);
+        delete L;
+        return fail(ctx, RBMOE_MEMORY_BUDGET, buf);
+    }
+    hipError_t e = hipSetDevice(ctx->device);
+    if (e != hipSuccess) {
+        delete L;
+        return hip_fail(ctx, e, "hipSetDevice");
+    }
+    for (auto& it : plan.items) {
+        void* p = nullptr;
+        e = hipMalloc(&p, it.second);
+        if (e != hipSuccess) {
+            size_t free_b = 0, total_b = 0;
+            (void)hipGetLastError();
+            (void)hipMemGetInfo(&free_b, &total_b);
+            char buf[200];
+            std::snprintf(buf, sizeof buf, "out of memory: an allocation of %zu MiB failed with %zu MiB free",
+                          it.second >> 20, free_b >> 20);
+            free_layer_buffers(L);
+            delete L;
+            return fail(ctx, RBMOE_OUT_OF_MEMORY, buf);
+        }
+        it.first->p = p;
+        it.first->bytes = it.second;
+        ctx->allocated += it.second;
+        L->all.push_back(it.first);
+        e = hipMemsetAsync(p, 0, it.second, ctx->stream);
+        if (e != hipSuccess) {
+            free_layer_buffers(L);
+            delete L;
+            return hip_fail(ctx, e, "hipMemsetAsync");
+        }
+    }
+    e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) {
+        free_layer_buffers(L);
+        delete L;
+        return hip_fail(ctx, e, "hipStreamSynchronize");
+    }
+    *out = L;
+    return RBMOE_OK;
+}
+
+void rbmoe_layer_destroy(rbmoe_layer* L) {
+    if (!L) return;
+    if (L->ctx) (void)hipStreamSynchronize(L->ctx->stream);
+    if (L->have_events)
+        for (auto& ev : L->ev)
+            if (ev) (void)hipEventDestroy(ev);
+    free_layer_buffers(L);
+    delete L;
+}
+
+int rbmoe_set_weight(rbmoe_layer* L, int32_t which, int32_t expert, const void* data, int32_t dtype,
+                     const float* scales, int32_t rows, int32_t cols) {
+    if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
+    rbmoe_ctx* ctx = L->ctx;
+    if (!data) return fail(ctx, RBMOE_NULL_POINTER, "data is NULL");
+    const rbmoe_config& c = L->cfg;
+    const int E = c.num_experts, d = c.d_model, F = c.d_ff, Fs = L->Fs;
+    int want_rows = 0, want_cols = 0;
+    char* dst = nullptr;        // destination of the matrix, in weight-dtype elements
+    float* sdst = nullptr;      // destination of the scales
+    size_t elem_off = 0, scale_off = 0;
+    bool is_router = false;
+    switch (which) {
+        case RBMOE_W_ROUTER:
+            want_rows = E; want_cols = d; is_router = true;
+            dst = static_cast<char*>(L->router.p);
+            break;
+        case RBMOE_W_GATE:
+        case RBMOE_W_UP:
+            want_rows = F; want_cols = d;
+            if (expert < 0 || expert >= E) return fail(ctx, RBMOE_INVALID_CONFIG, "expert index out of range");
+            elem_off = ((size_t)expert * 2 + (which == RBMOE_W_UP ? 1 : 0)) * F * d;
+            scale_off = ((size_t)expert * 2 + (which == RBMOE_W_UP ? 1 : 0)) * F;
+            dst = static_cast<char*>(L->wgu.p);
+            sdst = static_cast<float*>(L->sgu.p);
+            break;
+        case RBMOE_W_DOWN:
+            want_rows = d; want_cols = F;
+            if (expert < 0 || expert >= E) return fail(ctx, RBMOE_INVALID_CONFIG, "expert index out of range");
+            elem_off = (size_t)expert * d * F;
+            scale_off = (size_t)expert * d;
+            dst = static_cast<char*>(L->wd.p);
+            sdst = static_cast<float*>(L->sd.p);
+            break;
+        case RBMOE_W_SHARED_GATE:
+        case RBMOE_W_SHARED_UP:
+            if (!c.shared_expert) return fail(ctx, RBMOE_INVALID_CONFIG, "the layer has no shared expert");
+            want_rows = Fs; want_cols = d;
+            elem_off = (size_t)(which == RBMOE_W_SHARED_UP ? 1 : 0) * Fs * d;
+            scale_off = (size_t)(which == RBMOE_W_SHARED_UP ? 1 : 0) * Fs;
+            dst = static_cast<char*>(L->swgu.p);
+            sdst = static_cast<float*>(L->ssgu.p);
+            break;
+        case RBMOE_W_SHARED_DOWN:
+            if (!c.shared_expert) return fail(ctx, RBMOE_INVALID_CONFIG, "the layer has no shared expert");
+            want_rows = d; want_cols = Fs;
+            dst = static_cast<char*>(L->swd.p);
+            sdst = static_cast<float*>(L->ssd.p);
+            break;
+        default:
+            return fail(ctx, RBMOE_INVALID_CONFIG, "unknown weight id");
+    }
+    if (rows != want_rows || cols != want_cols) {
+        char buf[160];
+        std::snprintf(buf, sizeof buf, "weight shape [%d, %d] does not match expected [%d, %d]", rows, cols,
+                      want_rows, want_cols);
+        return fail(ctx, RBMOE_INVALID_INPUT, buf);
+    }
+    const size_t n = (size_t)rows * cols;
+    const int target = is_router ? RBMOE_F32 : c.weight_dtype;
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));  // no forward may still read the old weights
+
+    std::vector<unsigned char> staged;
+    std::vector<float> staged_scales;
+    const void* src = data;
+    if (dtype == target) {
+        if (target == RBMOE_I8) {
+            if (!scales) return fail(ctx, RBMOE_NULL_POINTER, "int8 weights need scales");
+        }
+    } else if (dtype == RBMOE_F32 && target == RBMOE_BF16) {
+        staged.resize(n * 2);
+        const float* f = static_cast<const float*>(data);
+        uint16_t* o = reinterpret_cast<uint16_t*>(staged.data());
+        for (size_t i = 0; i < n; ++i) o[i] = host_f32_to_bf16(f[i]);
+        src = staged.data();
+    } else if (dtype == RBMOE_BF16 && target == RBMOE_F32) {
+        staged.resize(n * 4);
+        const uint16_t* h = static_cast<const uint16_t*>(data);
+        float* o = reinterpret_cast<float*>(staged.data());
+        for (size_t i = 0; i < n; ++i) o[i] = host_bf16_to_f32(h[i]);
+        src = staged.data();
+    } else if (dtype == RBMOE_F32 && target == RBMOE_I8) {
+        // The checkpoint writer's rule (reference src/transformer.rs:512-519,
+        // :1839-1847): scale = absmax / 127, q = clamp(round(w / scale)).
+        staged.resize(n);
+        staged_scales.resize(rows);
+        const float* f = static_cast<const float*>(data);
+        int8_t* q = reinterpret_cast<int8_t*>(staged.data());
+        for (int r = 0; r < rows; ++r) {
+            float absmax = 0.0f;
+            for (int cc = 0; cc < cols; ++cc) absmax = std::fmax(absmax, std::fabs(f[(size_t)r * cols + cc]));
+            const float scale = absmax / 127.0f;
+            staged_scales[r] = scale;
+            for (int cc = 0; cc < cols; ++cc) {
+                float v = scale == 0.0f ? 0.0f : std::round(f[(size_t)r * cols + cc] / scale);
+                v = std::fmin(127.0f, std::fmax(-127.0f, v));
+                q[(size_t)r * cols + cc] = (int8_t)v;
+            }
+        }
+        src = staged.data();
+        scales = staged_scales.data();
+    } else {
+        return fail(ctx, RBMOE_UNSUPPORTED, "this conversion between weight dtypes is not supported");
+    }
+    const size_t es = dtype_size(target);
+    HIP_TRY(ctx, hipMemcpy(dst + elem_off * es, src, n * es, hipMemcpyHostToDevice));
+    if (target == RBMOE_I8)
+        HIP_TRY(ctx, hipMemcpy(sdst + scale_off, scales, (size_t)rows * 4, hipMemcpyHostToDevice));
+    return RBMOE_OK;
+}
+
+}  // extern "C"
+
+namespace {
+
+int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* valid, const float* router_bias,
+                 const void* residual, void* out, bool timed) {
+    if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
+    rbmoe_ctx* ctx = L->ctx;
+    const rbmoe_config& c = L->cfg;
+    const int E = c.num_experts, d = c.d_model, F = c.d_ff, k = c.experts_per_token, Fs = L->Fs;
+    // MoeLayer::forward_train's width check (reference src/moe.rs:248-253)
+    if (cols != d) {
+        char buf[120];
+        std::snprintf(buf, sizeof buf, "input length %d does not match expected length %d", cols, d);
+        return fail(ctx, RBMOE_INVALID_INPUT, buf);
+    }
+    if (T < 0) return fail(ctx, RBMOE_INVALID_INPUT, "negative token count");
+    if (T > L->max_T) {
+        char buf[120];
+        std::snprintf(buf, sizeof buf, "%d tokens exceed the layer's max_tokens %d", T, L->max_T);
+        return fail(ctx, RBMOE_INVALID_INPUT, buf);
+    }
+    if (T > 0 && (!x || !out)) return fail(ctx, RBMOE_NULL_POINTER, "x or out is NULL");
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    hipStream_t s = ctx->stream;
+    const bool abf = c.act_dtype == RBMOE_BF16;
+    const WeightKind wk = c.weight_dtype == RBMOE_F32 ? WeightKind::F32
+                          : c.weight_dtype == RBMOE_BF16 ? WeightKind::BF16 : WeightKind::I8;
+    if (timed && !L->have_events) {
+        for (auto& ev : L->ev) HIP_TRY(ctx, hipEventCreate(&ev));
+        L->have_events = true;
+    }
+    auto mark = [&](int i) -> hipError_t { return timed ? hipEventRecord(L->ev[i], s) : hipSuccess; };
+    HIP_TRY(ctx, mark(0));
+
+    const int nb = (T + kRouterTokens - 1) / kRouterTokens;
+    const int tile_m = kGenericTileM;
+    L->kernel_name = "generic";
+
+    RouterArgs ra{x, (const float*)L->router.p, router_bias, valid, T, d, E, k,
+                  (float*)L->P.p, (float*)L->lse.p, (int*)L->expert_of.p, (float*)L->gate_of.p,
+                  (int*)L->rank_in_block.p, (int*)L->blockcnt.p, (float*)L->partial.p};
+    HIP_TRY(ctx, launch_router(ra, abf, s));
+    HIP_TRY(ctx, mark(1));
+
+    ScanArgs sa{(const int*)L->blockcnt.p, (int*)L->blockbase.p, (const float*)L->partial.p, nb, E, k,
+                c.aux_loss_weight, c.router_z_loss_weight, tile_m, (int*)L->counts.p, (int*)L->offsets.p,
+                (int*)L->tile_expert.p, (int*)L->tile_row0.p, (int*)L->tile_rows.p, (int*)L->ntiles.p,
+                (float*)L->losses.p, (float*)L->mass.p};
+    HIP_TRY(ctx, launch_scan(sa, s));
+    HIP_TRY(ctx, mark(2));
+
+    DispatchArgs da{x, (const int*)L->expert_of.p, (const int*)L->rank_in_block.p, (const int*)L->blockbase.p,
+                    (const int*)L->offsets.p, T, d, E, k, (int*)L->perm_slot.p, (int*)L->perm_token.p,
+                    (int*)L->inv_pos.p, L->xg.p};
+    HIP_TRY(ctx, launch_dispatch(da, abf, s));
+    HIP_TRY(ctx, mark(3));
+
+    const int max_tiles = T > 0 ? (T * k) / tile_m + E : 0;
+    GroupedArgs g1{};
+    g1.a = L->xg.p;
+    g1.row_index = nullptr;
+    g1.w = L->wgu.p;
+    g1.w_expert_stride = (size_t)2 * F * d;
+    g1.scales = wk == WeightKind::I8 ? (const float*)L->sgu.p : nullptr;
+    g1.s_expert_stride = (size_t)2 * F;
+    g1.N = F;
+    g1.K = d;
+    g1.tile_expert = (const int*)L->tile_expert.p;
+    g1.tile_row0 = (const int*)L->tile_row0.p;
+    g1.tile_rows = (const int*)L->tile_rows.p;
+    g1.ntiles = (const int*)L->ntiles.p;
+    g1.max_tiles = max_tiles;
+    g1.dense_rows = -1;
+    g1.out = L->h.p;
+    g1.swiglu = true;
+    HIP_TRY(ctx, launch_grouped_generic(g1, abf, wk, tile_m, s));
+    HIP_TRY(ctx, mark(4));
+
+    GroupedArgs g2 = g1;
+    g2.a = L->h.p;
+    g2.w = L->wd.p;
+    g2.w_expert_stride = (size_t)d * F;
+    g2.scales = wk == WeightKind::I8 ? (const float*)L->sd.p : nullptr;
+    g2.s_expert_stride = (size_t)d;
+    g2.N = d;
+    g2.K = F;
+    g2.out = L->y.p;
+    g2.swiglu = false;
+    HIP_TRY(ctx, launch_grouped_generic(g2, abf, wk, tile_m, s));
+    HIP_TRY(ctx, mark(5));
+
+    if (c.shared_expert && T > 0) {
+        GroupedArgs s1 = g1;
+        s1.a = x;
+        s1.w = L->swgu.p;
+        s1.w_expert_stride = 0;
+        s1.scales = wk == WeightKind::I8 ? (const float*)L->ssgu.p : nullptr;
+        s1.s_expert_stride = 0;
+        s1.N = Fs;
+        s1.K = d;
+        s1.dense_rows = T;
+        s1.out = L->hs.p;
+        HIP_TRY(ctx, launch_grouped_generic(s1, abf, wk, tile_m, s));
+        GroupedArgs s2 = s1;
+        s2.a = L->hs.p;
+        s2.w = L->swd.p;
+        s2.scales = wk == WeightKind::I8 ? (const float*)L->ssd.p : nullptr;
+        s2.N = d;
+        s2.K = Fs;
+        s2.out = L->ys.p;
+        s2.swiglu = false;
+        HIP_TRY(ctx, launch_grouped_generic(s2, abf, wk, tile_m, s));
+    }
+    HIP_TRY(ctx, mark(6));
+
+    CombineArgs ca{L->y.p, c.shared_expert ? L->ys.p : nullptr, residual, (const int*)L->inv_pos.p,
+                   (const float*)L->gate_of.p, T, d, k, out};
+    HIP_TRY(ctx, launch_combine(ca, abf, s));
+    HIP_TRY(ctx, mark(7));
+    L->last_T = T;
+    return RBMOE_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rbmoe_forward(rbmoe_layer* L, const void* x, int32_t T, int32_t cols, const uint8_t* valid,
+                  const float* router_bias, const void* residual, void* out) {
+    return forward_impl(L, x, T, cols, valid, router_bias, residual, out, false);
+}
+
+int rbmoe_forward_timed(rbmoe_layer* L, const void* x, int32_t T, int32_t cols, const uint8_t* valid,
+                        const float* router_bias, const void* residual, void* out, float* ms) {
+    if (!ms) return fail(L ? L->ctx : nullptr, RBMOE_NULL_POINTER, "ms is NULL");
+    int rc = forward_impl(L, x, T, cols, valid, router_bias, residual, out, true);
+    if (rc != RBMOE_OK) return rc;
+    rbmoe_ctx* ctx = L->ctx;
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    for (int i = 0; i < RBMOE_NUM_STAGES - 1; ++i)
+        HIP_TRY(ctx, hipEventElapsedTime(&ms[i], L->ev[i], L->ev[i + 1]));
+    HIP_TRY(ctx, hipEventElapsedTime(&ms[RBMOE_STAGE_TOTAL], L->ev[0], L->ev[RBMOE_NUM_STAGES - 1]));
+    return RBMOE_OK;
+}
+
+int rbmoe_forward_host(rbmoe_layer* L, const void* x, int32_t T, int32_t cols, const uint8_t* valid,
+                       const float* router_bias, const void* residual, void* out) {
+    if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
+    rbmoe_ctx* ctx = L->ctx;
+    const rbmoe_config& c = L->cfg;
+    if (cols != c.d_model) {
+        char buf[120];
+        std::snprintf(buf, sizeof buf, "input length %d does not match expected length %d", cols, c.d_model);
+        return fail(ctx, RBMOE_INVALID_INPUT, buf);
+    }
+    if (T < 0 || T > L->max_T) return fail(ctx, RBMOE_INVALID_INPUT, "token count outside [0, max_tokens]");
+    if (T > 0 && (!x || !out)) return fail(ctx, RBMOE_NULL_POINTER, "x or out is NULL");
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    const size_t as = dtype_size(c.act_dtype);
+    const size_t nbytes = (size_t)T * c.d_model * as;
+    hipStream_t s = ctx->stream;
+    if (T > 0) {
+        HIP_TRY(ctx, hipMemcpyAsync(L->st_x.p, x, nbytes, hipMemcpyHostToDevice, s));
+        if (valid) HIP_TRY(ctx, hipMemcpyAsync(L->st_valid.p, valid, (size_t)T, hipMemcpyHostToDevice, s));
+        if (residual) HIP_TRY(ctx, hipMemcpyAsync(L->st_res.p, residual, nbytes, hipMemcpyHostToDevice, s));
+    }
+    if (router_bias)
+        HIP_TRY(ctx, hipMemcpyAsync(L->st_bias.p, router_bias, (size_t)c.num_experts * 4, hipMemcpyHostToDevice, s));
+    int rc = forward_impl(L, L->st_x.p, T, cols, valid ? (const uint8_t*)L->st_valid.p : nullptr,
+                          router_bias ? (const float*)L->st_bias.p : nullptr, residual ? L->st_res.p : nullptr,
+                          L->st_out.p, false);
+    if (rc != RBMOE_OK) return rc;
+    if (T > 0) HIP_TRY(ctx, hipMemcpyAsync(out, L->st_out.p, nbytes, hipMemcpyDeviceToHost, s));
+    HIP_TRY(ctx, hipStreamSynchronize(s));
+    return RBMOE_OK;
+}
+
+int rbmoe_get_losses(rbmoe_layer* L, float* aux_loss, float* z_loss) {
+    if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
+    rbmoe_ctx* ctx = L->ctx;
+    if (L->last_T < 0) return fail(ctx, RBMOE_INVALID_INPUT, "no forward pass has run yet");
+    float v[2] = {0.f, 0.f};
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    HIP_TRY(ctx, hipMemcpy(v, L->losses.p, 8, hipMemcpyDeviceToHost));
+    if (aux_loss) *aux_loss = v[0];
+    if (z_loss) *z_loss = v[1];
+    return RBMOE_OK;
+}
+
+int rbmoe_get_routing(rbmoe_layer* L, rbmoe_routing* r) {
+    if (!L || !r) return fail(L ? L->ctx : nullptr, RBMOE_NULL_POINTER, "layer or routing is NULL");
+    rbmoe_ctx* ctx = L->ctx;
+    if (L->last_T < 0) return fail(ctx, RBMOE_INVALID_INPUT, "no forward pass has run yet");
+    const int T = L->last_T, E = L->cfg.num_experts, k = L->cfg.experts_per_token;
+    const size_t S = (size_t)T * k;
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    if (r->counts) HIP_TRY(ctx, hipMemcpy(r->counts, L->counts.p, (size_t)E * 4, hipMemcpyDeviceToHost));
+    if (r->offsets) HIP_TRY(ctx, hipMemcpy(r->offsets, L->offsets.p, (size_t)(E + 1) * 4, hipMemcpyDeviceToHost));
+    if (S == 0) return RBMOE_OK;
+    if (r->expert_of) HIP_TRY(ctx, hipMemcpy(r->expert_of, L->expert_of.p, S * 4, hipMemcpyDeviceToHost));
+    if (r->gate_of) HIP_TRY(ctx, hipMemcpy(r->gate_of, L->gate_of.p, S * 4, hipMemcpyDeviceToHost));
+    if (r->perm_slot) HIP_TRY(ctx, hipMemcpy(r->perm_slot, L->perm_slot.p, S * 4, hipMemcpyDeviceToHost));
+    if (r->perm_token) HIP_TRY(ctx, hipMemcpy(r->perm_token, L->perm_token.p, S * 4, hipMemcpyDeviceToHost));
+    if (r->probabilities)
+        HIP_TRY(ctx, hipMemcpy(r->probabilities, L->P.p, (size_t)T * E * 4, hipMemcpyDeviceToHost));
+    if (r->log_sum_exp) HIP_TRY(ctx, hipMemcpy(r->log_sum_exp, L->lse.p, (size_t)T * 4, hipMemcpyDeviceToHost));
+    return RBMOE_OK;
+}
+
+int rbmoe_get_expert_rows(rbmoe_layer* L, float* hidden, float* expert_out) {
+    if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
+    rbmoe_ctx* ctx = L->ctx;
+    if (L->last_T < 0) return fail(ctx, RBMOE_INVALID_INPUT, "no forward pass has run yet");
+    const int E = L->cfg.num_experts, d = L->cfg.d_model, F = L->cfg.d_ff;
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    int R = 0;
+    HIP_TRY(ctx, hipMemcpy(&R, static_cast<int*>(L->offsets.p) + E, 4, hipMemcpyDeviceToHost));
+    const bool abf = L->cfg.act_dtype == RBMOE_BF16;
+    auto fetch = [&](float* dst, const Buf& src, size_t n) -> int {
+        if (!dst || n == 0) return RBMOE_OK;
+        if (!abf) {
+            HIP_TRY(ctx, hipMemcpy(dst, src.p, n * 4, hipMemcpyDeviceToHost));
+            return RBMOE_OK;
+        }
+        std::vector<uint16_t> tmp(n);
+        HIP_TRY(ctx, hipMemcpy(tmp.data(), src.p, n * 2, hipMemcpyDeviceToHost));
+        for (size_t i = 0; i < n; ++i) dst[i] = host_bf16_to_f32(tmp[i]);
+        return RBMOE_OK;
+    };
+    int rc = fetch(hidden, L->h, (size_t)R * F);
+    if (rc != RBMOE_OK) return rc;
+    return fetch(expert_out, L->y, (size_t)R * d);
+}
+
+const char* rbmoe_expert_kernel_name(const rbmoe_layer* L) { return L ? L->kernel_name : "none"; }
+
+int rbmoe_device_alloc(rbmoe_ctx* ctx, size_t bytes, void** out) {
+    if (!ctx || !out) return fail(ctx, RBMOE_NULL_POINTER, "ctx or out is NULL");
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    HIP_TRY(ctx, hipMalloc(out, bytes ? bytes : 1));
+    return RBMOE_OK;
+}
+
+int rbmoe_device_free(rbmoe_ctx* ctx, void* ptr) {
+    if (!ctx) return fail(nullptr, RBMOE_NULL_POINTER, "ctx is NULL");
+    if (ptr) HIP_TRY(ctx, hipFree(ptr));
+    return RBMOE_OK;
+}
+
+int rbmoe_copy_to_device(rbmoe_ctx* ctx, void* dst, const void* src, size_t bytes) {
+    if (!ctx) return fail(nullptr, RBMOE_NULL_POINTER, "ctx is NULL");
+    if (bytes == 0) return RBMOE_OK;
+    if (!dst || !src) return fail(ctx, RBMOE_NULL_POINTER, "dst or src is NULL");
+    HIP_TRY(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return RBMOE_OK;
+}
+
+int rbmoe_copy_to_host(rbmoe_ctx* ctx, void* dst, const void* src, size_t bytes) {
+    if (!ctx) return fail(nullptr, RBMOE_NULL_POINTER, "ctx is NULL");
+    if (bytes == 0) return RBMOE_OK;
+    if (!dst || !src) return fail(ctx, RBMOE_NULL_POINTER, "dst or src is NULL");
+    HIP_TRY(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return RBMOE_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,116 @@
+// Device-side helpers shared by the gfx950 kernels: element types, bf16
+// conversion and the fixed-sequence exp/log the router uses.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace rbmoe {
+
+constexpr int kWave = 64;
+
+// Raw bf16 storage.  Values are converted explicitly so that the rounding rule
+// (nearest even on the bit pattern) is visible and identical everywhere.
+struct bf16_t {
+    uint16_t bits;
+};
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16_t v) { return __uint_as_float((uint32_t)v.bits << 16); }
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
+
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+    uint32_t b = __float_as_uint(f);
+    if ((b & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((b >> 16) | 0x0040u);
+    b += 0x7fffu + ((b >> 16) & 1u);
+    return (uint16_t)(b >> 16);
+}
+
+template <typename T>
+__device__ __forceinline__ T from_f32(float v);
+template <>
+__device__ __forceinline__ float from_f32<float>(float v) {
+    return v;
+}
+template <>
+__device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) {
+    return bf16_t{f32_to_bf16_bits(v)};
+}
+
+// ---------------------------------------------------------------------------
+// exp and log as fixed sequences of binary32 operations (Cephes expf/logf).
+// Every step is either one fused multiply-add (__fmaf_rn) or one correctly
+// rounded multiply/add (__fmul_rn/__fadd_rn), so the compiler cannot reorder
+// or contract them and the result is the same on any IEEE-754 machine that
+// runs the same sequence.  Softmax probabilities and the log-sum-exp depend on
+// these bit for bit, and routing depends on the probabilities.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float rb_expf(float x) {
+    if (x != x) return x;
+    if (x > 88.72283935546875f) return __uint_as_float(0x7f800000u);
+    if (x < -103.97208404541015625f) return 0.0f;
+    const float t = __fmul_rn(x, 1.44269502162933349609375f);
+    const float kf = rintf(t);
+    float r = __fmaf_rn(kf, -0.693145751953125f, x);
+    r = __fmaf_rn(kf, -1.428606765330187045037746429443359375e-6f, r);
+    float p = 1.9875691500e-4f;
+    p = __fmaf_rn(p, r, 1.3981999507e-3f);
+    p = __fmaf_rn(p, r, 8.3334519073e-3f);
+    p = __fmaf_rn(p, r, 4.1665795894e-2f);
+    p = __fmaf_rn(p, r, 1.6666665459e-1f);
+    p = __fmaf_rn(p, r, 5.0000001201e-1f);
+    const float r2 = __fmul_rn(r, r);
+    p = __fmaf_rn(p, r2, r);
+    p = __fadd_rn(p, 1.0f);
+    const int k = (int)kf;
+    const int k1 = k / 2;
+    const int k2 = k - k1;
+    const float s1 = __uint_as_float((uint32_t)(k1 + 127) << 23);
+    const float s2 = __uint_as_float((uint32_t)(k2 + 127) << 23);
+    return __fmul_rn(__fmul_rn(p, s1), s2);
+}
+
+__device__ __forceinline__ float rb_logf(float x) {
+    if (x != x) return x;
+    if (x < 0.0f) return __uint_as_float(0x7fc00000u);
+    if (x == 0.0f) return __uint_as_float(0xff800000u);
+    if (__float_as_uint(x) == 0x7f800000u) return x;
+    int e = 0;
+    uint32_t b = __float_as_uint(x);
+    if (b < 0x00800000u) {
+        x = __fmul_rn(x, 8388608.0f);
+        b = __float_as_uint(x);
+        e = -23;
+    }
+    e += (int)(b >> 23) - 126;
+    float m = __uint_as_float((b & 0x007fffffu) | 0x3f000000u);
+    if (m < 0.707106769084930419921875f) {
+        e -= 1;
+        m = __fadd_rn(__fadd_rn(m, m), -1.0f);
+    } else {
+        m = __fadd_rn(m, -1.0f);
+    }
+    const float z = __fmul_rn(m, m);
+    float y = 7.0376836292e-2f;
+    y = __fmaf_rn(y, m, -1.1514610310e-1f);
+    y = __fmaf_rn(y, m, 1.1676998740e-1f);
+    y = __fmaf_rn(y, m, -1.2420140846e-1f);
+    y = __fmaf_rn(y, m, 1.4249322787e-1f);
+    y = __fmaf_rn(y, m, -1.6668057665e-1f);
+    y = __fmaf_rn(y, m, 2.0000714765e-1f);
+    y = __fmaf_rn(y, m, -2.4999993993e-1f);
+    y = __fmaf_rn(y, m, 3.3333331174e-1f);
+    y = __fmul_rn(__fmul_rn(y, m), z);
+    const float fe = (float)e;
+    y = __fmaf_rn(-2.12194440e-4f, fe, y);
+    y = __fmaf_rn(-0.5f, z, y);
+    float r = __fadd_rn(m, y);
+    r = __fmaf_rn(0.693359375f, fe, r);
+    return r;
+}
+
+// silu(x) = x * (1 / (1 + exp(-x))), the reference's operation order
+// (src/ffn.rs:223-229).  Tolerance-checked, so the fast exponential is used.
+__device__ __forceinline__ float silu_f32(float x) { return x * (1.0f / (1.0f + __expf(-x))); }
+
+}  // namespace rbmoe

@@ -1,0 +1,115 @@
+// Launch interfaces between the C ABI (rbmoe_api.hip) and the kernel files.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "rbmoe_device.h"
+
+namespace rbmoe {
+
+// Tokens owned by one router / dispatch block.  Slots are numbered
+// token * k + rank, so a block owns a contiguous slot range.
+constexpr int kRouterTokens = 32;
+
+// Largest expert count and top-k the routing kernels are laid out for.
+constexpr int kMaxExperts = 256;
+constexpr int kMaxTopK = 32;
+
+size_t router_lds_bytes(int E, int k);
+size_t scan_lds_bytes(int E);
+
+struct RouterArgs {
+    const void* x;       // [T, d] f32 or bf16
+    const float* wr;     // [E, d] f32
+    const float* bias;   // [E] or null
+    const uint8_t* valid;  // [T] or null
+    int T, d, E, k;
+    float* P;            // [T, E]
+    float* lse;          // [T]
+    int* expert_of;      // [T*k]
+    float* gate_of;      // [T*k]
+    int* rank_in_block;  // [T*k]
+    int* blockcnt;       // [nb, E]
+    float* partial;      // [nb, E+1]
+};
+hipError_t launch_router(const RouterArgs& a, bool bf16, hipStream_t s);
+
+struct ScanArgs {
+    const int* blockcnt;  // [nb, E]
+    int* blockbase;       // [nb, E]
+    const float* partial; // [nb, E+1]
+    int nb, E, k;
+    float w_aux, w_z;
+    int tile_m;
+    int* counts;       // [E]
+    int* offsets;      // [E+1]
+    int* tile_expert;  // [max_tiles]
+    int* tile_row0;
+    int* tile_rows;
+    int* ntiles;       // [1]
+    float* losses;     // [2]
+    float* mass;       // [E+1] or null: sum of probabilities per expert, sum of lse^2
+};
+hipError_t launch_scan(const ScanArgs& a, hipStream_t s);
+
+struct DispatchArgs {
+    const void* x;
+    const int* expert_of;
+    const int* rank_in_block;
+    const int* blockbase;
+    const int* offsets;
+    int T, d, E, k;
+    int* perm_slot;
+    int* perm_token;
+    int* inv_pos;
+    void* xg;  // [T*k, d] or null (rows are then gathered by the consumer)
+};
+hipError_t launch_dispatch(const DispatchArgs& a, bool bf16, hipStream_t s);
+
+struct CombineArgs {
+    const void* y;        // [R, d] expert output rows, activation dtype
+    const void* yshared;  // [T, d] or null
+    const void* residual; // [T, d] or null
+    const int* inv_pos;   // [T*k]
+    const float* gate_of; // [T*k]
+    int T, d, k;
+    void* out;            // [T, d]
+};
+hipError_t launch_combine(const CombineArgs& a, bool bf16, hipStream_t s);
+
+// ---------------------------------------------------------------------------
+// Grouped expert products.  Rows of `a` are grouped by expert through the tile
+// table written by the scan kernel; a tile never spans two experts.
+//   out[row, n] = sum_c a[row, c] * w[expert][n, c]        (SWIGLU = false)
+//   out[row, n] = silu(a . wg[n]) * (a . wu[n])            (SWIGLU = true; the
+//       expert's weight block holds the F gate rows, then the F up rows)
+// int8 weights carry one f32 scale per weight row; the product is
+// (sum_c a*q) * scale as in the reference (src/quantized.rs:55-62).
+// ---------------------------------------------------------------------------
+enum class WeightKind : int { F32 = 0, BF16 = 1, I8 = 2 };
+
+struct GroupedArgs {
+    const void* a;          // [rows, K] activation dtype
+    const int* row_index;   // null: row r of a tile is a[row0 + r]; else a[row_index[row0 + r]]
+    const void* w;          // expert 0's weight block
+    size_t w_expert_stride; // elements between experts
+    const float* scales;    // int8: expert 0's scales, one per weight row
+    size_t s_expert_stride;
+    int N;                  // output columns (F for SWIGLU, d for the down product)
+    int K;
+    const int* tile_expert;
+    const int* tile_row0;
+    const int* tile_rows;
+    const int* ntiles;
+    int max_tiles;
+    int dense_rows;         // >= 0: one group of this many rows, no tile table (shared expert)
+    void* out;              // [rows, N] activation dtype
+    bool swiglu;
+};
+hipError_t launch_grouped_generic(const GroupedArgs& a, bool act_bf16, WeightKind wk, int tile_m,
+                                  hipStream_t s);
+constexpr int kGenericTileM = 16;
+
+}  // namespace rbmoe

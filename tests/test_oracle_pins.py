@@ -1,0 +1,411 @@
+"""Pins the CPU oracle (oracle/rb_oracle.cpp) before anything trusts it.
+
+Each check is either a vector or known answer the reference's own tests hold
+(cited), a closed form, an invariant, or a brute-force / float64 evaluation on a
+small input — chosen so that a dropped term, a wrong index or a wrong order
+fails.  No GPU is involved.
+"""
+import numpy as np
+import pytest
+
+from conftest import rel_l2
+from helpers import f64_layer_forward, oracle_layer, small_workload
+from oracle import rb_oracle as orc
+from rustingbrain_amd import synth
+
+
+def ulp_diff(a, b):
+    ai = np.asarray(a, np.float32).view(np.int32).astype(np.int64)
+    bi = np.asarray(b, np.float32).view(np.int32).astype(np.int64)
+    return np.abs(ai - bi)
+
+
+# ------------------------------------------------------------------ exp / log
+def test_expf_within_one_ulp_of_float64_exp():
+    x = np.linspace(-103.9, 88.7, 400001, dtype=np.float32)
+    ref = np.exp(x.astype(np.float64))
+    with np.errstate(over="ignore"):
+        ref32 = ref.astype(np.float32)
+    m = np.isfinite(ref32) & (ref32 > 0)
+    assert ulp_diff(orc.expf_array(x)[m], ref32[m]).max() <= 1
+
+
+def test_expf_special_values():
+    assert orc.expf(0.0) == 1.0
+    assert orc.expf(-1000.0) == 0.0
+    assert orc.expf(1000.0) == float("inf")
+    assert np.isnan(orc.expf(float("nan")))
+    assert orc.expf(float("-inf")) == 0.0
+    # a subnormal result keeps its value instead of flushing to zero
+    assert abs(orc.expf(-100.0) - np.exp(-100.0)) < 2e-45
+
+
+def test_logf_within_one_ulp_of_float64_log():
+    x = np.exp(np.linspace(-100, 88, 400001)).astype(np.float32)
+    assert ulp_diff(orc.logf_array(x), np.log(x.astype(np.float64)).astype(np.float32)).max() <= 1
+    x = np.linspace(0.5, 300, 200001, dtype=np.float32)  # the range a softmax denominator lives in
+    assert ulp_diff(orc.logf_array(x), np.log(x.astype(np.float64)).astype(np.float32)).max() <= 1
+
+
+def test_logf_special_values():
+    assert orc.logf(1.0) == 0.0
+    assert orc.logf(0.0) == float("-inf")
+    assert np.isnan(orc.logf(-1.0))
+    assert orc.logf(float("inf")) == float("inf")
+
+
+# ------------------------------------------------------------------ products
+def test_linear_reproduces_the_reference_exact_integer_product():
+    # reference src/matrix.rs:304-312: [[1,2,3],[4,5,6]] . [[7,8],[9,10],[11,12]] = [[58,64],[139,154]].
+    # Our product takes the right operand transposed ([out, in]), so pass its transpose.
+    left = np.array([[1, 2, 3], [4, 5, 6]], np.float32)
+    right = np.array([[7, 8], [9, 10], [11, 12]], np.float32)
+    want = np.array([[58, 64], [139, 154]], np.float32)
+    for plain in (False, True):
+        assert np.array_equal(orc.linear(left, np.ascontiguousarray(right.T), plain=plain), want)
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 1, 1), (3, 7, 5), (9, 16, 2), (5, 37, 11), (64, 100, 33)])
+def test_linear_matches_float64_matmul(M, K, N):
+    x = synth.normal((M, K), 1.0, 1, 1)
+    w = synth.normal((N, K), 1.0, 1, 2)
+    ref = x.astype(np.float64) @ w.astype(np.float64).T
+    assert rel_l2(orc.linear(x, w), ref) < 1e-6
+    assert rel_l2(orc.linear(x, w, plain=True), ref) < 1e-6
+
+
+def test_dot8_follows_the_eight_lane_order_of_the_reference():
+    # Exact small integers: any order gives the same answer.
+    a = np.arange(1, 20, dtype=np.float32)
+    b = np.arange(2, 21, dtype=np.float32)
+    assert orc.dot8(a, b) == float(np.dot(a.astype(np.float64), b.astype(np.float64)))
+    # Order-sensitive vector.  lane 0 holds 2^24; columns 1 and 9 (both lane 1)
+    # hold 1.  The eight-lane order adds 1 + 1 first, so 2 survives: 2^24 + 2.
+    # A single running sum in index order loses both ones: 2^24.
+    b = np.zeros(16, np.float32)
+    b[0], b[1], b[9] = 2.0 ** 24, 1.0, 1.0
+    a = np.ones(16, np.float32)
+    assert orc.dot8(a, b) == 2.0 ** 24 + 2.0
+    assert float(orc.linear(a[None], b[None], plain=True)[0, 0]) == 2.0 ** 24
+    # The tail (columns past the last multiple of 8) is summed separately and
+    # added last: 2^24 in lane 0, then three ones in the tail -> 2^24 + 3 -> rounds
+    # to 2^24 + 4 (ties to even), while adding them one at a time would stay 2^24.
+    b = np.zeros(11, np.float32)
+    b[0], b[8], b[9], b[10] = 2.0 ** 24, 1.0, 1.0, 1.0
+    assert orc.dot8(np.ones(11, np.float32), b) == 2.0 ** 24 + 4.0
+
+
+def test_dot8_rounds_the_product_before_adding():
+    # (1 + 2^-12)^2 = 1 + 2^-11 + 2^-24: the product rounds to 1 + 2^-11 before
+    # the add, so subtracting 1 + 2^-11 leaves exactly 0; a fused multiply-add
+    # would leave 2^-24.
+    v = np.float32(1.0 + 2.0 ** -12)
+    a = np.zeros(8, np.float32)
+    b = np.zeros(8, np.float32)
+    a[0], b[0] = v, v
+    a[1], b[1] = np.float32(-(1.0 + 2.0 ** -11)), np.float32(1.0)
+    assert orc.dot8(a, b) == 0.0
+
+
+def test_router_logits_shape_and_bias():
+    x = synth.normal((5, 24), 1.0, 3, 1)
+    w = synth.normal((3, 24), 1.0, 3, 2)
+    bias = np.array([0.5, -1.0, 2.0], np.float32)
+    base = orc.router_logits(x, w)
+    assert rel_l2(base, x.astype(np.float64) @ w.astype(np.float64).T) < 1e-6
+    assert np.array_equal(orc.router_logits(x, w, bias), base + bias)
+    for t in range(5):
+        for e in range(3):
+            assert base[t, e] == np.float32(orc.dot8(x[t], w[e]))
+
+
+# ------------------------------------------------------------------ softmax
+def ramp(n):  # reference src/gpu_model.rs:3775-3779
+    return np.array([((i * 37) % 23) / 11.0 - 1.0 for i in range(n)], np.float32)
+
+
+def test_softmax_rows_closed_form_on_the_reference_ramp():
+    # reference src/gpu_model.rs:4102-4110: rows sum to 1 (1e-5), lse = max + ln sum exp(v - max) (1e-5)
+    logits = ramp(4 * 5).reshape(4, 5)
+    P, lse = orc.softmax_rows(logits)
+    assert np.all(np.abs(P.sum(axis=1) - 1.0) < 1e-5)
+    l64 = logits.astype(np.float64)
+    want = l64.max(axis=1) + np.log(np.exp(l64 - l64.max(axis=1, keepdims=True)).sum(axis=1))
+    assert np.all(np.abs(lse - want) < 1e-5)
+    wantP = np.exp(l64 - want[:, None])
+    assert np.all(np.abs(P - wantP) < 1e-6)
+
+
+def test_softmax_orders_like_the_reference_activation_test():
+    # reference src/activations.rs:77-85
+    P, _ = orc.softmax_rows(np.array([[1.0, 2.0, 3.0]], np.float32))
+    assert abs(P.sum() - 1.0) < 1e-6 and P[0, 2] > P[0, 1] > P[0, 0]
+
+
+def test_softmax_ignores_a_nan_when_taking_the_maximum():
+    P, lse = orc.softmax_rows(np.array([[1.0, np.nan, 3.0]], np.float32))
+    # max ignores the NaN (3.0); the sum is NaN, `sum > 0` is false, so the row is left as
+    # exp(v - max) without the division (reference src/activations.rs:65-69)
+    assert np.isnan(lse[0]) and np.isnan(P[0, 1])
+    assert P[0, 2] == 1.0 and abs(P[0, 0] - np.exp(-2.0)) < 1e-7
+
+
+# ------------------------------------------------------------------ route
+def test_route_hand_vector_from_the_reference():
+    # reference src/moe.rs:713-723
+    P = np.array([[0.1, 0.3, 0.05, 0.5, 0.05]], np.float32)
+    e, g = orc.route(P, 2)
+    assert e.tolist() == [3, 1]
+    assert np.allclose(g, [0.5 / 0.8, 0.3 / 0.8], atol=1e-7)
+
+
+def test_route_breaks_ties_to_the_lower_index():
+    P = np.array([[0.2, 0.3, 0.3, 0.2], [0.25, 0.25, 0.25, 0.25]], np.float32)
+    e, _ = orc.route(P, 2)
+    assert e.reshape(2, 2).tolist() == [[1, 2], [0, 1]]
+    e, _ = orc.route(np.full((1, 6), 1.0 / 6, np.float32), 4)
+    assert e.tolist() == [0, 1, 2, 3]
+
+
+def test_route_on_a_nan_row_takes_experts_in_index_order():
+    # reference semantics of `row[expert] > row[best]` with NaN (src/moe.rs:566-581)
+    e, _ = orc.route(np.full((1, 5), np.nan, np.float32), 3)
+    assert e.tolist() == [0, 1, 2]
+
+
+@pytest.mark.parametrize("k", [1, 2, 3, 4])
+def test_gates_sum_to_one(k):
+    # reference src/moe.rs:726-741 (tolerance 1e-5) and :744-754 (k = 1 -> gate 1 within 1e-6)
+    P, _ = orc.softmax_rows(synth.normal((7, 4), 1.0, 3, k))
+    _, g = orc.route(P, k)
+    assert np.all(np.abs(g.reshape(7, k).sum(axis=1) - 1.0) < 1e-5)
+    if k == 1:
+        assert np.all(np.abs(g - 1.0) < 1e-6)
+
+
+def test_route_equals_stable_descending_sort_prefix():
+    # reference src/gpu_model.rs:4121-4134: selected == order[..top_k]; gates == p / sum (1e-6)
+    P, _ = orc.softmax_rows(synth.normal((200, 9), 2.0, 4, 1))
+    for k in (1, 3, 9):
+        e, g = orc.route(P, k)
+        e = e.reshape(200, k)
+        g = g.reshape(200, k)
+        order = np.argsort(-P, axis=1, kind="stable")[:, :k]
+        assert np.array_equal(e, order)
+        sel = np.take_along_axis(P, order, axis=1)
+        assert np.all(np.abs(g - sel / sel.sum(axis=1, keepdims=True)) < 1e-6)
+
+
+def test_padding_rows_are_routed_nowhere():
+    # reference src/moe.rs:559-562, device test src/gpu_model.rs:4112-4119
+    P, _ = orc.softmax_rows(ramp(4 * 5).reshape(4, 5))
+    valid = np.array([1, 1, 1, 0], np.uint8)
+    e, g = orc.route(P, 2, valid)
+    assert e[6:].tolist() == [-1, -1] and g[6:].tolist() == [0.0, 0.0]
+    assert (e[:6] >= 0).all()
+
+
+# ------------------------------------------------------------------ bucket
+def test_bucket_is_a_stable_counting_sort():
+    rng = np.random.default_rng(0)
+    for E, k, T in [(4, 2, 50), (16, 2, 333), (5, 3, 17), (3, 1, 1)]:
+        expert_of = rng.integers(0, E, size=T * k).astype(np.int32)
+        expert_of[rng.random(T * k) < 0.1] = -1
+        counts, offsets, perm_slot, perm_token = orc.bucket(expert_of, E, k)
+        routed = np.nonzero(expert_of >= 0)[0]
+        want = routed[np.argsort(expert_of[routed], kind="stable")]
+        assert np.array_equal(perm_slot, want)
+        assert np.array_equal(perm_token, want // k)
+        assert np.array_equal(counts, np.bincount(expert_of[routed], minlength=E))
+        assert np.array_equal(offsets, np.concatenate([[0], np.cumsum(counts)]))
+        for e in range(E):
+            seg = perm_slot[offsets[e]:offsets[e + 1]]
+            assert np.all(np.diff(seg) > 0)
+
+
+# ------------------------------------------------------------------ int8
+def test_q8_product_agrees_with_the_float_product_on_the_reference_vectors():
+    # reference src/quantized.rs:202-217
+    w = np.array([v * 0.37 - 2.0 for v in range(12)], np.float32).reshape(3, 4)
+    x = np.array([0.5, -1.5, 2.0, 0.25, 1.0, 1.0, -1.0, 0.0], np.float32).reshape(2, 4)
+    want = orc.linear(x, w, plain=True)
+    for mode in (0, 1):
+        q, s = orc.q8_quantize(w, mode)
+        got = orc.q8_linear(x, q, s)
+        assert got.shape == (2, 3)
+        assert np.all(np.abs(got - want) < 0.05)
+
+
+def test_q8_zero_row_stays_zero_and_rows_dequantize_within_a_step():
+    # reference src/quantized.rs:219-237
+    q, s = orc.q8_quantize(np.zeros((2, 3), np.float32), 0)
+    assert not q.any() and not s.any()
+    w = np.array([[0.5, -1.0, 0.25], [4.0, -2.0, 0.0]], np.float32)
+    q, s = orc.q8_quantize(w, 0)
+    assert np.all(np.abs(q[1].astype(np.float32) * s[1] - w[1]) < 4.0 / 127.0)
+    assert np.all(np.abs(q.astype(np.float32) * s[:, None] - w) <= s[:, None] / 2 + 1e-7)
+    assert q.min() >= -127 and np.abs(q).max() == 127
+
+
+def test_q8_rounds_half_away_from_zero():
+    # scale = 127/127 = 1: values x.5 must round away from zero (Rust f32::round)
+    w = np.array([[127.0, 0.5, -0.5, 1.5, -2.5, 0.49999997]], np.float32)
+    q, s = orc.q8_quantize(w, 0)
+    assert s[0] == 1.0 and q[0].tolist() == [127, 1, -1, 2, -3, 0]
+    q2, s2 = synth.quantize_rows(w)
+    assert np.array_equal(q, q2) and np.array_equal(s, s2)
+
+
+# ------------------------------------------------------------------ silu / swiglu
+def test_silu_known_points():
+    # reference src/ffn.rs:346-352
+    assert abs(orc.silu(0.0)) < 1e-6
+    assert abs(orc.silu(10.0) - 10.0) < 1e-3
+    assert abs(orc.silu(-1.0) - (-1.0 / (1.0 + np.e))) < 1e-7
+
+
+def test_swiglu_matches_float64():
+    w = small_workload(d=12, F=9, E=1, k=1, T=6)
+    t = synth.make(w)
+    layer = oracle_layer(t)
+    out, g, u, h = layer.swiglu(layer.experts[0], t.x, w.d_ff)
+    e = t.experts[0]
+    g64 = t.x.astype(np.float64) @ e["gate"].astype(np.float64).T
+    u64 = t.x.astype(np.float64) @ e["up"].astype(np.float64).T
+    h64 = g64 / (1 + np.exp(-g64)) * u64
+    assert rel_l2(g, g64) < 1e-6 and rel_l2(u, u64) < 1e-6 and rel_l2(h, h64) < 1e-6
+    assert rel_l2(out, h64 @ e["down"].astype(np.float64).T) < 1e-6
+
+
+# ------------------------------------------------------------------ auxiliary losses
+def one_hot_router(E, d, strength):  # reference src/moe.rs:678-686
+    w = np.zeros((E, d), np.float32)
+    for e in range(E):
+        w[e, e % d] = strength
+    return w
+
+
+def one_hot_rows(rows, width):  # reference src/moe.rs:688-694
+    x = np.zeros((len(rows), width), np.float32)
+    for r, c in enumerate(rows):
+        x[r, c] = 1.0
+    return x
+
+
+def tiny_layer(E, k, F, d, seed, z_w=1e-3, aux_w=0.01, strength=None):
+    t = synth.make(small_workload(d=d, E=E, k=k, F=F, T=1, seed=seed))
+    layer = oracle_layer(t, aux_w, z_w)
+    if strength is not None:
+        layer.router = one_hot_router(E, d, strength)
+    return layer
+
+
+def test_balanced_routing_reaches_the_minimum_of_the_load_balancing_loss():
+    # reference src/moe.rs:768-787
+    layer = tiny_layer(4, 1, 4, 4, 6, z_w=0.0, strength=30.0)
+    r = layer.forward(one_hot_rows([0, 1, 2, 3], 4))
+    assert abs(r.aux_loss - 0.01) < 1e-3
+    assert np.all(np.abs(r.load_fractions() - 0.25) < 1e-6)
+
+
+def test_collapsed_routing_costs_num_experts_times_the_weight():
+    # reference src/moe.rs:790-802
+    layer = tiny_layer(4, 1, 4, 4, 6, z_w=0.0, strength=30.0)
+    r = layer.forward(one_hot_rows([0, 0, 0, 0], 4))
+    assert abs(r.aux_loss - 4 * 0.01) < 1e-3 and r.aux_loss > 0.01
+    assert r.load_fractions().tolist() == [1.0, 0.0, 0.0, 0.0]
+
+
+def test_z_loss_grows_with_the_logits_and_is_zero_when_disabled():
+    # reference src/moe.rs:805-836
+    x = one_hot_rows([0, 1, 2, 3], 4)
+    quiet = tiny_layer(4, 1, 4, 4, 7, strength=1.0).forward(x).z_loss
+    loud = tiny_layer(4, 1, 4, 4, 7, strength=20.0).forward(x).z_loss
+    assert loud > quiet > 0.0
+    layer = tiny_layer(4, 2, 6, 8, 8, z_w=0.0)
+    r = layer.forward(synth.uniform((4, 8), 1.0, 8, 77))
+    assert r.z_loss == 0.0
+
+
+def test_aux_losses_match_the_closed_form_in_float64():
+    # doc comment reference src/moe.rs:595-601
+    T, E, k = 50, 6, 2
+    P, lse = orc.softmax_rows(synth.normal((T, E), 1.5, 9, 1))
+    valid = (np.arange(T) % 7 != 3).astype(np.uint8)
+    e, _ = orc.route(P, k, valid)
+    counts, _, _, _ = orc.bucket(e, E, k)
+    aux, z = orc.aux_losses(P, lse, counts, k, 0.01, 1e-3, valid)
+    V = int(valid.sum())
+    f = counts.astype(np.float64) / (V * k)
+    Pm = P[valid.astype(bool)].astype(np.float64).mean(axis=0)
+    assert abs(aux - E * float(f @ Pm) * 0.01) < 1e-7
+    assert abs(z - 1e-3 * float((lse[valid.astype(bool)].astype(np.float64) ** 2).mean())) < 1e-7
+    assert 0.01 - 1e-6 <= aux <= E * 0.01 + 1e-6
+    assert orc.aux_losses(P, lse, np.zeros(E, np.int32), k, 0.01, 1e-3, np.zeros(T, np.uint8)) == (0.0, 0.0)
+
+
+# ------------------------------------------------------------------ whole layer
+def test_every_token_reaches_exactly_top_k_experts():
+    # reference src/moe.rs:757-765
+    t = synth.make(small_workload(d=8, E=6, k=3, F=4, T=9, seed=5))
+    r = oracle_layer(t).forward(t.x)
+    assert int(r.counts.sum()) == 9 * 3 and r.out.shape == (9, 8)
+
+
+def test_wrong_width_is_invalid_input():
+    # reference src/moe.rs:248-253
+    t = synth.make(small_workload())
+    with pytest.raises(ValueError, match="InvalidInput"):
+        oracle_layer(t).forward(np.zeros((3, 5), np.float32))
+
+
+@pytest.mark.parametrize("shared,k,wt", [(False, 2, "f32"), (True, 2, "f32"), (True, 3, "f32"), (False, 2, "int8")])
+def test_layer_output_matches_float64_given_the_same_routing(shared, k, wt):
+    w = small_workload(d=16, E=5, k=k, F=12, T=23, seed=21, shared=shared, shared_d_ff=20 if shared else 0, wt=wt)
+    t = synth.make(w)
+    valid = (np.arange(23) % 5 != 2).astype(np.uint8)
+    r = oracle_layer(t).forward(t.x, valid=valid, threads=3)
+    want = f64_layer_forward(t, routing=(r.expert_of, r.gate_of))
+    assert rel_l2(r.out, want) < 1e-6
+    # one thread and several threads agree bit for bit (work is split by rows)
+    r1 = oracle_layer(t).forward(t.x, valid=valid, threads=1)
+    assert np.array_equal(r.out, r1.out)
+    # padding rows are routed nowhere: without a shared expert they come out zero
+    if not shared:
+        assert not r.out[valid == 0].any()
+
+
+def test_top_one_with_a_one_hot_router_returns_that_experts_swiglu():
+    E, d, F = 4, 4, 5
+    t = synth.make(small_workload(d=d, E=E, k=1, F=F, T=1, seed=31))
+    layer = oracle_layer(t)
+    layer.router = one_hot_router(E, d, 30.0)
+    x = one_hot_rows([2, 0, 3, 1, 2], d)
+    r = layer.forward(x)
+    assert r.expert_of.tolist() == [2, 0, 3, 1, 2]
+    for tok, e in enumerate(r.expert_of):
+        want, _, _, _ = layer.swiglu(layer.experts[e], x[tok:tok + 1], F)
+        assert np.array_equal(r.out[tok], (r.gate_of[tok] * want[0]).astype(np.float32))
+
+
+def test_the_shared_expert_changes_every_token():
+    # reference src/moe.rs:839-859
+    t_plain = synth.make(small_workload(d=8, E=4, k=1, F=6, T=4, seed=9))
+    t_shared = synth.make(small_workload(d=8, E=4, k=1, F=6, T=4, seed=9, shared=True))
+    a = oracle_layer(t_plain).forward(t_plain.x).out
+    b = oracle_layer(t_shared).forward(t_shared.x).out
+    assert np.all(np.any(np.abs(a - b) > 1e-6, axis=1))
+
+
+def test_identical_tokens_collapse_onto_exactly_two_experts():
+    # reference tutorials/15_mixture_of_experts.md:310-312: 50% / 50% and E - 2 dead experts
+    t = synth.make(small_workload(d=64, E=8, k=2, F=32, T=1, seed=7))
+    x = np.repeat(synth.uniform((1, 64), 1.0, 7, 5), 512, axis=0)
+    r = oracle_layer(t).forward(x)
+    loads = sorted(r.load_fractions().tolist())
+    assert loads == [0.0] * 6 + [0.5, 0.5]
+
+
+def test_near_tie_census_counts_only_close_calls():
+    P = np.array([[0.5, 0.25, 0.25], [0.5, 0.3, 0.2]], np.float32)
+    assert orc.near_ties(P, 2, 4) == 1 and orc.near_ties(P, 1, 4) == 0
