@@ -1,0 +1,210 @@
+#!/usr/bin/env python3
+"""Benchmark of the mixture-of-experts layer forward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A step is one forward pass of the layer (router, dispatch, grouped SwiGLU expert
+products, combine, auxiliary losses) over one batch of seeded synthetic tokens
+already resident in HBM.  Prints ONE JSON line: tokens/s for the whole layer, the
+roofline of the dominant kernel (the grouped gate/up product) measured with HIP
+events on the library's stream, per-stage figures, and the CPU restatement of
+the reference's rayon path timed on this machine's host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+import rustingbrain_amd as rb  # noqa: E402
+from rustingbrain_amd import _lib as L  # noqa: E402
+from rustingbrain_amd import synth  # noqa: E402
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_F32_TFLOPS = 157.3     # MI355X fp32 matrix
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+
+class DeviceBuffer:
+    def __init__(self, dev: rb.Device, nbytes: int):
+        self.dev, self.nbytes = dev, nbytes
+        p = C.c_void_p()
+        rc = dev._lib.rbmoe_device_alloc(dev.handle, nbytes, C.byref(p))
+        if rc != L.OK:
+            raise RuntimeError(dev._lib.rbmoe_last_error(dev.handle).decode())
+        self.ptr = p.value
+
+    def upload(self, a: np.ndarray) -> "DeviceBuffer":
+        a = np.ascontiguousarray(a)
+        assert a.nbytes <= self.nbytes
+        rc = self.dev._lib.rbmoe_copy_to_device(self.dev.handle, C.c_void_p(self.ptr), a.ctypes.data_as(C.c_void_p),
+                                                a.nbytes)
+        assert rc == L.OK
+        return self
+
+    def download(self, a: np.ndarray) -> np.ndarray:
+        rc = self.dev._lib.rbmoe_copy_to_host(self.dev.handle, a.ctypes.data_as(C.c_void_p), C.c_void_p(self.ptr),
+                                              a.nbytes)
+        assert rc == L.OK
+        return a
+
+    def free(self):
+        if self.ptr:
+            self.dev._lib.rbmoe_device_free(self.dev.handle, C.c_void_p(self.ptr))
+            self.ptr = None
+
+
+def algorithmic(w: synth.Workload, T: int, routed: int, touched_experts: int) -> dict:
+    """Algorithmic flops / bytes per launch of each stage (padding and recomputation never count)."""
+    d, F, E, k = w.d_model, w.d_ff, w.num_experts, w.experts_per_token
+    Fs = w.shared_d_ff if w.shared_expert else 0
+    sa = 2 if w.act_dtype == "bf16" else 4
+    sw = {"f32": 4, "bf16": 2, "int8": 1}[w.weight_dtype]
+    S = routed
+    return {
+        "router_bytes": T * d * sa + E * d * 4 + T * k * 8,
+        "dispatch_bytes": T * d * sa + S * 4 + S * d * sa + S * 4,
+        "combine_bytes": S * d * sa + 2 * S * 4 + T * d * sa,
+        "gate_up_flops": 4 * d * F * S,
+        "down_flops": 2 * d * F * S,
+        "shared_flops": 6 * d * Fs * T,
+        "gemm_flops": 6 * d * F * S + 6 * d * Fs * T,
+        "layer_bytes_decode": touched_experts * 3 * d * F * sw + 3 * d * Fs * sw + E * d * 4 + 2 * T * d * sa + S * 8,
+    }
+
+
+def cpu_baseline(t: synth.Tensors, budget_s: float = 20.0) -> dict:
+    """The CPU restatement of the reference's rayon path (oracle/, C++), timed
+    on the host cores of this machine.  Only this function touches oracle/."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from helpers import oracle_layer
+    threads = max(1, min(16, os.cpu_count() or 1))
+    layer = oracle_layer(t)
+    T = t.x.shape[0]
+    layer.forward(t.x, router_bias=t.router_bias, threads=threads)  # warm-up
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while len(times) < 20 and (time.perf_counter() < t_end or len(times) < 2):
+        t0 = time.perf_counter()
+        layer.forward(t.x, router_bias=t.router_bias, threads=threads)
+        times.append(time.perf_counter() - t0)
+    best = float(np.median(times))
+    return {"value": T / best, "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": f"whole workload ({T} tokens), median of {len(times)} forwards after 1 warm-up; "
+                      "C++ restatement of the reference's rayon path, not the Rust binary",
+            "ms_per_forward": best * 1e3}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="c3_prefill_d768_e16", choices=list(synth.WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        return 2
+
+    w = synth.WORKLOADS[args.workload]
+    t = synth.make(w)
+    T = w.tokens
+    dev = rb.Device.open(0)
+    cfg = rb.MoeConfig(w.num_experts, w.experts_per_token, w.d_ff, w.shared_expert)
+    layer = rb.MoeLayer(w.d_model, cfg, dev, act_dtype=w.act_dtype, weight_dtype=w.weight_dtype, max_tokens=T,
+                        shared_d_ff=w.shared_d_ff if w.shared_expert else 0)
+    layer.load_tensors(t)
+
+    bf16 = w.act_dtype == "bf16"
+    xh = synth.f32_to_bf16_bits(t.x) if bf16 else t.x
+    x = DeviceBuffer(dev, xh.nbytes).upload(xh)
+    out = DeviceBuffer(dev, xh.nbytes)
+    bias = DeviceBuffer(dev, 4 * w.num_experts).upload(t.router_bias) if t.router_bias is not None else None
+    bp = bias.ptr if bias else 0
+
+    for _ in range(args.warmup):
+        layer.forward_device(x.ptr, T, out.ptr, bias_ptr=bp)
+    dev.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        layer.forward_device(x.ptr, T, out.ptr, bias_ptr=bp)
+    dev.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+
+    # per-stage durations from HIP events on the library's stream
+    nprof = max(10, min(100, args.steps))
+    acc = {}
+    for _ in range(nprof):
+        st = layer.forward_timed(x.ptr, T, out.ptr, bias_ptr=bp)
+        for name, v in st.items():
+            acc.setdefault(name, []).append(v)
+    stage_ms = {name: float(np.mean(v)) for name, v in acc.items()}
+    stage_ms_min = {name: float(np.min(v)) for name, v in acc.items()}
+
+    cache = layer.cache(T)
+    routed = int(cache.offsets[-1])
+    touched = int((cache.counts > 0).sum())
+    alg = algorithmic(w, T, routed, touched)
+    peak_tf = PEAK_F32_TFLOPS if (w.act_dtype == "f32") else PEAK_BF16_TFLOPS
+
+    def tflops(flops, ms):
+        return flops / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
+
+    def gbs(nbytes, ms):
+        return nbytes / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
+
+    gu = tflops(alg["gate_up_flops"], stage_ms["gate_up"])
+    decode = T <= 64
+    if decode:
+        whole = gbs(alg["layer_bytes_decode"], stage_ms["total"])
+        roofline = {"bound": "hbm", "kernel": "whole layer (weight streaming)", "achieved": whole,
+                    "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": whole / PEAK_HBM_GBS, "traffic": None}
+    else:
+        roofline = {"bound": "mfma", "kernel": "grouped gate/up product + SwiGLU (" + layer.kernel_name() + ")",
+                    "achieved": gu, "peak": peak_tf, "unit": "TFLOP/s", "frac": gu / peak_tf, "traffic": None,
+                    "flops_per_launch": alg["gate_up_flops"], "avg_launch_ms": stage_ms["gate_up"]}
+    both_ms = stage_ms["gate_up"] + stage_ms["down"] + stage_ms["shared"]
+    stages = {
+        "ms_mean": stage_ms, "ms_min": stage_ms_min,
+        "gate_up_tflops": gu,
+        "down_tflops": tflops(alg["down_flops"], stage_ms["down"]),
+        "grouped_gemms_tflops": tflops(alg["gemm_flops"], both_ms),
+        "grouped_gemms_frac_of_peak": tflops(alg["gemm_flops"], both_ms) / peak_tf,
+        "router_gbs": gbs(alg["router_bytes"], stage_ms["router"]),
+        "dispatch_gbs": gbs(alg["dispatch_bytes"], stage_ms["dispatch"]),
+        "dispatch_frac_of_hbm": gbs(alg["dispatch_bytes"], stage_ms["dispatch"]) / PEAK_HBM_GBS,
+        "combine_gbs": gbs(alg["combine_bytes"], stage_ms["combine"]),
+        "combine_frac_of_hbm": gbs(alg["combine_bytes"], stage_ms["combine"]) / PEAK_HBM_GBS,
+    }
+
+    result = {
+        "metric": "MoE-layer fwd tokens/sec at d768 E16 k2; grouped-GEMM % of bf16 MFMA peak",
+        "value": T / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16" if bf16 else "f32", "data": "synthetic",
+        "config": {"workload": w.name, "d_model": w.d_model, "num_experts": w.num_experts,
+                   "experts_per_token": w.experts_per_token, "d_ff": w.d_ff, "tokens": T,
+                   "shared_expert": w.shared_expert, "weight_dtype": w.weight_dtype, "seed": w.seed,
+                   "expert0_share": float(cache.load_fractions()[0]), "routed_slots": routed},
+        "roofline": roofline,
+        "stages": stages,
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(t)
+    print(json.dumps(result))
+    layer.close()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
