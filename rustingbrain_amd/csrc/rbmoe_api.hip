@@ -81,6 +81,7 @@ struct rbmoe_ctx {
     size_t budget_bytes = 0;
     size_t allocated = 0;
     std::string last_error;
+    int refs = 1;  // the caller's handle + one per live layer; torn down when the last one goes
 };
 
 namespace {
@@ -119,6 +120,10 @@ struct rbmoe_layer {
     int max_nb = 0;
     int max_tiles = 0;
     bool force_generic = false;
+    bool explicit_gather = false;  // materialise the gathered rows instead of gathering in the product
+    bool use_mfma = false;     // LDS-staged matrix-core kernels (plain weight layout)
+    bool use_bdirect = false;  // matrix-core kernels with packed weights streamed into registers
+    int cfg_gate_up = 0, cfg_down = 0, group_m = 4;
     const char* kernel_name = "none";
     int last_T = -1;
 
@@ -130,7 +135,7 @@ struct rbmoe_layer {
     Buf ssgu, ssd;         // shared scales
     // workspace
     Buf P, lse, expert_of, gate_of, rank_in_block, blockcnt, blockbase, partial;
-    Buf counts, offsets, tile_expert, tile_row0, tile_rows, ntiles, losses, mass;
+    Buf counts, offsets, tile_expert, tile_row0, tile_rows, tile_expert2, tile_row02, tile_rows2, ntiles, losses, mass;
     Buf perm_slot, perm_token, inv_pos;
     Buf xg, h, y, hs, ys;
     // staging for the host entry point
@@ -189,7 +194,10 @@ Plan make_plan(rbmoe_layer* L) {
     p.add(&L->tile_expert, (size_t)L->max_tiles * 4);
     p.add(&L->tile_row0, (size_t)L->max_tiles * 4);
     p.add(&L->tile_rows, (size_t)L->max_tiles * 4);
-    p.add(&L->ntiles, 4);
+    p.add(&L->tile_expert2, (size_t)L->max_tiles * 4);
+    p.add(&L->tile_row02, (size_t)L->max_tiles * 4);
+    p.add(&L->tile_rows2, (size_t)L->max_tiles * 4);
+    p.add(&L->ntiles, 8);
     p.add(&L->losses, 8);
     p.add(&L->mass, (E + 1) * 4);
     p.add(&L->perm_slot, S * 4);
@@ -301,14 +309,18 @@ int rbmoe_ctx_create(int32_t device, size_t budget_mib, rbmoe_ctx** out) {
     return RBMOE_OK;
 }
 
-void rbmoe_ctx_destroy(rbmoe_ctx* ctx) {
-    if (!ctx) return;
+static void ctx_release(rbmoe_ctx* ctx) {
+    if (!ctx || --ctx->refs > 0) return;
     if (ctx->own_stream) {
         (void)hipStreamSynchronize(ctx->own_stream);
         (void)hipStreamDestroy(ctx->own_stream);
     }
     delete ctx;
 }
+
+// Layers keep their context alive: destroying the context while layers exist
+// only drops the caller's reference.
+void rbmoe_ctx_destroy(rbmoe_ctx* ctx) { ctx_release(ctx); }
 
 int rbmoe_ctx_set_stream(rbmoe_ctx* ctx, void* hip_stream) {
     if (!ctx) return fail(nullptr, RBMOE_NULL_POINTER, "ctx is NULL");
@@ -344,8 +356,29 @@ int rbmoe_layer_create(rbmoe_ctx* ctx, const rbmoe_config* cfg, rbmoe_layer** ou
     L->max_S = cfg->max_tokens * cfg->experts_per_token;
     L->max_nb = (cfg->max_tokens + kRouterTokens - 1) / kRouterTokens;
     L->max_tiles = L->max_S / kGenericTileM + cfg->num_experts + 1;
-    const char* fg = std::getenv("RBMOE_FORCE_GENERIC");
-    L->force_generic = fg && fg[0] == '1';
+    auto env_int = [](const char* name, int fallback) {
+        const char* v = std::getenv(name);
+        return v && v[0] ? std::atoi(v) : fallback;
+    };
+    L->force_generic = env_int("RBMOE_FORCE_GENERIC", 0) == 1;
+    L->explicit_gather = env_int("RBMOE_EXPLICIT_GATHER", 0) == 1;
+    L->cfg_gate_up = env_int("RBMOE_GATE_UP_CFG", 0);
+    L->cfg_down = env_int("RBMOE_DOWN_CFG", 0);
+    L->group_m = env_int("RBMOE_GROUP_M", 4);
+    if (mfma_tile_m(true, L->cfg_gate_up) < 0 || mfma_tile_m(false, L->cfg_down) < 0 || L->group_m < 1) {
+        delete L;
+        return fail(ctx, RBMOE_INVALID_CONFIG, "unknown kernel configuration requested through the environment");
+    }
+    // bf16 matrix cores: bf16 activations, bf16 or int8 weights, reduction widths multiples of 64
+    const bool mc = !L->force_generic && cfg->act_dtype == RBMOE_BF16 && cfg->weight_dtype != RBMOE_F32;
+    const char* path = std::getenv("RBMOE_EXPERT_PATH");  // "bdirect" (default), "lds", "generic"
+    const std::string want = path ? path : "bdirect";
+    const bool bd_ok = mc && bdirect_shape_ok(cfg->d_ff, cfg->d_model) && bdirect_shape_ok(cfg->d_model, cfg->d_ff) &&
+                       (!cfg->shared_expert || (bdirect_shape_ok(L->Fs, cfg->d_model) && bdirect_shape_ok(cfg->d_model, L->Fs)));
+    const bool lds_ok = mc && mfma_shape_ok(cfg->d_model) && mfma_shape_ok(cfg->d_ff) &&
+                        (!cfg->shared_expert || mfma_shape_ok(L->Fs));
+    if (want == "bdirect" && bd_ok) L->use_bdirect = true;
+    else if (want != "generic" && lds_ok) L->use_mfma = true;
 
     Plan plan = make_plan(L);
     // Refuse before allocating anything, as the reference's budget check does
@@ -393,18 +426,21 @@ int rbmoe_layer_create(rbmoe_ctx* ctx, const rbmoe_config* cfg, rbmoe_layer** ou
         delete L;
         return hip_fail(ctx, e, "hipStreamSynchronize");
     }
+    ++ctx->refs;
     *out = L;
     return RBMOE_OK;
 }
 
 void rbmoe_layer_destroy(rbmoe_layer* L) {
     if (!L) return;
+    rbmoe_ctx* owner = L->ctx;
     if (L->ctx) (void)hipStreamSynchronize(L->ctx->stream);
     if (L->have_events)
         for (auto& ev : L->ev)
             if (ev) (void)hipEventDestroy(ev);
     free_layer_buffers(L);
     delete L;
+    ctx_release(owner);
 }
 
 int rbmoe_set_weight(rbmoe_layer* L, int32_t which, int32_t expert, const void* data, int32_t dtype,
@@ -513,6 +549,16 @@ int rbmoe_set_weight(rbmoe_layer* L, int32_t which, int32_t expert, const void* 
         return fail(ctx, RBMOE_UNSUPPORTED, "this conversion between weight dtypes is not supported");
     }
     const size_t es = dtype_size(target);
+    std::vector<unsigned char> packed;
+    if (L->use_bdirect && !is_router) {
+        // operand order of the matrix cores, matrix by matrix (same offsets, different inner layout)
+        packed.resize(n * es);
+        if (target == RBMOE_BF16)
+            pack_weight_bf16(static_cast<const uint16_t*>(src), rows, cols, reinterpret_cast<uint16_t*>(packed.data()));
+        else
+            pack_weight_i8(static_cast<const int8_t*>(src), rows, cols, reinterpret_cast<int8_t*>(packed.data()));
+        src = packed.data();
+    }
     HIP_TRY(ctx, hipMemcpy(dst + elem_off * es, src, n * es, hipMemcpyHostToDevice));
     if (target == RBMOE_I8)
         HIP_TRY(ctx, hipMemcpy(sdst + scale_off, scales, (size_t)rows * 4, hipMemcpyHostToDevice));
@@ -555,8 +601,14 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     HIP_TRY(ctx, mark(0));
 
     const int nb = (T + kRouterTokens - 1) / kRouterTokens;
-    const int tile_m = kGenericTileM;
-    L->kernel_name = "generic";
+    const bool bdirect = L->use_bdirect;
+    const bool mfma = L->use_mfma || bdirect;
+    const int tile_m0 = bdirect ? bdirect_tile_m() : mfma ? mfma_tile_m(true, L->cfg_gate_up) : kGenericTileM;
+    const int tile_m1 = bdirect ? bdirect_tile_m() : mfma ? mfma_tile_m(false, L->cfg_down) : kGenericTileM;
+    L->kernel_name = bdirect ? (wk == WeightKind::I8 ? "mfma_bf16_packed_int8w" : "mfma_bf16_packed")
+                     : mfma  ? (wk == WeightKind::I8 ? "mfma_bf16_lds_int8w" : "mfma_bf16_lds")
+                             : "generic";
+    const bool gather_in_product = mfma && !L->explicit_gather;
 
     RouterArgs ra{x, (const float*)L->router.p, router_bias, valid, T, d, E, k,
                   (float*)L->P.p, (float*)L->lse.p, (int*)L->expert_of.p, (float*)L->gate_of.p,
@@ -564,23 +616,34 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     HIP_TRY(ctx, launch_router(ra, abf, s));
     HIP_TRY(ctx, mark(1));
 
-    ScanArgs sa{(const int*)L->blockcnt.p, (int*)L->blockbase.p, (const float*)L->partial.p, nb, E, k,
-                c.aux_loss_weight, c.router_z_loss_weight, tile_m, (int*)L->counts.p, (int*)L->offsets.p,
-                (int*)L->tile_expert.p, (int*)L->tile_row0.p, (int*)L->tile_rows.p, (int*)L->ntiles.p,
-                (float*)L->losses.p, (float*)L->mass.p};
+    ScanArgs sa{};
+    sa.blockcnt = (const int*)L->blockcnt.p;
+    sa.blockbase = (int*)L->blockbase.p;
+    sa.partial = (const float*)L->partial.p;
+    sa.nb = nb; sa.E = E; sa.k = k;
+    sa.w_aux = c.aux_loss_weight; sa.w_z = c.router_z_loss_weight;
+    sa.tile_m[0] = tile_m0; sa.tile_m[1] = tile_m1;
+    sa.counts = (int*)L->counts.p; sa.offsets = (int*)L->offsets.p;
+    sa.tile_expert[0] = (int*)L->tile_expert.p; sa.tile_row0[0] = (int*)L->tile_row0.p; sa.tile_rows[0] = (int*)L->tile_rows.p;
+    sa.tile_expert[1] = (int*)L->tile_expert2.p; sa.tile_row0[1] = (int*)L->tile_row02.p; sa.tile_rows[1] = (int*)L->tile_rows2.p;
+    sa.ntiles = (int*)L->ntiles.p; sa.losses = (float*)L->losses.p; sa.mass = (float*)L->mass.p;
     HIP_TRY(ctx, launch_scan(sa, s));
     HIP_TRY(ctx, mark(2));
 
     DispatchArgs da{x, (const int*)L->expert_of.p, (const int*)L->rank_in_block.p, (const int*)L->blockbase.p,
                     (const int*)L->offsets.p, T, d, E, k, (int*)L->perm_slot.p, (int*)L->perm_token.p,
-                    (int*)L->inv_pos.p, L->xg.p};
+                    (int*)L->inv_pos.p, gather_in_product ? nullptr : L->xg.p};
     HIP_TRY(ctx, launch_dispatch(da, abf, s));
     HIP_TRY(ctx, mark(3));
 
-    const int max_tiles = T > 0 ? (T * k) / tile_m + E : 0;
+    auto run = [&](const GroupedArgs& g, bool swiglu) -> hipError_t {
+        if (bdirect) return launch_grouped_bdirect(g, wk, s);
+        if (mfma) return launch_grouped_mfma(g, wk, swiglu ? L->cfg_gate_up : L->cfg_down, s);
+        return launch_grouped_generic(g, abf, wk, kGenericTileM, s);
+    };
     GroupedArgs g1{};
-    g1.a = L->xg.p;
-    g1.row_index = nullptr;
+    g1.a = gather_in_product ? x : L->xg.p;
+    g1.row_index = gather_in_product ? (const int*)L->perm_token.p : nullptr;
     g1.w = L->wgu.p;
     g1.w_expert_stride = (size_t)2 * F * d;
     g1.scales = wk == WeightKind::I8 ? (const float*)L->sgu.p : nullptr;
@@ -591,29 +654,37 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     g1.tile_row0 = (const int*)L->tile_row0.p;
     g1.tile_rows = (const int*)L->tile_rows.p;
     g1.ntiles = (const int*)L->ntiles.p;
-    g1.max_tiles = max_tiles;
+    g1.max_tiles = T > 0 ? (T * k) / tile_m0 + E : 0;
     g1.dense_rows = -1;
     g1.out = L->h.p;
     g1.swiglu = true;
-    HIP_TRY(ctx, launch_grouped_generic(g1, abf, wk, tile_m, s));
+    g1.group_m = L->group_m;
+    HIP_TRY(ctx, run(g1, true));
     HIP_TRY(ctx, mark(4));
 
     GroupedArgs g2 = g1;
     g2.a = L->h.p;
+    g2.row_index = nullptr;
     g2.w = L->wd.p;
     g2.w_expert_stride = (size_t)d * F;
     g2.scales = wk == WeightKind::I8 ? (const float*)L->sd.p : nullptr;
     g2.s_expert_stride = (size_t)d;
     g2.N = d;
     g2.K = F;
+    g2.tile_expert = (const int*)L->tile_expert2.p;
+    g2.tile_row0 = (const int*)L->tile_row02.p;
+    g2.tile_rows = (const int*)L->tile_rows2.p;
+    g2.ntiles = (const int*)L->ntiles.p + 1;
+    g2.max_tiles = T > 0 ? (T * k) / tile_m1 + E : 0;
     g2.out = L->y.p;
     g2.swiglu = false;
-    HIP_TRY(ctx, launch_grouped_generic(g2, abf, wk, tile_m, s));
+    HIP_TRY(ctx, run(g2, false));
     HIP_TRY(ctx, mark(5));
 
     if (c.shared_expert && T > 0) {
         GroupedArgs s1 = g1;
         s1.a = x;
+        s1.row_index = nullptr;
         s1.w = L->swgu.p;
         s1.w_expert_stride = 0;
         s1.scales = wk == WeightKind::I8 ? (const float*)L->ssgu.p : nullptr;
@@ -622,7 +693,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
         s1.K = d;
         s1.dense_rows = T;
         s1.out = L->hs.p;
-        HIP_TRY(ctx, launch_grouped_generic(s1, abf, wk, tile_m, s));
+        HIP_TRY(ctx, run(s1, true));
         GroupedArgs s2 = s1;
         s2.a = L->hs.p;
         s2.w = L->swd.p;
@@ -631,7 +702,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
         s2.K = Fs;
         s2.out = L->ys.p;
         s2.swiglu = false;
-        HIP_TRY(ctx, launch_grouped_generic(s2, abf, wk, tile_m, s));
+        HIP_TRY(ctx, run(s2, false));
     }
     HIP_TRY(ctx, mark(6));
 

@@ -42,13 +42,13 @@ struct ScanArgs {
     const float* partial; // [nb, E+1]
     int nb, E, k;
     float w_aux, w_z;
-    int tile_m;
+    int tile_m[2];     // rows per tile of the two tile tables (gate/up product, down product)
     int* counts;       // [E]
     int* offsets;      // [E+1]
-    int* tile_expert;  // [max_tiles]
-    int* tile_row0;
-    int* tile_rows;
-    int* ntiles;       // [1]
+    int* tile_expert[2];  // [max_tiles] each
+    int* tile_row0[2];
+    int* tile_rows[2];
+    int* ntiles;       // [2]
     float* losses;     // [2]
     float* mass;       // [E+1] or null: sum of probabilities per expert, sum of lse^2
 };
@@ -107,9 +107,25 @@ struct GroupedArgs {
     int dense_rows;         // >= 0: one group of this many rows, no tile table (shared expert)
     void* out;              // [rows, N] activation dtype
     bool swiglu;
+    int group_m;            // MFMA path: M-tiles per scheduling group (0 = default)
 };
 hipError_t launch_grouped_generic(const GroupedArgs& a, bool act_bf16, WeightKind wk, int tile_m,
                                   hipStream_t s);
 constexpr int kGenericTileM = 16;
+
+// bf16 matrix-core path (bf16 activations; bf16 or int8 weights; K a multiple of 64).
+constexpr int kNumMfmaConfigs = 7;
+int mfma_tile_m(bool swiglu, int cfg);   // rows per tile of configuration `cfg`, -1 if unknown
+bool mfma_shape_ok(int K);
+hipError_t launch_grouped_mfma(const GroupedArgs& a, WeightKind wk, int cfg, hipStream_t s);
+
+// bf16 matrix-core path with weights repacked into operand order and streamed
+// from global memory into registers (no LDS for weights).  `w` must have been
+// packed with pack_weight_bf16 / pack_weight_i8, matrix by matrix.
+int bdirect_tile_m();
+bool bdirect_shape_ok(int N, int K);
+hipError_t launch_grouped_bdirect(const GroupedArgs& a, WeightKind wk, hipStream_t s);
+void pack_weight_bf16(const uint16_t* src, int rows, int cols, uint16_t* dst);
+void pack_weight_i8(const int8_t* src, int rows, int cols, int8_t* dst);
 
 }  // namespace rbmoe

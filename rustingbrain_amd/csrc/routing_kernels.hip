@@ -240,19 +240,20 @@ __global__ __launch_bounds__(256) void router_kernel(
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(1024) void scan_kernel(
     const int* __restrict__ blockcnt, int* __restrict__ blockbase, const float* __restrict__ partial,
-    int nb, int E, int k, float w_aux, float w_z, int tile_m, int* __restrict__ counts,
-    int* __restrict__ offsets, int* __restrict__ tile_expert, int* __restrict__ tile_row0,
-    int* __restrict__ tile_rows, int* __restrict__ ntiles, float* __restrict__ losses,
+    int nb, int E, int k, float w_aux, float w_z, int tile_m0, int tile_m1, int* __restrict__ counts,
+    int* __restrict__ offsets, int* __restrict__ tile_expert0, int* __restrict__ tile_row00,
+    int* __restrict__ tile_rows0, int* __restrict__ tile_expert1, int* __restrict__ tile_row01,
+    int* __restrict__ tile_rows1, int* __restrict__ ntiles, float* __restrict__ losses,
     float* __restrict__ mass_out) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
-    // LDS: partsum[parts][E] ints, partmass[parts][E+1] floats, cnt[E], off[E+1], toff[E+1]
+    // LDS: partsum[parts][E] ints, partmass[parts][E+1] floats, cnt[E], off[E+1], toff[2][E+1], mass[E+1]
     const int parts = 1024 / E;  // E <= 256 -> parts >= 4
     int* partsum = reinterpret_cast<int*>(lds_raw);
     float* partmass = reinterpret_cast<float*>(partsum + parts * E);
     int* cnt = reinterpret_cast<int*>(partmass + parts * (E + 1));
     int* off = cnt + E;
     int* toff = off + (E + 1);
-    float* mass = reinterpret_cast<float*>(toff + (E + 1));
+    float* mass = reinterpret_cast<float*>(toff + 2 * (E + 1));
 
     const int tid = threadIdx.x;
     const int len = (nb + parts - 1) / parts;
@@ -297,16 +298,20 @@ __global__ __launch_bounds__(1024) void scan_kernel(
     }
     __syncthreads();
     if (tid == 0) {
-        int run = 0, trun = 0;
+        int run = 0, trun0 = 0, trun1 = 0;
         for (int q = 0; q < E; ++q) {
             off[q] = run;
-            toff[q] = trun;
+            toff[q] = trun0;
+            toff[E + 1 + q] = trun1;
             run += cnt[q];
-            trun += (cnt[q] + tile_m - 1) / tile_m;
+            trun0 += (cnt[q] + tile_m0 - 1) / tile_m0;
+            trun1 += (cnt[q] + tile_m1 - 1) / tile_m1;
         }
         off[E] = run;
-        toff[E] = trun;
-        *ntiles = trun;
+        toff[E] = trun0;
+        toff[2 * E + 1] = trun1;
+        ntiles[0] = trun0;
+        ntiles[1] = trun1;
         // auxiliary losses: every valid token routes exactly k slots, so the
         // number of valid tokens is routed / k.
         const int V = run / k;
@@ -338,12 +343,19 @@ __global__ __launch_bounds__(1024) void scan_kernel(
         counts[tid] = cnt[tid];
         offsets[tid] = off[tid];
         if (mass_out) mass_out[tid] = mass[tid];
-        const int nt = toff[tid + 1] - toff[tid];
-        for (int i = 0; i < nt; ++i) {
+        const int nt0 = toff[tid + 1] - toff[tid];
+        for (int i = 0; i < nt0; ++i) {
             const int ti = toff[tid] + i;
-            tile_expert[ti] = tid;
-            tile_row0[ti] = off[tid] + i * tile_m;
-            tile_rows[ti] = min(tile_m, cnt[tid] - i * tile_m);
+            tile_expert0[ti] = tid;
+            tile_row00[ti] = off[tid] + i * tile_m0;
+            tile_rows0[ti] = min(tile_m0, cnt[tid] - i * tile_m0);
+        }
+        const int nt1 = toff[E + 1 + tid + 1] - toff[E + 1 + tid];
+        for (int i = 0; i < nt1; ++i) {
+            const int ti = toff[E + 1 + tid] + i;
+            tile_expert1[ti] = tid;
+            tile_row01[ti] = off[tid] + i * tile_m1;
+            tile_rows1[ti] = min(tile_m1, cnt[tid] - i * tile_m1);
         }
     }
     if (tid == 0) offsets[E] = off[E];
@@ -351,7 +363,7 @@ __global__ __launch_bounds__(1024) void scan_kernel(
 
 size_t scan_lds_bytes(int E) {
     const int parts = 1024 / E;
-    return ((size_t)parts * E + (size_t)parts * (E + 1) + E + 2 * (E + 1) + (E + 1)) * 4;
+    return ((size_t)parts * E + (size_t)parts * (E + 1) + E + 3 * (E + 1) + (E + 1)) * 4;
 }
 
 // ---------------------------------------------------------------------------
@@ -468,9 +480,9 @@ hipError_t launch_router(const RouterArgs& a, bool bf16, hipStream_t s) {
 
 hipError_t launch_scan(const ScanArgs& a, hipStream_t s) {
     hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), scan_lds_bytes(a.E), s, a.blockcnt,
-                       a.blockbase, a.partial, a.nb, a.E, a.k, a.w_aux, a.w_z, a.tile_m, a.counts,
-                       a.offsets, a.tile_expert, a.tile_row0, a.tile_rows, a.ntiles, a.losses,
-                       a.mass);
+                       a.blockbase, a.partial, a.nb, a.E, a.k, a.w_aux, a.w_z, a.tile_m[0], a.tile_m[1],
+                       a.counts, a.offsets, a.tile_expert[0], a.tile_row0[0], a.tile_rows[0],
+                       a.tile_expert[1], a.tile_row0[1], a.tile_rows[1], a.ntiles, a.losses, a.mass);
     return hipGetLastError();
 }
 

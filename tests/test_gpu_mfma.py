@@ -1,0 +1,124 @@
+"""The bf16 matrix-core path of the grouped expert products against the oracle,
+for every tile configuration the library carries: ragged groups, partial tiles
+in both directions, padding rows, empty experts, a shared expert of another
+width, int8 weights, and the explicit-gather variant."""
+import os
+
+import numpy as np
+import pytest
+
+import rustingbrain_amd as rb
+from conftest import rel_l2
+from helpers import assert_routing_identical, gpu_layer, oracle_layer, small_workload
+from rustingbrain_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+NUM_CONFIGS = 7
+
+
+@pytest.fixture
+def kernel_env():
+    keys = ("RBMOE_GATE_UP_CFG", "RBMOE_DOWN_CFG", "RBMOE_GROUP_M", "RBMOE_EXPLICIT_GATHER", "RBMOE_FORCE_GENERIC",
+            "RBMOE_EXPERT_PATH")
+    saved = {k: os.environ.get(k) for k in keys}
+    yield os.environ
+    for k, v in saved.items():
+        if v is None:
+            os.environ.pop(k, None)
+        else:
+            os.environ[k] = v
+
+
+def run(device, t, valid=None, bias=None):
+    ref = oracle_layer(t).forward(t.x, valid=valid, router_bias=bias, threads=8)
+    layer = gpu_layer(device, t)
+    assert layer.kernel_name().startswith("mfma") or layer.kernel_name() == "none"
+    layout = rb.Layout(valid=None if valid is None else [bool(v) for v in valid])
+    out, cache = layer.forward_train(t.x, layout, router_bias=bias)
+    assert layer.kernel_name().startswith("mfma")
+    assert_routing_identical(cache, ref)
+    h, y = layer.expert_rows(int(ref.offsets[-1]))
+    assert rel_l2(h, ref.hidden) <= 2e-2, "hidden rows"
+    assert rel_l2(y, ref.expert_out) <= 2e-2, "expert output rows"
+    err = rel_l2(out, ref.out)
+    assert err <= 2e-2, err
+    layer.close()
+    return err
+
+
+@pytest.mark.parametrize("cfg", range(NUM_CONFIGS))
+@pytest.mark.parametrize("wt", ["bf16", "int8"])
+def test_every_tile_configuration_of_the_lds_staged_kernels(device, kernel_env, cfg, wt):
+    kernel_env["RBMOE_EXPERT_PATH"] = "lds"
+    kernel_env["RBMOE_GATE_UP_CFG"] = str(cfg)
+    kernel_env["RBMOE_DOWN_CFG"] = str(cfg)
+    # F = 192 leaves a partial column tile; 700 tokens over 6 experts leave partial row tiles
+    t = synth.make(small_workload(d=128, E=6, k=2, F=192, T=700, seed=17, act="bf16", wt=wt, shared=True,
+                                  shared_d_ff=320))
+    bias = np.zeros(6, np.float32)
+    bias[1] = 1.5   # one large group ...
+    bias[4] = -50   # ... and one empty expert
+    valid = (np.arange(700) % 9 != 4).astype(np.uint8)
+    run(device, t, valid=valid, bias=bias)
+
+
+@pytest.mark.parametrize("wt", ["bf16", "int8"])
+@pytest.mark.parametrize("shape", [dict(d=128, E=6, k=2, F=192, T=700), dict(d=64, E=3, k=1, F=64, T=130),
+                                   dict(d=256, E=16, k=4, F=128, T=333), dict(d=192, E=5, k=2, F=320, T=1000)],
+                         ids=lambda s: "d{d}_E{E}_k{k}_F{F}_T{T}".format(**s))
+def test_packed_weight_kernels(device, kernel_env, shape, wt):
+    kernel_env["RBMOE_EXPERT_PATH"] = "bdirect"
+    E = shape["E"]
+    t = synth.make(small_workload(seed=19, act="bf16", wt=wt, shared=True, shared_d_ff=shape["F"] + 64, **shape))
+    bias = np.zeros(E, np.float32)
+    bias[1] = 1.5
+    bias[E - 1] = -50
+    T = shape["T"]
+    valid = (np.arange(T) % 9 != 4).astype(np.uint8)
+    layer_name = run(device, t, valid=valid, bias=bias)
+
+
+@pytest.mark.parametrize("group_m", [1, 3, 8])
+def test_scheduling_group_size_does_not_change_results(device, kernel_env, group_m):
+    kernel_env["RBMOE_GROUP_M"] = str(group_m)
+    t = synth.make(small_workload(d=64, E=8, k=2, F=128, T=1500, seed=23, act="bf16", wt="bf16"))
+    run(device, t)
+
+
+def test_explicit_gather_gives_the_same_bits_as_gathering_in_the_product(device, kernel_env):
+    t = synth.make(small_workload(d=128, E=8, k=3, F=256, T=900, seed=29, act="bf16", wt="bf16"))
+    layer = gpu_layer(device, t)
+    a, _ = layer.forward_train(t.x)
+    layer.close()
+    kernel_env["RBMOE_EXPLICIT_GATHER"] = "1"
+    layer = gpu_layer(device, t)
+    b, _ = layer.forward_train(t.x)
+    layer.close()
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+def test_matrix_core_and_generic_paths_agree(device, kernel_env):
+    t = synth.make(small_workload(d=64, E=4, k=2, F=64, T=257, seed=31, act="bf16", wt="bf16", shared=True))
+    layer = gpu_layer(device, t)
+    a, _ = layer.forward_train(t.x)
+    assert layer.kernel_name() == "mfma_bf16_packed"
+    layer.close()
+    kernel_env["RBMOE_EXPERT_PATH"] = "lds"
+    layer = gpu_layer(device, t)
+    c, _ = layer.forward_train(t.x)
+    assert layer.kernel_name() == "mfma_bf16_lds"
+    layer.close()
+    assert rel_l2(a, c) < 1e-2
+    kernel_env["RBMOE_FORCE_GENERIC"] = "1"
+    layer = gpu_layer(device, t)
+    b, _ = layer.forward_train(t.x)
+    assert layer.kernel_name() == "generic"
+    layer.close()
+    assert rel_l2(a, b) < 1e-2
+
+
+@pytest.mark.parametrize("T", [1, 8, 33, 127, 128, 129])
+def test_small_token_counts(device, T):
+    t = synth.make(small_workload(d=64, E=8, k=2, F=64, T=T, seed=37, act="bf16", wt="bf16", shared=True))
+    run(device, t)
