@@ -1,0 +1,399 @@
+// Grouped expert products on the bf16 matrix cores of gfx950.
+//
+//   out[row, n] = sum_c a[row, c] * w[expert][n, c]                 (down product)
+//   out[row, n] = silu(a . wgate[n]) * (a . wup[n])                 (gate/up product)
+//
+// Data paths (nothing is staged through registers on its way to LDS):
+//   weights      packed at upload into matrix-core operand order (see
+//                pack_weight_bf16 / pack_weight_i8); every wave streams its own
+//                fragments global -> VGPR through an 8-deep register ring, i.e.
+//                the load for reduction step g + 7 is issued while step g runs.
+//                int8 weights are widened to bf16 in registers right before the
+//                multiply; the per-row scale multiplies the accumulator.
+//   activations  128 token rows per workgroup (gathered through an index for
+//                the gate/up product) go global -> LDS with the LDS-DMA load
+//                (global_load_lds_dwordx4): lane l of a wave deposits its 16
+//                bytes at LDS base + 16 l, so the XOR swizzle that keeps the
+//                fragment reads free of bank conflicts is applied by choosing
+//                which global piece each lane fetches.  Two LDS stages; the DMA
+//                for slice k + 1 is issued when slice k starts and is awaited
+//                (vmcnt) just before the barrier that ends slice k.
+//   fragments    token fragments are read from LDS one step ahead of the
+//                multiplies that use them.
+// A workgroup is 4 waves side by side along the output features; a wave owns
+// 128 tokens x 64 weight rows (32 gate + the matching 32 up rows, or 64 down
+// rows).  The weight fragment is the matrix-core A operand and the token
+// fragment the B operand, so a lane ends with 4 consecutive output features of
+// one token and writes them with one 8-byte store.  Token blocks of 32 rows
+// that lie beyond the end of a group are skipped, so a ragged group costs at
+// most 31 rows of padding.
+#include <type_traits>
+
+#include "rbmoe_kernels.h"
+
+namespace rbmoe {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
+
+namespace {
+
+constexpr int BM = 128;   // token rows per workgroup
+constexpr int BK = 64;    // reduction slice held in one LDS stage
+constexpr int NW = 4;     // waves per workgroup
+constexpr int NT = NW * 64;
+constexpr int CPR = BK / 8;            // 16-byte pieces per LDS row
+constexpr int TT = BM / 32;            // token blocks per wave
+constexpr int KS = BK / 16;            // matrix-core steps per slice
+constexpr int DMA_PER_WAVE = BM * CPR / 64 / NW;  // LDS-DMA instructions per wave per slice (4)
+
+__device__ __forceinline__ uint32_t widen2(uint32_t word, int shift) {
+    const float lo = (float)(int)(int8_t)(word >> shift);
+    const float hi = (float)(int)(int8_t)(word >> (shift + 8));
+    return (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xffff0000u);  // small integers are exact in bf16
+}
+
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+    bf16x2 v = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(uint32_t, v);
+}
+
+__device__ __forceinline__ bf16x8 widen_i8(uint2 q) {
+    const uint4 w = make_uint4(widen2(q.x, 0), widen2(q.x, 16), widen2(q.y, 0), widen2(q.y, 16));
+    return __builtin_bit_cast(bf16x8, w);
+}
+
+// s_waitcnt vmcnt(N) only (expcnt and lgkmcnt left at their maxima), gfx9 encoding.
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt((N & 0xF) | (0x7 << 4) | (0xF << 8) | ((N >> 4) << 14));
+}
+
+// One ring slot: the wave's two weight fragments of one reduction step.
+// bf16: 16 bytes per lane per fragment.  int8: 8 bytes per lane per fragment.
+template <bool I8>
+struct Slot;
+template <>
+struct Slot<false> {
+    uint4 f0, f1;
+    __device__ __forceinline__ void load(const char* p0, const char* p1, int g, int lane) {
+        f0 = reinterpret_cast<const uint4*>(p0)[(size_t)g * 64 + lane];
+        f1 = reinterpret_cast<const uint4*>(p1)[(size_t)g * 64 + lane];
+    }
+    __device__ __forceinline__ bf16x8 a0() const { return __builtin_bit_cast(bf16x8, f0); }
+    __device__ __forceinline__ bf16x8 a1() const { return __builtin_bit_cast(bf16x8, f1); }
+};
+template <>
+struct Slot<true> {
+    uint2 f0, f1;
+    // packed int8 layout: [K/32][64 lanes][16 bytes]; bytes 0..7 belong to the even step, 8..15 to the odd one
+    __device__ __forceinline__ void load(const char* p0, const char* p1, int g, int lane) {
+        const size_t idx = ((size_t)(g >> 1) * 64 + lane) * 2 + (g & 1);
+        f0 = reinterpret_cast<const uint2*>(p0)[idx];
+        f1 = reinterpret_cast<const uint2*>(p1)[idx];
+    }
+    __device__ __forceinline__ bf16x8 a0() const { return widen_i8(f0); }
+    __device__ __forceinline__ bf16x8 a1() const { return widen_i8(f1); }
+};
+
+// RING = weight-fragment steps in flight per wave (register ring depth).
+template <bool SWIGLU, bool I8, int RING, int TFBUF>
+__global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
+    const bf16_t* __restrict__ a, const int* __restrict__ row_index, const void* __restrict__ wpacked,
+    size_t w_expert_stride_bytes, const float* __restrict__ scales, size_t s_expert_stride, int N, int K,
+    const int* __restrict__ tile_expert, const int* __restrict__ tile_row0, const int* __restrict__ tile_rows,
+    const int* __restrict__ ntiles, int dense_rows, bf16_t* __restrict__ out, int group_m) {
+    constexpr int BN = SWIGLU ? NW * 32 : NW * 64;  // output features per workgroup
+    __shared__ uint4 As[2][BM * CPR];
+
+    // ---- which tile (each XCD walks a contiguous range, M fastest inside a group)
+    const int tiles_n = (N + BN - 1) / BN;
+    const int tiles_m = dense_rows >= 0 ? (dense_rows + BM - 1) / BM : *ntiles;
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) / 8;
+    const int local = blockIdx.x >> 3;
+    if (local >= per_xcd) return;
+    const int pid = (blockIdx.x & 7) * per_xcd + local;
+    if (pid >= total) return;
+    const int per_group = group_m * tiles_n;
+    const int grp = pid / per_group;
+    const int first_m = grp * group_m;
+    const int gsize = min(group_m, tiles_m - first_m);
+    const int in_g = pid - grp * per_group;
+    const int tm_idx = first_m + in_g % gsize;
+    const int tn_idx = in_g / gsize;
+
+    int expert, row0, rows;
+    if (dense_rows >= 0) {
+        expert = 0;
+        row0 = tm_idx * BM;
+        rows = min(BM, dense_rows - row0);
+    } else {
+        expert = tile_expert[tm_idx];
+        row0 = tile_row0[tm_idx];
+        rows = tile_rows[tm_idx];
+    }
+    const int nblk = (rows + 31) >> 5;  // token blocks that hold at least one row
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    // ---- this wave's two blocks of 32 weight rows ---------------------------
+    const int nw = tn_idx * BN + wave * (SWIGLU ? 32 : 64);
+    const int r0 = nw, r1 = SWIGLU ? N + nw : nw + 32;
+    const bool act0 = nw < N;
+    const bool act1 = SWIGLU ? act0 : (nw + 32 < N);
+    const size_t block_bytes = (size_t)K * 32 * (I8 ? 1 : 2);  // one block of 32 weight rows over all of K
+    const char* wexp = static_cast<const char*>(wpacked) + (size_t)expert * w_expert_stride_bytes;
+    const char* wp0 = wexp + (size_t)(act0 ? r0 / 32 : 0) * block_bytes;
+    const char* wp1 = wexp + (size_t)(act1 ? r1 / 32 : 0) * block_bytes;
+
+    // ---- LDS-DMA of the activation slice --------------------------------------
+    // Wave w fills LDS rows [32 w, 32 w + 32): instruction j covers rows 32 w + 8 j .. + 7,
+    // lane l lands in row 8 j + l / 8 (of the wave's 32), position l % 8, and therefore
+    // fetches logical piece (l % 8) ^ (row % 8).  Rows past the end of the group are
+    // clamped to the tile's first row: their products are never stored.
+    const uint4* a_pieces = reinterpret_cast<const uint4*>(a);
+    const int kp = K / 8;
+    uint32_t a_off[DMA_PER_WAVE];
+#pragma unroll
+    for (int j = 0; j < DMA_PER_WAVE; ++j) {
+        const int r = wave * 32 + j * 8 + (lane >> 3);
+        const int rr = r < rows ? r : 0;
+        const int grow = row_index ? row_index[row0 + rr] : row0 + rr;
+        a_off[j] = (uint32_t)grow * (uint32_t)kp + ((lane & 7) ^ (r & 7));
+    }
+    auto dma_a = [&](int kt, int buf) {
+#pragma unroll
+        for (int j = 0; j < DMA_PER_WAVE; ++j) {
+            const uint4* src = a_pieces + a_off[j] + kt * CPR;
+            uint4* dst = &As[buf][(wave * 32 + j * 8) * CPR];
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                             (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+        }
+    };
+
+    floatx16 acc[2][TT];
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int t = 0; t < TT; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[b][t][v] = 0.0f;
+
+    const int lrow = lane & 31;
+    const int lhalf = lane >> 5;
+    const int lxor = lrow & 7;
+
+    const int KT = K / BK;
+    const int GS = KT * KS;  // reduction steps in all
+
+    // ---- prologue: first activation slice, first RING-1 weight steps ----------
+    dma_a(0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    Slot<I8> ring[RING];
+    if (act0) {
+#pragma unroll
+        for (int g = 0; g < RING - 1; ++g)
+            if (g < GS) ring[g].load(wp0, wp1, g, lane);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    wait_vmcnt<0>();  // first slice must be in LDS (this also drains the first weight loads: prologue only)
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+
+    // One slice = KS steps.  `G0` is the ring position of the slice's first step (0 or 4).
+    // NB = token blocks of this tile that hold rows, a compile-time constant inside the
+    // loop: a run-time branch per block between the multiplies costs far more than the
+    // skipped multiplies save, so the whole loop is specialised instead.
+    auto slice = [&](int kt, auto g0_tag, auto nb_tag) {
+        constexpr int G0 = decltype(g0_tag)::value;
+        constexpr int NB = decltype(nb_tag)::value;
+        const int buf = kt & 1;
+        const bool more = kt + 1 < KT;
+        if (more) dma_a(kt + 1, buf ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (act0) {
+            const uint4* Ab = As[buf];
+            bf16x8 tf[TFBUF][TT];
+#pragma unroll
+            for (int t = 0; t < NB; ++t) tf[0][t] = __builtin_bit_cast(bf16x8, Ab[(t * 32 + lrow) * CPR + (lhalf ^ lxor)]);
+#pragma unroll
+            for (int s = 0; s < KS; ++s) {
+                const int g = kt * KS + s;
+                // weight fragments for step g + RING - 1 go into the slot step g - 1 released
+                if (g + RING - 1 < GS) ring[(G0 + s + RING - 1) % RING].load(wp0, wp1, g + RING - 1, lane);
+                if constexpr (TFBUF == 2) {
+                    if (s + 1 < KS) {
+                        const int piece = (2 * (s + 1) + lhalf) ^ lxor;
+#pragma unroll
+                        for (int t = 0; t < NB; ++t)
+                            tf[(s + 1) & 1][t] = __builtin_bit_cast(bf16x8, Ab[(t * 32 + lrow) * CPR + piece]);
+                    }
+                } else if (s > 0) {
+                    const int piece = (2 * s + lhalf) ^ lxor;
+#pragma unroll
+                    for (int t = 0; t < NB; ++t) tf[0][t] = __builtin_bit_cast(bf16x8, Ab[(t * 32 + lrow) * CPR + piece]);
+                }
+                const bf16x8 w0 = ring[(G0 + s) % RING].a0();
+                const bf16x8 w1 = ring[(G0 + s) % RING].a1();
+#pragma unroll
+                for (int t = 0; t < NB; ++t) {
+                    acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w0, tf[s % TFBUF][t], acc[0][t], 0, 0, 0);
+                    acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w1, tf[s % TFBUF][t], acc[1][t], 0, 0, 0);
+                }
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // The DMA of the next slice was issued before this slice's weight loads.  Once at
+        // most that many loads are outstanding, the DMA has landed (loads retire in order).
+        if (more) {
+            if (act0 && (kt + 1) * KS - 1 + RING - 1 < GS)
+                wait_vmcnt<2 * KS>();  // every step of this slice issued its two weight loads
+            else
+                wait_vmcnt<0>();
+        }
+        // A bare barrier: every LDS read of this slice has already been consumed by a
+        // multiply, and the DMA wait above is the only other thing the next slice needs.
+        // (__syncthreads() would drain the whole weight ring with a vmcnt(0).)
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // The ring position of a slice's first step alternates between 0 and KS when the ring
+    // holds two slices, and is always 0 when it holds one.
+    static_assert(RING == KS || RING == 2 * KS, "ring depth is one or two slices");
+    auto run = [&](auto nb_tag) {
+        if constexpr (RING == KS) {
+            for (int kt = 0; kt < KT; ++kt) slice(kt, std::integral_constant<int, 0>{}, nb_tag);
+        } else {
+            int kt = 0;
+            for (; kt + 1 < KT; kt += 2) {
+                slice(kt, std::integral_constant<int, 0>{}, nb_tag);
+                slice(kt + 1, std::integral_constant<int, KS>{}, nb_tag);
+            }
+            if (kt < KT) slice(kt, std::integral_constant<int, 0>{}, nb_tag);
+        }
+    };
+    static_assert(TT == 4, "one specialisation per possible block count");
+    if (nblk == 4) run(std::integral_constant<int, 4>{});
+    else if (nblk == 3) run(std::integral_constant<int, 3>{});
+    else if (nblk == 2) run(std::integral_constant<int, 2>{});
+    else run(std::integral_constant<int, 1>{});
+    if (!act0) return;
+
+    // ---- epilogue -------------------------------------------------------------
+    // accumulator element v of block (b, t): feature 8*(v/4) + 4*(lane/32) + v%4 of the
+    // wave's row block b, token t*32 + lane%32.
+    const float* sc = I8 ? scales + (size_t)expert * s_expert_stride : nullptr;
+#pragma unroll
+    for (int t = 0; t < TT; ++t) {
+        const int m = t * 32 + lrow;
+        if (m >= rows) continue;
+        bf16_t* orow = out + (size_t)(row0 + m) * N;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int f = 8 * q + 4 * lhalf;  // first of 4 consecutive features inside a row block
+            if constexpr (SWIGLU) {
+                float h[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float gv = acc[0][t][4 * q + i], uv = acc[1][t][4 * q + i];
+                    if constexpr (I8) {
+                        gv *= sc[r0 + f + i];
+                        uv *= sc[r1 + f + i];
+                    }
+                    h[i] = silu_f32(gv) * uv;
+                }
+                *reinterpret_cast<uint2*>(orow + nw + f) = make_uint2(pack2(h[0], h[1]), pack2(h[2], h[3]));
+            } else {
+#pragma unroll
+                for (int b = 0; b < 2; ++b) {
+                    if (b == 1 && !act1) continue;
+                    const int rb = b ? r1 : r0;
+                    float y[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        y[i] = acc[b][t][4 * q + i];
+                        if constexpr (I8) y[i] *= sc[rb + f + i];
+                    }
+                    *reinterpret_cast<uint2*>(orow + rb + f) = make_uint2(pack2(y[0], y[1]), pack2(y[2], y[3]));
+                }
+            }
+        }
+    }
+}
+
+template <bool SWIGLU, bool I8, int RING, int TFBUF>
+hipError_t launch_t(const GroupedArgs& g, hipStream_t s) {
+    constexpr int BN = SWIGLU ? NW * 32 : NW * 64;
+    const int tiles_n = (g.N + BN - 1) / BN;
+    const int tiles_m = g.dense_rows >= 0 ? (g.dense_rows + BM - 1) / BM : g.max_tiles;
+    if (tiles_m <= 0) return hipSuccess;
+    const int total = tiles_m * tiles_n;
+    const int grid = ((total + 7) / 8) * 8;
+    hipLaunchKernelGGL((grouped_stream_kernel<SWIGLU, I8, RING, TFBUF>), dim3(grid), dim3(NT), 0, s,
+                       static_cast<const bf16_t*>(g.a), g.row_index, g.w, g.w_expert_stride * (I8 ? 1 : 2), g.scales,
+                       g.s_expert_stride, g.N, g.K, g.tile_expert, g.tile_row0, g.tile_rows, g.ntiles, g.dense_rows,
+                       static_cast<bf16_t*>(g.out), g.group_m > 0 ? g.group_m : 4);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+template <int RING, int TFBUF>
+static hipError_t launch_ring(const GroupedArgs& g, WeightKind wk, hipStream_t s) {
+    if (wk == WeightKind::BF16)
+        return g.swiglu ? launch_t<true, false, RING, TFBUF>(g, s) : launch_t<false, false, RING, TFBUF>(g, s);
+    if (wk == WeightKind::I8)
+        return g.swiglu ? launch_t<true, true, RING, TFBUF>(g, s) : launch_t<false, true, RING, TFBUF>(g, s);
+    return hipErrorInvalidValue;
+}
+
+// variant 0: ring of 4 steps, token fragments read one step ahead
+// variant 1: ring of 8 steps, token fragments read just in time
+int stream_tile_m() { return BM; }
+
+// K a multiple of 64 (one LDS slice), N a multiple of 32 (row blocks of the packed weights)
+bool stream_shape_ok(int N, int K) { return K % 64 == 0 && K >= 64 && N % 32 == 0 && N >= 32; }
+
+hipError_t launch_grouped_stream(const GroupedArgs& g, WeightKind wk, int variant, hipStream_t s) {
+    if (!stream_shape_ok(g.N, g.K)) return hipErrorInvalidValue;
+    switch (variant) {
+        case 0: return launch_ring<4, 2>(g, wk, s);
+        case 1: return launch_ring<8, 1>(g, wk, s);
+    }
+    return hipErrorInvalidValue;
+}
+
+// Host-side repacking of one [rows, cols] weight matrix into fragment order.
+// bf16: [rows/32][cols/16][64 lanes][8]; lane l holds row (l % 32), columns 16*s + 8*(l/32) + 0..7.
+void pack_weight_bf16(const uint16_t* src, int rows, int cols, uint16_t* dst) {
+    const int KS16 = cols / 16;
+    for (int nb = 0; nb < rows / 32; ++nb)
+        for (int s = 0; s < KS16; ++s)
+            for (int l = 0; l < 64; ++l) {
+                const uint16_t* p = src + (size_t)(nb * 32 + l % 32) * cols + 16 * s + 8 * (l / 32);
+                uint16_t* q = dst + (((size_t)nb * KS16 + s) * 64 + l) * 8;
+                for (int j = 0; j < 8; ++j) q[j] = p[j];
+            }
+}
+
+// int8: [rows/32][cols/32][64 lanes][16]; bytes 0..7 are the lane's piece of step 2s, bytes 8..15 of step 2s+1.
+void pack_weight_i8(const int8_t* src, int rows, int cols, int8_t* dst) {
+    const int KS32 = cols / 32;
+    for (int nb = 0; nb < rows / 32; ++nb)
+        for (int s = 0; s < KS32; ++s)
+            for (int l = 0; l < 64; ++l) {
+                const int8_t* p = src + (size_t)(nb * 32 + l % 32) * cols + 32 * s + 8 * (l / 32);
+                int8_t* q = dst + (((size_t)nb * KS32 + s) * 64 + l) * 16;
+                for (int j = 0; j < 8; ++j) {
+                    q[j] = p[j];
+                    q[8 + j] = p[16 + j];
+                }
+            }
+}
+
+}  // namespace rbmoe

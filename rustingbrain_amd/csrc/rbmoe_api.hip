@@ -121,9 +121,8 @@ struct rbmoe_layer {
     int max_tiles = 0;
     bool force_generic = false;
     bool explicit_gather = false;  // materialise the gathered rows instead of gathering in the product
-    bool use_mfma = false;     // LDS-staged matrix-core kernels (plain weight layout)
-    bool use_bdirect = false;  // matrix-core kernels with packed weights streamed into registers
-    int cfg_gate_up = 0, cfg_down = 0, group_m = 4;
+    bool use_stream = false;   // bf16 matrix-core kernels (packed weights); otherwise the generic kernels
+    int group_m = 4, variant = 0;
     const char* kernel_name = "none";
     int last_T = -1;
 
@@ -344,7 +343,7 @@ int rbmoe_layer_create(rbmoe_ctx* ctx, const rbmoe_config* cfg, rbmoe_layer** ou
     problem = limit_problem(cfg);
     if (!problem.empty()) return fail(ctx, RBMOE_UNSUPPORTED, problem);
     if (cfg->max_tokens <= 0) return fail(ctx, RBMOE_INVALID_CONFIG, "max_tokens must be positive");
-    if (router_lds_bytes(cfg->num_experts, cfg->experts_per_token) > 64 * 1024)
+    if (router_lds_bytes(cfg->num_experts, cfg->experts_per_token) > (size_t)kMaxRouterLds)
         return fail(ctx, RBMOE_UNSUPPORTED, "router tile does not fit in LDS for this expert count and top-k");
 
     rbmoe_layer* L = new rbmoe_layer();
@@ -362,23 +361,13 @@ int rbmoe_layer_create(rbmoe_ctx* ctx, const rbmoe_config* cfg, rbmoe_layer** ou
     };
     L->force_generic = env_int("RBMOE_FORCE_GENERIC", 0) == 1;
     L->explicit_gather = env_int("RBMOE_EXPLICIT_GATHER", 0) == 1;
-    L->cfg_gate_up = env_int("RBMOE_GATE_UP_CFG", 0);
-    L->cfg_down = env_int("RBMOE_DOWN_CFG", 0);
-    L->group_m = env_int("RBMOE_GROUP_M", 4);
-    if (mfma_tile_m(true, L->cfg_gate_up) < 0 || mfma_tile_m(false, L->cfg_down) < 0 || L->group_m < 1) {
-        delete L;
-        return fail(ctx, RBMOE_INVALID_CONFIG, "unknown kernel configuration requested through the environment");
-    }
-    // bf16 matrix cores: bf16 activations, bf16 or int8 weights, reduction widths multiples of 64
+    L->group_m = std::max(1, env_int("RBMOE_GROUP_M", 4));
+    L->variant = env_int("RBMOE_STREAM_VARIANT", 0) == 1 ? 1 : 0;
+    // bf16 matrix cores: bf16 activations, bf16 or int8 weights, widths that fit the packed layout
     const bool mc = !L->force_generic && cfg->act_dtype == RBMOE_BF16 && cfg->weight_dtype != RBMOE_F32;
-    const char* path = std::getenv("RBMOE_EXPERT_PATH");  // "bdirect" (default), "lds", "generic"
-    const std::string want = path ? path : "bdirect";
-    const bool bd_ok = mc && bdirect_shape_ok(cfg->d_ff, cfg->d_model) && bdirect_shape_ok(cfg->d_model, cfg->d_ff) &&
-                       (!cfg->shared_expert || (bdirect_shape_ok(L->Fs, cfg->d_model) && bdirect_shape_ok(cfg->d_model, L->Fs)));
-    const bool lds_ok = mc && mfma_shape_ok(cfg->d_model) && mfma_shape_ok(cfg->d_ff) &&
-                        (!cfg->shared_expert || mfma_shape_ok(L->Fs));
-    if (want == "bdirect" && bd_ok) L->use_bdirect = true;
-    else if (want != "generic" && lds_ok) L->use_mfma = true;
+    L->use_stream = mc && stream_shape_ok(cfg->d_ff, cfg->d_model) && stream_shape_ok(cfg->d_model, cfg->d_ff) &&
+                    (!cfg->shared_expert ||
+                     (stream_shape_ok(L->Fs, cfg->d_model) && stream_shape_ok(cfg->d_model, L->Fs)));
 
     Plan plan = make_plan(L);
     // Refuse before allocating anything, as the reference's budget check does
@@ -550,7 +539,7 @@ int rbmoe_set_weight(rbmoe_layer* L, int32_t which, int32_t expert, const void* 
     }
     const size_t es = dtype_size(target);
     std::vector<unsigned char> packed;
-    if (L->use_bdirect && !is_router) {
+    if (L->use_stream && !is_router) {
         // operand order of the matrix cores, matrix by matrix (same offsets, different inner layout)
         packed.resize(n * es);
         if (target == RBMOE_BF16)
@@ -601,13 +590,10 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     HIP_TRY(ctx, mark(0));
 
     const int nb = (T + kRouterTokens - 1) / kRouterTokens;
-    const bool bdirect = L->use_bdirect;
-    const bool mfma = L->use_mfma || bdirect;
-    const int tile_m0 = bdirect ? bdirect_tile_m() : mfma ? mfma_tile_m(true, L->cfg_gate_up) : kGenericTileM;
-    const int tile_m1 = bdirect ? bdirect_tile_m() : mfma ? mfma_tile_m(false, L->cfg_down) : kGenericTileM;
-    L->kernel_name = bdirect ? (wk == WeightKind::I8 ? "mfma_bf16_packed_int8w" : "mfma_bf16_packed")
-                     : mfma  ? (wk == WeightKind::I8 ? "mfma_bf16_lds_int8w" : "mfma_bf16_lds")
-                             : "generic";
+    const bool mfma = L->use_stream;
+    const int tile_m0 = mfma ? stream_tile_m() : kGenericTileM;
+    const int tile_m1 = tile_m0;
+    L->kernel_name = mfma ? (wk == WeightKind::I8 ? "mfma_bf16_stream_int8w" : "mfma_bf16_stream") : "generic";
     const bool gather_in_product = mfma && !L->explicit_gather;
 
     RouterArgs ra{x, (const float*)L->router.p, router_bias, valid, T, d, E, k,
@@ -637,8 +623,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     HIP_TRY(ctx, mark(3));
 
     auto run = [&](const GroupedArgs& g, bool swiglu) -> hipError_t {
-        if (bdirect) return launch_grouped_bdirect(g, wk, s);
-        if (mfma) return launch_grouped_mfma(g, wk, swiglu ? L->cfg_gate_up : L->cfg_down, s);
+        if (mfma) return launch_grouped_stream(g, wk, L->variant, s);
         return launch_grouped_generic(g, abf, wk, kGenericTileM, s);
     };
     GroupedArgs g1{};

@@ -18,6 +18,7 @@ constexpr int kMaxExperts = 256;
 constexpr int kMaxTopK = 32;
 
 size_t router_lds_bytes(int E, int k);
+constexpr int kMaxRouterLds = 160 * 1024;  // LDS per workgroup on gfx950
 size_t scan_lds_bytes(int E);
 
 struct RouterArgs {
@@ -113,18 +114,12 @@ hipError_t launch_grouped_generic(const GroupedArgs& a, bool act_bf16, WeightKin
                                   hipStream_t s);
 constexpr int kGenericTileM = 16;
 
-// bf16 matrix-core path (bf16 activations; bf16 or int8 weights; K a multiple of 64).
-constexpr int kNumMfmaConfigs = 7;
-int mfma_tile_m(bool swiglu, int cfg);   // rows per tile of configuration `cfg`, -1 if unknown
-bool mfma_shape_ok(int K);
-hipError_t launch_grouped_mfma(const GroupedArgs& a, WeightKind wk, int cfg, hipStream_t s);
-
-// bf16 matrix-core path with weights repacked into operand order and streamed
-// from global memory into registers (no LDS for weights).  `w` must have been
-// packed with pack_weight_bf16 / pack_weight_i8, matrix by matrix.
-int bdirect_tile_m();
-bool bdirect_shape_ok(int N, int K);
-hipError_t launch_grouped_bdirect(const GroupedArgs& a, WeightKind wk, hipStream_t s);
+// bf16 matrix-core path (bf16 activations; bf16 or int8 weights): weights repacked into
+// matrix-core operand order (pack_weight_*) and streamed global -> registers, activations
+// global -> LDS by DMA.  `w` must have been packed matrix by matrix.
+int stream_tile_m();
+bool stream_shape_ok(int N, int K);
+hipError_t launch_grouped_stream(const GroupedArgs& a, WeightKind wk, int variant, hipStream_t s);  // variant 0..1
 void pack_weight_bf16(const uint16_t* src, int rows, int cols, uint16_t* dst);
 void pack_weight_i8(const int8_t* src, int rows, int cols, int8_t* dst);
 

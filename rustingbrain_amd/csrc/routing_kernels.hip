@@ -16,60 +16,6 @@
 
 namespace rbmoe {
 
-// ---------------------------------------------------------------------------
-// Eight-lane dot product in the order of the reference's `dot`
-// (src/matrix.rs:26-40): lanes[c % 8] += x[c] * w[c] below the tail, a scalar
-// `rest` for the remaining columns, lanes folded left to right, rest last.
-// Multiply and add are rounded separately, as in the reference.
-// ---------------------------------------------------------------------------
-template <typename XT>
-__device__ __forceinline__ void load8(const XT* p, float (&v)[8]);
-
-template <>
-__device__ __forceinline__ void load8<float>(const float* p, float (&v)[8]) {
-    const float4 a = *reinterpret_cast<const float4*>(p);
-    const float4 b = *reinterpret_cast<const float4*>(p + 4);
-    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
-    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-}
-
-template <>
-__device__ __forceinline__ void load8<bf16_t>(const bf16_t* p, float (&v)[8]) {
-    const uint4 a = *reinterpret_cast<const uint4*>(p);
-    v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xffff0000u);
-    v[2] = __uint_as_float(a.y << 16); v[3] = __uint_as_float(a.y & 0xffff0000u);
-    v[4] = __uint_as_float(a.z << 16); v[5] = __uint_as_float(a.z & 0xffff0000u);
-    v[6] = __uint_as_float(a.w << 16); v[7] = __uint_as_float(a.w & 0xffff0000u);
-}
-
-template <typename XT>
-__device__ __forceinline__ float dot8(const XT* __restrict__ x, const float* __restrict__ w, int d,
-                                      bool vec) {
-    float lanes[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    const int tail = d - d % 8;
-    if (vec) {
-        for (int c = 0; c < tail; c += 8) {
-            float xv[8], wv[8];
-            load8<XT>(x + c, xv);
-            load8<float>(w + c, wv);
-#pragma unroll
-            for (int l = 0; l < 8; ++l) lanes[l] = __fadd_rn(lanes[l], __fmul_rn(xv[l], wv[l]));
-        }
-    } else {
-        for (int c = 0; c < tail; c += 8) {
-#pragma unroll
-            for (int l = 0; l < 8; ++l)
-                lanes[l] = __fadd_rn(lanes[l], __fmul_rn(to_f32(x[c + l]), w[c + l]));
-        }
-    }
-    float rest = 0.0f;
-    for (int c = tail; c < d; ++c) rest = __fadd_rn(rest, __fmul_rn(to_f32(x[c]), w[c]));
-    float sum = 0.0f;
-#pragma unroll
-    for (int l = 0; l < 8; ++l) sum = __fadd_rn(sum, lanes[l]);
-    return __fadd_rn(sum, rest);
-}
-
 // Dynamic LDS layout of router_kernel (floats / ints, in this order):
 //   prob   [TB][ES]   logits, then exp, then probabilities   (ES = E | 1)
 //   lsev   [TB]       log-sum-exp per token
@@ -77,12 +23,23 @@ __device__ __forceinline__ float dot8(const XT* __restrict__ x, const float* __r
 //   lexp   [TB][k]    selected expert per local slot (-1 = unrouted)
 //   wcount [4][E]     per-wave match counts of one ranking round
 //   running[E]        slots already ranked per expert
-//   taken  [TB][E]    bytes
-size_t router_lds_bytes(int E, int k) {
+//   taken  [TB][E]    bytes (padded to a multiple of 16)
+//   xs     [TB][kRouterChunk + 4]  f32 slice of the token rows
+//   ws     [min(E, 64)][kRouterChunk + 4]  f32 slice of the router rows of one pass
+constexpr int kRouterChunk = 128;              // columns staged per step (a multiple of 8)
+constexpr int kRouterStride = kRouterChunk + 4; // +4 floats: rows start 4 banks apart
+constexpr int kRouterPassExperts = 64;         // experts per pass (8 per thread)
+
+__host__ __device__ static size_t router_fixed_bytes(int E, int k) {
     const int ES = E | 1;
-    size_t n = (size_t)kRouterTokens * ES + kRouterTokens + 2 * (size_t)kRouterTokens * k +
-               4 * (size_t)E + E;
-    return n * 4 + (size_t)kRouterTokens * E;
+    size_t n = (size_t)kRouterTokens * ES + kRouterTokens + 2 * (size_t)kRouterTokens * k + 4 * (size_t)E + E;
+    size_t bytes = n * 4 + (size_t)kRouterTokens * E;
+    return (bytes + 15) & ~(size_t)15;
+}
+
+size_t router_lds_bytes(int E, int k) {
+    const int wrows = E < kRouterPassExperts ? E : kRouterPassExperts;
+    return router_fixed_bytes(E, k) + (size_t)(kRouterTokens + wrows) * kRouterStride * 4;
 }
 
 template <typename XT>
@@ -107,14 +64,74 @@ __global__ __launch_bounds__(256) void router_kernel(
     const int t0 = blk * TB;
     const int nt = min(TB, T - t0);
 
-    // ---- logits: one (token, expert) pair per thread per pass -------------
-    const bool vec = (d % 8 == 0);
-    for (int idx = tid; idx < nt * E; idx += 256) {
-        const int i = idx / E;
-        const int e = idx - i * E;
-        float v = dot8<XT>(x + (size_t)(t0 + i) * d, wr + (size_t)e * d, d, vec);
-        if (bias) v = __fadd_rn(v, bias[e]);
-        prob[i * ES + e] = v;
+    // ---- logits ----------------------------------------------------------------
+    // Thread (t = tid % 32, eg = tid / 32) owns token t and experts eg, eg + 8, ... of the
+    // current pass, eight lane accumulators each, exactly the reference `dot`: lanes[c % 8]
+    // += x[c] * w[c] in increasing c, a rounded multiply then a rounded add.  Token and
+    // router rows are staged in LDS slice by slice (coalesced loads, converted to f32).
+    float* xs = reinterpret_cast<float*>(lds_raw + router_fixed_bytes(E, k));
+    float* ws = xs + TB * kRouterStride;
+    const int tl = tid & 31;
+    const int eg = tid >> 5;
+    const int tail = d - d % 8;
+    for (int e0 = 0; e0 < E; e0 += kRouterPassExperts) {
+        const int pe = min(kRouterPassExperts, E - e0);  // experts in this pass
+        float lanes[8][8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+            for (int l = 0; l < 8; ++l) lanes[j][l] = 0.0f;
+        for (int c0 = 0; c0 < tail; c0 += kRouterChunk) {
+            const int clen = min(kRouterChunk, tail - c0);
+            __syncthreads();
+            for (int idx = tid; idx < TB * clen; idx += 256) {
+                const int r = idx / clen, c = idx - r * clen;
+                xs[r * kRouterStride + c] = r < nt ? to_f32(x[(size_t)(t0 + r) * d + c0 + c]) : 0.0f;
+            }
+            for (int idx = tid; idx < pe * clen; idx += 256) {
+                const int r = idx / clen, c = idx - r * clen;
+                ws[r * kRouterStride + c] = wr[(size_t)(e0 + r) * d + c0 + c];
+            }
+            __syncthreads();
+            const float* xrow = xs + tl * kRouterStride;
+            for (int c = 0; c < clen; c += 8) {
+                const float4 xa = *reinterpret_cast<const float4*>(xrow + c);
+                const float4 xb = *reinterpret_cast<const float4*>(xrow + c + 4);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int el = eg + 8 * j;
+                    if (el < pe) {
+                        const float* wrow = ws + el * kRouterStride + c;
+                        const float4 wa = *reinterpret_cast<const float4*>(wrow);
+                        const float4 wb = *reinterpret_cast<const float4*>(wrow + 4);
+                        lanes[j][0] = __fadd_rn(lanes[j][0], __fmul_rn(xa.x, wa.x));
+                        lanes[j][1] = __fadd_rn(lanes[j][1], __fmul_rn(xa.y, wa.y));
+                        lanes[j][2] = __fadd_rn(lanes[j][2], __fmul_rn(xa.z, wa.z));
+                        lanes[j][3] = __fadd_rn(lanes[j][3], __fmul_rn(xa.w, wa.w));
+                        lanes[j][4] = __fadd_rn(lanes[j][4], __fmul_rn(xb.x, wb.x));
+                        lanes[j][5] = __fadd_rn(lanes[j][5], __fmul_rn(xb.y, wb.y));
+                        lanes[j][6] = __fadd_rn(lanes[j][6], __fmul_rn(xb.z, wb.z));
+                        lanes[j][7] = __fadd_rn(lanes[j][7], __fmul_rn(xb.w, wb.w));
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int el = eg + 8 * j;
+            if (el < pe && tl < nt) {
+                const int e = e0 + el;
+                float rest = 0.0f;
+                for (int c = tail; c < d; ++c)
+                    rest = __fadd_rn(rest, __fmul_rn(to_f32(x[(size_t)(t0 + tl) * d + c]), wr[(size_t)e * d + c]));
+                float sum = 0.0f;
+#pragma unroll
+                for (int l = 0; l < 8; ++l) sum = __fadd_rn(sum, lanes[j][l]);
+                float v = __fadd_rn(sum, rest);
+                if (bias) v = __fadd_rn(v, bias[e]);
+                prob[tl * ES + e] = v;
+            }
+        }
     }
     for (int idx = tid; idx < TB * E; idx += 256) taken[idx] = 0;
     for (int idx = tid; idx < E; idx += 256) running[idx] = 0;
@@ -467,6 +484,13 @@ __global__ __launch_bounds__(256) void combine_kernel(
 template <typename XT>
 static hipError_t launch_router_t(const RouterArgs& a, hipStream_t s) {
     const int nb = (a.T + kRouterTokens - 1) / kRouterTokens;
+    static bool attr_set = false;
+    if (!attr_set) {  // allow more than the default 64 KiB of dynamic LDS (gfx950 has 160 KiB per CU)
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(router_kernel<XT>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kMaxRouterLds);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
     hipLaunchKernelGGL(router_kernel<XT>, dim3(nb), dim3(256), router_lds_bytes(a.E, a.k), s,
                        static_cast<const XT*>(a.x), a.wr, a.bias, a.valid, a.T, a.d, a.E, a.k, a.P,
                        a.lse, a.expert_of, a.gate_of, a.rank_in_block, a.blockcnt, a.partial);

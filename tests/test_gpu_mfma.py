@@ -1,6 +1,5 @@
 """The bf16 matrix-core path of the grouped expert products against the oracle,
-for every tile configuration the library carries: ragged groups, partial tiles
-in both directions, padding rows, empty experts, a shared expert of another
+ragged groups, partial tiles in both directions, padding rows, empty experts, a shared expert of another
 width, int8 weights, and the explicit-gather variant."""
 import os
 
@@ -14,13 +13,11 @@ from rustingbrain_amd import synth
 
 pytestmark = pytest.mark.gpu
 
-NUM_CONFIGS = 7
 
 
 @pytest.fixture
 def kernel_env():
-    keys = ("RBMOE_GATE_UP_CFG", "RBMOE_DOWN_CFG", "RBMOE_GROUP_M", "RBMOE_EXPLICIT_GATHER", "RBMOE_FORCE_GENERIC",
-            "RBMOE_EXPERT_PATH")
+    keys = ("RBMOE_GROUP_M", "RBMOE_EXPLICIT_GATHER", "RBMOE_FORCE_GENERIC", "RBMOE_STREAM_VARIANT")
     saved = {k: os.environ.get(k) for k in keys}
     yield os.environ
     for k, v in saved.items():
@@ -47,28 +44,13 @@ def run(device, t, valid=None, bias=None):
     return err
 
 
-@pytest.mark.parametrize("cfg", range(NUM_CONFIGS))
-@pytest.mark.parametrize("wt", ["bf16", "int8"])
-def test_every_tile_configuration_of_the_lds_staged_kernels(device, kernel_env, cfg, wt):
-    kernel_env["RBMOE_EXPERT_PATH"] = "lds"
-    kernel_env["RBMOE_GATE_UP_CFG"] = str(cfg)
-    kernel_env["RBMOE_DOWN_CFG"] = str(cfg)
-    # F = 192 leaves a partial column tile; 700 tokens over 6 experts leave partial row tiles
-    t = synth.make(small_workload(d=128, E=6, k=2, F=192, T=700, seed=17, act="bf16", wt=wt, shared=True,
-                                  shared_d_ff=320))
-    bias = np.zeros(6, np.float32)
-    bias[1] = 1.5   # one large group ...
-    bias[4] = -50   # ... and one empty expert
-    valid = (np.arange(700) % 9 != 4).astype(np.uint8)
-    run(device, t, valid=valid, bias=bias)
-
-
 @pytest.mark.parametrize("wt", ["bf16", "int8"])
 @pytest.mark.parametrize("shape", [dict(d=128, E=6, k=2, F=192, T=700), dict(d=64, E=3, k=1, F=64, T=130),
                                    dict(d=256, E=16, k=4, F=128, T=333), dict(d=192, E=5, k=2, F=320, T=1000)],
                          ids=lambda s: "d{d}_E{E}_k{k}_F{F}_T{T}".format(**s))
-def test_packed_weight_kernels(device, kernel_env, shape, wt):
-    kernel_env["RBMOE_EXPERT_PATH"] = "bdirect"
+@pytest.mark.parametrize("variant", [0, 1])
+def test_matrix_core_kernels(device, kernel_env, shape, wt, variant):
+    kernel_env["RBMOE_STREAM_VARIANT"] = str(variant)
     E = shape["E"]
     t = synth.make(small_workload(seed=19, act="bf16", wt=wt, shared=True, shared_d_ff=shape["F"] + 64, **shape))
     bias = np.zeros(E, np.float32)
@@ -102,14 +84,8 @@ def test_matrix_core_and_generic_paths_agree(device, kernel_env):
     t = synth.make(small_workload(d=64, E=4, k=2, F=64, T=257, seed=31, act="bf16", wt="bf16", shared=True))
     layer = gpu_layer(device, t)
     a, _ = layer.forward_train(t.x)
-    assert layer.kernel_name() == "mfma_bf16_packed"
+    assert layer.kernel_name() == "mfma_bf16_stream"
     layer.close()
-    kernel_env["RBMOE_EXPERT_PATH"] = "lds"
-    layer = gpu_layer(device, t)
-    c, _ = layer.forward_train(t.x)
-    assert layer.kernel_name() == "mfma_bf16_lds"
-    layer.close()
-    assert rel_l2(a, c) < 1e-2
     kernel_env["RBMOE_FORCE_GENERIC"] = "1"
     layer = gpu_layer(device, t)
     b, _ = layer.forward_train(t.x)
