@@ -1,9 +1,9 @@
 // Router, dispatch and combine kernels of the mixture-of-experts forward pass
 // for gfx950 (wave64).
 //
-//   router_kernel   logits (the reference's eight-lane `dot` order), softmax,
-//                   log-sum-exp, deterministic top-k, per-block ranks and
-//                   histogram, per-block partial sums for the auxiliary losses
+//   logits_kernel   router logits in the reference's eight-lane `dot` order
+//   router_kernel   softmax, log-sum-exp, deterministic top-k, per-block ranks
+//                   and histogram, per-block partial sums for the auxiliary losses
 //   scan_kernel     prefix scan over blocks and experts, tile table for the
 //                   grouped products, the two auxiliary losses
 //   dispatch_kernel stable permutation (slot -> position) and row gather
@@ -24,12 +24,6 @@ namespace rbmoe {
 //   wcount [4][E]     per-wave match counts of one ranking round
 //   running[E]        slots already ranked per expert
 //   taken  [TB][E]    bytes (padded to a multiple of 16)
-//   xs     [TB][kRouterChunk + 4]  f32 slice of the token rows
-//   ws     [min(E, 64)][kRouterChunk + 4]  f32 slice of the router rows of one pass
-constexpr int kRouterChunk = 128;              // columns staged per step (a multiple of 8)
-constexpr int kRouterStride = kRouterChunk + 4; // +4 floats: rows start 4 banks apart
-constexpr int kRouterPassExperts = 64;         // experts per pass (8 per thread)
-
 __host__ __device__ static size_t router_fixed_bytes(int E, int k) {
     const int ES = E | 1;
     size_t n = (size_t)kRouterTokens * ES + kRouterTokens + 2 * (size_t)kRouterTokens * k + 4 * (size_t)E + E;
@@ -38,8 +32,131 @@ __host__ __device__ static size_t router_fixed_bytes(int E, int k) {
 }
 
 size_t router_lds_bytes(int E, int k) {
-    const int wrows = E < kRouterPassExperts ? E : kRouterPassExperts;
-    return router_fixed_bytes(E, k) + (size_t)(kRouterTokens + wrows) * kRouterStride * 4;
+    return router_fixed_bytes(E, k);
+}
+
+// ---------------------------------------------------------------------------
+// logits_kernel: logits[t, e] = dot(x[t, :], w[e, :]) (+ bias[e]) in the order of the
+// reference's eight-lane `dot` (src/matrix.rs:26-40): lanes[c % 8] += x[c] * w[c] in
+// increasing c (a rounded multiply, then a rounded add), a scalar `rest` for the columns
+// past the last multiple of 8, lanes folded left to right, rest added last.
+//
+// A workgroup owns 64 tokens x 8 experts.  Lane = token; each of the 4 waves owns 2 experts,
+// so a router row is wave-uniform and is fetched with scalar loads (it costs neither vector
+// memory bandwidth nor LDS), while the token rows are staged through LDS in slices of
+// kLogitChunk columns (16-byte pieces, rows padded by 16 bytes so that a wave's 64 row reads
+// spread over all banks).
+// ---------------------------------------------------------------------------
+constexpr int kLogitTokens = 64;
+constexpr int kLogitExperts = 8;
+constexpr int kLogitChunk = 256;
+
+template <typename XT>
+struct XPiece;  // 8 consecutive elements of a token row
+template <>
+struct XPiece<bf16_t> {
+    typedef uint4 raw_t;
+    static __device__ __forceinline__ void widen(const raw_t& a, float (&v)[8]) {
+        v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xffff0000u);
+        v[2] = __uint_as_float(a.y << 16); v[3] = __uint_as_float(a.y & 0xffff0000u);
+        v[4] = __uint_as_float(a.z << 16); v[5] = __uint_as_float(a.z & 0xffff0000u);
+        v[6] = __uint_as_float(a.w << 16); v[7] = __uint_as_float(a.w & 0xffff0000u);
+    }
+};
+template <>
+struct XPiece<float> {
+    struct raw_t {
+        float4 a, b;
+    };
+    static __device__ __forceinline__ void widen(const raw_t& r, float (&v)[8]) {
+        v[0] = r.a.x; v[1] = r.a.y; v[2] = r.a.z; v[3] = r.a.w;
+        v[4] = r.b.x; v[5] = r.b.y; v[6] = r.b.z; v[7] = r.b.w;
+    }
+};
+
+template <typename XT>
+__global__ __launch_bounds__(256) void logits_kernel(const XT* __restrict__ x, const float* __restrict__ wr,
+                                                     const float* __restrict__ bias, int T, int d, int E,
+                                                     float* __restrict__ logits) {
+    typedef typename XPiece<XT>::raw_t piece_t;
+    constexpr int PIECES = kLogitChunk / 8;          // pieces per row per slice
+    constexpr int STRIDE = PIECES + (sizeof(piece_t) == 16 ? 1 : 1);  // +1 piece of padding per row
+    __shared__ piece_t xs[kLogitTokens * STRIDE];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int t0 = blockIdx.x * kLogitTokens;
+    const int nt = min(kLogitTokens, T - t0);
+    const int e0 = blockIdx.y * kLogitExperts + wave * 2;  // this wave's experts e0, e0 + 1
+    const bool has0 = e0 < E, has1 = e0 + 1 < E;
+    const float* w0 = wr + (size_t)(has0 ? e0 : 0) * d;
+    const float* w1 = wr + (size_t)(has1 ? e0 + 1 : 0) * d;
+    const int tail = d - d % 8;
+    float la[8], lb[8];
+#pragma unroll
+    for (int l = 0; l < 8; ++l) {
+        la[l] = 0.0f;
+        lb[l] = 0.0f;
+    }
+    const bool vec = d % 8 == 0;
+    for (int c0 = 0; c0 < tail; c0 += kLogitChunk) {
+        const int np = min(PIECES, (tail - c0) / 8);  // pieces in this slice
+        __syncthreads();
+        for (int idx = tid; idx < kLogitTokens * np; idx += 256) {
+            const int r = idx / np, q = idx - r * np;
+            piece_t v = {};
+            if (r < nt) {
+                const XT* src = x + (size_t)(t0 + r) * d + c0 + 8 * q;
+                if (vec) {
+                    v = *reinterpret_cast<const piece_t*>(src);
+                } else {  // rows are not 16-byte aligned: gather the eight elements
+                    XT tmp[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) tmp[j] = src[j];
+                    v = *reinterpret_cast<const piece_t*>(tmp);
+                }
+            }
+            xs[r * STRIDE + q] = v;
+        }
+        __syncthreads();
+        if (has0) {
+            const float* wa = w0 + c0;
+            const float* wb = w1 + c0;
+#pragma unroll 4
+            for (int q = 0; q < np; ++q) {
+                float xv[8];
+                XPiece<XT>::widen(xs[lane * STRIDE + q], xv);
+#pragma unroll
+                for (int l = 0; l < 8; ++l) la[l] = __fadd_rn(la[l], __fmul_rn(xv[l], wa[8 * q + l]));
+                if (has1) {
+#pragma unroll
+                    for (int l = 0; l < 8; ++l) lb[l] = __fadd_rn(lb[l], __fmul_rn(xv[l], wb[8 * q + l]));
+                }
+            }
+        }
+    }
+    if (lane < nt && has0) {
+        const XT* xr = x + (size_t)(t0 + lane) * d;
+        float rest0 = 0.0f, rest1 = 0.0f;
+        for (int c = tail; c < d; ++c) {
+            const float xv = to_f32(xr[c]);
+            rest0 = __fadd_rn(rest0, __fmul_rn(xv, w0[c]));
+            rest1 = __fadd_rn(rest1, __fmul_rn(xv, w1[c]));
+        }
+        float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+        for (int l = 0; l < 8; ++l) {
+            s0 = __fadd_rn(s0, la[l]);
+            s1 = __fadd_rn(s1, lb[l]);
+        }
+        float v0 = __fadd_rn(s0, rest0), v1 = __fadd_rn(s1, rest1);
+        if (bias) {
+            v0 = __fadd_rn(v0, bias[e0]);
+            if (has1) v1 = __fadd_rn(v1, bias[e0 + 1]);
+        }
+        logits[(size_t)(t0 + lane) * E + e0] = v0;
+        if (has1) logits[(size_t)(t0 + lane) * E + e0 + 1] = v1;
+    }
 }
 
 template <typename XT>
@@ -64,74 +181,10 @@ __global__ __launch_bounds__(256) void router_kernel(
     const int t0 = blk * TB;
     const int nt = min(TB, T - t0);
 
-    // ---- logits ----------------------------------------------------------------
-    // Thread (t = tid % 32, eg = tid / 32) owns token t and experts eg, eg + 8, ... of the
-    // current pass, eight lane accumulators each, exactly the reference `dot`: lanes[c % 8]
-    // += x[c] * w[c] in increasing c, a rounded multiply then a rounded add.  Token and
-    // router rows are staged in LDS slice by slice (coalesced loads, converted to f32).
-    float* xs = reinterpret_cast<float*>(lds_raw + router_fixed_bytes(E, k));
-    float* ws = xs + TB * kRouterStride;
-    const int tl = tid & 31;
-    const int eg = tid >> 5;
-    const int tail = d - d % 8;
-    for (int e0 = 0; e0 < E; e0 += kRouterPassExperts) {
-        const int pe = min(kRouterPassExperts, E - e0);  // experts in this pass
-        float lanes[8][8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-#pragma unroll
-            for (int l = 0; l < 8; ++l) lanes[j][l] = 0.0f;
-        for (int c0 = 0; c0 < tail; c0 += kRouterChunk) {
-            const int clen = min(kRouterChunk, tail - c0);
-            __syncthreads();
-            for (int idx = tid; idx < TB * clen; idx += 256) {
-                const int r = idx / clen, c = idx - r * clen;
-                xs[r * kRouterStride + c] = r < nt ? to_f32(x[(size_t)(t0 + r) * d + c0 + c]) : 0.0f;
-            }
-            for (int idx = tid; idx < pe * clen; idx += 256) {
-                const int r = idx / clen, c = idx - r * clen;
-                ws[r * kRouterStride + c] = wr[(size_t)(e0 + r) * d + c0 + c];
-            }
-            __syncthreads();
-            const float* xrow = xs + tl * kRouterStride;
-            for (int c = 0; c < clen; c += 8) {
-                const float4 xa = *reinterpret_cast<const float4*>(xrow + c);
-                const float4 xb = *reinterpret_cast<const float4*>(xrow + c + 4);
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const int el = eg + 8 * j;
-                    if (el < pe) {
-                        const float* wrow = ws + el * kRouterStride + c;
-                        const float4 wa = *reinterpret_cast<const float4*>(wrow);
-                        const float4 wb = *reinterpret_cast<const float4*>(wrow + 4);
-                        lanes[j][0] = __fadd_rn(lanes[j][0], __fmul_rn(xa.x, wa.x));
-                        lanes[j][1] = __fadd_rn(lanes[j][1], __fmul_rn(xa.y, wa.y));
-                        lanes[j][2] = __fadd_rn(lanes[j][2], __fmul_rn(xa.z, wa.z));
-                        lanes[j][3] = __fadd_rn(lanes[j][3], __fmul_rn(xa.w, wa.w));
-                        lanes[j][4] = __fadd_rn(lanes[j][4], __fmul_rn(xb.x, wb.x));
-                        lanes[j][5] = __fadd_rn(lanes[j][5], __fmul_rn(xb.y, wb.y));
-                        lanes[j][6] = __fadd_rn(lanes[j][6], __fmul_rn(xb.z, wb.z));
-                        lanes[j][7] = __fadd_rn(lanes[j][7], __fmul_rn(xb.w, wb.w));
-                    }
-                }
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int el = eg + 8 * j;
-            if (el < pe && tl < nt) {
-                const int e = e0 + el;
-                float rest = 0.0f;
-                for (int c = tail; c < d; ++c)
-                    rest = __fadd_rn(rest, __fmul_rn(to_f32(x[(size_t)(t0 + tl) * d + c]), wr[(size_t)e * d + c]));
-                float sum = 0.0f;
-#pragma unroll
-                for (int l = 0; l < 8; ++l) sum = __fadd_rn(sum, lanes[j][l]);
-                float v = __fadd_rn(sum, rest);
-                if (bias) v = __fadd_rn(v, bias[e]);
-                prob[tl * ES + e] = v;
-            }
-        }
+    // ---- logits were written to P by logits_kernel ------------------------------
+    for (int idx = tid; idx < nt * E; idx += 256) {
+        const int i = idx / E;
+        prob[i * ES + (idx - i * E)] = P[(size_t)t0 * E + idx];
     }
     for (int idx = tid; idx < TB * E; idx += 256) taken[idx] = 0;
     for (int idx = tid; idx < E; idx += 256) running[idx] = 0;
@@ -443,11 +496,114 @@ __global__ __launch_bounds__(256) void dispatch_kernel(
 // order of gate * y[pos,:] (a rounded multiply then a rounded add, as
 // src/moe.rs:294-311), then + shared[t,:] (src/moe.rs:313-319), then
 // + residual[t,:].  Ascending expert order is ascending position order.
-// One wave per token; eight columns per lane per step when d allows.
+// One thread per (token, 16-byte column piece); the token's slots are sorted
+// by position in registers when k <= KMAX, otherwise found by repeated search.
 // ---------------------------------------------------------------------------
-template <typename XT, typename YT>
-__global__ __launch_bounds__(256) void combine_kernel(
-    const YT* __restrict__ y, const YT* __restrict__ yshared, const XT* __restrict__ residual,
+template <typename T>
+struct Vec16;
+template <>
+struct Vec16<float> {
+    static constexpr int N = 4;
+    static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+        const float4 a = *reinterpret_cast<const float4*>(p);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    }
+    static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
+        *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    }
+};
+template <>
+struct Vec16<bf16_t> {
+    static constexpr int N = 8;
+    static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[8]) {
+        const uint4 a = *reinterpret_cast<const uint4*>(p);
+        v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xffff0000u);
+        v[2] = __uint_as_float(a.y << 16); v[3] = __uint_as_float(a.y & 0xffff0000u);
+        v[4] = __uint_as_float(a.z << 16); v[5] = __uint_as_float(a.z & 0xffff0000u);
+        v[6] = __uint_as_float(a.w << 16); v[7] = __uint_as_float(a.w & 0xffff0000u);
+    }
+    static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[8]) {
+        uint4 o;
+        o.x = f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16);
+        o.y = f32_to_bf16_bits(v[2]) | ((uint32_t)f32_to_bf16_bits(v[3]) << 16);
+        o.z = f32_to_bf16_bits(v[4]) | ((uint32_t)f32_to_bf16_bits(v[5]) << 16);
+        o.w = f32_to_bf16_bits(v[6]) | ((uint32_t)f32_to_bf16_bits(v[7]) << 16);
+        *reinterpret_cast<uint4*>(p) = o;
+    }
+};
+
+template <typename XT, int KMAX>
+__global__ __launch_bounds__(256) void combine_vec_kernel(
+    const XT* __restrict__ y, const XT* __restrict__ yshared, const XT* __restrict__ residual,
+    const int* __restrict__ inv_pos, const float* __restrict__ gate_of, int T, int d, int k,
+    XT* __restrict__ out) {
+    constexpr int VN = Vec16<XT>::N;
+    const int pieces = d / VN;
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (long long)T * pieces) return;
+    const int t = (int)(idx / pieces);
+    const int c = (int)(idx - (long long)t * pieces) * VN;
+    // the token's routed slots, sorted by position (insertion sort on registers)
+    int pos[KMAX];
+    float gate[KMAX];
+    int n = 0;
+#pragma unroll
+    for (int r = 0; r < KMAX; ++r) {
+        pos[r] = 0x7fffffff;
+        gate[r] = 0.0f;
+    }
+#pragma unroll
+    for (int r = 0; r < KMAX; ++r) {
+        if (r < k) {
+            int p = inv_pos[(size_t)t * k + r];
+            float g = gate_of[(size_t)t * k + r];
+            if (p >= 0) {
+                ++n;
+#pragma unroll
+                for (int q = 0; q < KMAX; ++q) {
+                    if (p < pos[q]) {
+                        const int tp = pos[q];
+                        const float tg = gate[q];
+                        pos[q] = p;
+                        gate[q] = g;
+                        p = tp;
+                        g = tg;
+                    }
+                }
+            }
+        }
+    }
+    float acc[VN];
+#pragma unroll
+    for (int i = 0; i < VN; ++i) acc[i] = 0.0f;
+#pragma unroll
+    for (int r = 0; r < KMAX; ++r) {
+        if (r < n) {
+            float v[VN];
+            Vec16<XT>::load(y + (size_t)pos[r] * d + c, v);
+#pragma unroll
+            for (int i = 0; i < VN; ++i) acc[i] = __fadd_rn(acc[i], __fmul_rn(gate[r], v[i]));
+        }
+    }
+    if (yshared) {
+        float v[VN];
+        Vec16<XT>::load(yshared + (size_t)t * d + c, v);
+#pragma unroll
+        for (int i = 0; i < VN; ++i) acc[i] = __fadd_rn(acc[i], v[i]);
+    }
+    if (residual) {
+        float v[VN];
+        Vec16<XT>::load(residual + (size_t)t * d + c, v);
+#pragma unroll
+        for (int i = 0; i < VN; ++i) acc[i] = __fadd_rn(acc[i], v[i]);
+    }
+    Vec16<XT>::store(out + (size_t)t * d + c, acc);
+}
+
+// Any k, any d: one wave per token, one column per lane per step.
+template <typename XT>
+__global__ __launch_bounds__(256) void combine_any_kernel(
+    const XT* __restrict__ y, const XT* __restrict__ yshared, const XT* __restrict__ residual,
     const int* __restrict__ inv_pos, const float* __restrict__ gate_of, int T, int d, int k,
     XT* __restrict__ out) {
     const int lane = threadIdx.x & 63;
@@ -459,8 +615,7 @@ __global__ __launch_bounds__(256) void combine_kernel(
         float acc = 0.0f;
         int last = -1;
         for (int r = 0; r < k; ++r) {
-            // next smallest position greater than `last`
-            int best = 0x7fffffff, bi = -1;
+            int best = 0x7fffffff, bi = -1;  // next smallest position greater than `last`
             for (int q = 0; q < k; ++q) {
                 const int p = ip[q];
                 if (p > last && p < best) {
@@ -491,9 +646,14 @@ static hipError_t launch_router_t(const RouterArgs& a, hipStream_t s) {
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    hipLaunchKernelGGL(router_kernel<XT>, dim3(nb), dim3(256), router_lds_bytes(a.E, a.k), s,
-                       static_cast<const XT*>(a.x), a.wr, a.bias, a.valid, a.T, a.d, a.E, a.k, a.P,
-                       a.lse, a.expert_of, a.gate_of, a.rank_in_block, a.blockcnt, a.partial);
+    const dim3 lgrid((a.T + kLogitTokens - 1) / kLogitTokens, (a.E + kLogitExperts - 1) / kLogitExperts);
+    hipLaunchKernelGGL((logits_kernel<XT>), lgrid, dim3(256), 0, s,
+                       static_cast<const XT*>(a.x), a.wr, a.bias, a.T, a.d, a.E, a.P);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((router_kernel<XT>), dim3(nb), dim3(256), router_lds_bytes(a.E, a.k), s,
+                       static_cast<const XT*>(a.x), a.wr, a.bias, a.valid, a.T, a.d, a.E, a.k, a.P, a.lse,
+                       a.expert_of, a.gate_of, a.rank_in_block, a.blockcnt, a.partial);
     return hipGetLastError();
 }
 
@@ -525,20 +685,32 @@ hipError_t launch_dispatch(const DispatchArgs& a, bool bf16, hipStream_t s) {
     return bf16 ? launch_dispatch_t<bf16_t>(a, s) : launch_dispatch_t<float>(a, s);
 }
 
+template <typename XT>
+static hipError_t launch_combine_t(const CombineArgs& a, hipStream_t s) {
+    const XT* y = static_cast<const XT*>(a.y);
+    const XT* ys = static_cast<const XT*>(a.yshared);
+    const XT* res = static_cast<const XT*>(a.residual);
+    XT* out = static_cast<XT*>(a.out);
+    constexpr int VN = Vec16<XT>::N;
+    if (a.d % VN == 0 && a.k <= 8) {
+        const long long total = (long long)a.T * (a.d / VN);
+        const dim3 grid((unsigned)((total + 255) / 256)), block(256);
+        if (a.k <= 2)
+            hipLaunchKernelGGL((combine_vec_kernel<XT, 2>), grid, block, 0, s, y, ys, res, a.inv_pos, a.gate_of, a.T, a.d, a.k, out);
+        else if (a.k <= 4)
+            hipLaunchKernelGGL((combine_vec_kernel<XT, 4>), grid, block, 0, s, y, ys, res, a.inv_pos, a.gate_of, a.T, a.d, a.k, out);
+        else
+            hipLaunchKernelGGL((combine_vec_kernel<XT, 8>), grid, block, 0, s, y, ys, res, a.inv_pos, a.gate_of, a.T, a.d, a.k, out);
+    } else {
+        hipLaunchKernelGGL((combine_any_kernel<XT>), dim3((a.T + 3) / 4), dim3(256), 0, s, y, ys, res, a.inv_pos,
+                           a.gate_of, a.T, a.d, a.k, out);
+    }
+    return hipGetLastError();
+}
+
 hipError_t launch_combine(const CombineArgs& a, bool bf16, hipStream_t s) {
     if (a.T <= 0) return hipSuccess;
-    const dim3 grid((a.T + 3) / 4), block(256);
-    if (bf16)
-        hipLaunchKernelGGL((combine_kernel<bf16_t, bf16_t>), grid, block, 0, s,
-                           static_cast<const bf16_t*>(a.y), static_cast<const bf16_t*>(a.yshared),
-                           static_cast<const bf16_t*>(a.residual), a.inv_pos, a.gate_of, a.T, a.d,
-                           a.k, static_cast<bf16_t*>(a.out));
-    else
-        hipLaunchKernelGGL((combine_kernel<float, float>), grid, block, 0, s,
-                           static_cast<const float*>(a.y), static_cast<const float*>(a.yshared),
-                           static_cast<const float*>(a.residual), a.inv_pos, a.gate_of, a.T, a.d,
-                           a.k, static_cast<float*>(a.out));
-    return hipGetLastError();
+    return bf16 ? launch_combine_t<bf16_t>(a, s) : launch_combine_t<float>(a, s);
 }
 
 }  // namespace rbmoe
