@@ -32,6 +32,11 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_F32_TFLOPS = 157.3     # MI355X fp32 matrix
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
+# HBM-side bytes per launch of the gate/up kernel, measured with rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (each scaled by the reading of a 256 MiB copy; profiles/c3_prefill_hbm_traffic.txt).
+# Valid only for the workload and kernel it was measured on.
+MEASURED_TRAFFIC = {("c3_prefill_d768_e16", "mfma_bf16_stream"): 264.6e6}
+
 
 class DeviceBuffer:
     def __init__(self, dev: rb.Device, nbytes: int):
@@ -110,6 +115,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="c3_prefill_d768_e16", choices=list(synth.WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 256 MiB device-to-device copy (the plain copy that FETCH_SIZE / "
+                         "WRITE_SIZE readings are scaled by when this command runs under rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -171,7 +179,8 @@ def main() -> int:
                     "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": whole / PEAK_HBM_GBS, "traffic": None}
     else:
         roofline = {"bound": "mfma", "kernel": "grouped gate/up product + SwiGLU (" + layer.kernel_name() + ")",
-                    "achieved": gu, "peak": peak_tf, "unit": "TFLOP/s", "frac": gu / peak_tf, "traffic": None,
+                    "achieved": gu, "peak": peak_tf, "unit": "TFLOP/s", "frac": gu / peak_tf,
+                    "traffic": MEASURED_TRAFFIC.get((w.name, layer.kernel_name())),
                     "flops_per_launch": alg["gate_up_flops"], "avg_launch_ms": stage_ms["gate_up"]}
     both_ms = stage_ms["gate_up"] + stage_ms["down"] + stage_ms["shared"]
     stages = {
@@ -199,6 +208,12 @@ def main() -> int:
         "roofline": roofline,
         "stages": stages,
     }
+    if args.calibrate_copy:
+        n = 256 << 20
+        a, b = DeviceBuffer(dev, n), DeviceBuffer(dev, n)
+        assert dev._lib.rbmoe_copy_device(dev.handle, C.c_void_p(b.ptr), C.c_void_p(a.ptr), n) == L.OK
+        a.free()
+        b.free()
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(t)
     print(json.dumps(result))

@@ -197,6 +197,9 @@ int rbmoe_device_alloc(rbmoe_ctx* ctx, size_t bytes, void** out);
 int rbmoe_device_free(rbmoe_ctx* ctx, void* ptr);
 int rbmoe_copy_to_device(rbmoe_ctx* ctx, void* dst, const void* src, size_t bytes);
 int rbmoe_copy_to_host(rbmoe_ctx* ctx, void* dst, const void* src, size_t bytes);
+/* Device-to-device copy on the context's stream, then synchronise (also serves as the
+ * plain copy of known size that hardware-counter readings are calibrated against). */
+int rbmoe_copy_device(rbmoe_ctx* ctx, void* dst, const void* src, size_t bytes);
 
 const char* rbmoe_version(void);
 

@@ -66,6 +66,7 @@ SIGNATURES = {
     "rbmoe_device_free": (C.c_int, [C.c_void_p, C.c_void_p]),
     "rbmoe_copy_to_device": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
     "rbmoe_copy_to_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
+    "rbmoe_copy_device": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
     "rbmoe_version": (C.c_char_p, []),
 }
 

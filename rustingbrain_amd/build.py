@@ -50,7 +50,22 @@ def build(jobs: int = 4) -> str:
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError("link failed:\n" + res.stderr)
+    build_host()
     return LIB
+
+
+HOST = os.path.join(HERE, "host")
+TUTORIAL = os.path.join(HOST, "moe_tutorial")
+
+
+def build_host() -> str:
+    """The C++ host mirror's driver (rustingbrain_amd/host/moe_tutorial), linked against librbmoe.so."""
+    cmd = ["g++", "-O2", "-std=c++17", "-Wall", os.path.join(HOST, "moe_tutorial.cpp"), "-o", TUTORIAL,
+           "-L" + HERE, "-lrbmoe", "-Wl,-rpath,$ORIGIN/.."]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("host build failed:\n" + res.stderr)
+    return TUTORIAL
 
 
 if __name__ == "__main__":

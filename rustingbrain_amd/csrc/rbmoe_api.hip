@@ -843,4 +843,13 @@ int rbmoe_copy_to_host(rbmoe_ctx* ctx, void* dst, const void* src, size_t bytes)
     return RBMOE_OK;
 }
 
+int rbmoe_copy_device(rbmoe_ctx* ctx, void* dst, const void* src, size_t bytes) {
+    if (!ctx) return fail(nullptr, RBMOE_NULL_POINTER, "ctx is NULL");
+    if (bytes == 0) return RBMOE_OK;
+    if (!dst || !src) return fail(ctx, RBMOE_NULL_POINTER, "dst or src is NULL");
+    HIP_TRY(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return RBMOE_OK;
+}
+
 }  // extern "C"

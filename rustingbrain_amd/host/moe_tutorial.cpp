@@ -1,0 +1,182 @@
+// Drives a bare mixture-of-experts layer through the C++ host mirror, the way the
+// reference's tutorial does (tutorials/code/15_mixture_of_experts.rs:58-120): the
+// total-vs-active parameter table, then the load fractions and the two auxiliary losses
+// for varied and for identical tokens.  It also asserts the reference's own unit-test
+// expectations, so it doubles as the test of the C++ host side.
+//
+//   moe_tutorial --cpu-checks   configuration, accounting and error paths only (no GPU)
+//   moe_tutorial                everything, on GPU 0
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+
+#include "rusting_brain_moe.hpp"
+
+using namespace rusting_brain;
+
+static int failures = 0;
+#define EXPECT(cond)                                                   \
+    do {                                                               \
+        if (!(cond)) {                                                 \
+            std::printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond); \
+            ++failures;                                                \
+        }                                                              \
+    } while (0)
+
+template <typename E, typename F>
+static bool throws(F f) {
+    try {
+        f();
+    } catch (const E&) {
+        return true;
+    } catch (...) {
+        return false;
+    }
+    return false;
+}
+
+// small deterministic generator (values in [-1, 1)); the tutorial's StdRng stream cannot be reproduced
+static float unit(uint64_t& s) {
+    s = s * 6364136223846793005ull + 1442695040888963407ull;
+    return (float)((s >> 40) & 0xffffff) / 8388608.0f - 1.0f;
+}
+static Matrix random_matrix(size_t r, size_t c, float bound, uint64_t seed) {
+    Matrix m(r, c);
+    uint64_t s = seed * 2654435761ull + 12345;
+    for (float& v : m.data) v = unit(s) * bound;
+    return m;
+}
+
+static void cpu_checks() {
+    // reference src/moe.rs:704-710
+    EXPECT(throws<InvalidConfig>([] { MoeConfig(4, 0, 6).validate(); }));
+    EXPECT(throws<InvalidConfig>([] { MoeConfig(4, 5, 6).validate(); }));
+    EXPECT(throws<InvalidConfig>([] { MoeConfig(0, 1, 6).validate(); }));
+    MoeConfig(4, 4, 6).validate();
+    // reference README.md:96: 55.2M total / 35.7M active for the default configuration
+    const ParameterCounts c = TransformerBuilder().parameter_counts();
+    EXPECT(c.total == 55181824ull && c.active == 35717632ull);
+    // reference src/transformer.rs:3020-3026
+    auto tiny = [] { return TransformerBuilder().n_layers(2).moe_layers({1}).experts(4, 2); };
+    EXPECT(throws<InvalidConfig>([&] { tiny().heads(4, 3, 4).validate(); }));
+    EXPECT(throws<InvalidConfig>([&] { tiny().heads(4, 2, 5).validate(); }));
+    EXPECT(throws<InvalidConfig>([&] { tiny().moe_layers({9}).validate(); }));
+    EXPECT(throws<InvalidConfig>([&] { tiny().experts(2, 4).validate(); }));
+    // reference src/batch.rs:254-268
+    std::vector<bool> mask = {true, false, true};
+    Layout bad;
+    bad.valid = &mask;
+    EXPECT(throws<InvalidConfig>([&] { bad.check(4); }));
+    Layout seq;
+    seq.seq_len = 4;
+    EXPECT(throws<InvalidConfig>([&] { seq.check(9); }));
+
+    std::printf("== Total vs active, as experts are added ==\n\nexperts   total    active    ratio\n");
+    for (size_t n : {1, 2, 4, 8, 16, 32}) {
+        const ParameterCounts p = TransformerBuilder().experts(n, n < 2 ? n : 2).parameter_counts();
+        std::printf("%7zu %6.1fM %7.1fM %7.2fx\n", n, p.total / 1e6, p.active / 1e6, (double)p.total / p.active);
+    }
+}
+
+static void report(const char* label, MoeLayer& layer, const Matrix& tokens, size_t experts) {
+    auto result = layer.forward_train(tokens, Layout{});
+    const MoeCache& cache = result.second;
+    const std::vector<float> loads = cache.load_fractions();
+    float busiest = 0.0f;
+    size_t dead = 0;
+    std::printf("%s\n  routing ", label);
+    for (float share : loads) {
+        std::printf("%6.1f%%", share * 100.0f);
+        busiest = std::fmax(busiest, share);
+        dead += share < 0.01f;
+    }
+    std::printf("\n  busiest %.1f%%   dead experts %zu/%zu   aux %.4f   z %.4f\n", busiest * 100.0f, dead, experts,
+                cache.aux_loss(), cache.z_loss());
+}
+
+static void gpu_checks() {
+    const size_t D = 64, E = 8, K = 2, F = 32, ROWS = 512;
+    auto device = Device::open(0);
+    MoeLayer layer(D, MoeConfig(E, K, F), device, ROWS);
+    const float bound = std::sqrt(6.0f / (float)(D + F));
+    layer.set_router(random_matrix(E, D, std::sqrt(6.0f / (float)(D + E)), 7));
+    for (size_t e = 0; e < E; ++e)
+        layer.set_expert(e, random_matrix(F, D, bound, 100 + 3 * e), random_matrix(F, D, bound, 101 + 3 * e),
+                         random_matrix(D, F, bound, 102 + 3 * e));
+
+    std::printf("\n== What the load-balancing loss measures ==\n\n");
+    const Matrix varied = random_matrix(ROWS, D, 1.0f, 11);
+    report("varied tokens, balanced routing:", layer, varied, E);
+    Matrix same(ROWS, D);
+    const Matrix one = random_matrix(1, D, 1.0f, 13);
+    for (size_t r = 0; r < ROWS; ++r) std::memcpy(same.row_mut(r), one.data.data(), D * sizeof(float));
+    report("identical tokens, collapsed routing:", layer, same, E);
+
+    // reference tutorials/15_mixture_of_experts.md:310-312: exactly two experts at 50 %, six dead
+    {
+        auto r = layer.forward_train(same, Layout{});
+        size_t half = 0, zero = 0;
+        for (float f : r.second.load_fractions()) {
+            half += f == 0.5f;
+            zero += f == 0.0f;
+        }
+        EXPECT(half == 2 && zero == E - 2);
+    }
+    // reference src/moe.rs:696-702, :726-741, :757-765
+    {
+        auto r = layer.forward_train(varied, Layout{});
+        EXPECT(r.first.rows == ROWS && r.first.cols == D);
+        size_t routed = 0;
+        for (const auto& v : r.second.expert_tokens) routed += v.size();
+        EXPECT(routed == ROWS * K);
+        bool sums_ok = true;
+        for (size_t t = 0; t < ROWS; ++t) {
+            float total = 0.0f;
+            for (size_t q = 0; q < K; ++q) total += r.second.assignments[t * K + q].second;
+            sums_ok = sums_ok && std::fabs(total - 1.0f) < 1e-5f;
+        }
+        EXPECT(sums_ok);
+        EXPECT(r.second.aux_loss() >= 0.01f - 1e-6f && r.second.aux_loss() <= (float)E * 0.01f + 1e-6f);
+        EXPECT(r.second.z_loss() > 0.0f);
+    }
+    // reference src/moe.rs:248-253
+    EXPECT(throws<InvalidInput>([&] { layer.forward(Matrix(3, D + 1)); }));
+    // padding rows are routed nowhere (reference src/moe.rs:559-562)
+    {
+        std::vector<bool> mask(ROWS, true);
+        mask[5] = false;
+        Layout layout;
+        layout.valid = &mask;
+        auto r = layer.forward_train(varied, layout);
+        EXPECT(r.second.assignments[5 * K].first == UNROUTED && r.second.assignments[5 * K].second == 0.0f);
+        EXPECT(r.second.valid_tokens == ROWS - 1);
+        bool zero_row = true;
+        for (size_t c = 0; c < D; ++c) zero_row = zero_row && r.first.row(5)[c] == 0.0f;
+        EXPECT(zero_row);
+    }
+    // the builder surface hands out one layer per index in moe_layers
+    {
+        auto layers = TransformerBuilder().d_model(16).n_layers(4).experts(4, 2).moe_layers({1, 3}).moe_d_ff(12)
+                          .shared_expert(true).build_moe_layers(device, 8);
+        EXPECT(layers.size() == 2 && layers.count(1) && layers.count(3));
+        EXPECT(layers[1]->num_parameters() == 4 * 16 + 5 * 3 * 16 * 12);
+    }
+    // a budget that cannot hold the layer is refused before anything is allocated
+    EXPECT(throws<MemoryBudget>([&] {
+        auto small = Device::open(0, 1);
+        MoeLayer big(768, MoeConfig(8, 2, 1408), small, 1024);
+    }));
+}
+
+int main(int argc, char** argv) {
+    const bool cpu_only = argc > 1 && std::strcmp(argv[1], "--cpu-checks") == 0;
+    try {
+        cpu_checks();
+        if (!cpu_only) gpu_checks();
+    } catch (const std::exception& e) {
+        std::printf("FAILED with exception: %s\n", e.what());
+        return 2;
+    }
+    std::printf(failures ? "\n%d check(s) FAILED\n" : "\nall checks passed%.0d\n", failures);
+    return failures ? 1 : 0;
+}
