@@ -64,40 +64,80 @@ __device__ __forceinline__ bf16x8 widen_i8(uint2 q) {
     return __builtin_bit_cast(bf16x8, w);
 }
 
-// s_waitcnt vmcnt(N) only (expcnt and lgkmcnt left at their maxima), gfx9 encoding.
+// Token fragment read from LDS.
+__device__ __forceinline__ bf16x8 lds_frag(const uint4* __restrict__ base, int idx) {
+    return __builtin_bit_cast(bf16x8, base[idx]);
+}
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// Every vector-memory instruction of the main loop is issued from inline assembly and waited
+// for by hand.  Left to the compiler, any wait that falls while an LDS-DMA is in flight
+// becomes vmcnt(0), which drains the whole weight ring and the DMA just issued once per
+// slice; and loads from read-only memory may be moved across the barriers the hand-written
+// counts rely on.  Loads retire in order, so "at most N outstanding" proves that everything
+// but the N youngest has landed; N is always the exact number of younger instructions.
+__device__ __forceinline__ void issue_load(u32x4& d, uint32_t byte_off, const char* base) {
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(d) : "v"(byte_off), "s"(base));
+}
+__device__ __forceinline__ void issue_load(u32x2& d, uint32_t byte_off, const char* base) {
+    asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(d) : "v"(byte_off), "s"(base));
+}
+// 64 lanes x 16 bytes from `src` (per lane) to LDS bytes [lds_addr, lds_addr + 1024).
+__device__ __forceinline__ void issue_dma(uint32_t lds_addr, const char* src) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(src) : "memory");
+}
+// Wait until at most N loads are outstanding; the two registers become usable only here.
+template <int N, typename V>
+__device__ __forceinline__ void wait_for(V& a, V& b) {
+    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+}
 template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-    __builtin_amdgcn_s_waitcnt((N & 0xF) | (0x7 << 4) | (0xF << 8) | ((N >> 4) << 14));
+__device__ __forceinline__ void wait_outstanding() {
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>), in order
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
 }
 
 // One ring slot: the wave's two weight fragments of one reduction step.
-// bf16: 16 bytes per lane per fragment.  int8: 8 bytes per lane per fragment.
+// bf16: 16 bytes per lane per fragment, step g at byte 1024 g + 16 lane of a row block.
+// int8: 8 bytes per lane per fragment; the packed layout is [K/32][64 lanes][16 bytes] with
+//       bytes 0..7 for the even step and 8..15 for the odd one.
 template <bool I8>
 struct Slot;
 template <>
 struct Slot<false> {
-    uint4 f0, f1;
-    __device__ __forceinline__ void load(const char* p0, const char* p1, int g, int lane) {
-        f0 = reinterpret_cast<const uint4*>(p0)[(size_t)g * 64 + lane];
-        f1 = reinterpret_cast<const uint4*>(p1)[(size_t)g * 64 + lane];
+    u32x4 f0, f1;
+    __device__ __forceinline__ void load(const char* p0, const char* p1, int g, uint32_t lane16) {
+        const uint32_t off = lane16 + (uint32_t)g * 1024u;
+        issue_load(f0, off, p0);
+        issue_load(f1, off, p1);
     }
     __device__ __forceinline__ bf16x8 a0() const { return __builtin_bit_cast(bf16x8, f0); }
     __device__ __forceinline__ bf16x8 a1() const { return __builtin_bit_cast(bf16x8, f1); }
 };
 template <>
 struct Slot<true> {
-    uint2 f0, f1;
-    // packed int8 layout: [K/32][64 lanes][16 bytes]; bytes 0..7 belong to the even step, 8..15 to the odd one
-    __device__ __forceinline__ void load(const char* p0, const char* p1, int g, int lane) {
-        const size_t idx = ((size_t)(g >> 1) * 64 + lane) * 2 + (g & 1);
-        f0 = reinterpret_cast<const uint2*>(p0)[idx];
-        f1 = reinterpret_cast<const uint2*>(p1)[idx];
+    u32x2 f0, f1;
+    __device__ __forceinline__ void load(const char* p0, const char* p1, int g, uint32_t lane16) {
+        const uint32_t off = lane16 + (uint32_t)(g >> 1) * 1024u + (uint32_t)(g & 1) * 8u;
+        issue_load(f0, off, p0);
+        issue_load(f1, off, p1);
     }
-    __device__ __forceinline__ bf16x8 a0() const { return widen_i8(f0); }
-    __device__ __forceinline__ bf16x8 a1() const { return widen_i8(f1); }
+    __device__ __forceinline__ bf16x8 a0() const { return widen_i8(make_uint2(f0.x, f0.y)); }
+    __device__ __forceinline__ bf16x8 a1() const { return widen_i8(make_uint2(f1.x, f1.y)); }
 };
 
-// RING = weight-fragment steps in flight per wave (register ring depth).
+// RING = weight-fragment steps in flight per wave (register ring depth);
+// TFBUF = 2: token fragments are read from LDS one step ahead, 1: just in time.
 template <bool SWIGLU, bool I8, int RING, int TFBUF>
 __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
     const bf16_t* __restrict__ a, const int* __restrict__ row_index, const void* __restrict__ wpacked,
@@ -105,7 +145,9 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
     const int* __restrict__ tile_expert, const int* __restrict__ tile_row0, const int* __restrict__ tile_rows,
     const int* __restrict__ ntiles, int dense_rows, bf16_t* __restrict__ out, int group_m) {
     constexpr int BN = SWIGLU ? NW * 32 : NW * 64;  // output features per workgroup
-    __shared__ uint4 As[2][BM * CPR];
+    // Two LDS stages, each always addressed through a compile-time constant.
+    __shared__ uint4 As0[BM * CPR];
+    __shared__ uint4 As1[BM * CPR];
 
     // ---- which tile (each XCD walks a contiguous range, M fastest inside a group)
     const int tiles_n = (N + BN - 1) / BN;
@@ -141,6 +183,9 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
     // ---- this wave's two blocks of 32 weight rows ---------------------------
+    // A wave whose rows lie past N (ragged last feature tile) runs the same loop on row
+    // block 0, so that every wave issues the same loads and meets the same barriers; it
+    // stores nothing.
     const int nw = tn_idx * BN + wave * (SWIGLU ? 32 : 64);
     const int r0 = nw, r1 = SWIGLU ? N + nw : nw + 32;
     const bool act0 = nw < N;
@@ -149,30 +194,28 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
     const char* wexp = static_cast<const char*>(wpacked) + (size_t)expert * w_expert_stride_bytes;
     const char* wp0 = wexp + (size_t)(act0 ? r0 / 32 : 0) * block_bytes;
     const char* wp1 = wexp + (size_t)(act1 ? r1 / 32 : 0) * block_bytes;
+    const uint32_t lane16 = (uint32_t)lane * 16u;
 
     // ---- LDS-DMA of the activation slice --------------------------------------
     // Wave w fills LDS rows [32 w, 32 w + 32): instruction j covers rows 32 w + 8 j .. + 7,
     // lane l lands in row 8 j + l / 8 (of the wave's 32), position l % 8, and therefore
     // fetches logical piece (l % 8) ^ (row % 8).  Rows past the end of the group are
     // clamped to the tile's first row: their products are never stored.
-    const uint4* a_pieces = reinterpret_cast<const uint4*>(a);
-    const int kp = K / 8;
-    uint32_t a_off[DMA_PER_WAVE];
+    const char* a_src[DMA_PER_WAVE];
 #pragma unroll
     for (int j = 0; j < DMA_PER_WAVE; ++j) {
         const int r = wave * 32 + j * 8 + (lane >> 3);
         const int rr = r < rows ? r : 0;
         const int grow = row_index ? row_index[row0 + rr] : row0 + rr;
-        a_off[j] = (uint32_t)grow * (uint32_t)kp + ((lane & 7) ^ (r & 7));
+        a_src[j] = reinterpret_cast<const char*>(a) + ((size_t)grow * K + 8 * ((lane & 7) ^ (r & 7))) * 2;
     }
-    auto dma_a = [&](int kt, int buf) {
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)As0 + wave * 32 * CPR * 16;
+    const uint32_t lds1 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)As1 + wave * 32 * CPR * 16;
+    auto dma_a = [&](int kt, auto buf_tag) {
+        constexpr int BUF = decltype(buf_tag)::value;
 #pragma unroll
-        for (int j = 0; j < DMA_PER_WAVE; ++j) {
-            const uint4* src = a_pieces + a_off[j] + kt * CPR;
-            uint4* dst = &As[buf][(wave * 32 + j * 8) * CPR];
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                             (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
-        }
+        for (int j = 0; j < DMA_PER_WAVE; ++j)
+            issue_dma((BUF ? lds1 : lds0) + j * 8 * CPR * 16, a_src[j] + (size_t)kt * (BK * 2));
     };
 
     floatx16 acc[2][TT];
@@ -189,99 +232,92 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
 
     const int KT = K / BK;
     const int GS = KT * KS;  // reduction steps in all
+    constexpr int D = RING - 1;  // the load for step g + D is issued while step g runs
 
-    // ---- prologue: first activation slice, first RING-1 weight steps ----------
-    dma_a(0, 0);
-    __builtin_amdgcn_sched_barrier(0);
+    // ---- prologue: first activation slice, first D weight steps -----------------
+    dma_a(0, std::integral_constant<int, 0>{});
     Slot<I8> ring[RING];
-    if (act0) {
 #pragma unroll
-        for (int g = 0; g < RING - 1; ++g)
-            if (g < GS) ring[g].load(wp0, wp1, g, lane);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    wait_vmcnt<0>();  // first slice must be in LDS (this also drains the first weight loads: prologue only)
+    for (int g = 0; g < D; ++g) ring[g].load(wp0, wp1, min(g, GS - 1), lane16);
+    wait_outstanding<0>();
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
 
-    // One slice = KS steps.  `G0` is the ring position of the slice's first step (0 or 4).
+    // One slice = KS steps.  BUF is the LDS stage the slice reads (its parity); the ring
+    // position of the slice's first step is 0, or BUF * KS when the ring holds two slices.
     // NB = token blocks of this tile that hold rows, a compile-time constant inside the
     // loop: a run-time branch per block between the multiplies costs far more than the
     // skipped multiplies save, so the whole loop is specialised instead.
-    auto slice = [&](int kt, auto g0_tag, auto nb_tag) {
-        constexpr int G0 = decltype(g0_tag)::value;
+    // The loop is straight-line and every wave issues, per slice, exactly: 4 DMA
+    // instructions, then 2 weight loads in each of the KS steps.  Past the end the last
+    // slice / step is fetched again, so that the counts below hold everywhere.
+    auto slice = [&](int kt, auto buf_tag, auto nb_tag) {
+        constexpr int BUF = decltype(buf_tag)::value;
+        constexpr int G0 = RING == 2 * KS ? BUF * KS : 0;
         constexpr int NB = decltype(nb_tag)::value;
-        const int buf = kt & 1;
-        const bool more = kt + 1 < KT;
-        if (more) dma_a(kt + 1, buf ^ 1);
-        __builtin_amdgcn_sched_barrier(0);
-        if (act0) {
-            const uint4* Ab = As[buf];
-            bf16x8 tf[TFBUF][TT];
+        dma_a(min(kt + 1, KT - 1), std::integral_constant<int, BUF ^ 1>{});
+        const uint4* Ab = BUF ? As1 : As0;
+        bf16x8 tf[TFBUF][TT];
 #pragma unroll
-            for (int t = 0; t < NB; ++t) tf[0][t] = __builtin_bit_cast(bf16x8, Ab[(t * 32 + lrow) * CPR + (lhalf ^ lxor)]);
+        for (int t = 0; t < NB; ++t) tf[0][t] = lds_frag(Ab, (t * 32 + lrow) * CPR + (lhalf ^ lxor));
+        static_for<0, KS>([&](auto s_tag) {
+            constexpr int s = decltype(s_tag)::value;
+            const int g = kt * KS + s;
+            Slot<I8>& cur = ring[(G0 + s) % RING];
+            // weight fragments for step g + D go into the slot step g - 1 released
+            ring[(G0 + s + D) % RING].load(wp0, wp1, min(g + D, GS - 1), lane16);
+            if constexpr (TFBUF == 2) {
+                if (s + 1 < KS) {
+                    const int piece = (2 * (s + 1) + lhalf) ^ lxor;
 #pragma unroll
-            for (int s = 0; s < KS; ++s) {
-                const int g = kt * KS + s;
-                // weight fragments for step g + RING - 1 go into the slot step g - 1 released
-                if (g + RING - 1 < GS) ring[(G0 + s + RING - 1) % RING].load(wp0, wp1, g + RING - 1, lane);
-                if constexpr (TFBUF == 2) {
-                    if (s + 1 < KS) {
-                        const int piece = (2 * (s + 1) + lhalf) ^ lxor;
-#pragma unroll
-                        for (int t = 0; t < NB; ++t)
-                            tf[(s + 1) & 1][t] = __builtin_bit_cast(bf16x8, Ab[(t * 32 + lrow) * CPR + piece]);
-                    }
-                } else if (s > 0) {
-                    const int piece = (2 * s + lhalf) ^ lxor;
-#pragma unroll
-                    for (int t = 0; t < NB; ++t) tf[0][t] = __builtin_bit_cast(bf16x8, Ab[(t * 32 + lrow) * CPR + piece]);
+                    for (int t = 0; t < NB; ++t) tf[(s + 1) & 1][t] = lds_frag(Ab, (t * 32 + lrow) * CPR + piece);
                 }
-                const bf16x8 w0 = ring[(G0 + s) % RING].a0();
-                const bf16x8 w1 = ring[(G0 + s) % RING].a1();
+            } else if (s > 0) {
+                const int piece = (2 * s + lhalf) ^ lxor;
 #pragma unroll
-                for (int t = 0; t < NB; ++t) {
-                    acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w0, tf[s % TFBUF][t], acc[0][t], 0, 0, 0);
-                    acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w1, tf[s % TFBUF][t], acc[1][t], 0, 0, 0);
-                }
+                for (int t = 0; t < NB; ++t) tf[0][t] = lds_frag(Ab, (t * 32 + lrow) * CPR + piece);
             }
-        }
+            // Younger than the loads of step g: the weight loads of steps g+1 .. g+D (2 each)
+            // and the DMA (4) of every slice that started after they were issued.
+            wait_for<2 * D + DMA_PER_WAVE * ((D - s + KS - 1) / KS)>(cur.f0, cur.f1);
+            const bf16x8 w0 = cur.a0();
+            const bf16x8 w1 = cur.a1();
+#pragma unroll
+            for (int t = 0; t < NB; ++t) {
+                acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w0, tf[s % TFBUF][t], acc[0][t], 0, 0, 0);
+                acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w1, tf[s % TFBUF][t], acc[1][t], 0, 0, 0);
+            }
+        });
+        // Every LDS read of this slice has been consumed by a multiply issued above this
+        // point.  The DMA of the next slice is older than this slice's 2 * KS weight loads.
         __builtin_amdgcn_sched_barrier(0);
-        // The DMA of the next slice was issued before this slice's weight loads.  Once at
-        // most that many loads are outstanding, the DMA has landed (loads retire in order).
-        if (more) {
-            if (act0 && (kt + 1) * KS - 1 + RING - 1 < GS)
-                wait_vmcnt<2 * KS>();  // every step of this slice issued its two weight loads
-            else
-                wait_vmcnt<0>();
-        }
-        // A bare barrier: every LDS read of this slice has already been consumed by a
-        // multiply, and the DMA wait above is the only other thing the next slice needs.
-        // (__syncthreads() would drain the whole weight ring with a vmcnt(0).)
+        wait_outstanding<2 * KS>();
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    // The ring position of a slice's first step alternates between 0 and KS when the ring
-    // holds two slices, and is always 0 when it holds one.
     static_assert(RING == KS || RING == 2 * KS, "ring depth is one or two slices");
+    static_assert(DMA_PER_WAVE == 4, "the wait counts assume 4 DMA instructions per wave per slice");
     auto run = [&](auto nb_tag) {
-        if constexpr (RING == KS) {
-            for (int kt = 0; kt < KT; ++kt) slice(kt, std::integral_constant<int, 0>{}, nb_tag);
-        } else {
-            int kt = 0;
-            for (; kt + 1 < KT; kt += 2) {
-                slice(kt, std::integral_constant<int, 0>{}, nb_tag);
-                slice(kt + 1, std::integral_constant<int, KS>{}, nb_tag);
-            }
-            if (kt < KT) slice(kt, std::integral_constant<int, 0>{}, nb_tag);
+        int kt = 0;
+        for (; kt + 1 < KT; kt += 2) {
+            slice(kt, std::integral_constant<int, 0>{}, nb_tag);
+            slice(kt + 1, std::integral_constant<int, 1>{}, nb_tag);
         }
+        if (kt < KT) slice(kt, std::integral_constant<int, 0>{}, nb_tag);
     };
     static_assert(TT == 4, "one specialisation per possible block count");
     if (nblk == 4) run(std::integral_constant<int, 4>{});
     else if (nblk == 3) run(std::integral_constant<int, 3>{});
     else if (nblk == 2) run(std::integral_constant<int, 2>{});
     else run(std::integral_constant<int, 1>{});
+    // The loads fetched again past the end still target ring registers and LDS.  Naming the
+    // registers after the wait keeps them allocated until their data has arrived: a loaded
+    // value the compiler sees no use for would otherwise hand its register to something
+    // live while the load is still in flight.
+    wait_outstanding<0>();
+#pragma unroll
+    for (int i = 0; i < RING; ++i) asm volatile("" : : "v"(ring[i].f0), "v"(ring[i].f1));
     if (!act0) return;
 
     // ---- epilogue -------------------------------------------------------------

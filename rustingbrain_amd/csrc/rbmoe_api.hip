@@ -133,8 +133,8 @@ struct rbmoe_layer {
     Buf swgu, swd;         // shared [2Fs, d], [d, Fs]
     Buf ssgu, ssd;         // shared scales
     // workspace
-    Buf P, lse, expert_of, gate_of, rank_in_block, blockcnt, blockbase, partial;
-    Buf counts, offsets, tile_expert, tile_row0, tile_rows, tile_expert2, tile_row02, tile_rows2, ntiles, losses, mass;
+    Buf P, lse, expert_of, gate_of, rank_in_block, blockcnt, partial;
+    Buf counts, offsets, tile_expert, tile_row0, tile_rows, ntiles, losses;
     Buf perm_slot, perm_token, inv_pos;
     Buf xg, h, y, hs, ys;
     // staging for the host entry point
@@ -186,19 +186,14 @@ Plan make_plan(rbmoe_layer* L) {
     p.add(&L->gate_of, S * 4);
     p.add(&L->rank_in_block, S * 4);
     p.add(&L->blockcnt, nb * E * 4);
-    p.add(&L->blockbase, nb * E * 4);
     p.add(&L->partial, nb * (E + 1) * 4);
     p.add(&L->counts, E * 4);
     p.add(&L->offsets, (E + 1) * 4);
     p.add(&L->tile_expert, (size_t)L->max_tiles * 4);
     p.add(&L->tile_row0, (size_t)L->max_tiles * 4);
     p.add(&L->tile_rows, (size_t)L->max_tiles * 4);
-    p.add(&L->tile_expert2, (size_t)L->max_tiles * 4);
-    p.add(&L->tile_row02, (size_t)L->max_tiles * 4);
-    p.add(&L->tile_rows2, (size_t)L->max_tiles * 4);
     p.add(&L->ntiles, 8);
     p.add(&L->losses, 8);
-    p.add(&L->mass, (E + 1) * 4);
     p.add(&L->perm_slot, S * 4);
     p.add(&L->perm_token, S * 4);
     p.add(&L->inv_pos, S * 4);
@@ -589,10 +584,8 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     auto mark = [&](int i) -> hipError_t { return timed ? hipEventRecord(L->ev[i], s) : hipSuccess; };
     HIP_TRY(ctx, mark(0));
 
-    const int nb = (T + kRouterTokens - 1) / kRouterTokens;
     const bool mfma = L->use_stream;
     const int tile_m0 = mfma ? stream_tile_m() : kGenericTileM;
-    const int tile_m1 = tile_m0;
     L->kernel_name = mfma ? (wk == WeightKind::I8 ? "mfma_bf16_stream_int8w" : "mfma_bf16_stream") : "generic";
     const bool gather_in_product = mfma && !L->explicit_gather;
 
@@ -602,23 +595,22 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     HIP_TRY(ctx, launch_router(ra, abf, s));
     HIP_TRY(ctx, mark(1));
 
-    ScanArgs sa{};
-    sa.blockcnt = (const int*)L->blockcnt.p;
-    sa.blockbase = (int*)L->blockbase.p;
-    sa.partial = (const float*)L->partial.p;
-    sa.nb = nb; sa.E = E; sa.k = k;
-    sa.w_aux = c.aux_loss_weight; sa.w_z = c.router_z_loss_weight;
-    sa.tile_m[0] = tile_m0; sa.tile_m[1] = tile_m1;
-    sa.counts = (int*)L->counts.p; sa.offsets = (int*)L->offsets.p;
-    sa.tile_expert[0] = (int*)L->tile_expert.p; sa.tile_row0[0] = (int*)L->tile_row0.p; sa.tile_rows[0] = (int*)L->tile_rows.p;
-    sa.tile_expert[1] = (int*)L->tile_expert2.p; sa.tile_row0[1] = (int*)L->tile_row02.p; sa.tile_rows[1] = (int*)L->tile_rows2.p;
-    sa.ntiles = (int*)L->ntiles.p; sa.losses = (float*)L->losses.p; sa.mass = (float*)L->mass.p;
-    HIP_TRY(ctx, launch_scan(sa, s));
-    HIP_TRY(ctx, mark(2));
+    HIP_TRY(ctx, mark(2));  // (the scan is part of the dispatch kernel)
 
-    DispatchArgs da{x, (const int*)L->expert_of.p, (const int*)L->rank_in_block.p, (const int*)L->blockbase.p,
-                    (const int*)L->offsets.p, T, d, E, k, (int*)L->perm_slot.p, (int*)L->perm_token.p,
-                    (int*)L->inv_pos.p, gather_in_product ? nullptr : L->xg.p};
+    DispatchArgs da{};
+    da.x = x;
+    da.expert_of = (const int*)L->expert_of.p;
+    da.rank_in_block = (const int*)L->rank_in_block.p;
+    da.blockcnt = (const int*)L->blockcnt.p;
+    da.partial = (const float*)L->partial.p;
+    da.T = T; da.d = d; da.E = E; da.k = k;
+    da.w_aux = c.aux_loss_weight; da.w_z = c.router_z_loss_weight;
+    da.tile_m = tile_m0;
+    da.counts = (int*)L->counts.p; da.offsets = (int*)L->offsets.p;
+    da.tile_expert = (int*)L->tile_expert.p; da.tile_row0 = (int*)L->tile_row0.p; da.tile_rows = (int*)L->tile_rows.p;
+    da.ntiles = (int*)L->ntiles.p; da.losses = (float*)L->losses.p;
+    da.perm_slot = (int*)L->perm_slot.p; da.perm_token = (int*)L->perm_token.p; da.inv_pos = (int*)L->inv_pos.p;
+    da.xg = gather_in_product ? nullptr : L->xg.p;
     HIP_TRY(ctx, launch_dispatch(da, abf, s));
     HIP_TRY(ctx, mark(3));
 
@@ -656,11 +648,6 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     g2.s_expert_stride = (size_t)d;
     g2.N = d;
     g2.K = F;
-    g2.tile_expert = (const int*)L->tile_expert2.p;
-    g2.tile_row0 = (const int*)L->tile_row02.p;
-    g2.tile_rows = (const int*)L->tile_rows2.p;
-    g2.ntiles = (const int*)L->ntiles.p + 1;
-    g2.max_tiles = T > 0 ? (T * k) / tile_m1 + E : 0;
     g2.out = L->y.p;
     g2.swiglu = false;
     HIP_TRY(ctx, run(g2, false));

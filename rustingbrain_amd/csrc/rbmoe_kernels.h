@@ -19,7 +19,7 @@ constexpr int kMaxTopK = 32;
 
 size_t router_lds_bytes(int E, int k);
 constexpr int kMaxRouterLds = 160 * 1024;  // LDS per workgroup on gfx950
-size_t scan_lds_bytes(int E);
+size_t dispatch_lds_bytes(int E, int k);
 
 struct RouterArgs {
     const void* x;       // [T, d] f32 or bf16
@@ -37,31 +37,22 @@ struct RouterArgs {
 };
 hipError_t launch_router(const RouterArgs& a, bool bf16, hipStream_t s);
 
-struct ScanArgs {
-    const int* blockcnt;  // [nb, E]
-    int* blockbase;       // [nb, E]
-    const float* partial; // [nb, E+1]
-    int nb, E, k;
-    float w_aux, w_z;
-    int tile_m[2];     // rows per tile of the two tile tables (gate/up product, down product)
-    int* counts;       // [E]
-    int* offsets;      // [E+1]
-    int* tile_expert[2];  // [max_tiles] each
-    int* tile_row0[2];
-    int* tile_rows[2];
-    int* ntiles;       // [2]
-    float* losses;     // [2]
-    float* mass;       // [E+1] or null: sum of probabilities per expert, sum of lse^2
-};
-hipError_t launch_scan(const ScanArgs& a, hipStream_t s);
-
 struct DispatchArgs {
     const void* x;
     const int* expert_of;
     const int* rank_in_block;
-    const int* blockbase;
-    const int* offsets;
+    const int* blockcnt;   // [nb, E]    per-block histogram from the router kernel
+    const float* partial;  // [nb, E+1]  per-block sums of probabilities and of lse^2
     int T, d, E, k;
+    float w_aux, w_z;
+    int tile_m;            // rows per tile of the grouped products
+    int* counts;           // [E]
+    int* offsets;          // [E+1]
+    int* tile_expert;      // [max_tiles]
+    int* tile_row0;
+    int* tile_rows;
+    int* ntiles;           // [1]
+    float* losses;         // [2]
     int* perm_slot;
     int* perm_token;
     int* inv_pos;

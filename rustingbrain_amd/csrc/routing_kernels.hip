@@ -4,14 +4,16 @@
 //   logits_kernel   router logits in the reference's eight-lane `dot` order
 //   router_kernel   softmax, log-sum-exp, deterministic top-k, per-block ranks
 //                   and histogram, per-block partial sums for the auxiliary losses
-//   scan_kernel     prefix scan over blocks and experts, tile table for the
-//                   grouped products, the two auxiliary losses
-//   dispatch_kernel stable permutation (slot -> position) and row gather
+//   dispatch_kernel prefix scan over blocks and experts, stable permutation
+//                   (slot -> position), optional row gather; block 0 also writes
+//                   the tile table of the grouped products and the two losses
 //   combine_kernel  gate-weighted sum in ascending expert order, then the
 //                   shared expert, then the optional residual
 //
 // Nothing here uses floating-point atomics: every sum has a fixed order, so two
 // runs give the same bits.
+#include <cstdlib>
+
 #include "rbmoe_kernels.h"
 
 namespace rbmoe {
@@ -23,12 +25,10 @@ namespace rbmoe {
 //   lexp   [TB][k]    selected expert per local slot (-1 = unrouted)
 //   wcount [4][E]     per-wave match counts of one ranking round
 //   running[E]        slots already ranked per expert
-//   taken  [TB][E]    bytes (padded to a multiple of 16)
 __host__ __device__ static size_t router_fixed_bytes(int E, int k) {
     const int ES = E | 1;
     size_t n = (size_t)kRouterTokens * ES + kRouterTokens + 2 * (size_t)kRouterTokens * k + 4 * (size_t)E + E;
-    size_t bytes = n * 4 + (size_t)kRouterTokens * E;
-    return (bytes + 15) & ~(size_t)15;
+    return (n * 4 + 15) & ~(size_t)15;
 }
 
 size_t router_lds_bytes(int E, int k) {
@@ -41,15 +41,15 @@ size_t router_lds_bytes(int E, int k) {
 // increasing c (a rounded multiply, then a rounded add), a scalar `rest` for the columns
 // past the last multiple of 8, lanes folded left to right, rest added last.
 //
-// A workgroup owns 64 tokens x 8 experts.  Lane = token; each of the 4 waves owns 2 experts,
-// so a router row is wave-uniform and is fetched with scalar loads (it costs neither vector
-// memory bandwidth nor LDS), while the token rows are staged through LDS in slices of
-// kLogitChunk columns (16-byte pieces, rows padded by 16 bytes so that a wave's 64 row reads
-// spread over all banks).
+// A workgroup owns 64 tokens x 8 experts: 8 waves, lane = token, one expert per wave, so a
+// router row is wave-uniform and is fetched with scalar loads (it costs neither vector
+// memory bandwidth nor LDS), 64 columns at a time so that their latency is paid once per
+// batch.  The token rows are staged through LDS in slices of kLogitChunk columns (16-byte
+// pieces, rows padded by one piece so that a wave's 64 row reads spread over all banks).
 // ---------------------------------------------------------------------------
 constexpr int kLogitTokens = 64;
-constexpr int kLogitExperts = 8;
 constexpr int kLogitChunk = 256;
+constexpr int kLogitBatch = 8;  // pieces (of 8 columns) per batch of scalar loads
 
 template <typename XT>
 struct XPiece;  // 8 consecutive elements of a token row
@@ -74,35 +74,34 @@ struct XPiece<float> {
     }
 };
 
-template <typename XT>
-__global__ __launch_bounds__(256) void logits_kernel(const XT* __restrict__ x, const float* __restrict__ wr,
-                                                     const float* __restrict__ bias, int T, int d, int E,
-                                                     float* __restrict__ logits) {
+// NE = experts (= waves) per workgroup.
+template <typename XT, int NE>
+__global__ __launch_bounds__(NE * 64) void logits_kernel(const XT* __restrict__ x,
+                                                                const float* __restrict__ wr,
+                                                                const float* __restrict__ bias, int T, int d, int E,
+                                                                float* __restrict__ logits) {
     typedef typename XPiece<XT>::raw_t piece_t;
-    constexpr int PIECES = kLogitChunk / 8;          // pieces per row per slice
-    constexpr int STRIDE = PIECES + (sizeof(piece_t) == 16 ? 1 : 1);  // +1 piece of padding per row
+    constexpr int PIECES = kLogitChunk / 8;  // pieces per row per slice
+    constexpr int STRIDE = PIECES + 1;       // one piece of padding per row
     __shared__ piece_t xs[kLogitTokens * STRIDE];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int t0 = blockIdx.x * kLogitTokens;
     const int nt = min(kLogitTokens, T - t0);
-    const int e0 = blockIdx.y * kLogitExperts + wave * 2;  // this wave's experts e0, e0 + 1
-    const bool has0 = e0 < E, has1 = e0 + 1 < E;
-    const float* w0 = wr + (size_t)(has0 ? e0 : 0) * d;
-    const float* w1 = wr + (size_t)(has1 ? e0 + 1 : 0) * d;
+    constexpr int kLogitThreads = NE * 64;
+    const int e = blockIdx.y * NE + wave;  // this wave's expert
+    const bool has = e < E;
+    const float* w0 = wr + (size_t)(has ? e : 0) * d;
     const int tail = d - d % 8;
-    float la[8], lb[8];
+    float la[8];
 #pragma unroll
-    for (int l = 0; l < 8; ++l) {
-        la[l] = 0.0f;
-        lb[l] = 0.0f;
-    }
+    for (int l = 0; l < 8; ++l) la[l] = 0.0f;
     const bool vec = d % 8 == 0;
     for (int c0 = 0; c0 < tail; c0 += kLogitChunk) {
         const int np = min(PIECES, (tail - c0) / 8);  // pieces in this slice
         __syncthreads();
-        for (int idx = tid; idx < kLogitTokens * np; idx += 256) {
+        for (int idx = tid; idx < kLogitTokens * np; idx += kLogitThreads) {
             const int r = idx / np, q = idx - r * np;
             piece_t v = {};
             if (r < nt) {
@@ -119,43 +118,43 @@ __global__ __launch_bounds__(256) void logits_kernel(const XT* __restrict__ x, c
             xs[r * STRIDE + q] = v;
         }
         __syncthreads();
-        if (has0) {
+        if (has) {
             const float* wa = w0 + c0;
-            const float* wb = w1 + c0;
-#pragma unroll 4
-            for (int q = 0; q < np; ++q) {
+            int q = 0;
+            for (; q + kLogitBatch <= np; q += kLogitBatch) {
+                // one batch: 32 router weights into scalar registers, 4 token pieces from LDS
+                float wv[8 * kLogitBatch];
+#pragma unroll
+                for (int j = 0; j < 8 * kLogitBatch; ++j) wv[j] = wa[8 * q + j];
+                piece_t xp[kLogitBatch];
+#pragma unroll
+                for (int b = 0; b < kLogitBatch; ++b) xp[b] = xs[lane * STRIDE + q + b];
+#pragma unroll
+                for (int b = 0; b < kLogitBatch; ++b) {
+                    float xv[8];
+                    XPiece<XT>::widen(xp[b], xv);
+#pragma unroll
+                    for (int l = 0; l < 8; ++l) la[l] = __fadd_rn(la[l], __fmul_rn(xv[l], wv[8 * b + l]));
+                }
+            }
+            for (; q < np; ++q) {
                 float xv[8];
                 XPiece<XT>::widen(xs[lane * STRIDE + q], xv);
 #pragma unroll
                 for (int l = 0; l < 8; ++l) la[l] = __fadd_rn(la[l], __fmul_rn(xv[l], wa[8 * q + l]));
-                if (has1) {
-#pragma unroll
-                    for (int l = 0; l < 8; ++l) lb[l] = __fadd_rn(lb[l], __fmul_rn(xv[l], wb[8 * q + l]));
-                }
             }
         }
     }
-    if (lane < nt && has0) {
+    if (lane < nt && has) {
         const XT* xr = x + (size_t)(t0 + lane) * d;
-        float rest0 = 0.0f, rest1 = 0.0f;
-        for (int c = tail; c < d; ++c) {
-            const float xv = to_f32(xr[c]);
-            rest0 = __fadd_rn(rest0, __fmul_rn(xv, w0[c]));
-            rest1 = __fadd_rn(rest1, __fmul_rn(xv, w1[c]));
-        }
-        float s0 = 0.0f, s1 = 0.0f;
+        float rest = 0.0f;
+        for (int c = tail; c < d; ++c) rest = __fadd_rn(rest, __fmul_rn(to_f32(xr[c]), w0[c]));
+        float sum = 0.0f;
 #pragma unroll
-        for (int l = 0; l < 8; ++l) {
-            s0 = __fadd_rn(s0, la[l]);
-            s1 = __fadd_rn(s1, lb[l]);
-        }
-        float v0 = __fadd_rn(s0, rest0), v1 = __fadd_rn(s1, rest1);
-        if (bias) {
-            v0 = __fadd_rn(v0, bias[e0]);
-            if (has1) v1 = __fadd_rn(v1, bias[e0 + 1]);
-        }
-        logits[(size_t)(t0 + lane) * E + e0] = v0;
-        if (has1) logits[(size_t)(t0 + lane) * E + e0 + 1] = v1;
+        for (int l = 0; l < 8; ++l) sum = __fadd_rn(sum, la[l]);
+        float v = __fadd_rn(sum, rest);
+        if (bias) v = __fadd_rn(v, bias[e]);
+        logits[(size_t)(t0 + lane) * E + e] = v;
     }
 }
 
@@ -174,7 +173,6 @@ __global__ __launch_bounds__(256) void router_kernel(
     int* lexp = reinterpret_cast<int*>(gates + TB * k);
     int* wcount = lexp + TB * k;
     int* running = wcount + 4 * E;
-    unsigned char* taken = reinterpret_cast<unsigned char*>(running + E);
 
     const int tid = threadIdx.x;
     const int blk = blockIdx.x;
@@ -186,57 +184,121 @@ __global__ __launch_bounds__(256) void router_kernel(
         const int i = idx / E;
         prob[i * ES + (idx - i * E)] = P[(size_t)t0 * E + idx];
     }
-    for (int idx = tid; idx < TB * E; idx += 256) taken[idx] = 0;
     for (int idx = tid; idx < E; idx += 256) running[idx] = 0;
     __syncthreads();
 
-    // ---- softmax + top-k: one token per thread, sequential over experts ---
-    if (tid < nt) {
-        float* row = prob + tid * ES;
-        float mx = __uint_as_float(0xff800000u);
-        for (int e = 0; e < E; ++e) {
-            const float v = row[e];
-            if (v > mx) mx = v;
-        }
-        float sum = 0.0f;
-        for (int e = 0; e < E; ++e) {
-            const float ex = rb_expf(__fadd_rn(row[e], -mx));
-            row[e] = ex;
-            sum = __fadd_rn(sum, ex);
-        }
-        lsev[tid] = __fadd_rn(mx, rb_logf(sum));
-        if (sum > 0.0f)
-            for (int e = 0; e < E; ++e) row[e] = __fdiv_rn(row[e], sum);
-
-        const bool ok = (valid == nullptr) || (valid[t0 + tid] != 0);
-        float* g = gates + tid * k;
-        int* le = lexp + tid * k;
-        if (!ok) {
-            for (int r = 0; r < k; ++r) {
-                le[r] = -1;
-                g[r] = 0.0f;
+    // ---- softmax + top-k: G lanes per token, lane j of a group owns experts j, j + G, ... ----
+    // Everything order-sensitive keeps the reference's order: the maximum ignores NaN
+    // (f32::max), exp(v - max) is summed one expert after the other in index order (every
+    // lane of the group walks the same chain from LDS), the k argmax rounds prefer the
+    // lower index on equal probabilities, and the gates are summed in rank order.
+    {
+        int G = 1;
+        while (G < E && G < 64) G <<= 1;
+        const int lane_ = tid & 63, wave_ = tid >> 6;
+        const int lig = lane_ & (G - 1);          // lane in group
+        const int gbase = lane_ & ~(G - 1);       // first lane of the group
+        const int tpw = 64 / G;                   // tokens a wave handles at once
+        const unsigned long long gmask = (G == 64 ? ~0ull : ((1ull << G) - 1ull)) << gbase;
+        constexpr int MAXJ = kMaxExperts / 64;    // experts per lane when G == 64
+        const float neg_inf = __uint_as_float(0xff800000u);
+        for (int i0 = wave_ * (TB / 4); i0 < (wave_ + 1) * (TB / 4); i0 += tpw) {
+            const int i = i0 + lane_ / G;         // token of this group
+            const bool live = i < nt && i < (wave_ + 1) * (TB / 4);
+            float* row = prob + (live ? i : 0) * ES;
+            float pv[MAXJ];
+            float mx = neg_inf;
+#pragma unroll
+            for (int j = 0; j < MAXJ; ++j) {
+                const int e = lig + G * j;
+                pv[j] = (live && e < E) ? row[e] : neg_inf;
+                const float vv = (pv[j] == pv[j]) ? pv[j] : neg_inf;  // a NaN never becomes the maximum
+                mx = vv > mx ? vv : mx;
             }
-        } else {
-            unsigned char* tk = taken + tid * E;
+            for (int o = 1; o < G; o <<= 1) {
+                const float other = __shfl_xor(mx, o);
+                mx = other > mx ? other : mx;
+            }
+#pragma unroll
+            for (int j = 0; j < MAXJ; ++j) {
+                const int e = lig + G * j;
+                if (live && e < E) {
+                    pv[j] = rb_expf(__fadd_rn(pv[j], -mx));
+                    row[e] = pv[j];
+                }
+            }
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the group's LDS writes have landed
+            __builtin_amdgcn_wave_barrier();
+            float sum = 0.0f;
+            if (live)
+                for (int e = 0; e < E; ++e) sum = __fadd_rn(sum, row[e]);
+            __builtin_amdgcn_wave_barrier();
+            if (live && lig == 0) lsev[i] = __fadd_rn(mx, rb_logf(sum));
+#pragma unroll
+            for (int j = 0; j < MAXJ; ++j) {
+                const int e = lig + G * j;
+                if (live && e < E) {
+                    if (sum > 0.0f) pv[j] = __fdiv_rn(pv[j], sum);
+                    row[e] = pv[j];
+                }
+            }
+            // ---- k rounds of argmax over the experts not yet taken ----
+            const bool ok = live && ((valid == nullptr) || (valid[t0 + i] != 0));
+            unsigned taken_bits = 0;  // bit j: expert lig + G j is taken
+            float total = 0.0f;
             for (int r = 0; r < k; ++r) {
-                int best = -1;
-                float bestv = 0.0f;
-                for (int e = 0; e < E; ++e) {
-                    if (tk[e]) continue;
-                    const float v = row[e];
-                    if (best < 0 || v > bestv) {
-                        best = e;
-                        bestv = v;
+                // first expert not yet taken, and the best non-NaN candidate of this lane
+                int first = 0x7fffffff, ci = 0x7fffffff;
+                float cv = neg_inf;
+#pragma unroll
+                for (int j = MAXJ - 1; j >= 0; --j) {
+                    const int e = lig + G * j;
+                    if (e < E && !((taken_bits >> j) & 1u)) first = e;
+                }
+#pragma unroll
+                for (int j = 0; j < MAXJ; ++j) {
+                    const int e = lig + G * j;
+                    if (e < E && !((taken_bits >> j) & 1u) && pv[j] == pv[j] && (ci == 0x7fffffff || pv[j] > cv)) {
+                        cv = pv[j];
+                        ci = e;
                     }
                 }
-                tk[best] = 1;
-                le[r] = best;
-                g[r] = bestv;
+                for (int o = 1; o < G; o <<= 1) {
+                    const int of = __shfl_xor(first, o);
+                    first = of < first ? of : first;
+                    const float ov = __shfl_xor(cv, o);
+                    const int oi = __shfl_xor(ci, o);
+                    if (oi != 0x7fffffff && (ci == 0x7fffffff || ov > cv || (ov == cv && oi < ci))) {
+                        cv = ov;
+                        ci = oi;
+                    }
+                }
+                // the reference starts from the first untaken expert and replaces it only on a
+                // strictly greater probability: if that first one is NaN nothing replaces it
+                bool first_nan = false;
+#pragma unroll
+                for (int j = 0; j < MAXJ; ++j)
+                    if (lig + G * j == first && pv[j] != pv[j]) first_nan = true;
+                const bool nan_wins = (__ballot(first_nan) & gmask) != 0ull;
+                const int best = (nan_wins || ci == 0x7fffffff) ? first : ci;
+                float mine = 0.0f;
+#pragma unroll
+                for (int j = 0; j < MAXJ; ++j)
+                    if (lig + G * j == best) {
+                        mine = pv[j];
+                        taken_bits |= 1u << j;
+                    }
+                const float bestv = __shfl(mine, gbase + (best & (G - 1)));
+                total = __fadd_rn(total, bestv);
+                if (live && lig == 0) {
+                    lexp[i * k + r] = ok ? best : -1;
+                    gates[i * k + r] = ok ? bestv : 0.0f;
+                }
             }
-            float total = 0.0f;
-            for (int r = 0; r < k; ++r) total = __fadd_rn(total, g[r]);
-            if (total > 0.0f)
-                for (int r = 0; r < k; ++r) g[r] = __fdiv_rn(g[r], total);
+            __builtin_amdgcn_s_waitcnt(0xc07f);
+            __builtin_amdgcn_wave_barrier();
+            if (ok && total > 0.0f)
+                for (int r = lig; r < k; r += G) gates[i * k + r] = __fdiv_rn(gates[i * k + r], total);
         }
     }
     __syncthreads();
@@ -301,169 +363,147 @@ __global__ __launch_bounds__(256) void router_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// scan_kernel: one block of 1024 threads.
-//   blockbase[b][e] = number of slots of expert e in blocks before b
-//   counts[e], offsets[e] (exclusive prefix, offsets[E] = routed slots)
-//   tile table for the grouped products: tile i covers rows
-//   [tile_row0[i], tile_row0[i] + tile_rows[i]) of expert tile_expert[i]
-//   losses[0] = aux, losses[1] = z   (reference src/moe.rs:602-639)
+// dispatch_kernel: block b owns the same 32 tokens as router block b.
+//
+// Prologue (every block, redundantly — the table is a few KB and sits in L2): column sums
+// of the per-block histogram give counts[e], their exclusive prefix gives offsets[e], and
+// the sums over the blocks before b give this block's base per expert.  Block 0 also
+// writes counts / offsets, the tile table of the grouped products (tile i = rows
+// [tile_row0[i], tile_row0[i] + tile_rows[i]) of expert tile_expert[i]; a tile never spans
+// two experts) and the two auxiliary losses (reference src/moe.rs:602-639), folding the
+// per-block partial sums in a fixed order.
+//
+// Position of a routed slot = offsets[e] + base[e] + rank_in_block[slot]: slots are numbered
+// token-major, so this is exactly the order in which the reference appends slots to an
+// expert's list (src/moe.rs:266-274).  The optional row copy is `gather_rows`
+// (src/moe.rs:658-664); rows move as 16-byte pieces.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(1024) void scan_kernel(
-    const int* __restrict__ blockcnt, int* __restrict__ blockbase, const float* __restrict__ partial,
-    int nb, int E, int k, float w_aux, float w_z, int tile_m0, int tile_m1, int* __restrict__ counts,
-    int* __restrict__ offsets, int* __restrict__ tile_expert0, int* __restrict__ tile_row00,
-    int* __restrict__ tile_rows0, int* __restrict__ tile_expert1, int* __restrict__ tile_row01,
-    int* __restrict__ tile_rows1, int* __restrict__ ntiles, float* __restrict__ losses,
-    float* __restrict__ mass_out) {
+size_t dispatch_lds_bytes(int E, int k) {
+    const int parts = 256 / E;
+    return ((size_t)2 * parts * E + (size_t)parts * (E + 1) + 4 * (size_t)(E + 1) + (size_t)kRouterTokens * k) * 4;
+}
+
+template <typename XT>
+__global__ __launch_bounds__(256) void dispatch_kernel(
+    const XT* __restrict__ x, const int* __restrict__ expert_of, const int* __restrict__ rank_in_block,
+    const int* __restrict__ blockcnt, const float* __restrict__ partial, int T, int d, int E, int k,
+    float w_aux, float w_z, int tile_m, int* __restrict__ counts, int* __restrict__ offsets,
+    int* __restrict__ tile_expert, int* __restrict__ tile_row0, int* __restrict__ tile_rows,
+    int* __restrict__ ntiles, float* __restrict__ losses, int* __restrict__ perm_slot,
+    int* __restrict__ perm_token, int* __restrict__ inv_pos, XT* __restrict__ xg) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
-    // LDS: partsum[parts][E] ints, partmass[parts][E+1] floats, cnt[E], off[E+1], toff[2][E+1], mass[E+1]
-    const int parts = 1024 / E;  // E <= 256 -> parts >= 4
-    int* partsum = reinterpret_cast<int*>(lds_raw);
-    float* partmass = reinterpret_cast<float*>(partsum + parts * E);
-    int* cnt = reinterpret_cast<int*>(partmass + parts * (E + 1));
-    int* off = cnt + E;
-    int* toff = off + (E + 1);
-    float* mass = reinterpret_cast<float*>(toff + 2 * (E + 1));
+    constexpr int TB = kRouterTokens;
+    const int parts = 256 / E;  // E <= 256
+    int* part_all = reinterpret_cast<int*>(lds_raw);           // [parts][E]
+    int* part_before = part_all + parts * E;                   // [parts][E]
+    float* part_mass = reinterpret_cast<float*>(part_before + parts * E);  // [parts][E+1] (block 0)
+    int* cnt = reinterpret_cast<int*>(part_mass + parts * (E + 1));        // [E+1]
+    int* base = cnt + (E + 1);                                 // [E+1]
+    int* off = base + (E + 1);                                 // [E+1]
+    float* mass = reinterpret_cast<float*>(off + (E + 1));     // [E+1]
+    int* lpos = reinterpret_cast<int*>(mass + (E + 1));        // [TB * k]
 
     const int tid = threadIdx.x;
+    const int blk = blockIdx.x;
+    const int nb = (T + TB - 1) / TB;
     const int len = (nb + parts - 1) / parts;
     const int p = tid / E;
     const int e = tid - p * E;
     const bool active = p < parts;
-    const int b0 = active ? min(nb, p * len) : 0;
-    const int b1 = active ? min(nb, b0 + len) : 0;
-
     if (active) {
-        int s = 0;
-        float m = 0.0f;
+        const int b0 = min(nb, p * len), b1 = min(nb, b0 + len);
+        int s_all = 0, s_before = 0;
         for (int b = b0; b < b1; ++b) {
-            s += blockcnt[(size_t)b * E + e];
-            m += partial[(size_t)b * (E + 1) + e];
+            const int c = blockcnt[(size_t)b * E + e];
+            s_all += c;
+            s_before += b < blk ? c : 0;
         }
-        partsum[p * E + e] = s;
-        partmass[p * (E + 1) + e] = m;
-        if (e == 0) {
-            float zs = 0.0f;
-            for (int b = b0; b < b1; ++b) zs += partial[(size_t)b * (E + 1) + E];
-            partmass[p * (E + 1) + E] = zs;
+        part_all[p * E + e] = s_all;
+        part_before[p * E + e] = s_before;
+        if (blk == 0) {
+            float m = 0.0f;
+            for (int b = b0; b < b1; ++b) m += partial[(size_t)b * (E + 1) + e];
+            part_mass[p * (E + 1) + e] = m;
+            if (e == 0) {
+                float zs = 0.0f;
+                for (int b = b0; b < b1; ++b) zs += partial[(size_t)b * (E + 1) + E];
+                part_mass[p * (E + 1) + E] = zs;
+            }
         }
     }
     __syncthreads();
     if (tid < E) {
-        int run = 0;
+        int ca = 0, cb = 0;
         float m = 0.0f;
         for (int q = 0; q < parts; ++q) {
-            const int s = partsum[q * E + tid];
-            partsum[q * E + tid] = run;
-            run += s;
-            m += partmass[q * (E + 1) + tid];
+            ca += part_all[q * E + tid];
+            cb += part_before[q * E + tid];
+            if (blk == 0) m += part_mass[q * (E + 1) + tid];
         }
-        cnt[tid] = run;
+        cnt[tid] = ca;
+        base[tid] = cb;
         mass[tid] = m;
     }
-    if (tid == E) {
+    if (blk == 0 && tid == E) {
         float zs = 0.0f;
-        for (int q = 0; q < parts; ++q) zs += partmass[q * (E + 1) + E];
+        for (int q = 0; q < parts; ++q) zs += part_mass[q * (E + 1) + E];
         mass[E] = zs;
     }
     __syncthreads();
-    if (tid == 0) {
-        int run = 0, trun0 = 0, trun1 = 0;
+    if (tid == 0) {  // exclusive prefix over the experts (E <= 256)
+        int run = 0;
         for (int q = 0; q < E; ++q) {
             off[q] = run;
-            toff[q] = trun0;
-            toff[E + 1 + q] = trun1;
             run += cnt[q];
-            trun0 += (cnt[q] + tile_m0 - 1) / tile_m0;
-            trun1 += (cnt[q] + tile_m1 - 1) / tile_m1;
         }
         off[E] = run;
-        toff[E] = trun0;
-        toff[2 * E + 1] = trun1;
-        ntiles[0] = trun0;
-        ntiles[1] = trun1;
-        // auxiliary losses: every valid token routes exactly k slots, so the
-        // number of valid tokens is routed / k.
-        const int V = run / k;
-        float aux = 0.0f, z = 0.0f;
-        if (V > 0) {
-            const float tokens = (float)V;
-            const float slots = (float)V * (float)k;
-            for (int q = 0; q < E; ++q) {
-                const float load = (float)cnt[q] / slots;
-                const float ms = mass[q] / tokens;
-                aux = aux + load * ms;
-            }
-            aux = aux * ((float)E * w_aux);
-            z = w_z * mass[E] / tokens;
-        }
-        losses[0] = aux;
-        losses[1] = z;
     }
     __syncthreads();
-    if (active) {
-        int run = partsum[p * E + e];
-        for (int b = b0; b < b1; ++b) {
-            const int c = blockcnt[(size_t)b * E + e];
-            blockbase[(size_t)b * E + e] = run;
-            run += c;
+    if (blk == 0) {
+        if (tid < E) {
+            counts[tid] = cnt[tid];
+            offsets[tid] = off[tid];
+            // tiles of this expert start after the tiles of the experts before it
+            int first = 0;
+            for (int q = 0; q < tid; ++q) first += (cnt[q] + tile_m - 1) / tile_m;
+            const int n = (cnt[tid] + tile_m - 1) / tile_m;
+            for (int i = 0; i < n; ++i) {
+                tile_expert[first + i] = tid;
+                tile_row0[first + i] = off[tid] + i * tile_m;
+                tile_rows[first + i] = min(tile_m, cnt[tid] - i * tile_m);
+            }
+            if (tid == E - 1) ntiles[0] = first + n;
+        }
+        if (tid == 0) {
+            offsets[E] = off[E];
+            // every valid token routes exactly k slots, so the valid-token count is routed / k
+            const int V = off[E] / k;
+            float aux = 0.0f, z = 0.0f;
+            if (V > 0) {
+                const float tokens = (float)V;
+                const float slots = (float)V * (float)k;
+                for (int q = 0; q < E; ++q) {
+                    const float load = (float)cnt[q] / slots;
+                    const float ms = mass[q] / tokens;
+                    aux = aux + load * ms;
+                }
+                aux = aux * ((float)E * w_aux);
+                z = w_z * mass[E] / tokens;
+            }
+            losses[0] = aux;
+            losses[1] = z;
         }
     }
-    if (tid < E) {
-        counts[tid] = cnt[tid];
-        offsets[tid] = off[tid];
-        if (mass_out) mass_out[tid] = mass[tid];
-        const int nt0 = toff[tid + 1] - toff[tid];
-        for (int i = 0; i < nt0; ++i) {
-            const int ti = toff[tid] + i;
-            tile_expert0[ti] = tid;
-            tile_row00[ti] = off[tid] + i * tile_m0;
-            tile_rows0[ti] = min(tile_m0, cnt[tid] - i * tile_m0);
-        }
-        const int nt1 = toff[E + 1 + tid + 1] - toff[E + 1 + tid];
-        for (int i = 0; i < nt1; ++i) {
-            const int ti = toff[E + 1 + tid] + i;
-            tile_expert1[ti] = tid;
-            tile_row01[ti] = off[tid] + i * tile_m1;
-            tile_rows1[ti] = min(tile_m1, cnt[tid] - i * tile_m1);
-        }
-    }
-    if (tid == 0) offsets[E] = off[E];
-}
 
-size_t scan_lds_bytes(int E) {
-    const int parts = 1024 / E;
-    return ((size_t)parts * E + (size_t)parts * (E + 1) + E + 3 * (E + 1) + (E + 1)) * 4;
-}
-
-// ---------------------------------------------------------------------------
-// dispatch_kernel: block b owns the same tokens as router block b.  Position
-// of a routed slot = offsets[e] + blockbase[b][e] + rank_in_block[slot]: slots
-// are numbered token-major, so this is exactly the order in which the
-// reference appends slots to an expert's list (src/moe.rs:266-274).  The row
-// copy is `gather_rows` (src/moe.rs:658-664); the slot table of the block is
-// staged in LDS, rows move as 16-byte pieces.
-// ---------------------------------------------------------------------------
-template <typename XT>
-__global__ __launch_bounds__(256) void dispatch_kernel(
-    const XT* __restrict__ x, const int* __restrict__ expert_of, const int* __restrict__ rank_in_block,
-    const int* __restrict__ blockbase, const int* __restrict__ offsets, int T, int d, int E, int k,
-    int* __restrict__ perm_slot, int* __restrict__ perm_token, int* __restrict__ inv_pos,
-    XT* __restrict__ xg) {
-    extern __shared__ __align__(16) unsigned char lds_raw[];
-    int* lpos = reinterpret_cast<int*>(lds_raw);  // [TB * k]
-    constexpr int TB = kRouterTokens;
-    const int tid = threadIdx.x;
-    const int blk = blockIdx.x;
     const int t0 = blk * TB;
     const int nt = min(TB, T - t0);
     const int nls = nt * k;
     for (int ls = tid; ls < nls; ls += 256) {
         const int s = t0 * k + ls;
-        const int e = expert_of[s];
+        const int ex = expert_of[s];
         int pos = -1;
-        if (e >= 0) {
-            pos = offsets[e] + blockbase[(size_t)blk * E + e] + rank_in_block[s];
+        if (ex >= 0) {
+            pos = off[ex] + base[ex] + rank_in_block[s];
             perm_slot[pos] = s;
             perm_token[pos] = s / k;
         }
@@ -646,8 +686,10 @@ static hipError_t launch_router_t(const RouterArgs& a, hipStream_t s) {
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    const dim3 lgrid((a.T + kLogitTokens - 1) / kLogitTokens, (a.E + kLogitExperts - 1) / kLogitExperts);
-    hipLaunchKernelGGL((logits_kernel<XT>), lgrid, dim3(256), 0, s,
+    // eight experts (waves) per workgroup share one staged slice of 64 token rows
+    constexpr int NE = 8;
+    const int tiles_t = (a.T + kLogitTokens - 1) / kLogitTokens;
+    hipLaunchKernelGGL((logits_kernel<XT, NE>), dim3(tiles_t, (a.E + NE - 1) / NE), dim3(NE * 64), 0, s,
                        static_cast<const XT*>(a.x), a.wr, a.bias, a.T, a.d, a.E, a.P);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
@@ -662,26 +704,19 @@ hipError_t launch_router(const RouterArgs& a, bool bf16, hipStream_t s) {
     return bf16 ? launch_router_t<bf16_t>(a, s) : launch_router_t<float>(a, s);
 }
 
-hipError_t launch_scan(const ScanArgs& a, hipStream_t s) {
-    hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), scan_lds_bytes(a.E), s, a.blockcnt,
-                       a.blockbase, a.partial, a.nb, a.E, a.k, a.w_aux, a.w_z, a.tile_m[0], a.tile_m[1],
-                       a.counts, a.offsets, a.tile_expert[0], a.tile_row0[0], a.tile_rows[0],
-                       a.tile_expert[1], a.tile_row0[1], a.tile_rows[1], a.ntiles, a.losses, a.mass);
-    return hipGetLastError();
-}
-
 template <typename XT>
 static hipError_t launch_dispatch_t(const DispatchArgs& a, hipStream_t s) {
     const int nb = (a.T + kRouterTokens - 1) / kRouterTokens;
-    hipLaunchKernelGGL(dispatch_kernel<XT>, dim3(nb), dim3(256),
-                       (size_t)kRouterTokens * a.k * sizeof(int), s, static_cast<const XT*>(a.x),
-                       a.expert_of, a.rank_in_block, a.blockbase, a.offsets, a.T, a.d, a.E, a.k,
-                       a.perm_slot, a.perm_token, a.inv_pos, static_cast<XT*>(a.xg));
+    hipLaunchKernelGGL(dispatch_kernel<XT>, dim3(nb > 0 ? nb : 1), dim3(256), dispatch_lds_bytes(a.E, a.k), s,
+                       static_cast<const XT*>(a.x), a.expert_of, a.rank_in_block, a.blockcnt, a.partial, a.T, a.d,
+                       a.E, a.k, a.w_aux, a.w_z, a.tile_m, a.counts, a.offsets, a.tile_expert, a.tile_row0,
+                       a.tile_rows, a.ntiles, a.losses, a.perm_slot, a.perm_token, a.inv_pos,
+                       static_cast<XT*>(a.xg));
     return hipGetLastError();
 }
 
+// Runs for T == 0 too: block 0 then writes zero counts, an empty tile table and zero losses.
 hipError_t launch_dispatch(const DispatchArgs& a, bool bf16, hipStream_t s) {
-    if (a.T <= 0) return hipSuccess;
     return bf16 ? launch_dispatch_t<bf16_t>(a, s) : launch_dispatch_t<float>(a, s);
 }
 
