@@ -145,9 +145,11 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
     const int* __restrict__ tile_expert, const int* __restrict__ tile_row0, const int* __restrict__ tile_rows,
     const int* __restrict__ ntiles, int dense_rows, bf16_t* __restrict__ out, int group_m) {
     constexpr int BN = SWIGLU ? NW * 32 : NW * 64;  // output features per workgroup
-    // Two LDS stages, each always addressed through a compile-time constant.
-    __shared__ uint4 As0[BM * CPR];
-    __shared__ uint4 As1[BM * CPR];
+    // Two LDS stages of one activation slice each; the epilogue reuses both as one
+    // 128 x 128 staging tile for the output.
+    __shared__ uint4 As[2 * BM * CPR];
+    uint4* const As0 = As;
+    uint4* const As1 = As + BM * CPR;
 
     // ---- which tile (each XCD walks a contiguous range, M fastest inside a group)
     const int tiles_n = (N + BN - 1) / BN;
@@ -186,10 +188,13 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
     // A wave whose rows lie past N (ragged last feature tile) runs the same loop on row
     // block 0, so that every wave issues the same loads and meets the same barriers; it
     // stores nothing.
-    const int nw = tn_idx * BN + wave * (SWIGLU ? 32 : 64);
-    const int r0 = nw, r1 = SWIGLU ? N + nw : nw + 32;
+    // gate/up: gate rows nw .. nw + 31 and the matching up rows; down: rows nw .. nw + 31 and
+    // the rows 128 further on, so that each block index covers 128 consecutive features of
+    // the workgroup's tile.
+    const int nw = tn_idx * BN + wave * 32;
+    const int r0 = nw, r1 = SWIGLU ? N + nw : nw + NW * 32;
     const bool act0 = nw < N;
-    const bool act1 = SWIGLU ? act0 : (nw + 32 < N);
+    const bool act1 = SWIGLU ? act0 : (nw + NW * 32 < N);
     const size_t block_bytes = (size_t)K * 32 * (I8 ? 1 : 2);  // one block of 32 weight rows over all of K
     const char* wexp = static_cast<const char*>(wpacked) + (size_t)expert * w_expert_stride_bytes;
     const char* wp0 = wexp + (size_t)(act0 ? r0 / 32 : 0) * block_bytes;
@@ -199,7 +204,9 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
     // ---- LDS-DMA of the activation slice --------------------------------------
     // Wave w fills LDS rows [32 w, 32 w + 32): instruction j covers rows 32 w + 8 j .. + 7,
     // lane l lands in row 8 j + l / 8 (of the wave's 32), position l % 8, and therefore
-    // fetches logical piece (l % 8) ^ (row % 8).  Rows past the end of the group are
+    // fetches logical piece (l % 8) ^ ((row / 2) % 8): a 16-lane group of a fragment read
+    // (16 consecutive rows, one logical piece) then touches 8 distinct pieces in the even rows
+    // and 8 in the odd rows, i.e. all 64 banks once.  Rows past the end of the group are
     // clamped to the tile's first row: their products are never stored.
     const char* a_src[DMA_PER_WAVE];
 #pragma unroll
@@ -207,7 +214,7 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
         const int r = wave * 32 + j * 8 + (lane >> 3);
         const int rr = r < rows ? r : 0;
         const int grow = row_index ? row_index[row0 + rr] : row0 + rr;
-        a_src[j] = reinterpret_cast<const char*>(a) + ((size_t)grow * K + 8 * ((lane & 7) ^ (r & 7))) * 2;
+        a_src[j] = reinterpret_cast<const char*>(a) + ((size_t)grow * K + 8 * ((lane & 7) ^ ((r >> 1) & 7))) * 2;
     }
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)As0 + wave * 32 * CPR * 16;
     const uint32_t lds1 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)As1 + wave * 32 * CPR * 16;
@@ -228,7 +235,7 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
 
     const int lrow = lane & 31;
     const int lhalf = lane >> 5;
-    const int lxor = lrow & 7;
+    const int lxor = (lrow >> 1) & 7;
 
     const int KT = K / BK;
     const int GS = KT * KS;  // reduction steps in all
@@ -318,45 +325,60 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
     wait_outstanding<0>();
 #pragma unroll
     for (int i = 0; i < RING; ++i) asm volatile("" : : "v"(ring[i].f0), "v"(ring[i].f1));
-    if (!act0) return;
 
     // ---- epilogue -------------------------------------------------------------
-    // accumulator element v of block (b, t): feature 8*(v/4) + 4*(lane/32) + v%4 of the
-    // wave's row block b, token t*32 + lane%32.
+    // Accumulator element v of block (b, t): feature 8*(v/4) + 4*(lane/32) + v%4 of the
+    // wave's row block b, token t*32 + lane%32 - a lane holds 4 consecutive features of a
+    // token, so a direct store would scatter 8-byte pieces over 32 rows per instruction.
+    // Instead each block index goes through LDS as a 128-token x 128-feature tile (16-byte
+    // pieces, piece p of row r kept at position p ^ (r % 16)), and is written out with
+    // 16-byte stores, 16 consecutive lanes covering the 256 contiguous bytes of a row.
     const float* sc = I8 ? scales + (size_t)expert * s_expert_stride : nullptr;
+    char* const stage = reinterpret_cast<char*>(As);
+    constexpr int PASSES = SWIGLU ? 1 : 2;
+    __syncthreads();  // every wave's last DMA has landed and its last fragment reads are done
 #pragma unroll
-    for (int t = 0; t < TT; ++t) {
-        const int m = t * 32 + lrow;
-        if (m >= rows) continue;
-        bf16_t* orow = out + (size_t)(row0 + m) * N;
+    for (int b = 0; b < PASSES; ++b) {
+        if (b) __syncthreads();  // the previous pass has been read out
+        if (b ? act1 : act0) {
+            const int rb = b ? r1 : r0;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int f = 8 * q + 4 * lhalf;  // first of 4 consecutive features inside a row block
-            if constexpr (SWIGLU) {
-                float h[4];
+            for (int t = 0; t < TT; ++t) {
+                if (t * 32 >= rows) continue;
+                const int m = t * 32 + lrow;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    float gv = acc[0][t][4 * q + i], uv = acc[1][t][4 * q + i];
-                    if constexpr (I8) {
-                        gv *= sc[r0 + f + i];
-                        uv *= sc[r1 + f + i];
-                    }
-                    h[i] = silu_f32(gv) * uv;
-                }
-                *reinterpret_cast<uint2*>(orow + nw + f) = make_uint2(pack2(h[0], h[1]), pack2(h[2], h[3]));
-            } else {
-#pragma unroll
-                for (int b = 0; b < 2; ++b) {
-                    if (b == 1 && !act1) continue;
-                    const int rb = b ? r1 : r0;
+                for (int q = 0; q < 4; ++q) {
+                    const int f = 8 * q + 4 * lhalf;  // first of 4 consecutive features inside the row block
                     float y[4];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        y[i] = acc[b][t][4 * q + i];
-                        if constexpr (I8) y[i] *= sc[rb + f + i];
+                        if constexpr (SWIGLU) {
+                            float gv = acc[0][t][4 * q + i], uv = acc[1][t][4 * q + i];
+                            if constexpr (I8) {
+                                gv *= sc[r0 + f + i];
+                                uv *= sc[r1 + f + i];
+                            }
+                            y[i] = silu_f32(gv) * uv;
+                        } else {
+                            y[i] = acc[b][t][4 * q + i];
+                            if constexpr (I8) y[i] *= sc[rb + f + i];
+                        }
                     }
-                    *reinterpret_cast<uint2*>(orow + rb + f) = make_uint2(pack2(y[0], y[1]), pack2(y[2], y[3]));
+                    const int piece = (wave * 4 + q) ^ (m & 15);
+                    *reinterpret_cast<uint2*>(stage + m * 256 + piece * 16 + lhalf * 8) =
+                        make_uint2(pack2(y[0], y[1]), pack2(y[2], y[3]));
                 }
+            }
+        }
+        __syncthreads();
+        const int col0 = tn_idx * BN + b * (NW * 32);
+#pragma unroll
+        for (int i = 0; i < BM * 16 / NT; ++i) {
+            const int idx = i * NT + tid;
+            const int r = idx >> 4, p = idx & 15;
+            if (r < rows && col0 + 8 * p < N) {
+                const uint4 v = *reinterpret_cast<const uint4*>(stage + r * 256 + ((p ^ (r & 15)) * 16));
+                *reinterpret_cast<uint4*>(out + (size_t)(row0 + r) * N + col0 + 8 * p) = v;
             }
         }
     }
