@@ -85,8 +85,8 @@ __device__ __forceinline__ void issue_load(u32x2& d, uint32_t byte_off, const ch
     asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(d) : "v"(byte_off), "s"(base));
 }
 // 64 lanes x 16 bytes from `src` (per lane) to LDS bytes [lds_addr, lds_addr + 1024).
-__device__ __forceinline__ void issue_dma(uint32_t lds_addr, const char* src) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(src) : "memory");
+__device__ __forceinline__ void issue_dma(uint32_t lds_addr, uint32_t byte_off, const char* base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(byte_off), "s"(base) : "memory");
 }
 // Wait until at most N loads are outstanding; the two registers become usable only here.
 template <int N, typename V>
@@ -138,7 +138,7 @@ struct Slot<true> {
 
 // RING = weight-fragment steps in flight per wave (register ring depth);
 // TFBUF = 2: token fragments are read from LDS one step ahead, 1: just in time.
-template <bool SWIGLU, bool I8, int RING, int TFBUF>
+template <bool SWIGLU, bool I8, int RING, int TFBUF, bool AREG>
 __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
     const bf16_t* __restrict__ a, const int* __restrict__ row_index, const void* __restrict__ wpacked,
     size_t w_expert_stride_bytes, const float* __restrict__ scales, size_t s_expert_stride, int N, int K,
@@ -208,13 +208,15 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
     // (16 consecutive rows, one logical piece) then touches 8 distinct pieces in the even rows
     // and 8 in the odd rows, i.e. all 64 banks once.  Rows past the end of the group are
     // clamped to the tile's first row: their products are never stored.
-    const char* a_src[DMA_PER_WAVE];
+    // Byte offsets from `a` fit 32 bits (the launcher checks rows * K * 2 < 4 GiB).
+    const char* const a_base = reinterpret_cast<const char*>(a);
+    uint32_t a_src[DMA_PER_WAVE];
 #pragma unroll
     for (int j = 0; j < DMA_PER_WAVE; ++j) {
         const int r = wave * 32 + j * 8 + (lane >> 3);
         const int rr = r < rows ? r : 0;
         const int grow = row_index ? row_index[row0 + rr] : row0 + rr;
-        a_src[j] = reinterpret_cast<const char*>(a) + ((size_t)grow * K + 8 * ((lane & 7) ^ ((r >> 1) & 7))) * 2;
+        a_src[j] = ((uint32_t)grow * (uint32_t)K + 8u * ((lane & 7) ^ ((r >> 1) & 7))) * 2u;
     }
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)As0 + wave * 32 * CPR * 16;
     const uint32_t lds1 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)As1 + wave * 32 * CPR * 16;
@@ -222,7 +224,7 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
         constexpr int BUF = decltype(buf_tag)::value;
 #pragma unroll
         for (int j = 0; j < DMA_PER_WAVE; ++j)
-            issue_dma((BUF ? lds1 : lds0) + j * 8 * CPR * 16, a_src[j] + (size_t)kt * (BK * 2));
+            issue_dma((BUF ? lds1 : lds0) + j * 8 * CPR * 16, a_src[j] + (uint32_t)kt * (BK * 2), a_base);
     };
 
     floatx16 acc[2][TT];
@@ -242,11 +244,39 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
     constexpr int D = RING - 1;  // the load for step g + D is issued while step g runs
 
     // ---- prologue: first activation slice, first D weight steps -----------------
-    dma_a(0, std::integral_constant<int, 0>{});
+    // AREG: the activation slice travels global -> VGPR -> LDS instead of by LDS-DMA, one
+    // 1 KB piece per wave per step: piece j of slice k + 2 is fetched in step j of slice k and
+    // written to LDS in step j of slice k + 1 (into the stage slice k read).  Slices 0 and 1
+    // are placed by the prologue, so that no load is in flight where the loop is entered
+    // (the compiler may copy registers there); the first slice's writes go to a spare row.
+    u32x4 areg[DMA_PER_WAVE];
+    uint4* const a_dst0 = As0 + (wave * 32) * CPR + lane;
+    uint4* const a_dst1 = As1 + (wave * 32) * CPR + lane;
+    __shared__ uint4 spare[AREG ? NT : 1];
     Slot<I8> ring[RING];
+    if constexpr (AREG) {
+        u32x4 first[DMA_PER_WAVE];
 #pragma unroll
-    for (int g = 0; g < D; ++g) ring[g].load(wp0, wp1, min(g, GS - 1), lane16);
-    wait_outstanding<0>();
+        for (int j = 0; j < DMA_PER_WAVE; ++j) issue_load(first[j], a_src[j], a_base);
+#pragma unroll
+        for (int j = 0; j < DMA_PER_WAVE; ++j)
+            issue_load(areg[j], a_src[j] + (uint32_t)min(1, KT - 1) * (BK * 2), a_base);
+#pragma unroll
+        for (int g = 0; g < D; ++g) ring[g].load(wp0, wp1, min(g, GS - 1), lane16);
+        wait_outstanding<0>();
+#pragma unroll
+        for (int j = 0; j < DMA_PER_WAVE; ++j) {
+            asm volatile("" : "+v"(first[j]), "+v"(areg[j]));
+            a_dst0[j * 8 * CPR] = make_uint4(first[j].x, first[j].y, first[j].z, first[j].w);
+            a_dst1[j * 8 * CPR] = make_uint4(areg[j].x, areg[j].y, areg[j].z, areg[j].w);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
+    } else {
+        dma_a(0, std::integral_constant<int, 0>{});
+#pragma unroll
+        for (int g = 0; g < D; ++g) ring[g].load(wp0, wp1, min(g, GS - 1), lane16);
+        wait_outstanding<0>();
+    }
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
 
@@ -262,7 +292,7 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
         constexpr int BUF = decltype(buf_tag)::value;
         constexpr int G0 = RING == 2 * KS ? BUF * KS : 0;
         constexpr int NB = decltype(nb_tag)::value;
-        dma_a(min(kt + 1, KT - 1), std::integral_constant<int, BUF ^ 1>{});
+        if constexpr (!AREG) dma_a(min(kt + 1, KT - 1), std::integral_constant<int, BUF ^ 1>{});
         const uint4* Ab = BUF ? As1 : As0;
         bf16x8 tf[TFBUF][TT];
 #pragma unroll
@@ -284,9 +314,21 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
 #pragma unroll
                 for (int t = 0; t < NB; ++t) tf[0][t] = lds_frag(Ab, (t * 32 + lrow) * CPR + piece);
             }
-            // Younger than the loads of step g: the weight loads of steps g+1 .. g+D (2 each)
-            // and the DMA (4) of every slice that started after they were issued.
-            wait_for<2 * D + DMA_PER_WAVE * ((D - s + KS - 1) / KS)>(cur.f0, cur.f1);
+            if constexpr (AREG) {
+                // Per step: 2 weight loads, then 1 activation load.  Younger than the weight loads
+                // of step g: 3 per step for D steps.  The activation piece this step writes to LDS
+                // was fetched a whole slice ago, i.e. is older still.
+                static_assert(KS == DMA_PER_WAVE && D <= KS, "one activation piece per step, fetched KS steps before use");
+                wait_for<3 * D>(cur.f0, cur.f1);
+                asm volatile("" : "+v"(areg[s]));
+                uint4* const dst = kt > 0 ? (BUF ? a_dst0 : a_dst1) + s * 8 * CPR : spare + tid;
+                *dst = make_uint4(areg[s].x, areg[s].y, areg[s].z, areg[s].w);
+                issue_load(areg[s], a_src[s] + (uint32_t)min(kt + 2, KT - 1) * (BK * 2), a_base);
+            } else {
+                // Younger than the loads of step g: the weight loads of steps g+1 .. g+D (2 each)
+                // and the DMA (4) of every slice that started after they were issued.
+                wait_for<2 * D + DMA_PER_WAVE * ((D - s + KS - 1) / KS)>(cur.f0, cur.f1);
+            }
             const bf16x8 w0 = cur.a0();
             const bf16x8 w1 = cur.a1();
 #pragma unroll
@@ -298,7 +340,10 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
         // Every LDS read of this slice has been consumed by a multiply issued above this
         // point.  The DMA of the next slice is older than this slice's 2 * KS weight loads.
         __builtin_amdgcn_sched_barrier(0);
-        wait_outstanding<2 * KS>();
+        if constexpr (AREG)
+            asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");  // this wave's pieces of the next slice are in LDS
+        else
+            wait_outstanding<2 * KS>();
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
     };
@@ -312,20 +357,24 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
             slice(kt + 1, std::integral_constant<int, 1>{}, nb_tag);
         }
         if (kt < KT) slice(kt, std::integral_constant<int, 0>{}, nb_tag);
+        // The loads fetched again past the end still target ring registers and LDS.  Naming
+        // the registers after the wait keeps them allocated until their data has arrived: a
+        // loaded value the compiler sees no use for would otherwise hand its register to
+        // something live while the load is still in flight.  (Done here, inside each
+        // specialisation, so that no path leaves it with loads outstanding.)
+        wait_outstanding<0>();
+        auto& ring_ref = ring;
+        auto& areg_ref = areg;
+#pragma unroll
+        for (int i = 0; i < RING; ++i) asm volatile("" : : "v"(ring_ref[i].f0), "v"(ring_ref[i].f1));
+#pragma unroll
+        for (int j = 0; j < DMA_PER_WAVE; ++j) asm volatile("" : : "v"(areg_ref[j]));
     };
     static_assert(TT == 4, "one specialisation per possible block count");
     if (nblk == 4) run(std::integral_constant<int, 4>{});
     else if (nblk == 3) run(std::integral_constant<int, 3>{});
     else if (nblk == 2) run(std::integral_constant<int, 2>{});
     else run(std::integral_constant<int, 1>{});
-    // The loads fetched again past the end still target ring registers and LDS.  Naming the
-    // registers after the wait keeps them allocated until their data has arrived: a loaded
-    // value the compiler sees no use for would otherwise hand its register to something
-    // live while the load is still in flight.
-    wait_outstanding<0>();
-#pragma unroll
-    for (int i = 0; i < RING; ++i) asm volatile("" : : "v"(ring[i].f0), "v"(ring[i].f1));
-
     // ---- epilogue -------------------------------------------------------------
     // Accumulator element v of block (b, t): feature 8*(v/4) + 4*(lane/32) + v%4 of the
     // wave's row block b, token t*32 + lane%32 - a lane holds 4 consecutive features of a
@@ -358,7 +407,7 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
                                 gv *= sc[r0 + f + i];
                                 uv *= sc[r1 + f + i];
                             }
-                            y[i] = silu_f32(gv) * uv;
+                            y[i] = silu_bf16_grade(gv) * uv;
                         } else {
                             y[i] = acc[b][t][4 * q + i];
                             if constexpr (I8) y[i] *= sc[rb + f + i];
@@ -384,7 +433,7 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
     }
 }
 
-template <bool SWIGLU, bool I8, int RING, int TFBUF>
+template <bool SWIGLU, bool I8, int RING, int TFBUF, bool AREG>
 hipError_t launch_t(const GroupedArgs& g, hipStream_t s) {
     constexpr int BN = SWIGLU ? NW * 32 : NW * 64;
     const int tiles_n = (g.N + BN - 1) / BN;
@@ -392,7 +441,7 @@ hipError_t launch_t(const GroupedArgs& g, hipStream_t s) {
     if (tiles_m <= 0) return hipSuccess;
     const int total = tiles_m * tiles_n;
     const int grid = ((total + 7) / 8) * 8;
-    hipLaunchKernelGGL((grouped_stream_kernel<SWIGLU, I8, RING, TFBUF>), dim3(grid), dim3(NT), 0, s,
+    hipLaunchKernelGGL((grouped_stream_kernel<SWIGLU, I8, RING, TFBUF, AREG>), dim3(grid), dim3(NT), 0, s,
                        static_cast<const bf16_t*>(g.a), g.row_index, g.w, g.w_expert_stride * (I8 ? 1 : 2), g.scales,
                        g.s_expert_stride, g.N, g.K, g.tile_expert, g.tile_row0, g.tile_rows, g.ntiles, g.dense_rows,
                        static_cast<bf16_t*>(g.out), g.group_m > 0 ? g.group_m : 4);
@@ -401,12 +450,12 @@ hipError_t launch_t(const GroupedArgs& g, hipStream_t s) {
 
 }  // namespace
 
-template <int RING, int TFBUF>
+template <int RING, int TFBUF, bool AREG>
 static hipError_t launch_ring(const GroupedArgs& g, WeightKind wk, hipStream_t s) {
     if (wk == WeightKind::BF16)
-        return g.swiglu ? launch_t<true, false, RING, TFBUF>(g, s) : launch_t<false, false, RING, TFBUF>(g, s);
+        return g.swiglu ? launch_t<true, false, RING, TFBUF, AREG>(g, s) : launch_t<false, false, RING, TFBUF, AREG>(g, s);
     if (wk == WeightKind::I8)
-        return g.swiglu ? launch_t<true, true, RING, TFBUF>(g, s) : launch_t<false, true, RING, TFBUF>(g, s);
+        return g.swiglu ? launch_t<true, true, RING, TFBUF, AREG>(g, s) : launch_t<false, true, RING, TFBUF, AREG>(g, s);
     return hipErrorInvalidValue;
 }
 
@@ -420,8 +469,8 @@ bool stream_shape_ok(int N, int K) { return K % 64 == 0 && K >= 64 && N % 32 == 
 hipError_t launch_grouped_stream(const GroupedArgs& g, WeightKind wk, int variant, hipStream_t s) {
     if (!stream_shape_ok(g.N, g.K)) return hipErrorInvalidValue;
     switch (variant) {
-        case 0: return launch_ring<4, 2>(g, wk, s);
-        case 1: return launch_ring<8, 1>(g, wk, s);
+        case 0: return launch_ring<4, 2, false>(g, wk, s);
+        case 1: return launch_ring<4, 1, true>(g, wk, s);
     }
     return hipErrorInvalidValue;
 }
