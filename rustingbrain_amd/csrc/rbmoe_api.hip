@@ -363,6 +363,12 @@ int rbmoe_layer_create(rbmoe_ctx* ctx, const rbmoe_config* cfg, rbmoe_layer** ou
     L->use_stream = mc && stream_shape_ok(cfg->d_ff, cfg->d_model) && stream_shape_ok(cfg->d_model, cfg->d_ff) &&
                     (!cfg->shared_expert ||
                      (stream_shape_ok(L->Fs, cfg->d_model) && stream_shape_ok(cfg->d_model, L->Fs)));
+    {
+        // the streaming kernel addresses activation rows with 32-bit byte offsets
+        const size_t widest = (size_t)std::max(std::max(cfg->d_model, cfg->d_ff), L->Fs);
+        const size_t rows = (size_t)cfg->max_tokens * (size_t)std::max(1, cfg->experts_per_token);
+        if (rows * widest * 2 >= ((size_t)1 << 32)) L->use_stream = false;
+    }
 
     Plan plan = make_plan(L);
     // Refuse before allocating anything, as the reference's budget check does

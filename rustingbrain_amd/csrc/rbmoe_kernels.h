@@ -12,6 +12,8 @@ namespace rbmoe {
 // Tokens owned by one router / dispatch block.  Slots are numbered
 // token * k + rank, so a block owns a contiguous slot range.
 constexpr int kRouterTokens = 32;
+constexpr int kRouterThreads = 512;     // router_kernel workgroup
+constexpr int kRouterWaves = kRouterThreads / 64;
 
 // Largest expert count and top-k the routing kernels are laid out for.
 constexpr int kMaxExperts = 256;

@@ -23,11 +23,11 @@ namespace rbmoe {
 //   lsev   [TB]       log-sum-exp per token
 //   gates  [TB][k]    selected probabilities, then gates
 //   lexp   [TB][k]    selected expert per local slot (-1 = unrouted)
-//   wcount [4][E]     per-wave match counts of one ranking round
+//   wcount [waves][E] per-wave match counts of one ranking round
 //   running[E]        slots already ranked per expert
 __host__ __device__ static size_t router_fixed_bytes(int E, int k) {
     const int ES = E | 1;
-    size_t n = (size_t)kRouterTokens * ES + kRouterTokens + 2 * (size_t)kRouterTokens * k + 4 * (size_t)E + E;
+    size_t n = (size_t)kRouterTokens * ES + kRouterTokens + 2 * (size_t)kRouterTokens * k + (size_t)kRouterWaves * E + E;
     return (n * 4 + 15) & ~(size_t)15;
 }
 
@@ -159,7 +159,7 @@ __global__ __launch_bounds__(NE * 64) void logits_kernel(const XT* __restrict__ 
 }
 
 template <typename XT>
-__global__ __launch_bounds__(256) void router_kernel(
+__global__ __launch_bounds__(kRouterThreads) void router_kernel(
     const XT* __restrict__ x, const float* __restrict__ wr, const float* __restrict__ bias,
     const uint8_t* __restrict__ valid, int T, int d, int E, int k, float* __restrict__ P,
     float* __restrict__ lse, int* __restrict__ expert_of, float* __restrict__ gate_of,
@@ -172,7 +172,7 @@ __global__ __launch_bounds__(256) void router_kernel(
     float* gates = lsev + TB;
     int* lexp = reinterpret_cast<int*>(gates + TB * k);
     int* wcount = lexp + TB * k;
-    int* running = wcount + 4 * E;
+    int* running = wcount + kRouterWaves * E;
 
     const int tid = threadIdx.x;
     const int blk = blockIdx.x;
@@ -180,11 +180,11 @@ __global__ __launch_bounds__(256) void router_kernel(
     const int nt = min(TB, T - t0);
 
     // ---- logits were written to P by logits_kernel ------------------------------
-    for (int idx = tid; idx < nt * E; idx += 256) {
+    for (int idx = tid; idx < nt * E; idx += kRouterThreads) {
         const int i = idx / E;
         prob[i * ES + (idx - i * E)] = P[(size_t)t0 * E + idx];
     }
-    for (int idx = tid; idx < E; idx += 256) running[idx] = 0;
+    for (int idx = tid; idx < E; idx += kRouterThreads) running[idx] = 0;
     __syncthreads();
 
     // ---- softmax + top-k: G lanes per token, lane j of a group owns experts j, j + G, ... ----
@@ -202,9 +202,9 @@ __global__ __launch_bounds__(256) void router_kernel(
         const unsigned long long gmask = (G == 64 ? ~0ull : ((1ull << G) - 1ull)) << gbase;
         constexpr int MAXJ = kMaxExperts / 64;    // experts per lane when G == 64
         const float neg_inf = __uint_as_float(0xff800000u);
-        for (int i0 = wave_ * (TB / 4); i0 < (wave_ + 1) * (TB / 4); i0 += tpw) {
+        for (int i0 = wave_ * (TB / kRouterWaves); i0 < (wave_ + 1) * (TB / kRouterWaves); i0 += tpw) {
             const int i = i0 + lane_ / G;         // token of this group
-            const bool live = i < nt && i < (wave_ + 1) * (TB / 4);
+            const bool live = i < nt && i < (wave_ + 1) * (TB / kRouterWaves);
             float* row = prob + (live ? i : 0) * ES;
             float pv[MAXJ];
             float mx = neg_inf;
@@ -304,20 +304,20 @@ __global__ __launch_bounds__(256) void router_kernel(
     __syncthreads();
 
     // ---- write probabilities, lse, assignments (coalesced) ----------------
-    for (int idx = tid; idx < nt * E; idx += 256) {
+    for (int idx = tid; idx < nt * E; idx += kRouterThreads) {
         const int i = idx / E;
         const int e = idx - i * E;
         P[(size_t)t0 * E + idx] = prob[i * ES + e];
     }
     if (tid < nt) lse[t0 + tid] = lsev[tid];
     const int nls = nt * k;
-    for (int ls = tid; ls < nls; ls += 256) {
+    for (int ls = tid; ls < nls; ls += kRouterThreads) {
         expert_of[(size_t)t0 * k + ls] = lexp[ls];
         gate_of[(size_t)t0 * k + ls] = gates[ls];
     }
 
     // ---- partial sums for the auxiliary losses (fixed order) --------------
-    for (int e = tid; e <= E; e += 256) {
+    for (int e = tid; e <= E; e += kRouterThreads) {
         float s = 0.0f;
         if (e < E) {
             for (int i = 0; i < nt; ++i)
@@ -334,11 +334,11 @@ __global__ __launch_bounds__(256) void router_kernel(
     const int wave = tid >> 6;
     int ebits = 0;
     while ((1 << ebits) < E) ++ebits;
-    const int rounds = (nls + 255) / 256;
+    const int rounds = (nls + kRouterThreads - 1) / kRouterThreads;
     for (int rd = 0; rd < rounds; ++rd) {
-        for (int idx = tid; idx < 4 * E; idx += 256) wcount[idx] = 0;
+        for (int idx = tid; idx < kRouterWaves * E; idx += kRouterThreads) wcount[idx] = 0;
         __syncthreads();
-        const int ls = rd * 256 + tid;
+        const int ls = rd * kRouterThreads + tid;
         const int e = (ls < nls) ? lexp[ls] : -1;
         unsigned long long mask = __ballot(e >= 0);
         for (int b = 0; b < ebits; ++b) {
@@ -355,11 +355,11 @@ __global__ __launch_bounds__(256) void router_kernel(
             rank_in_block[(size_t)t0 * k + ls] = pre + rank_w;
         }
         __syncthreads();
-        for (int idx = tid; idx < E; idx += 256)
-            running[idx] += wcount[idx] + wcount[E + idx] + wcount[2 * E + idx] + wcount[3 * E + idx];
+        for (int idx = tid; idx < E; idx += kRouterThreads)
+            for (int w = 0; w < kRouterWaves; ++w) running[idx] += wcount[w * E + idx];
         __syncthreads();
     }
-    for (int idx = tid; idx < E; idx += 256) blockcnt[(size_t)blk * E + idx] = running[idx];
+    for (int idx = tid; idx < E; idx += kRouterThreads) blockcnt[(size_t)blk * E + idx] = running[idx];
 }
 
 // ---------------------------------------------------------------------------
@@ -410,25 +410,51 @@ __global__ __launch_bounds__(256) void dispatch_kernel(
     const int p = tid / E;
     const int e = tid - p * E;
     const bool active = p < parts;
+    // this thread's first slot does not depend on the scan: fetch it before anything else
+    const int t0 = blk * TB;
+    const int nt = min(TB, T - t0);
+    const int nls = nt * k;
+    int ex_first = -1, rank_first = 0;
+    if (tid < nls) {
+        ex_first = expert_of[(size_t)t0 * k + tid];
+        rank_first = rank_in_block[(size_t)t0 * k + tid];
+    }
     if (active) {
         const int b0 = min(nb, p * len), b1 = min(nb, b0 + len);
+        // Loads in batches of 16 that do not depend on one another: one round trip to L2 per
+        // batch instead of one per block.
         int s_all = 0, s_before = 0;
-        for (int b = b0; b < b1; ++b) {
-            const int c = blockcnt[(size_t)b * E + e];
-            s_all += c;
-            s_before += b < blk ? c : 0;
+        for (int b = b0; b < b1; b += 16) {
+            int c[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) c[u] = b + u < b1 ? blockcnt[(size_t)(b + u) * E + e] : 0;
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                s_all += c[u];
+                s_before += b + u < blk ? c[u] : 0;
+            }
         }
         part_all[p * E + e] = s_all;
         part_before[p * E + e] = s_before;
         if (blk == 0) {
-            float m = 0.0f;
-            for (int b = b0; b < b1; ++b) m += partial[(size_t)b * (E + 1) + e];
-            part_mass[p * (E + 1) + e] = m;
-            if (e == 0) {
-                float zs = 0.0f;
-                for (int b = b0; b < b1; ++b) zs += partial[(size_t)b * (E + 1) + E];
-                part_mass[p * (E + 1) + E] = zs;
+            float m = 0.0f, zs = 0.0f;
+            for (int b = b0; b < b1; b += 16) {
+                float v[16], z[16];
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    v[u] = b + u < b1 ? partial[(size_t)(b + u) * (E + 1) + e] : 0.0f;
+                    z[u] = (e == 0 && b + u < b1) ? partial[(size_t)(b + u) * (E + 1) + E] : 0.0f;
+                }
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    if (b + u < b1) {
+                        m += v[u];
+                        zs += z[u];
+                    }
+                }
             }
+            part_mass[p * (E + 1) + e] = m;
+            if (e == 0) part_mass[p * (E + 1) + E] = zs;
         }
     }
     __syncthreads();
@@ -450,7 +476,19 @@ __global__ __launch_bounds__(256) void dispatch_kernel(
         mass[E] = zs;
     }
     __syncthreads();
-    if (tid == 0) {  // exclusive prefix over the experts (E <= 256)
+    if (E <= 64) {  // exclusive prefix over the experts: one wave, log2(64) shuffle steps
+        if (tid < 64) {
+            const int c = tid < E ? cnt[tid] : 0;
+            int incl = c;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const int up = __shfl_up(incl, o);
+                if (tid >= o) incl += up;
+            }
+            if (tid < E) off[tid] = incl - c;
+            if (tid == E - 1) off[E] = incl;
+        }
+    } else if (tid == 0) {
         int run = 0;
         for (int q = 0; q < E; ++q) {
             off[q] = run;
@@ -495,15 +533,12 @@ __global__ __launch_bounds__(256) void dispatch_kernel(
         }
     }
 
-    const int t0 = blk * TB;
-    const int nt = min(TB, T - t0);
-    const int nls = nt * k;
     for (int ls = tid; ls < nls; ls += 256) {
         const int s = t0 * k + ls;
-        const int ex = expert_of[s];
+        const int ex = ls == tid ? ex_first : expert_of[s];
         int pos = -1;
         if (ex >= 0) {
-            pos = off[ex] + base[ex] + rank_in_block[s];
+            pos = off[ex] + base[ex] + (ls == tid ? rank_first : rank_in_block[s]);
             perm_slot[pos] = s;
             perm_token[pos] = s / k;
         }
@@ -693,7 +728,7 @@ static hipError_t launch_router_t(const RouterArgs& a, hipStream_t s) {
                        static_cast<const XT*>(a.x), a.wr, a.bias, a.T, a.d, a.E, a.P);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((router_kernel<XT>), dim3(nb), dim3(256), router_lds_bytes(a.E, a.k), s,
+    hipLaunchKernelGGL((router_kernel<XT>), dim3(nb), dim3(kRouterThreads), router_lds_bytes(a.E, a.k), s,
                        static_cast<const XT*>(a.x), a.wr, a.bias, a.valid, a.T, a.d, a.E, a.k, a.P, a.lse,
                        a.expert_of, a.gate_of, a.rank_in_block, a.blockcnt, a.partial);
     return hipGetLastError();
