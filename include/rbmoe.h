@@ -172,12 +172,14 @@ int rbmoe_get_routing(rbmoe_layer* layer, rbmoe_routing* routing);
 int rbmoe_get_expert_rows(rbmoe_layer* layer, float* hidden, float* expert_out);
 
 /* Per-stage timing of one forward with HIP events on the context's stream.
- * `ms` receives RBMOE_NUM_STAGES durations in milliseconds.  Synchronises. */
+ * `ms` receives RBMOE_NUM_STAGES durations in milliseconds.  Synchronises.
+ * Stage 1 brackets no work at all: it reads what one pair of event records adds to
+ * every other stage (about 5 us), so callers can subtract it. */
 #define RBMOE_NUM_STAGES 8
 enum {
-    RBMOE_STAGE_ROUTER = 0,   /* logits + softmax + top-k + block histogram     */
-    RBMOE_STAGE_SCAN = 1,     /* prefix scan, tile table, auxiliary losses      */
-    RBMOE_STAGE_DISPATCH = 2, /* permutation + row gather                       */
+    RBMOE_STAGE_ROUTER = 0,   /* logits, softmax, top-k, block histograms       */
+    RBMOE_STAGE_EMPTY = 1,    /* nothing: the cost of one event interval        */
+    RBMOE_STAGE_DISPATCH = 2, /* layout scan, losses, permutation (+ row gather) */
     RBMOE_STAGE_GATE_UP = 3,  /* grouped gate/up product + SwiGLU               */
     RBMOE_STAGE_DOWN = 4,     /* grouped down product                           */
     RBMOE_STAGE_SHARED = 5,   /* shared expert (both products)                  */

@@ -20,7 +20,7 @@ DTYPES = {"f32": F32, "bf16": BF16, "int8": I8}
 # rbmoe_weight
 W_ROUTER, W_GATE, W_UP, W_DOWN, W_SHARED_GATE, W_SHARED_UP, W_SHARED_DOWN = range(7)
 NUM_STAGES = 8
-STAGE_NAMES = ("router", "scan", "dispatch", "gate_up", "down", "shared", "combine", "total")
+STAGE_NAMES = ("router", "empty", "dispatch", "gate_up", "down", "shared", "combine", "total")
 
 
 class Config(C.Structure):

@@ -601,7 +601,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     HIP_TRY(ctx, launch_router(ra, abf, s));
     HIP_TRY(ctx, mark(1));
 
-    HIP_TRY(ctx, mark(2));  // (the scan is part of the dispatch kernel)
+    HIP_TRY(ctx, mark(2));  // an interval with no work in it: the cost of one pair of event records
 
     DispatchArgs da{};
     da.x = x;
