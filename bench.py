@@ -83,6 +83,10 @@ def algorithmic(w: synth.Workload, T: int, routed: int, touched_experts: int) ->
         "shared_flops": 6 * d * Fs * T,
         "gemm_flops": 6 * d * F * S + 6 * d * Fs * T,
         "layer_bytes_decode": touched_experts * 3 * d * F * sw + 3 * d * Fs * sw + E * d * 4 + 2 * T * d * sa + S * 8,
+        # decode-shaped products: every touched expert's weights once, token rows in, hidden / output rows out
+        "decode_gate_up_bytes": touched_experts * 2 * d * F * sw + 2 * d * Fs * sw + (S + T) * d * sa
+                                + (S * F + T * Fs) * sa,
+        "decode_down_bytes": touched_experts * d * F * sw + d * Fs * sw + (S * F + T * Fs) * sa + (S + T) * d * sa,
     }
 
 
@@ -178,9 +182,14 @@ def main() -> int:
     gu = tflops(alg["gate_up_flops"], stage_ms["gate_up"])
     decode = T <= 64
     if decode:
-        whole = gbs(alg["layer_bytes_decode"], stage_ms["total"])
-        roofline = {"bound": "hbm", "kernel": "whole layer (weight streaming)", "achieved": whole,
-                    "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": whole / PEAK_HBM_GBS, "traffic": None}
+        # the dominant kernel of the decode-shaped path streams the gate/up weights of the touched experts
+        # (and of the shared expert) once: it is bound by HBM
+        gu_gbs = gbs(alg["decode_gate_up_bytes"], stage_ms["gate_up"])
+        roofline = {"bound": "hbm", "kernel": "decode gate/up product + SwiGLU, routed and shared (" +
+                                              layer.kernel_name() + ")",
+                    "achieved": gu_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gu_gbs / PEAK_HBM_GBS,
+                    "traffic": None, "bytes_per_launch": alg["decode_gate_up_bytes"],
+                    "avg_launch_ms": stage_ms["gate_up"], "touched_experts": touched}
     else:
         roofline = {"bound": "mfma", "kernel": "grouped gate/up product + SwiGLU (" + layer.kernel_name() + ")",
                     "achieved": gu, "peak": peak_tf, "unit": "TFLOP/s", "frac": gu / peak_tf,
@@ -200,6 +209,12 @@ def main() -> int:
         "combine_gbs": gbs(alg["combine_bytes"], stage_ms["combine"]),
         "combine_frac_of_hbm": gbs(alg["combine_bytes"], stage_ms["combine"]) / PEAK_HBM_GBS,
     }
+    if decode:
+        whole = gbs(alg["layer_bytes_decode"], ms_per_step)
+        stages.update({"decode_down_gbs": gbs(alg["decode_down_bytes"], stage_ms["down"]),
+                       "decode_down_frac_of_hbm": gbs(alg["decode_down_bytes"], stage_ms["down"]) / PEAK_HBM_GBS,
+                       "whole_layer_gbs": whole, "whole_layer_frac_of_hbm": whole / PEAK_HBM_GBS,
+                       "whole_layer_bytes": alg["layer_bytes_decode"]})
 
     result = {
         "metric": "MoE-layer fwd tokens/sec at d768 E16 k2; grouped-GEMM % of bf16 MFMA peak",

@@ -1,0 +1,476 @@
+// Decode-shaped forward (a few tokens): the layer is bound by streaming the touched experts'
+// weights once from HBM and by launch latency, so the work is cut into four launches
+//
+//   route_small_kernel   one workgroup: logits, softmax, top-k, counting sort, tile table,
+//                        auxiliary losses (MoeLayer::forward_train, src/moe.rs:243-341, up to
+//                        the bucket loop; route src/moe.rs:553-593; losses src/moe.rs:325-337)
+//   decode_gemm_kernel   gate/up + SwiGLU of every routed tile and of the shared expert
+//   decode_gemm_kernel   down product of both
+//   combine              (the same kernel as the large path)
+//
+// and the products are spread over (tile, 32-feature block) workgroups whose four waves
+// split the reduction dimension, so that a few hundred kilobytes of weight fragments are in
+// flight per CU and every byte of a touched expert is fetched exactly once per 32-row tile.
+#include "rbmoe_kernels.h"
+
+namespace rbmoe {
+
+// ---------------------------------------------------------------------------
+// route_small_kernel.  Everything is written the way the reference walks it, one token or
+// one expert per thread, because at this size the order of operations matters and the time
+// does not: logits in the order of the eight-lane `dot` (src/matrix.rs:26-40) with the
+// eight lanes of a pair on eight neighbouring threads, softmax_rows and route per token,
+// the bucket loop per expert (a stable counting sort), losses per expert in token order.
+// ---------------------------------------------------------------------------
+constexpr int kSmallThreads = 512;
+
+// softmax_rows (src/moe.rs, softmax over one row) and route (src/moe.rs:553-593) of one token, by one
+// thread.  EMAX > 0: the row is copied into EMAX registers and every loop over the experts is
+// unrolled with the tail predicated off; EMAX == 0: the row is used where it lies (LDS).
+template <int EMAX>
+__device__ __forceinline__ void token_phase(float* row_lds, int t, int E, int k, const uint8_t* valid, float* P,
+                                            float* lse, float* lsev, int* sexp, int* expert_of, float* gate_of) {
+    constexpr int N = EMAX > 0 ? EMAX : 1;
+    float reg[N];
+    auto get = [&](int e) -> float {
+        if constexpr (EMAX > 0) return reg[e];
+        else return row_lds[e];
+    };
+    auto set = [&](int e, float v) {
+        if constexpr (EMAX > 0) reg[e] = v;
+        else row_lds[e] = v;
+    };
+    const int EB = EMAX > 0 ? EMAX : E;  // loop bound (a compile-time constant when EMAX > 0)
+    if constexpr (EMAX > 0) {
+#pragma unroll
+        for (int e = 0; e < EMAX; ++e) reg[e] = e < E ? row_lds[e] : 0.0f;
+    }
+    const float neg_inf = __uint_as_float(0xff800000u);
+    float mx = neg_inf;
+#pragma unroll
+    for (int e = 0; e < EB; ++e)
+        if (e < E && get(e) > mx) mx = get(e);  // a NaN never replaces the maximum
+    float sum = 0.0f;
+#pragma unroll
+    for (int e = 0; e < EB; ++e)
+        if (e < E) {
+            set(e, rb_expf(__fadd_rn(get(e), -mx)));
+            sum = __fadd_rn(sum, get(e));
+        }
+    const float l = __fadd_rn(mx, rb_logf(sum));
+    lsev[t] = l;
+    lse[t] = l;
+#pragma unroll
+    for (int e = 0; e < EB; ++e)
+        if (e < E) {
+            if (sum > 0.0f) set(e, __fdiv_rn(get(e), sum));
+            P[(size_t)t * E + e] = get(e);
+            if constexpr (EMAX > 0) row_lds[e] = get(e);  // the loss phase reads the probabilities from LDS
+        }
+
+    int* eo = sexp + t * k;
+    const bool ok = (valid == nullptr) || (valid[t] != 0);
+    if (!ok) {
+        for (int r = 0; r < k; ++r) {
+            eo[r] = -1;
+            expert_of[t * k + r] = -1;
+            gate_of[t * k + r] = 0.0f;
+        }
+        return;
+    }
+    // taken experts as a bit set when they fit one (EMAX <= 64), else through the slot list
+    unsigned long long taken_bits = 0ull;
+    float total = 0.0f;
+    for (int r = 0; r < k; ++r) {
+        int best = -1;
+        float bestv = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EB; ++e) {
+            if (e >= E) continue;
+            bool taken;
+            if constexpr (EMAX > 0) {
+                taken = (taken_bits >> e) & 1ull;
+            } else {
+                taken = false;
+                for (int q = 0; q < r; ++q) taken = taken || (eo[q] == e);
+            }
+            if (taken) continue;
+            const float v = get(e);
+            if (best < 0 || v > bestv) {
+                best = e;
+                bestv = v;
+            }
+        }
+        eo[r] = best;
+        if constexpr (EMAX > 0) taken_bits |= 1ull << best;
+        total = __fadd_rn(total, bestv);
+        gate_of[t * k + r] = bestv;  // rewritten below once the sum is known
+        expert_of[t * k + r] = best;
+    }
+    if (total > 0.0f)
+        for (int r = 0; r < k; ++r) {
+            float g;
+            if constexpr (EMAX > 0) {
+                g = 0.0f;
+#pragma unroll
+                for (int e = 0; e < EMAX; ++e)
+                    if (e == eo[r]) g = reg[e];
+            } else {
+                g = row_lds[eo[r]];
+            }
+            gate_of[t * k + r] = __fdiv_rn(g, total);
+        }
+}
+
+template <typename XT>
+__global__ __launch_bounds__(kSmallThreads) void route_small_kernel(
+    const XT* __restrict__ x, const float* __restrict__ wr, const float* __restrict__ bias,
+    const uint8_t* __restrict__ valid, int T, int d, int E, int k, float w_aux, float w_z, int tile_m,
+    float* __restrict__ P, float* __restrict__ lse, int* __restrict__ expert_of, float* __restrict__ gate_of,
+    int* __restrict__ counts, int* __restrict__ offsets, int* __restrict__ tile_expert,
+    int* __restrict__ tile_row0, int* __restrict__ tile_rows, int* __restrict__ ntiles,
+    float* __restrict__ losses, int* __restrict__ perm_slot, int* __restrict__ perm_token,
+    int* __restrict__ inv_pos) {
+    __shared__ float prob[kSmallRouteMaxPairs];
+    __shared__ float lsev[kSmallRouteMaxTokens];
+    __shared__ int sexp[kSmallRouteMaxTokens * kMaxTopK];
+    __shared__ int cnt[kMaxExperts + 1];
+    __shared__ int off[kMaxExperts + 1];
+    __shared__ float aux_term[kMaxExperts];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int S = T * k;
+
+    // ---- logits ---------------------------------------------------------------
+    const int tail = d - d % 8;
+    const int tasks = T * E * 8;
+    for (int base = 0; base < tasks; base += kSmallThreads) {
+        const int task = base + tid;
+        const bool live = task < tasks;
+        const int pair = live ? task >> 3 : 0;
+        const int j = task & 7;
+        const int t = pair / E;
+        const int e = pair - t * E;
+        const XT* xr = x + (size_t)t * d;
+        const float* wrow = wr + (size_t)e * d;
+        // lane j of the pair: columns j, j + 8, ... in increasing order.  The loads of 32 steps
+        // are issued together (they do not depend on one another); the adds stay a chain.
+        float acc = 0.0f;
+        if (live) {
+            constexpr int U = 32;
+            for (int c0 = j; c0 < tail; c0 += 8 * U) {
+                float xv[U], wv[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int c = c0 + 8 * u;
+                    const int cc = c < tail ? c : j;  // always a valid column: no branch around the load
+                    xv[u] = to_f32(xr[cc]);
+                    wv[u] = wrow[cc];
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    if (c0 + 8 * u < tail) acc = __fadd_rn(acc, __fmul_rn(xv[u], wv[u]));
+            }
+        }
+        // lanes folded left to right, by the first thread of the group of eight
+        float sum = 0.0f;
+#pragma unroll
+        for (int l = 0; l < 8; ++l) sum = __fadd_rn(sum, __shfl(acc, (lane & ~7) + l));
+        if (live && j == 0) {
+            float rest = 0.0f;
+            for (int c = tail; c < d; ++c) rest = __fadd_rn(rest, __fmul_rn(to_f32(xr[c]), wrow[c]));
+            float v = __fadd_rn(sum, rest);
+            if (bias) v = __fadd_rn(v, bias[e]);
+            prob[pair] = v;
+        }
+    }
+    __syncthreads();
+
+    // ---- softmax_rows and route: one token per thread --------------------------
+    // With few experts the token's row lives in registers (every loop fully unrolled, the
+    // same operations in the same order); otherwise it stays in LDS.
+    if (tid < T) {
+        if (E <= 16)
+            token_phase<16>(prob + tid * E, tid, E, k, valid, P, lse, lsev, sexp, expert_of, gate_of);
+        else if (E <= 64)
+            token_phase<64>(prob + tid * E, tid, E, k, valid, P, lse, lsev, sexp, expert_of, gate_of);
+        else
+            token_phase<0>(prob + tid * E, tid, E, k, valid, P, lse, lsev, sexp, expert_of, gate_of);
+    }
+    __syncthreads();
+
+    // ---- bucket loop: a stable counting sort of the slots by expert ----------------
+    if (S <= 64) {
+        // one wave, slot = lane: a ballot per expert gives its count and every slot's rank
+        if (tid < 64) {
+            const int my = tid < S ? sexp[tid] : -1;
+            int run = 0, tiles = 0;
+            for (int e = 0; e < E; ++e) {
+                const unsigned long long mask = __ballot(my == e);
+                const int c = __popcll(mask);
+                if (my == e) {
+                    const int pos = run + __popcll(mask & ((1ull << tid) - 1ull));
+                    perm_slot[pos] = tid;
+                    perm_token[pos] = tid / k;
+                    inv_pos[tid] = pos;
+                }
+                if (tid == 0) {
+                    cnt[e] = c;
+                    counts[e] = c;
+                    offsets[e] = run;
+                    for (int r0 = 0; r0 < c; r0 += tile_m) {
+                        tile_expert[tiles] = e;
+                        tile_row0[tiles] = run + r0;
+                        tile_rows[tiles] = min(tile_m, c - r0);
+                        ++tiles;
+                    }
+                }
+                run += c;
+            }
+            if (tid < S && my < 0) inv_pos[tid] = -1;
+            if (tid == 0) {
+                offsets[E] = run;
+                ntiles[0] = tiles;
+            }
+        }
+    } else {
+        // one expert per thread, slots in increasing order
+        for (int e = tid; e < E; e += kSmallThreads) {
+            int c = 0;
+            for (int s = 0; s < S; ++s) c += (sexp[s] == e) ? 1 : 0;
+            cnt[e] = c;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            int run = 0, tiles = 0;
+            for (int e = 0; e < E; ++e) {
+                off[e] = run;
+                counts[e] = cnt[e];
+                offsets[e] = run;
+                for (int r0 = 0; r0 < cnt[e]; r0 += tile_m) {
+                    tile_expert[tiles] = e;
+                    tile_row0[tiles] = run + r0;
+                    tile_rows[tiles] = min(tile_m, cnt[e] - r0);
+                    ++tiles;
+                }
+                run += cnt[e];
+            }
+            off[E] = run;
+            offsets[E] = run;
+            ntiles[0] = tiles;
+        }
+        for (int s = tid; s < S; s += kSmallThreads)
+            if (sexp[s] < 0) inv_pos[s] = -1;
+        __syncthreads();
+        for (int e = tid; e < E; e += kSmallThreads) {
+            int pos = off[e];
+            for (int s = 0; s < S; ++s)
+                if (sexp[s] == e) {
+                    perm_slot[pos] = s;
+                    perm_token[pos] = s / k;
+                    inv_pos[s] = pos;
+                    ++pos;
+                }
+        }
+    }
+    __syncthreads();
+
+    // ---- auxiliary losses (src/moe.rs:325-337): per expert in token order ---------
+    int V = 0;
+    for (int t = 0; t < T; ++t) V += ((valid == nullptr) || valid[t]) ? 1 : 0;
+    for (int e = tid; e < E; e += kSmallThreads) {
+        float term = 0.0f;
+        if (V > 0) {
+            const float load = (float)cnt[e] / ((float)V * (float)k);
+            float mass = 0.0f;
+            for (int t = 0; t < T; ++t)
+                if ((valid == nullptr) || valid[t]) mass = mass + prob[t * E + e];
+            mass = mass / (float)V;
+            term = load * mass;
+        }
+        aux_term[e] = term;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        float aux = 0.0f, z = 0.0f;
+        if (V > 0) {
+            for (int e = 0; e < E; ++e) aux = aux + aux_term[e];
+            aux = aux * ((float)E * w_aux);
+            float zs = 0.0f;
+            for (int t = 0; t < T; ++t)
+                if ((valid == nullptr) || valid[t]) zs = zs + lsev[t] * lsev[t];
+            z = w_z * zs / (float)V;
+        }
+        losses[0] = aux;
+        losses[1] = z;
+    }
+}
+
+bool small_route_ok(int T, int E, int k) {
+    return T >= 1 && T <= kSmallRouteMaxTokens && E <= kMaxExperts && k <= kMaxTopK &&
+           T * E <= kSmallRouteMaxPairs;
+}
+
+hipError_t launch_route_small(const SmallRouteArgs& a, bool bf16, hipStream_t s) {
+    if (!small_route_ok(a.T, a.E, a.k)) return hipErrorInvalidValue;
+    if (bf16)
+        hipLaunchKernelGGL(route_small_kernel<bf16_t>, dim3(1), dim3(kSmallThreads), 0, s,
+                           static_cast<const bf16_t*>(a.x), a.wr, a.bias, a.valid, a.T, a.d, a.E, a.k, a.w_aux, a.w_z,
+                           a.tile_m, a.P, a.lse, a.expert_of, a.gate_of, a.counts, a.offsets, a.tile_expert,
+                           a.tile_row0, a.tile_rows, a.ntiles, a.losses, a.perm_slot, a.perm_token, a.inv_pos);
+    else
+        hipLaunchKernelGGL(route_small_kernel<float>, dim3(1), dim3(kSmallThreads), 0, s,
+                           static_cast<const float*>(a.x), a.wr, a.bias, a.valid, a.T, a.d, a.E, a.k, a.w_aux, a.w_z,
+                           a.tile_m, a.P, a.lse, a.expert_of, a.gate_of, a.counts, a.offsets, a.tile_expert,
+                           a.tile_row0, a.tile_rows, a.ntiles, a.losses, a.perm_slot, a.perm_token, a.inv_pos);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// decode_gemm_kernel: out[row, n] for one tile of at most 32 rows and one block of 32
+// output features (gate/up: 32 gate rows and the matching 32 up rows of the packed weights).
+// The four waves of a workgroup take a quarter of the reduction steps each; a wave fetches
+// its weight fragments (1 KB per step and row block, straight from the packed layout) in
+// batches of kBatch steps so that tens of kilobytes are in flight, multiplies them on the
+// matrix cores against token fragments read from global memory (32 rows x K: they stay in
+// L2), and the partial sums meet in LDS, in a fixed order.
+// blockIdx.y < max_tiles: routed tiles (those past *ntiles exit); the rest: 32-row blocks of
+// the shared expert, which takes every token.
+// ---------------------------------------------------------------------------
+constexpr int kBatch = 12;
+
+struct DecodeSide {
+    const bf16_t* a;
+    const int* row_index;
+    const char* w;
+    const float* scales;
+    bf16_t* out;
+    int N, K, row0, rows;
+};
+
+template <bool SWIGLU, bool I8>
+__global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs g) {
+    __shared__ float red[4][2][16][64];
+    const int fb = blockIdx.x;
+    const int ty = blockIdx.y;
+    DecodeSide sd;
+    if (ty < g.max_tiles) {
+        if (ty >= *g.ntiles) return;
+        const int expert = g.tile_expert[ty];
+        sd.a = static_cast<const bf16_t*>(g.a);
+        sd.row_index = g.row_index;
+        sd.w = static_cast<const char*>(g.w) + (size_t)expert * g.w_expert_stride * (I8 ? 1 : 2);
+        sd.scales = I8 ? g.scales + (size_t)expert * g.s_expert_stride : nullptr;
+        sd.out = static_cast<bf16_t*>(g.out);
+        sd.N = g.N;
+        sd.K = g.K;
+        sd.row0 = g.tile_row0[ty];
+        sd.rows = g.tile_rows[ty];
+    } else {
+        const int st = ty - g.max_tiles;
+        sd.a = static_cast<const bf16_t*>(g.a_shared);
+        sd.row_index = nullptr;
+        sd.w = static_cast<const char*>(g.w_shared);
+        sd.scales = I8 ? g.scales_shared : nullptr;
+        sd.out = static_cast<bf16_t*>(g.out_shared);
+        sd.N = g.N_shared;
+        sd.K = g.K_shared;
+        sd.row0 = st * 32;
+        sd.rows = min(32, g.T_shared - sd.row0);
+    }
+    if (fb * 32 >= sd.N) return;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int K = sd.K;
+    const int steps = K / 16;
+    const int chunk = (steps + 3) / 4;
+    const int g0 = min(steps, wave * chunk), g1 = min(steps, g0 + chunk);
+
+    // packed weights: row block rb starts at rb * K * 32 elements; step s, lane l at (s * 64 + l) * 16 bytes
+    // (int8: steps come in pairs, 16 bytes per lane and pair, the even step first)
+    const size_t block_bytes = (size_t)K * 32 * (I8 ? 1 : 2);
+    const char* w0 = sd.w + (size_t)fb * block_bytes;
+    const char* w1 = sd.w + (size_t)(sd.N / 32 + fb) * block_bytes;  // the matching up rows
+    auto wfrag = [&](const char* base, int s) -> bf16x8 {
+        if constexpr (I8) {
+            const uint2 q = *reinterpret_cast<const uint2*>(base + ((size_t)(s >> 1) * 64 + lane) * 16 + (s & 1) * 8);
+            return widen_i8(q);
+        } else {
+            const uint4 q = *reinterpret_cast<const uint4*>(base + ((size_t)s * 64 + lane) * 16);
+            return __builtin_bit_cast(bf16x8, q);
+        }
+    };
+    // token fragment: lane -> token lane % 32, columns 16 s + 8 (lane / 32) .. + 7
+    const int trow = (lane & 31) < sd.rows ? (lane & 31) : 0;
+    const int grow = sd.row_index ? sd.row_index[sd.row0 + trow] : sd.row0 + trow;
+    const bf16_t* arow = sd.a + (size_t)grow * K + 8 * (lane >> 5);
+
+    floatx16 acc0, acc1;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc0[v] = acc1[v] = 0.0f;
+
+    for (int s0 = g0; s0 < g1; s0 += kBatch) {
+        bf16x8 wa[kBatch], wb[kBatch], tf[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const int s = min(s0 + u, g1 - 1);
+            wa[u] = wfrag(w0, s);
+            if constexpr (SWIGLU) wb[u] = wfrag(w1, s);
+            tf[u] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(arow + 16 * s));
+        }
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            if (s0 + u < g1) {
+                acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wa[u], tf[u], acc0, 0, 0, 0);
+                if constexpr (SWIGLU) acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[u], tf[u], acc1, 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        red[wave][0][v][lane] = acc0[v];
+        if constexpr (SWIGLU) red[wave][1][v][lane] = acc1[v];
+    }
+    __syncthreads();
+    // accumulator element v of lane l: feature 8 (v / 4) + 4 (l / 32) + v % 4, token l % 32
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int idx = i * 256 + tid;
+        const int v = idx >> 6, l = idx & 63;
+        const int token = l & 31;
+        const int f = 8 * (v >> 2) + 4 * (l >> 5) + (v & 3);
+        float y = ((red[0][0][v][l] + red[1][0][v][l]) + red[2][0][v][l]) + red[3][0][v][l];
+        if constexpr (I8) y *= sd.scales[fb * 32 + f];
+        if constexpr (SWIGLU) {
+            float u = ((red[0][1][v][l] + red[1][1][v][l]) + red[2][1][v][l]) + red[3][1][v][l];
+            if constexpr (I8) u *= sd.scales[sd.N + fb * 32 + f];
+            y = silu_bf16_grade(y) * u;
+        }
+        if (token < sd.rows) sd.out[(size_t)(sd.row0 + token) * sd.N + fb * 32 + f] = from_f32<bf16_t>(y);
+    }
+}
+
+bool decode_shape_ok(int N, int K) { return K % 32 == 0 && K >= 32 && N % 32 == 0 && N >= 32; }
+
+hipError_t launch_decode_gemm(const DecodeGemmArgs& g, WeightKind wk, hipStream_t s) {
+    const int shared_tiles = g.a_shared ? (g.T_shared + 31) / 32 : 0;
+    const int tiles = g.max_tiles + shared_tiles;
+    if (tiles <= 0) return hipSuccess;
+    const int widest = g.a_shared ? (g.N > g.N_shared ? g.N : g.N_shared) : g.N;
+    const dim3 grid(widest / 32, tiles), block(256);
+    if (wk == WeightKind::BF16) {
+        if (g.swiglu) hipLaunchKernelGGL((decode_gemm_kernel<true, false>), grid, block, 0, s, g);
+        else hipLaunchKernelGGL((decode_gemm_kernel<false, false>), grid, block, 0, s, g);
+    } else if (wk == WeightKind::I8) {
+        if (g.swiglu) hipLaunchKernelGGL((decode_gemm_kernel<true, true>), grid, block, 0, s, g);
+        else hipLaunchKernelGGL((decode_gemm_kernel<false, true>), grid, block, 0, s, g);
+    } else {
+        return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+}  // namespace rbmoe

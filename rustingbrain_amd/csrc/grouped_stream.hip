@@ -33,9 +33,6 @@
 
 namespace rbmoe {
 
-typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
-typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
-
 namespace {
 
 constexpr int BM = 128;   // token rows per workgroup
@@ -46,23 +43,6 @@ constexpr int CPR = BK / 8;            // 16-byte pieces per LDS row
 constexpr int TT = BM / 32;            // token blocks per wave
 constexpr int KS = BK / 16;            // matrix-core steps per slice
 constexpr int DMA_PER_WAVE = BM * CPR / 64 / NW;  // LDS-DMA instructions per wave per slice (4)
-
-__device__ __forceinline__ uint32_t widen2(uint32_t word, int shift) {
-    const float lo = (float)(int)(int8_t)(word >> shift);
-    const float hi = (float)(int)(int8_t)(word >> (shift + 8));
-    return (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xffff0000u);  // small integers are exact in bf16
-}
-
-__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-    typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
-    bf16x2 v = {(__bf16)lo, (__bf16)hi};
-    return __builtin_bit_cast(uint32_t, v);
-}
-
-__device__ __forceinline__ bf16x8 widen_i8(uint2 q) {
-    const uint4 w = make_uint4(widen2(q.x, 0), widen2(q.x, 16), widen2(q.y, 0), widen2(q.y, 16));
-    return __builtin_bit_cast(bf16x8, w);
-}
 
 // Token fragment read from LDS.
 __device__ __forceinline__ bf16x8 lds_frag(const uint4* __restrict__ base, int idx) {

@@ -122,6 +122,7 @@ struct rbmoe_layer {
     bool force_generic = false;
     bool explicit_gather = false;  // materialise the gathered rows instead of gathering in the product
     bool use_stream = false;   // bf16 matrix-core kernels (packed weights); otherwise the generic kernels
+    bool decode_path = true;   // few tokens: four launches that stream every touched weight once
     int group_m = 4, variant = 0;
     const char* kernel_name = "none";
     int last_T = -1;
@@ -358,6 +359,7 @@ int rbmoe_layer_create(rbmoe_ctx* ctx, const rbmoe_config* cfg, rbmoe_layer** ou
     L->explicit_gather = env_int("RBMOE_EXPLICIT_GATHER", 0) == 1;
     L->group_m = std::max(1, env_int("RBMOE_GROUP_M", 4));
     L->variant = env_int("RBMOE_STREAM_VARIANT", 0) == 1 ? 1 : 0;
+    L->decode_path = env_int("RBMOE_NO_DECODE_PATH", 0) != 1;
     // bf16 matrix cores: bf16 activations, bf16 or int8 weights, widths that fit the packed layout
     const bool mc = !L->force_generic && cfg->act_dtype == RBMOE_BF16 && cfg->weight_dtype != RBMOE_F32;
     L->use_stream = mc && stream_shape_ok(cfg->d_ff, cfg->d_model) && stream_shape_ok(cfg->d_model, cfg->d_ff) &&
@@ -594,6 +596,67 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     const int tile_m0 = mfma ? stream_tile_m() : kGenericTileM;
     L->kernel_name = mfma ? (wk == WeightKind::I8 ? "mfma_bf16_stream_int8w" : "mfma_bf16_stream") : "generic";
     const bool gather_in_product = mfma && !L->explicit_gather;
+
+    // ---- a few tokens: route in one workgroup, then stream the touched weights once -------
+    if (mfma && L->decode_path && small_route_ok(T, E, k) && decode_shape_ok(F, d) && decode_shape_ok(d, F) &&
+        (!c.shared_expert || (decode_shape_ok(Fs, d) && decode_shape_ok(d, Fs)))) {
+        L->kernel_name = wk == WeightKind::I8 ? "mfma_bf16_decode_int8w" : "mfma_bf16_decode";
+        SmallRouteArgs sr{};
+        sr.x = x; sr.wr = (const float*)L->router.p; sr.bias = router_bias; sr.valid = valid;
+        sr.T = T; sr.d = d; sr.E = E; sr.k = k;
+        sr.w_aux = c.aux_loss_weight; sr.w_z = c.router_z_loss_weight;
+        sr.tile_m = kDecodeTileM;
+        sr.P = (float*)L->P.p; sr.lse = (float*)L->lse.p;
+        sr.expert_of = (int*)L->expert_of.p; sr.gate_of = (float*)L->gate_of.p;
+        sr.counts = (int*)L->counts.p; sr.offsets = (int*)L->offsets.p;
+        sr.tile_expert = (int*)L->tile_expert.p; sr.tile_row0 = (int*)L->tile_row0.p; sr.tile_rows = (int*)L->tile_rows.p;
+        sr.ntiles = (int*)L->ntiles.p; sr.losses = (float*)L->losses.p;
+        sr.perm_slot = (int*)L->perm_slot.p; sr.perm_token = (int*)L->perm_token.p; sr.inv_pos = (int*)L->inv_pos.p;
+        HIP_TRY(ctx, launch_route_small(sr, abf, s));
+        HIP_TRY(ctx, mark(1));
+        HIP_TRY(ctx, mark(2));
+        HIP_TRY(ctx, mark(3));
+
+        DecodeGemmArgs d1{};
+        d1.a = x; d1.row_index = (const int*)L->perm_token.p;
+        d1.w = L->wgu.p; d1.w_expert_stride = (size_t)2 * F * d;
+        d1.scales = wk == WeightKind::I8 ? (const float*)L->sgu.p : nullptr; d1.s_expert_stride = (size_t)2 * F;
+        d1.N = F; d1.K = d;
+        d1.tile_expert = (const int*)L->tile_expert.p; d1.tile_row0 = (const int*)L->tile_row0.p;
+        d1.tile_rows = (const int*)L->tile_rows.p; d1.ntiles = (const int*)L->ntiles.p;
+        d1.max_tiles = (T * k) / kDecodeTileM + E;
+        d1.out = L->h.p;
+        d1.swiglu = 1;
+        if (c.shared_expert) {
+            d1.a_shared = x; d1.w_shared = L->swgu.p;
+            d1.scales_shared = wk == WeightKind::I8 ? (const float*)L->ssgu.p : nullptr;
+            d1.N_shared = Fs; d1.K_shared = d; d1.T_shared = T; d1.out_shared = L->hs.p;
+        }
+        HIP_TRY(ctx, launch_decode_gemm(d1, wk, s));
+        HIP_TRY(ctx, mark(4));
+
+        DecodeGemmArgs d2 = d1;
+        d2.a = L->h.p; d2.row_index = nullptr;
+        d2.w = L->wd.p; d2.w_expert_stride = (size_t)d * F;
+        d2.scales = wk == WeightKind::I8 ? (const float*)L->sd.p : nullptr; d2.s_expert_stride = (size_t)d;
+        d2.N = d; d2.K = F;
+        d2.out = L->y.p;
+        d2.swiglu = 0;
+        if (c.shared_expert) {
+            d2.a_shared = L->hs.p; d2.w_shared = L->swd.p;
+            d2.scales_shared = wk == WeightKind::I8 ? (const float*)L->ssd.p : nullptr;
+            d2.N_shared = d; d2.K_shared = Fs; d2.out_shared = L->ys.p;
+        }
+        HIP_TRY(ctx, launch_decode_gemm(d2, wk, s));
+        HIP_TRY(ctx, mark(5));
+        HIP_TRY(ctx, mark(6));
+        CombineArgs cd{L->y.p, c.shared_expert ? L->ys.p : nullptr, residual, (const int*)L->inv_pos.p,
+                       (const float*)L->gate_of.p, T, d, k, out};
+        HIP_TRY(ctx, launch_combine(cd, abf, s));
+        HIP_TRY(ctx, mark(7));
+        L->last_T = T;
+        return RBMOE_OK;
+    }
 
     RouterArgs ra{x, (const float*)L->router.p, router_bias, valid, T, d, E, k,
                   (float*)L->P.p, (float*)L->lse.p, (int*)L->expert_of.p, (float*)L->gate_of.p,

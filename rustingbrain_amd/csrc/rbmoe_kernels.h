@@ -116,4 +116,61 @@ hipError_t launch_grouped_stream(const GroupedArgs& a, WeightKind wk, int varian
 void pack_weight_bf16(const uint16_t* src, int rows, int cols, uint16_t* dst);
 void pack_weight_i8(const int8_t* src, int rows, int cols, int8_t* dst);
 
+// ---- decode-shaped path (a few tokens) -------------------------------------------
+constexpr int kSmallRouteMaxTokens = 32;
+constexpr int kSmallRouteMaxPairs = 8192;  // T * E
+constexpr int kDecodeTileM = 32;
+
+struct SmallRouteArgs {
+    const void* x;
+    const float* wr;
+    const float* bias;
+    const uint8_t* valid;
+    int T, d, E, k;
+    float w_aux, w_z;
+    int tile_m;
+    float* P;
+    float* lse;
+    int* expert_of;
+    float* gate_of;
+    int* counts;
+    int* offsets;
+    int* tile_expert;
+    int* tile_row0;
+    int* tile_rows;
+    int* ntiles;
+    float* losses;
+    int* perm_slot;
+    int* perm_token;
+    int* inv_pos;
+};
+bool small_route_ok(int T, int E, int k);
+hipError_t launch_route_small(const SmallRouteArgs& a, bool bf16, hipStream_t s);
+
+// One launch covers the routed tiles (<= 32 rows each) and, when a_shared is set, the shared
+// expert over rows [0, T_shared).  Weights are in the packed layout of pack_weight_*.
+struct DecodeGemmArgs {
+    const void* a;
+    const int* row_index;
+    const void* w;
+    size_t w_expert_stride;  // elements
+    const float* scales;
+    size_t s_expert_stride;
+    int N, K;
+    const int* tile_expert;
+    const int* tile_row0;
+    const int* tile_rows;
+    const int* ntiles;
+    int max_tiles;
+    void* out;
+    const void* a_shared;
+    const void* w_shared;
+    const float* scales_shared;
+    int N_shared, K_shared, T_shared;
+    void* out_shared;
+    int swiglu;
+};
+bool decode_shape_ok(int N, int K);
+hipError_t launch_decode_gemm(const DecodeGemmArgs& g, WeightKind wk, hipStream_t s);
+
 }  // namespace rbmoe

@@ -1,0 +1,120 @@
+"""The decode-shaped path (at most 32 tokens, packed bf16 / int8 weights): one routing workgroup and two
+weight-streaming launches, against the oracle and against the large-batch path of the same library."""
+import os
+
+import numpy as np
+import pytest
+
+import rustingbrain_amd as rb
+from conftest import rel_l2
+from helpers import assert_routing_identical, gpu_layer, oracle_layer, small_workload
+from rustingbrain_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture
+def env():
+    saved = os.environ.get("RBMOE_NO_DECODE_PATH")
+    yield os.environ
+    if saved is None:
+        os.environ.pop("RBMOE_NO_DECODE_PATH", None)
+    else:
+        os.environ["RBMOE_NO_DECODE_PATH"] = saved
+
+
+def run(device, t, valid=None, bias=None, residual=None):
+    ref = oracle_layer(t).forward(t.x, valid=valid, router_bias=bias, threads=4)
+    layer = gpu_layer(device, t)
+    layout = rb.Layout(valid=None if valid is None else [bool(v) for v in valid])
+    out, cache = layer.forward_train(t.x, layout, router_bias=bias, residual=residual)
+    name = layer.kernel_name()
+    assert_routing_identical(cache, ref)
+    R = int(ref.offsets[-1])
+    if R:
+        h, y = layer.expert_rows(R)
+        assert rel_l2(h, ref.hidden) <= 2e-2, "hidden rows"
+        assert rel_l2(y, ref.expert_out) <= 2e-2, "expert output rows"
+    want = ref.out if residual is None else ref.out + residual
+    assert rel_l2(out, want) <= 2e-2
+    assert abs(cache.aux_loss() - ref.aux_loss) <= 1e-6 + 1e-5 * abs(ref.aux_loss)
+    assert abs(cache.z_loss() - ref.z_loss) <= 1e-6 + 1e-5 * abs(ref.z_loss)
+    layer.close()
+    return name, out, cache
+
+
+# widths are multiples of 64: the packed-weight kernels need that in both directions
+SHAPES = [dict(d=64, E=4, k=1, F=64, T=1), dict(d=128, E=8, k=2, F=128, T=8), dict(d=192, E=6, k=3, F=192, T=7),
+          dict(d=256, E=64, k=6, F=64, T=32), dict(d=128, E=5, k=2, F=320, T=19)]
+
+
+@pytest.mark.parametrize("wt", ["bf16", "int8"])
+@pytest.mark.parametrize("shared", [False, True])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "d{d}_E{E}_k{k}_F{F}_T{T}".format(**s))
+def test_decode_path_matches_the_oracle(device, env, shape, shared, wt):
+    env.pop("RBMOE_NO_DECODE_PATH", None)
+    t = synth.make(small_workload(seed=23, act="bf16", wt=wt, shared=shared, shared_d_ff=shape["F"] + 64, **shape))
+    name, _, _ = run(device, t)
+    assert name.startswith("mfma_bf16_decode"), name
+
+
+def test_decode_path_with_padding_bias_and_residual(device, env):
+    env.pop("RBMOE_NO_DECODE_PATH", None)
+    shape = dict(d=128, E=8, k=2, F=128, T=13)
+    t = synth.make(small_workload(seed=29, act="bf16", wt="bf16", shared=True, **shape))
+    valid = (np.arange(13) % 4 != 1).astype(np.uint8)
+    bias = np.zeros(8, np.float32)
+    bias[5] = 3.0  # nearly every token takes expert 5 first
+    residual = synth.round_bf16(synth.normal((13, 128), 1.0, 7, 5))
+    name, out, cache = run(device, t, valid=valid, bias=bias, residual=residual)
+    assert name.startswith("mfma_bf16_decode")
+    assert cache.counts[5] >= 8
+    assert (cache.expert_of.reshape(13, 2)[valid == 0] == -1).all()
+
+
+def test_decode_path_all_tokens_on_one_expert_fill_one_tile(device, env):
+    env.pop("RBMOE_NO_DECODE_PATH", None)
+    t = synth.make(small_workload(seed=31, act="bf16", wt="bf16", d=64, E=4, k=1, F=64, T=32))
+    bias = np.array([0, 50, 0, 0], np.float32)
+    name, out, cache = run(device, t, bias=bias)
+    assert name.startswith("mfma_bf16_decode")
+    assert cache.counts.tolist() == [0, 32, 0, 0]
+
+
+def test_decode_path_ties_and_nan_rows(device, env):
+    env.pop("RBMOE_NO_DECODE_PATH", None)
+    t = synth.make(small_workload(seed=2, act="bf16", wt="bf16", d=64, E=6, k=3, F=64, T=4))
+    t.router = np.zeros((6, 64), np.float32)  # all logits equal -> experts 0, 1, 2
+    name, out, cache = run(device, t)
+    assert name.startswith("mfma_bf16_decode")
+    assert cache.expert_of.reshape(4, 3).tolist() == [[0, 1, 2]] * 4
+    t = synth.make(small_workload(seed=2, act="bf16", wt="bf16", d=64, E=5, k=2, F=64, T=3))
+    t.x[1, 0] = np.nan
+    ref = oracle_layer(t).forward(t.x)
+    layer = gpu_layer(device, t)
+    out, cache = layer.forward_train(t.x)
+    assert layer.kernel_name().startswith("mfma_bf16_decode")
+    assert np.array_equal(cache.expert_of, ref.expert_of)
+    assert cache.expert_of.reshape(3, 2)[1].tolist() == [0, 1]
+    assert np.array_equal(np.isnan(cache.probabilities), np.isnan(ref.probabilities))
+    layer.close()
+
+
+def test_decode_and_large_batch_paths_agree(device, env):
+    shape = dict(d=128, E=8, k=2, F=192, T=24)
+    t = synth.make(small_workload(seed=37, act="bf16", wt="bf16", shared=True, **shape))
+    env.pop("RBMOE_NO_DECODE_PATH", None)
+    small = gpu_layer(device, t)
+    out_s, cache_s = small.forward_train(t.x)
+    assert small.kernel_name() == "mfma_bf16_decode"
+    env["RBMOE_NO_DECODE_PATH"] = "1"
+    large = gpu_layer(device, t)
+    out_l, cache_l = large.forward_train(t.x)
+    assert large.kernel_name() == "mfma_bf16_stream"
+    for f in ("expert_of", "counts", "offsets", "perm_slot", "perm_token"):
+        assert np.array_equal(getattr(cache_s, f), getattr(cache_l, f)), f
+    assert np.array_equal(cache_s.probabilities.view(np.uint32), cache_l.probabilities.view(np.uint32))
+    assert np.array_equal(cache_s.gate_of.view(np.uint32), cache_l.gate_of.view(np.uint32))
+    assert rel_l2(out_s, out_l) <= 5e-3
+    small.close()
+    large.close()
