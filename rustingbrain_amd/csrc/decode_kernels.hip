@@ -23,6 +23,7 @@ namespace rbmoe {
 // the bucket loop per expert (a stable counting sort), losses per expert in token order.
 // ---------------------------------------------------------------------------
 constexpr int kSmallThreads = 512;
+constexpr int kStageBytes = 44 * 1024;  // LDS for the staged router and token rows
 
 // softmax_rows (src/moe.rs, softmax over one row) and route (src/moe.rs:553-593) of one token, by one
 // thread.  EMAX > 0: the row is copied into EMAX registers and every loop over the experts is
@@ -131,6 +132,7 @@ __global__ __launch_bounds__(kSmallThreads) void route_small_kernel(
     int* __restrict__ tile_row0, int* __restrict__ tile_rows, int* __restrict__ ntiles,
     float* __restrict__ losses, int* __restrict__ perm_slot, int* __restrict__ perm_token,
     int* __restrict__ inv_pos) {
+    __shared__ __align__(16) unsigned char stage[kStageBytes];
     __shared__ float prob[kSmallRouteMaxPairs];
     __shared__ float lsev[kSmallRouteMaxTokens];
     __shared__ int sexp[kSmallRouteMaxTokens * kMaxTopK];
@@ -143,46 +145,106 @@ __global__ __launch_bounds__(kSmallThreads) void route_small_kernel(
     const int S = T * k;
 
     // ---- logits ---------------------------------------------------------------
-    const int tail = d - d % 8;
-    const int tasks = T * E * 8;
-    for (int base = 0; base < tasks; base += kSmallThreads) {
-        const int task = base + tid;
-        const bool live = task < tasks;
-        const int pair = live ? task >> 3 : 0;
-        const int j = task & 7;
-        const int t = pair / E;
-        const int e = pair - t * E;
-        const XT* xr = x + (size_t)t * d;
-        const float* wrow = wr + (size_t)e * d;
-        // lane j of the pair: columns j, j + 8, ... in increasing order.  The loads of 32 steps
-        // are issued together (they do not depend on one another); the adds stay a chain.
-        float acc = 0.0f;
-        if (live) {
-            constexpr int U = 32;
-            for (int c0 = j; c0 < tail; c0 += 8 * U) {
-                float xv[U], wv[U];
+    // When they fit, the router rows and the token rows are first copied to LDS with wide
+    // coalesced loads (one round trip to memory instead of one per batch of columns); rows are
+    // padded by 8 elements so that the eight pairs a wave works on fall into different banks.
+    const int ds = d + 8;
+    const bool staged = (d % 8 == 0) && ((size_t)E * ds * 4 + (size_t)T * ds * sizeof(XT) <= (size_t)kStageBytes) &&
+                        (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(wr) % 16 == 0);
+    if (staged) {
+        float* ws = reinterpret_cast<float*>(stage);
+        XT* xs = reinterpret_cast<XT*>(stage + (size_t)E * ds * 4);
+        const int wp = d / 4, xp = d * (int)sizeof(XT) / 16;  // 16-byte pieces per row
+        const int nw = E * wp, nx = T * xp;
+        const uint4* wsrc = reinterpret_cast<const uint4*>(wr);
+        const uint4* xsrc = reinterpret_cast<const uint4*>(x);
+        for (int i0 = 0; i0 < nw + nx; i0 += 4 * kSmallThreads) {
+            uint4 v[4];
 #pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int c = c0 + 8 * u;
-                    const int cc = c < tail ? c : j;  // always a valid column: no branch around the load
-                    xv[u] = to_f32(xr[cc]);
-                    wv[u] = wrow[cc];
+            for (int u = 0; u < 4; ++u) {
+                const int i = min(i0 + u * kSmallThreads + tid, nw + nx - 1);
+                v[u] = i < nw ? wsrc[i] : xsrc[i - nw];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int i = i0 + u * kSmallThreads + tid;
+                if (i < nw) {
+                    const int r = i / wp, c = i - r * wp;
+                    *reinterpret_cast<uint4*>(ws + (size_t)r * ds + 4 * c) = v[u];
+                } else if (i < nw + nx) {
+                    const int r = (i - nw) / xp, c = (i - nw) - r * xp;
+                    *reinterpret_cast<uint4*>(reinterpret_cast<char*>(xs + (size_t)r * ds) + 16 * c) = v[u];
                 }
-#pragma unroll
-                for (int u = 0; u < U; ++u)
-                    if (c0 + 8 * u < tail) acc = __fadd_rn(acc, __fmul_rn(xv[u], wv[u]));
             }
         }
-        // lanes folded left to right, by the first thread of the group of eight
-        float sum = 0.0f;
+        __syncthreads();
+        const int tasks = T * E * 8;
+        for (int base = 0; base < tasks; base += kSmallThreads) {
+            const int task = base + tid;
+            const bool live = task < tasks;
+            const int pair = live ? task >> 3 : 0;
+            const int j = task & 7;
+            const int t = pair / E;
+            const int e = pair - t * E;
+            const XT* xr = xs + (size_t)t * ds;
+            const float* wrow = ws + (size_t)e * ds;
+            const float bv = (bias && live && j == 0) ? bias[e] : 0.0f;  // fetched while the dot product runs
+            float acc = 0.0f;
+            if (live) {
+#pragma unroll 16
+                for (int c = j; c < d; c += 8) acc = __fadd_rn(acc, __fmul_rn(to_f32(xr[c]), wrow[c]));
+            }
+            float sum = 0.0f;
 #pragma unroll
-        for (int l = 0; l < 8; ++l) sum = __fadd_rn(sum, __shfl(acc, (lane & ~7) + l));
-        if (live && j == 0) {
-            float rest = 0.0f;
-            for (int c = tail; c < d; ++c) rest = __fadd_rn(rest, __fmul_rn(to_f32(xr[c]), wrow[c]));
-            float v = __fadd_rn(sum, rest);
-            if (bias) v = __fadd_rn(v, bias[e]);
-            prob[pair] = v;
+            for (int l = 0; l < 8; ++l) sum = __fadd_rn(sum, __shfl(acc, (lane & ~7) + l));
+            if (live && j == 0) {
+                float v = __fadd_rn(sum, 0.0f);  // the reference adds its (empty) scalar rest: sum + 0
+                if (bias) v = __fadd_rn(v, bv);
+                prob[pair] = v;
+            }
+        }
+    } else {
+        const int tail = d - d % 8;
+        const int tasks = T * E * 8;
+        for (int base = 0; base < tasks; base += kSmallThreads) {
+            const int task = base + tid;
+            const bool live = task < tasks;
+            const int pair = live ? task >> 3 : 0;
+            const int j = task & 7;
+            const int t = pair / E;
+            const int e = pair - t * E;
+            const XT* xr = x + (size_t)t * d;
+            const float* wrow = wr + (size_t)e * d;
+            // lane j of the pair: columns j, j + 8, ... in increasing order.  The loads of 32 steps
+            // are issued together (they do not depend on one another); the adds stay a chain.
+            float acc = 0.0f;
+            if (live) {
+                constexpr int U = 32;
+                for (int c0 = j; c0 < tail; c0 += 8 * U) {
+                    float xv[U], wv[U];
+    #pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        const int c = c0 + 8 * u;
+                        const int cc = c < tail ? c : j;  // always a valid column: no branch around the load
+                        xv[u] = to_f32(xr[cc]);
+                        wv[u] = wrow[cc];
+                    }
+    #pragma unroll
+                    for (int u = 0; u < U; ++u)
+                        if (c0 + 8 * u < tail) acc = __fadd_rn(acc, __fmul_rn(xv[u], wv[u]));
+                }
+            }
+            // lanes folded left to right, by the first thread of the group of eight
+            float sum = 0.0f;
+    #pragma unroll
+            for (int l = 0; l < 8; ++l) sum = __fadd_rn(sum, __shfl(acc, (lane & ~7) + l));
+            if (live && j == 0) {
+                float rest = 0.0f;
+                for (int c = tail; c < d; ++c) rest = __fadd_rn(rest, __fmul_rn(to_f32(xr[c]), wrow[c]));
+                float v = __fadd_rn(sum, rest);
+                if (bias) v = __fadd_rn(v, bias[e]);
+                prob[pair] = v;
+            }
         }
     }
     __syncthreads();

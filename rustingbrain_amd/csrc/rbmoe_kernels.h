@@ -118,7 +118,7 @@ void pack_weight_i8(const int8_t* src, int rows, int cols, int8_t* dst);
 
 // ---- decode-shaped path (a few tokens) -------------------------------------------
 constexpr int kSmallRouteMaxTokens = 32;
-constexpr int kSmallRouteMaxPairs = 8192;  // T * E
+constexpr int kSmallRouteMaxPairs = 2048;  // T * E
 constexpr int kDecodeTileM = 32;
 
 struct SmallRouteArgs {
