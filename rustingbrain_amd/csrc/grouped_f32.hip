@@ -1,0 +1,172 @@
+// Grouped expert products for all-f32 layers on the f32 matrix cores of gfx950
+// (v_mfma_f32_32x32x2_f32: f32 products, f32 accumulation).
+//
+//   out[row, n] = sum_c a[row, c] * w[expert][n, c]                 (down product)
+//   out[row, n] = silu(a . wgate[n]) * (a . wup[n])                 (gate/up product)
+//
+// A workgroup of 4 waves (2 x 2) owns 64 token rows x 64 output features; a wave owns 32 x 32
+// (gate/up: two accumulators, the gate rows and the matching up rows).  Both operands go
+// global -> registers -> LDS in slices of 32 reduction columns; the loads of slice k + 1 are in
+// flight while slice k is multiplied.  Rows are fetched through `row_index`, so the gather of
+// the routed rows (gather_rows, src/moe.rs:658-664) never materialises.  The weight fragment
+// is the matrix-core A operand and the token fragment B, so a lane ends with 4 consecutive
+// features of one token (one 16-byte store).  SiLU uses the exact division: this path is held
+// to 1e-5.
+#include "rbmoe_kernels.h"
+
+namespace rbmoe {
+
+namespace {
+
+constexpr int FM = 64;   // token rows per workgroup
+constexpr int FN = 64;   // output features per workgroup
+constexpr int FK = 32;   // reduction columns per slice
+constexpr int LS = FK + 1;  // LDS row stride: lanes of a fragment read fall into 64 distinct banks
+
+template <bool SWIGLU>
+__global__ __launch_bounds__(256) void grouped_f32_kernel(
+    const float* __restrict__ a, const int* __restrict__ row_index, const float* __restrict__ w,
+    size_t w_expert_stride, int N, int K, const int* __restrict__ tile_expert, const int* __restrict__ tile_row0,
+    const int* __restrict__ tile_rows, const int* __restrict__ ntiles, int dense_rows, float* __restrict__ out) {
+    constexpr int WR = SWIGLU ? 2 * FN : FN;  // weight rows staged per slice
+    __shared__ float As[FM * LS];
+    __shared__ float Ws[WR * LS];
+
+    int expert, row0, rows;
+    if (dense_rows >= 0) {
+        expert = 0;
+        row0 = blockIdx.y * FM;
+        rows = min(FM, dense_rows - row0);
+        if (rows <= 0) return;
+    } else {
+        if ((int)blockIdx.y >= *ntiles) return;
+        expert = tile_expert[blockIdx.y];
+        row0 = tile_row0[blockIdx.y];
+        rows = tile_rows[blockIdx.y];
+    }
+    const int n0 = blockIdx.x * FN;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wy = wave >> 1, wx = wave & 1;  // token half, feature half
+    const float* wbase = w + (size_t)expert * w_expert_stride;
+
+    // ---- staging: 16-byte pieces; thread -> (row, piece) ----------------------
+    // activations: 64 rows x 8 pieces = 512 pieces, 2 per thread; weights: WR rows x 8 pieces
+    constexpr int AP = FM * (FK / 4) / 256;  // 2
+    constexpr int WP = WR * (FK / 4) / 256;  // 2 or 4
+    const float* a_src[AP];
+    int a_dst[AP];
+#pragma unroll
+    for (int i = 0; i < AP; ++i) {
+        const int p = i * 256 + tid;
+        const int r = p >> 3, c = p & 7;
+        const int rr = r < rows ? r : 0;  // rows past the end of the group: products never stored
+        const int grow = row_index ? row_index[row0 + rr] : row0 + rr;
+        a_src[i] = a + (size_t)grow * K + 4 * c;
+        a_dst[i] = r * LS + 4 * c;
+    }
+    const float* w_src[WP];
+    int w_dst[WP];
+#pragma unroll
+    for (int i = 0; i < WP; ++i) {
+        const int p = i * 256 + tid;
+        const int r = p >> 3, c = p & 7;
+        // staged row r < FN: gate (or plain) feature n0 + r; r >= FN: the matching up row
+        const int feat = n0 + (r % FN);
+        const int fr = feat < N ? feat : 0;
+        const int wrow = (SWIGLU && r >= FN) ? N + fr : fr;
+        w_src[i] = wbase + (size_t)wrow * K + 4 * c;
+        w_dst[i] = r * LS + 4 * c;
+    }
+    float4 areg[AP], wreg[WP];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < AP; ++i) areg[i] = *reinterpret_cast<const float4*>(a_src[i] + k0);
+#pragma unroll
+        for (int i = 0; i < WP; ++i) wreg[i] = *reinterpret_cast<const float4*>(w_src[i] + k0);
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int i = 0; i < AP; ++i) {
+            float* d = As + a_dst[i];
+            d[0] = areg[i].x; d[1] = areg[i].y; d[2] = areg[i].z; d[3] = areg[i].w;
+        }
+#pragma unroll
+        for (int i = 0; i < WP; ++i) {
+            float* d = Ws + w_dst[i];
+            d[0] = wreg[i].x; d[1] = wreg[i].y; d[2] = wreg[i].z; d[3] = wreg[i].w;
+        }
+    };
+
+    floatx16 acc0, acc1;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc0[v] = acc1[v] = 0.0f;
+
+    // fragment addresses: lane l -> row l % 32 of the wave's block, reduction column 2 s + l / 32
+    const float* a_frag = As + (wy * 32 + (lane & 31)) * LS + (lane >> 5);
+    const float* w_frag = Ws + (wx * 32 + (lane & 31)) * LS + (lane >> 5);
+
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += FK) {
+        stage();
+        __syncthreads();
+        if (k0 + FK < K) fetch(k0 + FK);
+#pragma unroll
+        for (int s = 0; s < FK / 2; ++s) {
+            const float tv = a_frag[2 * s];
+            const float gv = w_frag[2 * s];
+            acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(gv, tv, acc0, 0, 0, 0);
+            if constexpr (SWIGLU) {
+                const float uv = w_frag[FN * LS + 2 * s];
+                acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(uv, tv, acc1, 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+
+    // accumulator element v of lane l: feature 8 (v / 4) + 4 (l / 32) + v % 4 of the wave's
+    // block, token l % 32
+    const int tok = wy * 32 + (lane & 31);
+    if (tok >= rows) return;
+    float* orow = out + (size_t)(row0 + tok) * N + n0 + wx * 32;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int f = 8 * q + 4 * (lane >> 5);
+        if (n0 + wx * 32 + f >= N) continue;  // N is a multiple of 4: a group of 4 is in or out as a whole
+        float4 y;
+        if constexpr (SWIGLU) {
+            y.x = silu_f32(acc0[4 * q + 0]) * acc1[4 * q + 0];
+            y.y = silu_f32(acc0[4 * q + 1]) * acc1[4 * q + 1];
+            y.z = silu_f32(acc0[4 * q + 2]) * acc1[4 * q + 2];
+            y.w = silu_f32(acc0[4 * q + 3]) * acc1[4 * q + 3];
+        } else {
+            y = make_float4(acc0[4 * q + 0], acc0[4 * q + 1], acc0[4 * q + 2], acc0[4 * q + 3]);
+        }
+        *reinterpret_cast<float4*>(orow + f) = y;
+    }
+}
+
+}  // namespace
+
+int f32_tile_m() { return FM; }
+
+// reduction width a multiple of the slice, output width a multiple of 4 (16-byte stores)
+bool f32_shape_ok(int N, int K) { return K % FK == 0 && K >= FK && N % 4 == 0 && N >= 4; }
+
+hipError_t launch_grouped_f32(const GroupedArgs& g, hipStream_t s) {
+    const int tiles_m = g.dense_rows >= 0 ? (g.dense_rows + FM - 1) / FM : g.max_tiles;
+    if (tiles_m <= 0) return hipSuccess;
+    const dim3 grid((g.N + FN - 1) / FN, tiles_m), block(256);
+    if (g.swiglu)
+        hipLaunchKernelGGL((grouped_f32_kernel<true>), grid, block, 0, s, static_cast<const float*>(g.a), g.row_index,
+                           static_cast<const float*>(g.w), g.w_expert_stride, g.N, g.K, g.tile_expert, g.tile_row0,
+                           g.tile_rows, g.ntiles, g.dense_rows, static_cast<float*>(g.out));
+    else
+        hipLaunchKernelGGL((grouped_f32_kernel<false>), grid, block, 0, s, static_cast<const float*>(g.a), g.row_index,
+                           static_cast<const float*>(g.w), g.w_expert_stride, g.N, g.K, g.tile_expert, g.tile_row0,
+                           g.tile_rows, g.ntiles, g.dense_rows, static_cast<float*>(g.out));
+    return hipGetLastError();
+}
+
+}  // namespace rbmoe

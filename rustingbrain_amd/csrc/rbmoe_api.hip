@@ -122,6 +122,7 @@ struct rbmoe_layer {
     bool force_generic = false;
     bool explicit_gather = false;  // materialise the gathered rows instead of gathering in the product
     bool use_stream = false;   // bf16 matrix-core kernels (packed weights); otherwise the generic kernels
+    bool use_f32_mc = false;   // all-f32 layer on the f32 matrix cores
     bool decode_path = true;   // few tokens: four launches that stream every touched weight once
     int group_m = 4, variant = 0;
     const char* kernel_name = "none";
@@ -365,6 +366,9 @@ int rbmoe_layer_create(rbmoe_ctx* ctx, const rbmoe_config* cfg, rbmoe_layer** ou
     L->use_stream = mc && stream_shape_ok(cfg->d_ff, cfg->d_model) && stream_shape_ok(cfg->d_model, cfg->d_ff) &&
                     (!cfg->shared_expert ||
                      (stream_shape_ok(L->Fs, cfg->d_model) && stream_shape_ok(cfg->d_model, L->Fs)));
+    L->use_f32_mc = !L->force_generic && cfg->act_dtype == RBMOE_F32 && cfg->weight_dtype == RBMOE_F32 &&
+                    f32_shape_ok(cfg->d_ff, cfg->d_model) && f32_shape_ok(cfg->d_model, cfg->d_ff) &&
+                    (!cfg->shared_expert || (f32_shape_ok(L->Fs, cfg->d_model) && f32_shape_ok(cfg->d_model, L->Fs)));
     {
         // the streaming kernel addresses activation rows with 32-bit byte offsets
         const size_t widest = (size_t)std::max(std::max(cfg->d_model, cfg->d_ff), L->Fs);
@@ -593,9 +597,11 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     HIP_TRY(ctx, mark(0));
 
     const bool mfma = L->use_stream;
-    const int tile_m0 = mfma ? stream_tile_m() : kGenericTileM;
-    L->kernel_name = mfma ? (wk == WeightKind::I8 ? "mfma_bf16_stream_int8w" : "mfma_bf16_stream") : "generic";
-    const bool gather_in_product = mfma && !L->explicit_gather;
+    const bool f32mc = L->use_f32_mc;
+    const int tile_m0 = mfma ? stream_tile_m() : (f32mc ? f32_tile_m() : kGenericTileM);
+    L->kernel_name = mfma ? (wk == WeightKind::I8 ? "mfma_bf16_stream_int8w" : "mfma_bf16_stream")
+                          : (f32mc ? "mfma_f32" : "generic");
+    const bool gather_in_product = (mfma || f32mc) && !L->explicit_gather;
 
     // ---- a few tokens: route in one workgroup, then stream the touched weights once -------
     if (mfma && L->decode_path && small_route_ok(T, E, k) && decode_shape_ok(F, d) && decode_shape_ok(d, F) &&
@@ -685,6 +691,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
 
     auto run = [&](const GroupedArgs& g, bool swiglu) -> hipError_t {
         if (mfma) return launch_grouped_stream(g, wk, L->variant, s);
+        if (f32mc) return launch_grouped_f32(g, s);
         return launch_grouped_generic(g, abf, wk, kGenericTileM, s);
     };
     GroupedArgs g1{};

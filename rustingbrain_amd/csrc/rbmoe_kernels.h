@@ -116,6 +116,11 @@ hipError_t launch_grouped_stream(const GroupedArgs& a, WeightKind wk, int varian
 void pack_weight_bf16(const uint16_t* src, int rows, int cols, uint16_t* dst);
 void pack_weight_i8(const int8_t* src, int rows, int cols, int8_t* dst);
 
+// f32 matrix cores (all-f32 layers): 64-row tiles, plain row-major weights.
+int f32_tile_m();
+bool f32_shape_ok(int N, int K);
+hipError_t launch_grouped_f32(const GroupedArgs& a, hipStream_t s);
+
 // ---- decode-shaped path (a few tokens) -------------------------------------------
 constexpr int kSmallRouteMaxTokens = 32;
 constexpr int kSmallRouteMaxPairs = 2048;  // T * E
