@@ -135,7 +135,7 @@ struct rbmoe_layer {
     Buf swgu, swd;         // shared [2Fs, d], [d, Fs]
     Buf ssgu, ssd;         // shared scales
     // workspace
-    Buf P, lse, expert_of, gate_of, rank_in_block, blockcnt, partial;
+    Buf P, lse, expert_of, gate_of, rank_in_block, blockcnt, partial, blockbase;
     Buf counts, offsets, tile_expert, tile_row0, tile_rows, ntiles, losses;
     Buf perm_slot, perm_token, inv_pos;
     Buf xg, h, y, hs, ys;
@@ -189,6 +189,7 @@ Plan make_plan(rbmoe_layer* L) {
     p.add(&L->rank_in_block, S * 4);
     p.add(&L->blockcnt, nb * E * 4);
     p.add(&L->partial, nb * (E + 1) * 4);
+    p.add(&L->blockbase, nb * E * 4);
     p.add(&L->counts, E * 4);
     p.add(&L->offsets, (E + 1) * 4);
     p.add(&L->tile_expert, (size_t)L->max_tiles * 4);
@@ -678,6 +679,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     da.rank_in_block = (const int*)L->rank_in_block.p;
     da.blockcnt = (const int*)L->blockcnt.p;
     da.partial = (const float*)L->partial.p;
+    da.blockbase = (int*)L->blockbase.p;
     da.T = T; da.d = d; da.E = E; da.k = k;
     da.w_aux = c.aux_loss_weight; da.w_z = c.router_z_loss_weight;
     da.tile_m = tile_m0;

@@ -55,6 +55,7 @@ struct DispatchArgs {
     int* tile_rows;
     int* ntiles;           // [1]
     float* losses;         // [2]
+    int* blockbase;        // [nb, E]  scratch: slots of expert e routed by the blocks before block b
     int* perm_slot;
     int* perm_token;
     int* inv_pos;

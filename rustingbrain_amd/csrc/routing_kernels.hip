@@ -378,13 +378,17 @@ __global__ __launch_bounds__(kRouterThreads) void router_kernel(
 // expert's list (src/moe.rs:266-274).  The optional row copy is `gather_rows`
 // (src/moe.rs:658-664); rows move as 16-byte pieces.
 // ---------------------------------------------------------------------------
-size_t dispatch_lds_bytes(int E, int k) {
+// dispatch_fused_kernel: for a modest number of router blocks the layout scan is folded into the
+// dispatch launch: every block re-derives counts, offsets and its own base from all the block
+// histograms (O(blocks^2 x experts) reads in total, but one launch less on the critical path);
+// block 0 also writes counts, offsets, the tile table and the losses.
+size_t dispatch_fused_lds_bytes(int E, int k) {
     const int parts = 256 / E;
     return ((size_t)2 * parts * E + (size_t)parts * (E + 1) + 4 * (size_t)(E + 1) + (size_t)kRouterTokens * k) * 4;
 }
 
 template <typename XT>
-__global__ __launch_bounds__(256) void dispatch_kernel(
+__global__ __launch_bounds__(256) void dispatch_fused_kernel(
     const XT* __restrict__ x, const int* __restrict__ expert_of, const int* __restrict__ rank_in_block,
     const int* __restrict__ blockcnt, const float* __restrict__ partial, int T, int d, int E, int k,
     float w_aux, float w_z, int tile_m, int* __restrict__ counts, int* __restrict__ offsets,
@@ -532,6 +536,257 @@ __global__ __launch_bounds__(256) void dispatch_kernel(
             losses[1] = z;
         }
     }
+
+    for (int ls = tid; ls < nls; ls += 256) {
+        const int s = t0 * k + ls;
+        const int ex = ls == tid ? ex_first : expert_of[s];
+        int pos = -1;
+        if (ex >= 0) {
+            pos = off[ex] + base[ex] + (ls == tid ? rank_first : rank_in_block[s]);
+            perm_slot[pos] = s;
+            perm_token[pos] = s / k;
+        }
+        inv_pos[s] = pos;
+        lpos[ls] = pos;
+    }
+    __syncthreads();
+    if (xg == nullptr) return;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    constexpr int VE = 16 / (int)sizeof(XT);  // elements per 16 bytes
+    const bool vec = (d % VE == 0);
+    for (int ls = wave; ls < nls; ls += 4) {
+        const int pos = lpos[ls];
+        if (pos < 0) continue;
+        const XT* src = x + (size_t)(t0 + ls / k) * d;
+        XT* dst = xg + (size_t)pos * d;
+        if (vec) {
+            const uint4* s4 = reinterpret_cast<const uint4*>(src);
+            uint4* d4 = reinterpret_cast<uint4*>(dst);
+            for (int c = lane; c < d / VE; c += 64) d4[c] = s4[c];
+        } else {
+            for (int c = lane; c < d; c += 64) dst[c] = src[c];
+        }
+    }
+}
+
+
+// layout_scan_kernel: one workgroup turns the per-block histograms into the global layout in
+// O(blocks x experts): counts and offsets per expert, for every router block the number of
+// slots of each expert routed by the blocks before it, the tile table of the grouped
+// products, and the two auxiliary losses (src/moe.rs:602-639) from the per-block partial sums.
+constexpr int kScanThreads = 1024;
+// router blocks x experts up to which the scan is folded into the dispatch launch
+constexpr long long kFusedScanLimit = 4096;
+
+// the blocks are cut into at most 16 consecutive parts: their partial results are folded serially
+__host__ __device__ static int scan_parts(int E) { return kScanThreads / E < 16 ? kScanThreads / E : 16; }
+
+size_t scan_lds_bytes(int E) {
+    const int parts = scan_parts(E);
+    return ((size_t)parts * E + (size_t)parts * (E + 1) + 3 * (size_t)(E + 1)) * 4;
+}
+
+__global__ __launch_bounds__(kScanThreads) void layout_scan_kernel(
+    const int* __restrict__ blockcnt, const float* __restrict__ partial, int nb, int E, int k, float w_aux,
+    float w_z, int tile_m, int* __restrict__ blockbase, int* __restrict__ counts, int* __restrict__ offsets,
+    int* __restrict__ tile_expert, int* __restrict__ tile_row0, int* __restrict__ tile_rows,
+    int* __restrict__ ntiles, float* __restrict__ losses) {
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    const int parts = scan_parts(E);  // E <= 256: at least 4 parts
+    int* part_sum = reinterpret_cast<int*>(lds_raw);                      // [parts][E]
+    float* part_mass = reinterpret_cast<float*>(part_sum + parts * E);   // [parts][E+1]
+    int* cnt = reinterpret_cast<int*>(part_mass + parts * (E + 1));      // [E+1]
+    int* off = cnt + (E + 1);                                             // [E+1]
+    float* mass = reinterpret_cast<float*>(off + (E + 1));               // [E+1]
+
+    const int tid = threadIdx.x;
+    const int len = (nb + parts - 1) / parts;
+    const int p = tid / E;
+    const int e = tid - p * E;
+    const bool active = p < parts;
+    const int b0 = min(nb, p * len), b1 = min(nb, b0 + len);
+    // Loads come in batches of 8 that do not depend on one another: one round trip per batch.
+    // The first kKeep histogram entries of a thread stay in registers for the second pass.
+    constexpr int kKeep = 32;
+    int keep[kKeep];
+    if (active) {
+        int sc = 0;
+        float m = 0.0f, zs = 0.0f;
+#pragma unroll
+        for (int i = 0; i < kKeep; i += 8) {
+            float v[8], z[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int bb = max(0, min(b0 + i + u, nb - 1));  // always a valid row: no branch around the loads
+                keep[i + u] = blockcnt[(size_t)bb * E + e];
+                v[u] = partial[(size_t)bb * (E + 1) + e];
+                z[u] = partial[(size_t)bb * (E + 1) + E];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                if (b0 + i + u < b1) {
+                    sc += keep[i + u];
+                    m += v[u];
+                    zs += z[u];
+                }
+            }
+        }
+        for (int b = b0 + kKeep; b < b1; b += 8) {
+            int c[8];
+            float v[8], z[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int bb = min(b + u, b1 - 1);
+                c[u] = blockcnt[(size_t)bb * E + e];
+                v[u] = partial[(size_t)bb * (E + 1) + e];
+                z[u] = partial[(size_t)bb * (E + 1) + E];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                if (b + u < b1) {
+                    sc += c[u];
+                    m += v[u];
+                    zs += z[u];
+                }
+            }
+        }
+        part_sum[p * E + e] = sc;
+        part_mass[p * (E + 1) + e] = m;
+        if (e == 0) part_mass[p * (E + 1) + E] = zs;
+    }
+    __syncthreads();
+    if (tid < E) {  // exclusive prefix over the parts, per expert
+        int run = 0;
+        float m = 0.0f;
+        for (int q = 0; q < parts; ++q) {
+            const int c = part_sum[q * E + tid];
+            part_sum[q * E + tid] = run;
+            run += c;
+            m += part_mass[q * (E + 1) + tid];
+        }
+        cnt[tid] = run;
+        mass[tid] = m;
+    }
+    if (tid == E) {
+        float zs = 0.0f;
+        for (int q = 0; q < parts; ++q) zs += part_mass[q * (E + 1) + E];
+        mass[E] = zs;
+    }
+    __syncthreads();
+    if (E <= 64) {  // exclusive prefix over the experts: one wave, log2(64) shuffle steps
+        if (tid < 64) {
+            const int c = tid < E ? cnt[tid] : 0;
+            int incl = c;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const int up = __shfl_up(incl, o);
+                if (tid >= o) incl += up;
+            }
+            if (tid < E) off[tid] = incl - c;
+            if (tid == E - 1) off[E] = incl;
+        }
+    } else if (tid == 0) {
+        int run = 0;
+        for (int q = 0; q < E; ++q) {
+            off[q] = run;
+            run += cnt[q];
+        }
+        off[E] = run;
+    }
+    __syncthreads();
+    if (active) {  // slots of expert e routed by the blocks before block b
+        int run = part_sum[p * E + e];
+#pragma unroll
+        for (int i = 0; i < kKeep; ++i) {
+            if (b0 + i < b1) {
+                blockbase[(size_t)(b0 + i) * E + e] = run;
+                run += keep[i];
+            }
+        }
+        for (int b = b0 + kKeep; b < b1; b += 8) {
+            int c[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) c[u] = blockcnt[(size_t)min(b + u, b1 - 1) * E + e];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                if (b + u < b1) {
+                    blockbase[(size_t)(b + u) * E + e] = run;
+                    run += c[u];
+                }
+            }
+        }
+    }
+    if (tid < E) {
+        counts[tid] = cnt[tid];
+        offsets[tid] = off[tid];
+        // tiles of this expert start after the tiles of the experts before it
+        int first = 0;
+        for (int q = 0; q < tid; ++q) first += (cnt[q] + tile_m - 1) / tile_m;
+        const int n = (cnt[tid] + tile_m - 1) / tile_m;
+        for (int i = 0; i < n; ++i) {
+            tile_expert[first + i] = tid;
+            tile_row0[first + i] = off[tid] + i * tile_m;
+            tile_rows[first + i] = min(tile_m, cnt[tid] - i * tile_m);
+        }
+        if (tid == E - 1) ntiles[0] = first + n;
+    }
+    if (tid == 0) {
+        offsets[E] = off[E];
+        // every valid token routes exactly k slots, so the valid-token count is routed / k
+        const int V = off[E] / k;
+        float aux = 0.0f, z = 0.0f;
+        if (V > 0) {
+            const float tokens = (float)V;
+            const float slots = (float)V * (float)k;
+            for (int q = 0; q < E; ++q) {
+                const float load = (float)cnt[q] / slots;
+                const float ms = mass[q] / tokens;
+                aux = aux + load * ms;
+            }
+            aux = aux * ((float)E * w_aux);
+            z = w_z * mass[E] / tokens;
+        }
+        losses[0] = aux;
+        losses[1] = z;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// dispatch_kernel: block b owns the same 32 tokens as router block b:
+// position = offsets[e] + blockbase[b][e] + rank in block.
+// ---------------------------------------------------------------------------
+size_t dispatch_lds_bytes(int E, int k) {
+    return ((size_t)2 * (E + 1) + (size_t)kRouterTokens * k) * 4;
+}
+
+template <typename XT>
+__global__ __launch_bounds__(256) void dispatch_kernel(
+    const XT* __restrict__ x, const int* __restrict__ expert_of, const int* __restrict__ rank_in_block,
+    const int* __restrict__ blockbase, const int* __restrict__ offsets, int T, int d, int E, int k,
+    int* __restrict__ perm_slot, int* __restrict__ perm_token, int* __restrict__ inv_pos, XT* __restrict__ xg) {
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    constexpr int TB = kRouterTokens;
+    int* base = reinterpret_cast<int*>(lds_raw);  // [E+1] slots of each expert routed by earlier blocks
+    int* off = base + (E + 1);                    // [E+1] first row of each expert group
+    int* lpos = off + (E + 1);                    // [TB * k]
+
+    const int tid = threadIdx.x;
+    const int blk = blockIdx.x;
+    const int t0 = blk * TB;
+    const int nt = min(TB, T - t0);
+    const int nls = nt * k;
+    // this thread's first slot and the block's two table rows are independent loads
+    int ex_first = -1, rank_first = 0;
+    if (tid < nls) {
+        ex_first = expert_of[(size_t)t0 * k + tid];
+        rank_first = rank_in_block[(size_t)t0 * k + tid];
+    }
+    for (int q = tid; q < E; q += 256) {
+        base[q] = blockbase[(size_t)blk * E + q];
+        off[q] = offsets[q];
+    }
+    __syncthreads();
 
     for (int ls = tid; ls < nls; ls += 256) {
         const int s = t0 * k + ls;
@@ -742,15 +997,33 @@ hipError_t launch_router(const RouterArgs& a, bool bf16, hipStream_t s) {
 template <typename XT>
 static hipError_t launch_dispatch_t(const DispatchArgs& a, hipStream_t s) {
     const int nb = (a.T + kRouterTokens - 1) / kRouterTokens;
-    hipLaunchKernelGGL(dispatch_kernel<XT>, dim3(nb > 0 ? nb : 1), dim3(256), dispatch_lds_bytes(a.E, a.k), s,
-                       static_cast<const XT*>(a.x), a.expert_of, a.rank_in_block, a.blockcnt, a.partial, a.T, a.d,
-                       a.E, a.k, a.w_aux, a.w_z, a.tile_m, a.counts, a.offsets, a.tile_expert, a.tile_row0,
-                       a.tile_rows, a.ntiles, a.losses, a.perm_slot, a.perm_token, a.inv_pos,
-                       static_cast<XT*>(a.xg));
+    if ((long long)nb * a.E <= kFusedScanLimit) {
+        hipLaunchKernelGGL(dispatch_fused_kernel<XT>, dim3(nb > 0 ? nb : 1), dim3(256),
+                           dispatch_fused_lds_bytes(a.E, a.k), s, static_cast<const XT*>(a.x), a.expert_of,
+                           a.rank_in_block, a.blockcnt, a.partial, a.T, a.d, a.E, a.k, a.w_aux, a.w_z, a.tile_m,
+                           a.counts, a.offsets, a.tile_expert, a.tile_row0, a.tile_rows, a.ntiles, a.losses,
+                           a.perm_slot, a.perm_token, a.inv_pos, static_cast<XT*>(a.xg));
+        return hipGetLastError();
+    }
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(layout_scan_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    // runs for T == 0 too: it then writes zero counts, an empty tile table and zero losses
+    hipLaunchKernelGGL(layout_scan_kernel, dim3(1), dim3(kScanThreads), scan_lds_bytes(a.E), s, a.blockcnt, a.partial,
+                       nb, a.E, a.k, a.w_aux, a.w_z, a.tile_m, a.blockbase, a.counts, a.offsets, a.tile_expert,
+                       a.tile_row0, a.tile_rows, a.ntiles, a.losses);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || nb == 0) return e;
+    hipLaunchKernelGGL(dispatch_kernel<XT>, dim3(nb), dim3(256), dispatch_lds_bytes(a.E, a.k), s,
+                       static_cast<const XT*>(a.x), a.expert_of, a.rank_in_block, a.blockbase, a.offsets, a.T, a.d,
+                       a.E, a.k, a.perm_slot, a.perm_token, a.inv_pos, static_cast<XT*>(a.xg));
     return hipGetLastError();
 }
 
-// Runs for T == 0 too: block 0 then writes zero counts, an empty tile table and zero losses.
 hipError_t launch_dispatch(const DispatchArgs& a, bool bf16, hipStream_t s) {
     return bf16 ? launch_dispatch_t<bf16_t>(a, s) : launch_dispatch_t<float>(a, s);
 }

@@ -258,3 +258,11 @@ def test_builder_surface_builds_the_sparse_layers(device):
     assert sorted(layers) == [1, 3]
     assert layers[1].num_parameters() == 4 * 16 + 5 * 3 * 16 * 12
     assert layers[1].active_parameters() == 4 * 16 + 3 * 3 * 16 * 12
+
+
+def test_many_router_blocks_take_the_separate_layout_scan(device):
+    # 66 router blocks x 64 experts is past the size up to which the layout scan rides in the dispatch launch
+    t = synth.make(small_workload(d=16, E=64, k=3, F=8, T=2100, seed=17))
+    valid = (np.arange(2100) % 13 != 5).astype(np.uint8)
+    out, cache, ref = check_parity(device, t, valid=valid)
+    assert int(cache.offsets[-1]) == int(valid.sum()) * 3
