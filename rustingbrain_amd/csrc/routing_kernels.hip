@@ -158,7 +158,8 @@ __global__ __launch_bounds__(NE * 64) void logits_kernel(const XT* __restrict__ 
     }
 }
 
-template <typename XT>
+// MAXJ = experts a lane may own: 1 when E <= 64 (a lane owns one expert), kMaxExperts / 64 otherwise.
+template <typename XT, int MAXJ>
 __global__ __launch_bounds__(kRouterThreads) void router_kernel(
     const XT* __restrict__ x, const float* __restrict__ wr, const float* __restrict__ bias,
     const uint8_t* __restrict__ valid, int T, int d, int E, int k, float* __restrict__ P,
@@ -200,7 +201,6 @@ __global__ __launch_bounds__(kRouterThreads) void router_kernel(
         const int gbase = lane_ & ~(G - 1);       // first lane of the group
         const int tpw = 64 / G;                   // tokens a wave handles at once
         const unsigned long long gmask = (G == 64 ? ~0ull : ((1ull << G) - 1ull)) << gbase;
-        constexpr int MAXJ = kMaxExperts / 64;    // experts per lane when G == 64
         const float neg_inf = __uint_as_float(0xff800000u);
         for (int i0 = wave_ * (TB / kRouterWaves); i0 < (wave_ + 1) * (TB / kRouterWaves); i0 += tpw) {
             const int i = i0 + lane_ / G;         // token of this group
@@ -229,9 +229,19 @@ __global__ __launch_bounds__(kRouterThreads) void router_kernel(
             }
             __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the group's LDS writes have landed
             __builtin_amdgcn_wave_barrier();
+            // the sum stays one chain of adds in index order; the LDS reads feeding it are issued
+            // eight at a time
             float sum = 0.0f;
-            if (live)
-                for (int e = 0; e < E; ++e) sum = __fadd_rn(sum, row[e]);
+            if (live) {
+                for (int e0 = 0; e0 < E; e0 += 8) {
+                    float ev[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) ev[u] = row[min(e0 + u, E - 1)];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+                        if (e0 + u < E) sum = __fadd_rn(sum, ev[u]);
+                }
+            }
             __builtin_amdgcn_wave_barrier();
             if (live && lig == 0) lsev[i] = __fadd_rn(mx, rb_logf(sum));
 #pragma unroll
@@ -247,32 +257,33 @@ __global__ __launch_bounds__(kRouterThreads) void router_kernel(
             unsigned taken_bits = 0;  // bit j: expert lig + G j is taken
             float total = 0.0f;
             for (int r = 0; r < k; ++r) {
-                // first expert not yet taken, and the best non-NaN candidate of this lane
-                int first = 0x7fffffff, ci = 0x7fffffff;
-                float cv = neg_inf;
+                // First expert not yet taken: the lowest set bit of a ballot over the group, taking
+                // the expert slices j in increasing order (slice j holds experts G j .. G j + G - 1).
+                int first = 0x7fffffff;
 #pragma unroll
                 for (int j = MAXJ - 1; j >= 0; --j) {
                     const int e = lig + G * j;
-                    if (e < E && !((taken_bits >> j) & 1u)) first = e;
+                    const unsigned long long m = __ballot(e < E && !((taken_bits >> j) & 1u)) & gmask;
+                    if (m != 0ull) first = (__ffsll((long long)m) - 1 - gbase) + G * j;
                 }
+                // Best non-NaN candidate: probabilities are never negative, so their bit patterns
+                // order like the values; with the inverted index below them, one 64-bit maximum over
+                // the group yields the greatest probability and, among equals, the lowest index.
+                unsigned long long key = 0ull;  // no candidate
 #pragma unroll
                 for (int j = 0; j < MAXJ; ++j) {
                     const int e = lig + G * j;
-                    if (e < E && !((taken_bits >> j) & 1u) && pv[j] == pv[j] && (ci == 0x7fffffff || pv[j] > cv)) {
-                        cv = pv[j];
-                        ci = e;
+                    if (e < E && !((taken_bits >> j) & 1u) && pv[j] == pv[j]) {
+                        const unsigned long long kj =
+                            ((unsigned long long)__float_as_uint(pv[j]) << 32) | (unsigned long long)(0xffffffffu - (unsigned)e);
+                        key = kj > key ? kj : key;
                     }
                 }
                 for (int o = 1; o < G; o <<= 1) {
-                    const int of = __shfl_xor(first, o);
-                    first = of < first ? of : first;
-                    const float ov = __shfl_xor(cv, o);
-                    const int oi = __shfl_xor(ci, o);
-                    if (oi != 0x7fffffff && (ci == 0x7fffffff || ov > cv || (ov == cv && oi < ci))) {
-                        cv = ov;
-                        ci = oi;
-                    }
+                    const unsigned long long other = __shfl_xor(key, o);
+                    key = other > key ? other : key;
                 }
+                const int ci = key != 0ull ? (int)(0xffffffffu - (unsigned)(key & 0xffffffffull)) : 0x7fffffff;
                 // the reference starts from the first untaken expert and replaces it only on a
                 // strictly greater probability: if that first one is NaN nothing replaces it
                 bool first_nan = false;
@@ -319,12 +330,18 @@ __global__ __launch_bounds__(kRouterThreads) void router_kernel(
     // ---- partial sums for the auxiliary losses (fixed order) --------------
     for (int e = tid; e <= E; e += kRouterThreads) {
         float s = 0.0f;
-        if (e < E) {
-            for (int i = 0; i < nt; ++i)
-                if (lexp[i * k] >= 0) s += prob[i * ES + e];
-        } else {
-            for (int i = 0; i < nt; ++i)
-                if (lexp[i * k] >= 0) s += lsev[i] * lsev[i];
+        for (int i0 = 0; i0 < nt; i0 += 8) {
+            float pvv[8];
+            int okv[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int i = min(i0 + u, nt - 1);
+                okv[u] = lexp[i * k];
+                pvv[u] = e < E ? prob[i * ES + e] : lsev[i] * lsev[i];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (i0 + u < nt && okv[u] >= 0) s += pvv[u];
         }
         partial[(size_t)blk * (E + 1) + e] = s;
     }
@@ -834,6 +851,10 @@ struct Vec16;
 template <>
 struct Vec16<float> {
     static constexpr int N = 4;
+    static __device__ __forceinline__ uint4 load_raw(const float* p) { return *reinterpret_cast<const uint4*>(p); }
+    static __device__ __forceinline__ void widen(const uint4& a, float (&v)[4]) {
+        v[0] = __uint_as_float(a.x); v[1] = __uint_as_float(a.y); v[2] = __uint_as_float(a.z); v[3] = __uint_as_float(a.w);
+    }
     static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
         const float4 a = *reinterpret_cast<const float4*>(p);
         v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
@@ -845,6 +866,13 @@ struct Vec16<float> {
 template <>
 struct Vec16<bf16_t> {
     static constexpr int N = 8;
+    static __device__ __forceinline__ uint4 load_raw(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
+    static __device__ __forceinline__ void widen(const uint4& a, float (&v)[8]) {
+        v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xffff0000u);
+        v[2] = __uint_as_float(a.y << 16); v[3] = __uint_as_float(a.y & 0xffff0000u);
+        v[4] = __uint_as_float(a.z << 16); v[5] = __uint_as_float(a.z & 0xffff0000u);
+        v[6] = __uint_as_float(a.w << 16); v[7] = __uint_as_float(a.w & 0xffff0000u);
+    }
     static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[8]) {
         const uint4 a = *reinterpret_cast<const uint4*>(p);
         v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xffff0000u);
@@ -906,24 +934,32 @@ __global__ __launch_bounds__(256) void combine_vec_kernel(
     float acc[VN];
 #pragma unroll
     for (int i = 0; i < VN; ++i) acc[i] = 0.0f;
+    // every row piece is fetched before the first add (no branch around a load: an unused slot
+    // re-reads row 0), so the k loads of a token are one round trip instead of k
+    uint4 raw[KMAX], raw_s, raw_r;
+#pragma unroll
+    for (int r = 0; r < KMAX; ++r) raw[r] = Vec16<XT>::load_raw(y + (size_t)(r < n ? pos[r] : 0) * d + c);
+    raw_s = raw_r = make_uint4(0, 0, 0, 0);
+    if (yshared) raw_s = Vec16<XT>::load_raw(yshared + (size_t)t * d + c);    // uniform over the launch
+    if (residual) raw_r = Vec16<XT>::load_raw(residual + (size_t)t * d + c);
 #pragma unroll
     for (int r = 0; r < KMAX; ++r) {
         if (r < n) {
             float v[VN];
-            Vec16<XT>::load(y + (size_t)pos[r] * d + c, v);
+            Vec16<XT>::widen(raw[r], v);
 #pragma unroll
             for (int i = 0; i < VN; ++i) acc[i] = __fadd_rn(acc[i], __fmul_rn(gate[r], v[i]));
         }
     }
     if (yshared) {
         float v[VN];
-        Vec16<XT>::load(yshared + (size_t)t * d + c, v);
+        Vec16<XT>::widen(raw_s, v);
 #pragma unroll
         for (int i = 0; i < VN; ++i) acc[i] = __fadd_rn(acc[i], v[i]);
     }
     if (residual) {
         float v[VN];
-        Vec16<XT>::load(residual + (size_t)t * d + c, v);
+        Vec16<XT>::widen(raw_r, v);
 #pragma unroll
         for (int i = 0; i < VN; ++i) acc[i] = __fadd_rn(acc[i], v[i]);
     }
@@ -971,8 +1007,11 @@ static hipError_t launch_router_t(const RouterArgs& a, hipStream_t s) {
     const int nb = (a.T + kRouterTokens - 1) / kRouterTokens;
     static bool attr_set = false;
     if (!attr_set) {  // allow more than the default 64 KiB of dynamic LDS (gfx950 has 160 KiB per CU)
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(router_kernel<XT>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(router_kernel<XT, 1>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kMaxRouterLds);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(router_kernel<XT, kMaxExperts / 64>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, kMaxRouterLds);
         if (e != hipSuccess) return e;
         attr_set = true;
     }
@@ -983,9 +1022,14 @@ static hipError_t launch_router_t(const RouterArgs& a, hipStream_t s) {
                        static_cast<const XT*>(a.x), a.wr, a.bias, a.T, a.d, a.E, a.P);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((router_kernel<XT>), dim3(nb), dim3(kRouterThreads), router_lds_bytes(a.E, a.k), s,
-                       static_cast<const XT*>(a.x), a.wr, a.bias, a.valid, a.T, a.d, a.E, a.k, a.P, a.lse,
-                       a.expert_of, a.gate_of, a.rank_in_block, a.blockcnt, a.partial);
+    if (a.E <= 64)
+        hipLaunchKernelGGL((router_kernel<XT, 1>), dim3(nb), dim3(kRouterThreads), router_lds_bytes(a.E, a.k), s,
+                           static_cast<const XT*>(a.x), a.wr, a.bias, a.valid, a.T, a.d, a.E, a.k, a.P, a.lse,
+                           a.expert_of, a.gate_of, a.rank_in_block, a.blockcnt, a.partial);
+    else
+        hipLaunchKernelGGL((router_kernel<XT, kMaxExperts / 64>), dim3(nb), dim3(kRouterThreads),
+                           router_lds_bytes(a.E, a.k), s, static_cast<const XT*>(a.x), a.wr, a.bias, a.valid, a.T, a.d,
+                           a.E, a.k, a.P, a.lse, a.expert_of, a.gate_of, a.rank_in_block, a.blockcnt, a.partial);
     return hipGetLastError();
 }
 
