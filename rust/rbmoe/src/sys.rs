@@ -1,0 +1,99 @@
+//! Raw declarations of `include/rbmoe.h`, one to one.
+#![allow(non_camel_case_types)]
+
+use std::os::raw::{c_char, c_int, c_void};
+
+pub const RBMOE_OK: c_int = 0;
+pub const RBMOE_INVALID_INPUT: c_int = 1;
+pub const RBMOE_INVALID_CONFIG: c_int = 2;
+pub const RBMOE_DEVICE_ERROR: c_int = 3;
+pub const RBMOE_BACKEND_UNAVAILABLE: c_int = 4;
+pub const RBMOE_MEMORY_BUDGET: c_int = 5;
+pub const RBMOE_OUT_OF_MEMORY: c_int = 6;
+pub const RBMOE_UNSUPPORTED: c_int = 7;
+pub const RBMOE_NULL_POINTER: c_int = 8;
+
+pub const RBMOE_F32: i32 = 0;
+pub const RBMOE_BF16: i32 = 1;
+pub const RBMOE_I8: i32 = 2;
+
+pub const RBMOE_W_ROUTER: i32 = 0;
+pub const RBMOE_W_GATE: i32 = 1;
+pub const RBMOE_W_UP: i32 = 2;
+pub const RBMOE_W_DOWN: i32 = 3;
+pub const RBMOE_W_SHARED_GATE: i32 = 4;
+pub const RBMOE_W_SHARED_UP: i32 = 5;
+pub const RBMOE_W_SHARED_DOWN: i32 = 6;
+
+pub const RBMOE_NUM_STAGES: usize = 8;
+
+#[repr(C)]
+#[derive(Clone, Copy, Debug, Default)]
+pub struct rbmoe_config {
+    pub d_model: i32,
+    pub num_experts: i32,
+    pub experts_per_token: i32,
+    pub d_ff: i32,
+    pub shared_expert: i32,
+    pub shared_d_ff: i32,
+    pub aux_loss_weight: f32,
+    pub router_z_loss_weight: f32,
+    pub weight_dtype: i32,
+    pub act_dtype: i32,
+    pub max_tokens: i32,
+}
+
+#[repr(C)]
+pub struct rbmoe_routing {
+    pub expert_of: *mut i32,
+    pub gate_of: *mut f32,
+    pub counts: *mut i32,
+    pub offsets: *mut i32,
+    pub perm_slot: *mut i32,
+    pub perm_token: *mut i32,
+    pub probabilities: *mut f32,
+    pub log_sum_exp: *mut f32,
+}
+
+#[repr(C)]
+pub struct rbmoe_ctx {
+    _private: [u8; 0],
+}
+#[repr(C)]
+pub struct rbmoe_layer {
+    _private: [u8; 0],
+}
+
+extern "C" {
+    pub fn rbmoe_config_init(cfg: *mut rbmoe_config, d_model: i32, num_experts: i32, experts_per_token: i32,
+                             d_ff: i32) -> c_int;
+    pub fn rbmoe_validate(cfg: *const rbmoe_config, msg: *mut c_char, msg_cap: usize) -> c_int;
+    pub fn rbmoe_parameter_counts(cfg: *const rbmoe_config, total: *mut u64, active: *mut u64) -> c_int;
+    pub fn rbmoe_ctx_create(device: i32, budget_mib: usize, out: *mut *mut rbmoe_ctx) -> c_int;
+    pub fn rbmoe_ctx_destroy(ctx: *mut rbmoe_ctx);
+    pub fn rbmoe_ctx_set_stream(ctx: *mut rbmoe_ctx, hip_stream: *mut c_void) -> c_int;
+    pub fn rbmoe_synchronize(ctx: *mut rbmoe_ctx) -> c_int;
+    pub fn rbmoe_last_error(ctx: *const rbmoe_ctx) -> *const c_char;
+    pub fn rbmoe_last_global_error() -> *const c_char;
+    pub fn rbmoe_layer_create(ctx: *mut rbmoe_ctx, cfg: *const rbmoe_config, out: *mut *mut rbmoe_layer) -> c_int;
+    pub fn rbmoe_layer_destroy(layer: *mut rbmoe_layer);
+    pub fn rbmoe_set_weight(layer: *mut rbmoe_layer, which: i32, expert: i32, data: *const c_void, dtype: i32,
+                            scales: *const f32, rows: i32, cols: i32) -> c_int;
+    pub fn rbmoe_forward(layer: *mut rbmoe_layer, x: *const c_void, tokens: i32, cols: i32, valid: *const u8,
+                         router_bias: *const f32, residual: *const c_void, out: *mut c_void) -> c_int;
+    pub fn rbmoe_forward_host(layer: *mut rbmoe_layer, x: *const c_void, tokens: i32, cols: i32, valid: *const u8,
+                              router_bias: *const f32, residual: *const c_void, out: *mut c_void) -> c_int;
+    pub fn rbmoe_forward_timed(layer: *mut rbmoe_layer, x: *const c_void, tokens: i32, cols: i32, valid: *const u8,
+                               router_bias: *const f32, residual: *const c_void, out: *mut c_void,
+                               ms: *mut f32) -> c_int;
+    pub fn rbmoe_get_losses(layer: *mut rbmoe_layer, aux_loss: *mut f32, z_loss: *mut f32) -> c_int;
+    pub fn rbmoe_get_routing(layer: *mut rbmoe_layer, routing: *mut rbmoe_routing) -> c_int;
+    pub fn rbmoe_get_expert_rows(layer: *mut rbmoe_layer, hidden: *mut f32, expert_out: *mut f32) -> c_int;
+    pub fn rbmoe_expert_kernel_name(layer: *const rbmoe_layer) -> *const c_char;
+    pub fn rbmoe_device_alloc(ctx: *mut rbmoe_ctx, bytes: usize, out: *mut *mut c_void) -> c_int;
+    pub fn rbmoe_device_free(ctx: *mut rbmoe_ctx, ptr: *mut c_void) -> c_int;
+    pub fn rbmoe_copy_to_device(ctx: *mut rbmoe_ctx, dst: *mut c_void, src: *const c_void, bytes: usize) -> c_int;
+    pub fn rbmoe_copy_to_host(ctx: *mut rbmoe_ctx, dst: *mut c_void, src: *const c_void, bytes: usize) -> c_int;
+    pub fn rbmoe_copy_device(ctx: *mut rbmoe_ctx, dst: *mut c_void, src: *const c_void, bytes: usize) -> c_int;
+    pub fn rbmoe_version() -> *const c_char;
+}
