@@ -1,8 +1,8 @@
-// TEST INFRASTRUCTURE — CPU oracle for the mixture-of-experts forward pass.
+// TEST INFRASTRUCTURE — CPU oracle for the mixture-of-experts layer.
 //
 // This file restates, on the CPU and in plain C++, the algorithm of
-// RustingBrain's `MoeLayer::forward_train` (reference src/moe.rs:243-341) and
-// the helpers under it.  It is NOT the Rust binary: no Rust toolchain exists
+// RustingBrain's `MoeLayer::forward_train` (reference src/moe.rs:243-341), of
+// `MoeLayer::backward` (src/moe.rs:348-489) and of the helpers under them.  It is NOT the Rust binary: no Rust toolchain exists
 // where this is built, so every function below follows the reference source
 // text line by line and cites the lines it follows.  Nothing in the shipped
 // library links, loads or calls this file; only tests, the smoke check and
@@ -25,7 +25,9 @@
 //     counts them.
 //
 // Pinned by: tests/test_oracle_*.py (hand vectors and known answers from the
-// reference's own unit tests, closed forms, brute force on small inputs).
+// reference's own unit tests, closed forms, brute force on small inputs; the
+// backward pass by the reference's four gradient tests and by finite
+// differences of an independent float64 evaluation of the layer).
 //
 // Build: see oracle/Makefile (g++ -O2 -ffp-contract=off -mavx2 -mfma).
 
@@ -704,6 +706,208 @@ int rbo_near_ties(const float* P, int T, int E, int k, int ulps) {
         if (a - b < ulps) ++n;
     }
     return n;
+}
+
+
+// ---------------------------------------------------------------------------
+// Backward pass: MoeLayer::backward (src/moe.rs:348-489) with SwiGlu::backward
+// (src/ffn.rs:87-120), Linear::backward (src/param.rs:799-825: weight.grad +=
+// grad_output^T . input, grad_input = grad_output . weight) and
+// silu_derivative (src/ffn.rs:235-238).  f32 expert weights only (the
+// reference's quantized experts have no backward).  The forward pass is
+// recomputed here to obtain what MoeCache holds.  Gradients are ACCUMULATED
+// into the weight-gradient buffers, as the reference accumulates into
+// Param.grad; grad_input is overwritten.
+// Order of the contributions to grad_input, as in the reference: shared expert,
+// then the routed experts in ascending expert index (rows ascending), then the
+// router.  The auxiliary losses' gradients reach the router here (the load
+// fractions are constants, as in the reference).
+// ---------------------------------------------------------------------------
+struct rbo_grads {
+    float* grad_input;    // [T, d]
+    float* grad_router;   // [E, d]
+    float* grad_gate;     // [E, F, d]
+    float* grad_up;       // [E, F, d]
+    float* grad_down;     // [E, d, F]
+    float* grad_sgate;    // [Fs, d] or NULL
+    float* grad_sup;      // [Fs, d] or NULL
+    float* grad_sdown;    // [d, Fs] or NULL
+    float* grad_gates;    // [T*k] dL/dgate per slot, or NULL (diagnostic)
+    float* grad_logits;   // [T, E] or NULL (diagnostic)
+};
+
+static float silu_derivative_ref(float x) {
+    const float s = 1.0f / (1.0f + std::exp(-x));
+    return s * (1.0f + x * (1.0f - s));
+}
+
+// y[M, K] = g[M, N] . w[N, K]      (grad_input = grad_output . weight)
+static void matmul_nn(const float* g, const float* w, int M, int N, int K, float* y) {
+    for (int m = 0; m < M; ++m) {
+        float* yr = y + (int64_t)m * K;
+        for (int c = 0; c < K; ++c) yr[c] = 0.0f;
+        for (int n = 0; n < N; ++n) {
+            const float gv = g[(int64_t)m * N + n];
+            const float* wr = w + (int64_t)n * K;
+            for (int c = 0; c < K; ++c) yr[c] = yr[c] + gv * wr[c];
+        }
+    }
+}
+
+// dw[N, K] += g[M, N]^T . x[M, K]  (weight.grad += grad_output^T . input)
+static void matmul_tn_acc(const float* g, const float* x, int M, int N, int K, float* dw) {
+    for (int m = 0; m < M; ++m) {
+        const float* xr = x + (int64_t)m * K;
+        for (int n = 0; n < N; ++n) {
+            const float gv = g[(int64_t)m * N + n];
+            float* dr = dw + (int64_t)n * K;
+            for (int c = 0; c < K; ++c) dr[c] = dr[c] + gv * xr[c];
+        }
+    }
+}
+
+// SwiGlu::backward for `rows` rows; returns grad_input in gx [rows, d]
+static void swiglu_backward(const rbo_expert_weights* w, const float* x, const float* gate, const float* up,
+                            const float* hidden, const float* gy, int rows, int d, int F, float* dgate_w,
+                            float* dup_w, float* ddown_w, float* gx) {
+    std::vector<float> gh((size_t)rows * F), gg((size_t)rows * F), gu((size_t)rows * F), tmp((size_t)rows * d);
+    matmul_tn_acc(gy, hidden, rows, d, F, ddown_w);       // down.weight.grad += gy^T . hidden
+    matmul_nn(gy, w->down, rows, d, F, gh.data());        // grad_hidden = gy . Wdown
+    for (int64_t i = 0; i < (int64_t)rows * F; ++i) {
+        const float g = gate[i];
+        gg[i] = gh[i] * up[i] * silu_derivative_ref(g);
+        gu[i] = gh[i] * silu_ref(g);
+    }
+    matmul_tn_acc(gg.data(), x, rows, F, d, dgate_w);
+    matmul_nn(gg.data(), w->gate, rows, F, d, gx);
+    matmul_tn_acc(gu.data(), x, rows, F, d, dup_w);
+    matmul_nn(gu.data(), w->up, rows, F, d, tmp.data());
+    for (int64_t i = 0; i < (int64_t)rows * d; ++i) gx[i] = gx[i] + tmp[i];
+}
+
+// Returns 0; 1 when cols != d_model; 2 when an expert is quantized.
+int rbo_moe_backward(const rbo_layer* L, const float* x, int T, int cols, const uint8_t* valid,
+                     const float* router_bias, const float* grad_output, rbo_grads* G) {
+    const int d = L->d_model, E = L->num_experts, k = L->experts_per_token, F = L->d_ff;
+    if (cols != d) return 1;
+    for (int e = 0; e < E; ++e)
+        if (L->experts[e].gate_q) return 2;
+    if (L->shared && L->shared->gate_q) return 2;
+    const int S = T * k;
+    const int Fs = L->shared_d_ff > 0 ? L->shared_d_ff : F;
+
+    // ---- what the forward pass cached ------------------------------------------
+    std::vector<float> logits((size_t)T * E), P((size_t)T * E), lse((size_t)T), gate_of((size_t)S);
+    std::vector<int32_t> expert_of((size_t)S), counts((size_t)E), offsets((size_t)E + 1), perm_slot((size_t)S),
+        perm_token((size_t)S);
+    rbo_router_logits(x, L->router, router_bias, T, d, E, logits.data());
+    rbo_softmax_rows(logits.data(), T, E, P.data(), lse.data());
+    rbo_route(P.data(), valid, T, E, k, expert_of.data(), gate_of.data());
+    rbo_bucket(expert_of.data(), S, E, k, counts.data(), offsets.data(), perm_slot.data(), perm_token.data());
+    const int R = offsets[E];
+    int V = 0;
+    for (int t = 0; t < T; ++t) V += (!valid || valid[t]) ? 1 : 0;
+    const size_t Rn = (size_t)std::max(R, 1);
+    std::vector<float> xg(Rn * d), gate(Rn * F), up(Rn * F), hidden(Rn * F), eout(Rn * d);
+    for (int i = 0; i < R; ++i)
+        std::memcpy(xg.data() + (int64_t)i * d, x + (int64_t)perm_token[i] * d, sizeof(float) * d);
+    for (int e = 0; e < E; ++e)
+        swiglu_rows(&L->experts[e], xg.data() + (int64_t)offsets[e] * d, 0, counts[e], d, F,
+                    gate.data() + (int64_t)offsets[e] * F, up.data() + (int64_t)offsets[e] * F,
+                    hidden.data() + (int64_t)offsets[e] * F, eout.data() + (int64_t)offsets[e] * d);
+
+    float* gin = G->grad_input;
+    std::memset(gin, 0, sizeof(float) * (size_t)T * d);
+
+    // ---- shared expert (src/moe.rs:356-361) ----------------------------------------
+    if (L->shared) {
+        std::vector<float> sg((size_t)T * Fs), su((size_t)T * Fs), sh((size_t)T * Fs), so((size_t)T * d),
+            sgx((size_t)T * d);
+        swiglu_rows(L->shared, x, 0, T, d, Fs, sg.data(), su.data(), sh.data(), so.data());
+        swiglu_backward(L->shared, x, sg.data(), su.data(), sh.data(), grad_output, T, d, Fs, G->grad_sgate,
+                        G->grad_sup, G->grad_sdown, sgx.data());
+        for (int64_t i = 0; i < (int64_t)T * d; ++i) gin[i] = gin[i] + sgx[i];
+    }
+
+    // ---- routed experts (src/moe.rs:366-399) -----------------------------------------
+    std::vector<float> grad_gates((size_t)std::max(S, 1), 0.0f);
+    for (int e = 0; e < E; ++e) {
+        const int rows = counts[e];
+        if (rows == 0) continue;
+        const int64_t base = offsets[e];
+        std::vector<float> scaled((size_t)rows * d), gx((size_t)rows * d);
+        for (int i = 0; i < rows; ++i) {
+            const float g = gate_of[perm_slot[base + i]];
+            const float* upstream = grad_output + (int64_t)perm_token[base + i] * d;
+            for (int c = 0; c < d; ++c) scaled[(int64_t)i * d + c] = g * upstream[c];
+        }
+        swiglu_backward(&L->experts[e], xg.data() + base * d, gate.data() + base * F, up.data() + base * F,
+                        hidden.data() + base * F, scaled.data(), rows, d, F, G->grad_gate + (int64_t)e * F * d,
+                        G->grad_up + (int64_t)e * F * d, G->grad_down + (int64_t)e * d * F, gx.data());
+        for (int i = 0; i < rows; ++i) {
+            float* dst = gin + (int64_t)perm_token[base + i] * d;
+            for (int c = 0; c < d; ++c) dst[c] = dst[c] + gx[(int64_t)i * d + c];
+        }
+    }
+    // gate gradients: one dot product per routed slot (src/moe.rs:404-416)
+    for (int e = 0; e < E; ++e)
+        for (int i = 0; i < counts[e]; ++i) {
+            const int64_t pos = offsets[e] + i;
+            const float* go = grad_output + (int64_t)perm_token[pos] * d;
+            const float* eo = eout.data() + pos * d;
+            float sum = 0.0f;
+            for (int c = 0; c < d; ++c) sum = sum + go[c] * eo[c];
+            grad_gates[perm_slot[pos]] = sum;
+        }
+
+    // ---- through the renormalisation, the softmax and the two losses (src/moe.rs:421-478) ----
+    std::vector<float> gp((size_t)T * E, 0.0f), gl((size_t)T * E, 0.0f);
+    for (int t = 0; t < T; ++t) {
+        const int32_t* sel = expert_of.data() + (int64_t)t * k;
+        if (sel[0] < 0) continue;
+        const float* p = P.data() + (int64_t)t * E;
+        float total = 0.0f;
+        for (int r = 0; r < k; ++r) total = total + p[sel[r]];
+        if (total <= 0.0f) continue;
+        float weighted = 0.0f;
+        for (int r = 0; r < k; ++r) weighted = weighted + grad_gates[(int64_t)t * k + r] * p[sel[r]];
+        float* row = gp.data() + (int64_t)t * E;
+        for (int r = 0; r < k; ++r)
+            row[sel[r]] = row[sel[r]] + (grad_gates[(int64_t)t * k + r] / total - weighted / (total * total));
+    }
+    if (L->aux_loss_weight != 0.0f && V > 0) {
+        const float scale = L->aux_loss_weight * (float)E / (float)V;
+        const float slots = (float)(V * k);
+        for (int e = 0; e < E; ++e) {
+            const float load = (float)counts[e] / slots;
+            for (int t = 0; t < T; ++t) {
+                if (expert_of[(int64_t)t * k] < 0) continue;
+                gp[(int64_t)t * E + e] = gp[(int64_t)t * E + e] + scale * load;
+            }
+        }
+    }
+    for (int t = 0; t < T; ++t) {
+        if (expert_of[(int64_t)t * k] < 0) continue;
+        const float* p = P.data() + (int64_t)t * E;
+        const float* upstream = gp.data() + (int64_t)t * E;
+        float dot = 0.0f;
+        for (int e = 0; e < E; ++e) dot = dot + p[e] * upstream[e];
+        float* row = gl.data() + (int64_t)t * E;
+        for (int e = 0; e < E; ++e) row[e] = p[e] * (upstream[e] - dot);
+        if (L->router_z_loss_weight != 0.0f) {
+            const float factor = 2.0f * L->router_z_loss_weight * lse[t] / (float)std::max(V, 1);
+            for (int e = 0; e < E; ++e) row[e] = row[e] + factor * p[e];
+        }
+    }
+    // ---- router (src/moe.rs:480-484) ------------------------------------------------
+    matmul_tn_acc(gl.data(), x, T, E, d, G->grad_router);
+    std::vector<float> from_router((size_t)T * d);
+    matmul_nn(gl.data(), L->router, T, E, d, from_router.data());
+    for (int64_t i = 0; i < (int64_t)T * d; ++i) gin[i] = gin[i] + from_router[i];
+
+    if (G->grad_gates && S > 0) std::memcpy(G->grad_gates, grad_gates.data(), sizeof(float) * (size_t)S);
+    if (G->grad_logits) std::memcpy(G->grad_logits, gl.data(), sizeof(float) * (size_t)T * E);
+    return 0;
 }
 
 }  // extern "C"

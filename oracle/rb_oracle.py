@@ -282,6 +282,29 @@ class ForwardResult:
         return self.counts.astype(np.float32) / np.float32(slots)
 
 
+class _Grads(C.Structure):
+    _fields_ = [("grad_input", _f32p), ("grad_router", _f32p), ("grad_gate", _f32p), ("grad_up", _f32p),
+                ("grad_down", _f32p), ("grad_sgate", _f32p), ("grad_sup", _f32p), ("grad_sdown", _f32p),
+                ("grad_gates", _f32p), ("grad_logits", _f32p)]
+
+
+_lib.rbo_moe_backward.restype = C.c_int
+_lib.rbo_moe_backward.argtypes = [C.POINTER(_Layer), _f32p, C.c_int, C.c_int, _u8p, _f32p, _f32p, C.POINTER(_Grads)]
+
+
+@dataclass
+class BackwardResult:
+    """Gradients of MoeLayer::backward (src/moe.rs:348-489); the weight gradients start from zero here."""
+    grad_input: np.ndarray     # [T, d]
+    grad_router: np.ndarray    # [E, d]
+    grad_gate: np.ndarray      # [E, F, d]
+    grad_up: np.ndarray        # [E, F, d]
+    grad_down: np.ndarray      # [E, d, F]
+    grad_shared: Optional[tuple]  # (gate [Fs, d], up [Fs, d], down [d, Fs]) or None
+    grad_gates: np.ndarray     # [T*k]
+    grad_logits: np.ndarray    # [T, E]
+
+
 @dataclass
 class OracleLayer:
     d_model: int
@@ -342,3 +365,39 @@ class OracleLayer:
         res["hidden"] = res["hidden"][:R]
         res["expert_out"] = res["expert_out"][:R]
         return ForwardResult(aux_loss=float(outs.aux_loss), z_loss=float(outs.z_loss), **res)
+
+    def backward(self, x: np.ndarray, grad_output: np.ndarray, valid: Optional[np.ndarray] = None,
+                 router_bias: Optional[np.ndarray] = None) -> BackwardResult:
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        grad_output = np.ascontiguousarray(grad_output, dtype=np.float32)
+        T, cols = x.shape
+        E, k, F, d = self.num_experts, self.experts_per_token, self.d_ff, self.d_model
+        Fs = self.shared_d_ff or F
+        arr = (_ExpertWeights * E)(*[w._c() for w in self.experts])
+        shared_c = self.shared._c() if self.shared is not None else None
+        layer = _Layer(d, E, k, F, 1 if self.shared is not None else 0, self.shared_d_ff,
+                       self.aux_loss_weight, self.router_z_loss_weight, _fp(self.router),
+                       C.cast(arr, C.POINTER(_ExpertWeights)),
+                       C.pointer(shared_c) if shared_c is not None else None)
+        gi = np.zeros((T, d), np.float32)
+        gr = np.zeros((E, d), np.float32)
+        gg = np.zeros((E, F, d), np.float32)
+        gu = np.zeros((E, F, d), np.float32)
+        gd = np.zeros((E, d, F), np.float32)
+        sh = (np.zeros((Fs, d), np.float32), np.zeros((Fs, d), np.float32), np.zeros((d, Fs), np.float32)) \
+            if self.shared is not None else None
+        ggates = np.zeros((max(T * k, 1),), np.float32)
+        gl = np.zeros((T, E), np.float32)
+        grads = _Grads(_fp(gi), _fp(gr), _fp(gg), _fp(gu), _fp(gd), _fp(sh[0]) if sh else None,
+                       _fp(sh[1]) if sh else None, _fp(sh[2]) if sh else None, _fp(ggates), _fp(gl))
+        if valid is not None:
+            valid = np.ascontiguousarray(valid, dtype=np.uint8)
+        if router_bias is not None:
+            router_bias = np.ascontiguousarray(router_bias, dtype=np.float32)
+        rc = _lib.rbo_moe_backward(C.byref(layer), _fp(x), T, cols, _up(valid), _fp(router_bias), _fp(grad_output),
+                                   C.byref(grads))
+        if rc == 1:
+            raise ValueError(f"InvalidInput: expected {d} columns, got {cols}")
+        if rc == 2:
+            raise ValueError("quantized experts have no backward pass")
+        return BackwardResult(gi, gr, gg, gu, gd, sh, ggates[:T * k], gl)
