@@ -171,6 +171,27 @@ int rbmoe_get_routing(rbmoe_layer* layer, rbmoe_routing* routing);
  * (src/moe.rs:150-152, src/ffn.rs:27-33).  Synchronises. */
 int rbmoe_get_expert_rows(rbmoe_layer* layer, float* hidden, float* expert_out);
 
+/* ---- backward pass (MoeLayer::backward, src/moe.rs:348-489) ------------------------------
+ * Training mode makes the forward keep what MoeCache keeps for the backward pass (the input,
+ * src/moe.rs:133-135; gate and up pre-activations, src/ffn.rs:27-33) and allocates f32 gradient
+ * accumulators, the role of Param.grad (src/param.rs).  bf16 layers on the matrix-core path only;
+ * call it before the weights are set.  A training layer always takes the large-batch kernels. */
+int rbmoe_layer_enable_training(rbmoe_layer* layer);
+
+/* MoeLayer::backward on DEVICE pointers for the last forward: `grad_output` [T, d] act_dtype in,
+ * `grad_input` [T, d] act_dtype out; weight gradients are ACCUMULATED (as Param.grad is) until
+ * rbmoe_zero_grads.  The gradients of the two auxiliary losses reach the router here, as in the
+ * reference (src/moe.rs:343-347).  Enqueued on the context's stream. */
+int rbmoe_backward(rbmoe_layer* layer, const void* grad_output, void* grad_input);
+/* Same on HOST pointers; synchronises. */
+int rbmoe_backward_host(rbmoe_layer* layer, const void* grad_output, void* grad_input);
+/* Param::zero_grad for every weight of the layer. */
+int rbmoe_zero_grads(rbmoe_layer* layer);
+/* One accumulated weight gradient as f32 [rows, cols] into host memory (same ids and shapes as
+ * rbmoe_set_weight).  Synchronises. */
+int rbmoe_get_weight_grad(rbmoe_layer* layer, int32_t which, int32_t expert, float* host, int32_t rows,
+                          int32_t cols);
+
 /* Per-stage timing of one forward with HIP events on the context's stream.
  * `ms` receives RBMOE_NUM_STAGES durations in milliseconds.  Synchronises.
  * Stage 1 brackets no work at all: it reads what one pair of event records adds to

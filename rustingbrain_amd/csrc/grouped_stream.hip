@@ -123,7 +123,8 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
     const bf16_t* __restrict__ a, const int* __restrict__ row_index, const void* __restrict__ wpacked,
     size_t w_expert_stride_bytes, const float* __restrict__ scales, size_t s_expert_stride, int N, int K,
     const int* __restrict__ tile_expert, const int* __restrict__ tile_row0, const int* __restrict__ tile_rows,
-    const int* __restrict__ ntiles, int dense_rows, bf16_t* __restrict__ out, int group_m) {
+    const int* __restrict__ ntiles, int dense_rows, bf16_t* __restrict__ out, bf16_t* __restrict__ gu_out,
+    int group_m) {
     constexpr int BN = SWIGLU ? NW * 32 : NW * 64;  // output features per workgroup
     // Two LDS stages of one activation slice each; the epilogue reuses both as one
     // 128 x 128 staging tile for the output.
@@ -364,12 +365,18 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
     // 16-byte stores, 16 consecutive lanes covering the 256 contiguous bytes of a row.
     const float* sc = I8 ? scales + (size_t)expert * s_expert_stride : nullptr;
     char* const stage = reinterpret_cast<char*>(As);
-    constexpr int PASSES = SWIGLU ? 1 : 2;
+    // Passes through the staging tile: down product: the two blocks of 128 features; gate/up: the
+    // hidden rows, then (only when the caller keeps them for a backward pass) the gate and the
+    // up pre-activations, which go to `gu_out` [rows, 2N] with the gate half in columns [0, N).
+    constexpr int PASSES = SWIGLU ? 3 : 2;
     __syncthreads();  // every wave's last DMA has landed and its last fragment reads are done
 #pragma unroll
     for (int b = 0; b < PASSES; ++b) {
+        if constexpr (SWIGLU) {
+            if (b > 0 && gu_out == nullptr) break;  // uniform over the launch
+        }
         if (b) __syncthreads();  // the previous pass has been read out
-        if (b ? act1 : act0) {
+        if (SWIGLU ? act0 : (b ? act1 : act0)) {
             const int rb = b ? r1 : r0;
 #pragma unroll
             for (int t = 0; t < TT; ++t) {
@@ -387,7 +394,7 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
                                 gv *= sc[r0 + f + i];
                                 uv *= sc[r1 + f + i];
                             }
-                            y[i] = silu_bf16_grade(gv) * uv;
+                            y[i] = b == 0 ? silu_bf16_grade(gv) * uv : (b == 1 ? gv : uv);
                         } else {
                             y[i] = acc[b][t][4 * q + i];
                             if constexpr (I8) y[i] *= sc[rb + f + i];
@@ -400,14 +407,18 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
             }
         }
         __syncthreads();
-        const int col0 = tn_idx * BN + b * (NW * 32);
+        // where this pass goes: hidden rows and down rows into `out` (row stride N), the
+        // pre-activations into `gu_out` (row stride 2 N)
+        const int col0 = tn_idx * BN + (SWIGLU ? 0 : b * (NW * 32));
+        bf16_t* const dst = (SWIGLU && b > 0) ? gu_out + (b == 2 ? N : 0) : out;
+        const size_t dstride = (SWIGLU && b > 0) ? (size_t)2 * N : (size_t)N;
 #pragma unroll
         for (int i = 0; i < BM * 16 / NT; ++i) {
             const int idx = i * NT + tid;
             const int r = idx >> 4, p = idx & 15;
             if (r < rows && col0 + 8 * p < N) {
                 const uint4 v = *reinterpret_cast<const uint4*>(stage + r * 256 + ((p ^ (r & 15)) * 16));
-                *reinterpret_cast<uint4*>(out + (size_t)(row0 + r) * N + col0 + 8 * p) = v;
+                *reinterpret_cast<uint4*>(dst + (size_t)(row0 + r) * dstride + col0 + 8 * p) = v;
             }
         }
     }
@@ -424,7 +435,7 @@ hipError_t launch_t(const GroupedArgs& g, hipStream_t s) {
     hipLaunchKernelGGL((grouped_stream_kernel<SWIGLU, I8, RING, TFBUF, AREG>), dim3(grid), dim3(NT), 0, s,
                        static_cast<const bf16_t*>(g.a), g.row_index, g.w, g.w_expert_stride * (I8 ? 1 : 2), g.scales,
                        g.s_expert_stride, g.N, g.K, g.tile_expert, g.tile_row0, g.tile_rows, g.ntiles, g.dense_rows,
-                       static_cast<bf16_t*>(g.out), g.group_m > 0 ? g.group_m : 4);
+                       static_cast<bf16_t*>(g.out), static_cast<bf16_t*>(g.gu_out), g.group_m > 0 ? g.group_m : 4);
     return hipGetLastError();
 }
 

@@ -139,6 +139,17 @@ struct rbmoe_layer {
     Buf counts, offsets, tile_expert, tile_row0, tile_rows, ntiles, losses;
     Buf perm_slot, perm_token, inv_pos;
     Buf xg, h, y, hs, ys;
+    // training (allocated by rbmoe_layer_enable_training)
+    bool training = false;
+    bool weights_set = false;
+    Buf xc;                               // copy of the last input [T, d]
+    Buf gu, gus;                          // pre-activations (gate | up): [S, 2F], shared [T, 2Fs]
+    Buf dy, dh, dgu, dxg;                 // [S, d], [S, F], [S, 2F], [S, d]
+    Buf dhs, dgus, dxs;                   // shared: [T, Fs], [T, 2Fs], [T, d]
+    Buf grad_gates, ones, dlogits, dxr, rpartial;
+    Buf g_router, g_gu, g_down, g_sgu, g_sdown;   // f32 weight gradients, accumulated
+    Buf wdT, wguT, swdT, swguT;           // transposed packed weights: [E][F, d], [E][d, 2F], [Fs, d], [d, 2Fs]
+    Buf st_gout, st_gin;
     // staging for the host entry point
     Buf st_x, st_out, st_valid, st_bias, st_res;
     std::vector<Buf*> all;
@@ -559,6 +570,38 @@ int rbmoe_set_weight(rbmoe_layer* L, int32_t which, int32_t expert, const void* 
     HIP_TRY(ctx, hipMemcpy(dst + elem_off * es, src, n * es, hipMemcpyHostToDevice));
     if (target == RBMOE_I8)
         HIP_TRY(ctx, hipMemcpy(sdst + scale_off, scales, (size_t)rows * 4, hipMemcpyHostToDevice));
+    L->weights_set = true;
+    if (L->training && !is_router) {
+        // The backward products multiply by the weight itself, not by its transpose (grad_input =
+        // grad_output . W, src/param.rs:822-823): keep a transposed copy in the packed layout.  Gate and up
+        // share one matrix [d, 2F] (gate^T in columns [0, F), up^T in [F, 2F)) so that dX = dG . Wg + dU . Wu is
+        // one product; packed column steps of 16 never straddle the two halves.
+        std::vector<uint16_t> plain(n), tr(n), trp(n);
+        if (dtype == RBMOE_BF16) {
+            std::memcpy(plain.data(), data, n * 2);
+        } else {
+            const float* f = static_cast<const float*>(data);
+            for (size_t i = 0; i < n; ++i) plain[i] = host_f32_to_bf16(f[i]);
+        }
+        for (int r = 0; r < rows; ++r)
+            for (int cc = 0; cc < cols; ++cc) tr[(size_t)cc * rows + r] = plain[(size_t)r * cols + cc];
+        pack_weight_bf16(tr.data(), cols, rows, trp.data());  // [cols, rows] matrix
+        const bool shared_w = which >= RBMOE_W_SHARED_GATE;
+        const int Fw = shared_w ? Fs : F;
+        if (which == RBMOE_W_DOWN || which == RBMOE_W_SHARED_DOWN) {
+            char* tdst = static_cast<char*>(shared_w ? L->swdT.p : L->wdT.p) + (shared_w ? 0 : (size_t)expert * Fw * d * 2);
+            HIP_TRY(ctx, hipMemcpy(tdst, trp.data(), n * 2, hipMemcpyHostToDevice));
+        } else {
+            // [d, Fw] packed as [d/32][Fw/16][512]; destination [d/32][2Fw/16][512]
+            const bool is_up = which == RBMOE_W_UP || which == RBMOE_W_SHARED_UP;
+            char* base = static_cast<char*>(shared_w ? L->swguT.p : L->wguT.p) +
+                         (shared_w ? 0 : (size_t)expert * d * 2 * Fw * 2);
+            const size_t half = (size_t)(Fw / 16) * 512;  // elements per row block and half
+            for (int rb = 0; rb < d / 32; ++rb)
+                HIP_TRY(ctx, hipMemcpy(base + ((size_t)rb * 2 * half + (is_up ? half : 0)) * 2,
+                                       trp.data() + (size_t)rb * half, half * 2, hipMemcpyHostToDevice));
+        }
+    }
     return RBMOE_OK;
 }
 
@@ -605,7 +648,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     const bool gather_in_product = (mfma || f32mc) && !L->explicit_gather;
 
     // ---- a few tokens: route in one workgroup, then stream the touched weights once -------
-    if (mfma && L->decode_path && small_route_ok(T, E, k) && decode_shape_ok(F, d) && decode_shape_ok(d, F) &&
+    if (mfma && L->decode_path && !L->training && small_route_ok(T, E, k) && decode_shape_ok(F, d) && decode_shape_ok(d, F) &&
         (!c.shared_expert || (decode_shape_ok(Fs, d) && decode_shape_ok(d, Fs)))) {
         L->kernel_name = wk == WeightKind::I8 ? "mfma_bf16_decode_int8w" : "mfma_bf16_decode";
         SmallRouteArgs sr{};
@@ -665,6 +708,9 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
         return RBMOE_OK;
     }
 
+    if (L->training && T > 0)  // MoeCache keeps the input (src/moe.rs:133-135)
+        HIP_TRY(ctx, hipMemcpyAsync(L->xc.p, x, (size_t)T * d * dtype_size(c.act_dtype), hipMemcpyDeviceToDevice, s));
+
     RouterArgs ra{x, (const float*)L->router.p, router_bias, valid, T, d, E, k,
                   (float*)L->P.p, (float*)L->lse.p, (int*)L->expert_of.p, (float*)L->gate_of.p,
                   (int*)L->rank_in_block.p, (int*)L->blockcnt.p, (float*)L->partial.p};
@@ -714,11 +760,13 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     g1.out = L->h.p;
     g1.swiglu = true;
     g1.group_m = L->group_m;
+    if (L->training) g1.gu_out = L->gu.p;
     HIP_TRY(ctx, run(g1, true));
     HIP_TRY(ctx, mark(4));
 
     GroupedArgs g2 = g1;
     g2.a = L->h.p;
+    g2.gu_out = nullptr;
     g2.row_index = nullptr;
     g2.w = L->wd.p;
     g2.w_expert_stride = (size_t)d * F;
@@ -743,11 +791,13 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
         s1.K = d;
         s1.dense_rows = T;
         s1.out = L->hs.p;
+        if (L->training) s1.gu_out = L->gus.p;
         HIP_TRY(ctx, run(s1, true));
         GroupedArgs s2 = s1;
         s2.a = L->hs.p;
         s2.w = L->swd.p;
         s2.scales = wk == WeightKind::I8 ? (const float*)L->ssd.p : nullptr;
+        s2.gu_out = nullptr;
         s2.N = d;
         s2.K = Fs;
         s2.out = L->ys.p;
@@ -815,6 +865,223 @@ int rbmoe_forward_host(rbmoe_layer* L, const void* x, int32_t T, int32_t cols, c
     if (rc != RBMOE_OK) return rc;
     if (T > 0) HIP_TRY(ctx, hipMemcpyAsync(out, L->st_out.p, nbytes, hipMemcpyDeviceToHost, s));
     HIP_TRY(ctx, hipStreamSynchronize(s));
+    return RBMOE_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Training: MoeLayer::backward (reference src/moe.rs:348-489).
+// ---------------------------------------------------------------------------
+int rbmoe_layer_enable_training(rbmoe_layer* L) {
+    if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
+    rbmoe_ctx* ctx = L->ctx;
+    if (L->training) return RBMOE_OK;
+    const rbmoe_config& c = L->cfg;
+    if (!L->use_stream || c.weight_dtype != RBMOE_BF16)
+        return fail(ctx, RBMOE_UNSUPPORTED,
+                    "the backward pass needs bf16 activations and weights with widths that are multiples of 64");
+    if (L->weights_set)
+        return fail(ctx, RBMOE_INVALID_CONFIG, "enable training before the weights are set");
+    const size_t E = c.num_experts, d = c.d_model, F = c.d_ff, Fs = L->Fs, T = L->max_T, S = L->max_S;
+    if (!stream_shape_ok((int)d, (int)(2 * F)) || (c.shared_expert && !stream_shape_ok((int)d, (int)(2 * Fs))))
+        return fail(ctx, RBMOE_UNSUPPORTED, "expert width not supported by the backward products");
+    // 32-bit byte offsets into the widest operand of the backward products: [S, 2F] bf16
+    if (std::max(S * 2 * F, T * 2 * Fs) * 2 >= ((size_t)1 << 32))
+        return fail(ctx, RBMOE_UNSUPPORTED, "max_tokens x expert width too large for the backward products");
+    const size_t as = dtype_size(c.act_dtype);
+    Plan p;
+    p.add(&L->xc, T * d * as);
+    p.add(&L->gu, S * 2 * F * as);
+    p.add(&L->dy, S * d * as);
+    p.add(&L->dh, S * F * as);
+    p.add(&L->dgu, S * 2 * F * as);
+    p.add(&L->dxg, S * d * as);
+    p.add(&L->grad_gates, S * 4);
+    p.add(&L->ones, S * 4);
+    p.add(&L->dlogits, T * E * 4);
+    p.add(&L->dxr, T * d * as);
+    p.add(&L->rpartial, (size_t)router_grad_chunks((int)T) * E * d * 4);
+    p.add(&L->g_router, E * d * 4);
+    p.add(&L->g_gu, E * 2 * F * d * 4);
+    p.add(&L->g_down, E * d * F * 4);
+    p.add(&L->wdT, E * F * d * 2);
+    p.add(&L->wguT, E * d * 2 * F * 2);
+    p.add(&L->st_gout, T * d * as);
+    p.add(&L->st_gin, T * d * as);
+    if (c.shared_expert) {
+        p.add(&L->gus, T * 2 * Fs * as);
+        p.add(&L->dhs, T * Fs * as);
+        p.add(&L->dgus, T * 2 * Fs * as);
+        p.add(&L->dxs, T * d * as);
+        p.add(&L->g_sgu, 2 * Fs * d * 4);
+        p.add(&L->g_sdown, d * Fs * 4);
+        p.add(&L->swdT, Fs * d * 2);
+        p.add(&L->swguT, d * 2 * Fs * 2);
+    }
+    if (ctx->budget_bytes && ctx->allocated + p.total > ctx->budget_bytes) {
+        char buf[200];
+        std::snprintf(buf, sizeof buf, "memory budget exceeded: estimated %zu MiB exceeds budget %zu MiB",
+                      (ctx->allocated + p.total + (1 << 20) - 1) >> 20, ctx->budget_bytes >> 20);
+        return fail(ctx, RBMOE_MEMORY_BUDGET, buf);
+    }
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    for (auto& it : p.items) {
+        void* q = nullptr;
+        hipError_t e = hipMalloc(&q, it.second);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(ctx, RBMOE_OUT_OF_MEMORY, "out of memory while allocating the training buffers");
+        }
+        it.first->p = q;
+        it.first->bytes = it.second;
+        ctx->allocated += it.second;
+        L->all.push_back(it.first);
+        HIP_TRY(ctx, hipMemsetAsync(q, 0, it.second, ctx->stream));
+    }
+    HIP_TRY(ctx, launch_fill_f32((float*)L->ones.p, 1.0f, (long long)S, ctx->stream));
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    L->training = true;
+    return RBMOE_OK;
+}
+
+int rbmoe_zero_grads(rbmoe_layer* L) {
+    if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
+    rbmoe_ctx* ctx = L->ctx;
+    if (!L->training) return fail(ctx, RBMOE_INVALID_CONFIG, "training is not enabled on this layer");
+    for (Buf* b : {&L->g_router, &L->g_gu, &L->g_down, &L->g_sgu, &L->g_sdown})
+        if (b->p) HIP_TRY(ctx, hipMemsetAsync(b->p, 0, b->bytes, ctx->stream));
+    return RBMOE_OK;
+}
+
+int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
+    if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
+    rbmoe_ctx* ctx = L->ctx;
+    if (!L->training) return fail(ctx, RBMOE_INVALID_CONFIG, "training is not enabled on this layer");
+    if (L->last_T < 0) return fail(ctx, RBMOE_INVALID_INPUT, "no forward pass has run yet");
+    const rbmoe_config& c = L->cfg;
+    const int E = c.num_experts, d = c.d_model, F = c.d_ff, k = c.experts_per_token, Fs = L->Fs, T = L->last_T;
+    if (T == 0) return RBMOE_OK;
+    if (!grad_output || !grad_input) return fail(ctx, RBMOE_NULL_POINTER, "grad_output or grad_input is NULL");
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    hipStream_t s = ctx->stream;
+    const bool abf = c.act_dtype == RBMOE_BF16;
+    const int S = T * k;
+    const int* offsets = (const int*)L->offsets.p;
+    const int* counts = (const int*)L->counts.p;
+
+    // upstream of every expert: gate * dOut[token]; gate gradient: dOut[token] . Y[row]
+    HIP_TRY(ctx, hipMemsetAsync(L->grad_gates.p, 0, (size_t)S * 4, s));
+    HIP_TRY(ctx, launch_scale_rows(grad_output, L->y.p, (const int*)L->perm_slot.p, (const int*)L->perm_token.p,
+                                   (const float*)L->gate_of.p, offsets, E, d, S, L->dy.p, (float*)L->grad_gates.p, abf,
+                                   s));
+    // SwiGlu::backward over the routed rows (src/ffn.rs:87-120)
+    GroupedArgs g{};
+    g.tile_expert = (const int*)L->tile_expert.p;
+    g.tile_row0 = (const int*)L->tile_row0.p;
+    g.tile_rows = (const int*)L->tile_rows.p;
+    g.ntiles = (const int*)L->ntiles.p;
+    g.max_tiles = S / stream_tile_m() + E;
+    g.dense_rows = -1;
+    g.swiglu = false;
+    g.group_m = L->group_m;
+    GroupedArgs gh = g;  // grad_hidden = dY . Wdown
+    gh.a = L->dy.p; gh.w = L->wdT.p; gh.w_expert_stride = (size_t)F * d; gh.N = F; gh.K = d; gh.out = L->dh.p;
+    HIP_TRY(ctx, launch_grouped_stream(gh, WeightKind::BF16, L->variant, s));
+    HIP_TRY(ctx, launch_swiglu_grad(L->dh.p, L->gu.p, offsets, E, S, F, L->dgu.p, abf, s));
+    GroupedArgs gx = g;  // grad_input rows = dG . Wgate + dU . Wup
+    gx.a = L->dgu.p; gx.w = L->wguT.p; gx.w_expert_stride = (size_t)d * 2 * F; gx.N = d; gx.K = 2 * F; gx.out = L->dxg.p;
+    HIP_TRY(ctx, launch_grouped_stream(gx, WeightKind::BF16, L->variant, s));
+    // weight gradients (src/param.rs:819-821): down += dY^T . H; (gate | up) += (dG | dU)^T . X[token]
+    HIP_TRY(ctx, launch_grouped_tn(L->dy.p, d, L->h.p, nullptr, F, counts, offsets, E, -1, (float*)L->g_down.p,
+                                   (size_t)d * F, abf, s));
+    HIP_TRY(ctx, launch_grouped_tn(L->dgu.p, 2 * F, L->xc.p, (const int*)L->perm_token.p, d, counts, offsets, E, -1,
+                                   (float*)L->g_gu.p, (size_t)2 * F * d, abf, s));
+    // shared expert over every row (src/moe.rs:356-361)
+    if (c.shared_expert) {
+        GroupedArgs sh = g;
+        sh.dense_rows = T;
+        sh.a = grad_output; sh.w = L->swdT.p; sh.w_expert_stride = 0; sh.N = Fs; sh.K = d; sh.out = L->dhs.p;
+        HIP_TRY(ctx, launch_grouped_stream(sh, WeightKind::BF16, L->variant, s));
+        HIP_TRY(ctx, launch_swiglu_grad(L->dhs.p, L->gus.p, nullptr, 0, T, Fs, L->dgus.p, abf, s));
+        GroupedArgs sx = sh;
+        sx.a = L->dgus.p; sx.w = L->swguT.p; sx.N = d; sx.K = 2 * Fs; sx.out = L->dxs.p;
+        HIP_TRY(ctx, launch_grouped_stream(sx, WeightKind::BF16, L->variant, s));
+        HIP_TRY(ctx, launch_grouped_tn(grad_output, d, L->hs.p, nullptr, Fs, nullptr, nullptr, 1, T,
+                                       (float*)L->g_sdown.p, 0, abf, s));
+        HIP_TRY(ctx, launch_grouped_tn(L->dgus.p, 2 * Fs, L->xc.p, nullptr, d, nullptr, nullptr, 1, T,
+                                       (float*)L->g_sgu.p, 0, abf, s));
+    }
+    // gates -> probabilities -> logits, with the two auxiliary losses (src/moe.rs:421-478), then the router
+    HIP_TRY(ctx, launch_route_backward((const float*)L->P.p, (const float*)L->lse.p, (const int*)L->expert_of.p,
+                                       (const float*)L->grad_gates.p, counts, offsets, T, E, k, c.aux_loss_weight,
+                                       c.router_z_loss_weight, (float*)L->dlogits.p, s));
+    HIP_TRY(ctx, launch_router_grad((const float*)L->dlogits.p, L->xc.p, (const float*)L->router.p, T, d, E,
+                                    (float*)L->rpartial.p, (float*)L->g_router.p, L->dxr.p, abf, s));
+    // grad_input = sum over a token's slots of its expert rows + shared + router
+    CombineArgs ca{L->dxg.p, c.shared_expert ? L->dxs.p : nullptr, L->dxr.p, (const int*)L->inv_pos.p,
+                   (const float*)L->ones.p, T, d, k, grad_input};
+    HIP_TRY(ctx, launch_combine(ca, abf, s));
+    return RBMOE_OK;
+}
+
+int rbmoe_backward_host(rbmoe_layer* L, const void* grad_output, void* grad_input) {
+    if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
+    rbmoe_ctx* ctx = L->ctx;
+    if (!L->training) return fail(ctx, RBMOE_INVALID_CONFIG, "training is not enabled on this layer");
+    if (L->last_T < 0) return fail(ctx, RBMOE_INVALID_INPUT, "no forward pass has run yet");
+    const int T = L->last_T;
+    if (T == 0) return RBMOE_OK;
+    if (!grad_output || !grad_input) return fail(ctx, RBMOE_NULL_POINTER, "grad_output or grad_input is NULL");
+    const size_t nbytes = (size_t)T * L->cfg.d_model * dtype_size(L->cfg.act_dtype);
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    HIP_TRY(ctx, hipMemcpyAsync(L->st_gout.p, grad_output, nbytes, hipMemcpyHostToDevice, ctx->stream));
+    int rc = rbmoe_backward(L, L->st_gout.p, L->st_gin.p);
+    if (rc != RBMOE_OK) return rc;
+    HIP_TRY(ctx, hipMemcpyAsync(grad_input, L->st_gin.p, nbytes, hipMemcpyDeviceToHost, ctx->stream));
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return RBMOE_OK;
+}
+
+int rbmoe_get_weight_grad(rbmoe_layer* L, int32_t which, int32_t expert, float* host, int32_t rows, int32_t cols) {
+    if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
+    rbmoe_ctx* ctx = L->ctx;
+    if (!L->training) return fail(ctx, RBMOE_INVALID_CONFIG, "training is not enabled on this layer");
+    if (!host) return fail(ctx, RBMOE_NULL_POINTER, "host buffer is NULL");
+    const rbmoe_config& c = L->cfg;
+    const size_t E = c.num_experts, d = c.d_model, F = c.d_ff, Fs = L->Fs;
+    const float* src = nullptr;
+    size_t want_rows = 0, want_cols = 0;
+    const bool bad_expert = expert < 0 || (size_t)expert >= E;
+    switch (which) {
+        case RBMOE_W_ROUTER: src = (const float*)L->g_router.p; want_rows = E; want_cols = d; break;
+        case RBMOE_W_GATE:
+        case RBMOE_W_UP:
+            if (bad_expert) return fail(ctx, RBMOE_INVALID_CONFIG, "expert index out of range");
+            src = (const float*)L->g_gu.p + ((size_t)expert * 2 + (which == RBMOE_W_UP ? 1 : 0)) * F * d;
+            want_rows = F; want_cols = d;
+            break;
+        case RBMOE_W_DOWN:
+            if (bad_expert) return fail(ctx, RBMOE_INVALID_CONFIG, "expert index out of range");
+            src = (const float*)L->g_down.p + (size_t)expert * d * F;
+            want_rows = d; want_cols = F;
+            break;
+        case RBMOE_W_SHARED_GATE:
+        case RBMOE_W_SHARED_UP:
+            if (!c.shared_expert) return fail(ctx, RBMOE_INVALID_CONFIG, "the layer has no shared expert");
+            src = (const float*)L->g_sgu.p + (size_t)(which == RBMOE_W_SHARED_UP ? 1 : 0) * Fs * d;
+            want_rows = Fs; want_cols = d;
+            break;
+        case RBMOE_W_SHARED_DOWN:
+            if (!c.shared_expert) return fail(ctx, RBMOE_INVALID_CONFIG, "the layer has no shared expert");
+            src = (const float*)L->g_sdown.p;
+            want_rows = d; want_cols = Fs;
+            break;
+        default:
+            return fail(ctx, RBMOE_INVALID_CONFIG, "unknown weight id");
+    }
+    if ((size_t)rows != want_rows || (size_t)cols != want_cols)
+        return fail(ctx, RBMOE_INVALID_INPUT, "gradient shape does not match the weight");
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    HIP_TRY(ctx, hipMemcpy(host, src, want_rows * want_cols * 4, hipMemcpyDeviceToHost));
     return RBMOE_OK;
 }
 

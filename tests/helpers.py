@@ -59,13 +59,15 @@ def f64_layer_forward(t: synth.Tensors, valid: Optional[np.ndarray] = None,
 
 
 def gpu_layer(device, t: synth.Tensors, max_tokens: Optional[int] = None, aux_w: float = 0.01,
-              z_w: float = 1e-3):
+              z_w: float = 1e-3, training: bool = False):
     import rustingbrain_amd as rb
     w = t.workload
     cfg = rb.MoeConfig(w.num_experts, w.experts_per_token, w.d_ff, w.shared_expert, aux_w, z_w)
     layer = rb.MoeLayer(w.d_model, cfg, device, act_dtype=w.act_dtype, weight_dtype=w.weight_dtype,
                         max_tokens=max_tokens or max(t.x.shape[0], 1),
                         shared_d_ff=w.shared_d_ff if w.shared_expert else 0)
+    if training:
+        layer.enable_training()
     layer.load_tensors(t)
     return layer
 

@@ -1,0 +1,187 @@
+"""GPU parity of the backward pass (MoeLayer::backward, src/moe.rs:348-489) through the C ABI against the CPU
+oracle's backward on the same seeded inputs.  The routing of the forward is bit-identical, so both sides
+differentiate the same selection; every gradient must agree within rel-L2 2e-2 (bf16 activations and weights; the
+oracle computes in f32 from the same bf16-representable values).
+"""
+import numpy as np
+import pytest
+
+import rustingbrain_amd as rb
+from conftest import rel_l2
+from helpers import assert_routing_identical, gpu_layer, oracle_layer, small_workload
+from rustingbrain_amd import _lib as L
+from rustingbrain_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+TOL = 2e-2
+
+
+def grad_output_for(t, seed):
+    rng = np.random.default_rng(seed)
+    return synth.round_bf16(rng.standard_normal(t.x.shape).astype(np.float32))
+
+
+def check_backward(device, t, valid=None, bias=None, aux_w=0.01, z_w=1e-3, seed=1, tol=TOL):
+    w = t.workload
+    E = w.num_experts
+    gout = grad_output_for(t, seed)
+    ref_layer = oracle_layer(t, aux_w=aux_w, z_w=z_w)
+    ref_fwd = ref_layer.forward(t.x, valid=valid, router_bias=bias)
+    ref = ref_layer.backward(t.x, gout, valid=valid, router_bias=bias)
+    layer = gpu_layer(device, t, aux_w=aux_w, z_w=z_w, training=True)
+    layout = rb.Layout(valid=None if valid is None else [bool(v) for v in valid])
+    out, cache = layer.forward_train(t.x, layout, router_bias=bias)
+    assert_routing_identical(cache, ref_fwd)
+    assert rel_l2(out, ref_fwd.out) <= tol
+    gin = layer.backward(gout)
+
+    def close(name, got, want):
+        if not want.any():
+            assert not got.any(), f"{name}: expected exactly zero"
+            return
+        err = rel_l2(got, want)
+        assert err <= tol, f"{name}: rel-L2 {err} > {tol}"
+
+    close("grad_input", gin, ref.grad_input)
+    close("grad_router", layer.weight_grad(L.W_ROUTER), ref.grad_router)
+    for e in range(E):
+        close(f"grad_gate[{e}]", layer.weight_grad(L.W_GATE, e), ref.grad_gate[e])
+        close(f"grad_up[{e}]", layer.weight_grad(L.W_UP, e), ref.grad_up[e])
+        close(f"grad_down[{e}]", layer.weight_grad(L.W_DOWN, e), ref.grad_down[e])
+    if t.shared is not None:
+        close("grad_shared_gate", layer.weight_grad(L.W_SHARED_GATE), ref.grad_shared[0])
+        close("grad_shared_up", layer.weight_grad(L.W_SHARED_UP), ref.grad_shared[1])
+        close("grad_shared_down", layer.weight_grad(L.W_SHARED_DOWN), ref.grad_shared[2])
+    return layer, ref, gout
+
+
+SHAPES = [
+    dict(d=64, E=4, k=2, F=64, T=50),
+    dict(d=64, E=4, k=1, F=128, T=7),
+    dict(d=128, E=8, k=3, F=192, T=300, shared=True, shared_d_ff=128),
+    dict(d=192, E=16, k=2, F=64, T=1000, shared=True),
+    dict(d=64, E=3, k=3, F=64, T=129),
+]
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "d{d}_E{E}_k{k}_F{F}_T{T}".format(**s))
+def test_backward_matches_the_oracle(device, shape):
+    t = synth.make(small_workload(seed=21, act="bf16", wt="bf16", **shape))
+    layer, _, _ = check_backward(device, t)
+    layer.close()
+
+
+def test_backward_with_padding_rows_and_router_bias(device):
+    # padding rows get no gradient from the routed experts or the router, only from the shared expert
+    # (src/moe.rs:356-361 runs it over every row)
+    t = synth.make(small_workload(d=64, E=6, k=2, F=128, T=90, seed=22, act="bf16", wt="bf16", shared=True))
+    valid = (np.arange(90) % 5 != 2).astype(np.uint8)
+    bias = np.linspace(-0.5, 0.5, 6).astype(np.float32)
+    layer, ref, _ = check_backward(device, t, valid=valid, bias=bias)
+    layer.close()
+
+
+def test_an_expert_without_tokens_gets_exactly_zero_gradients(device):
+    # reference test src/moe.rs:861-890: gradients reach only the experts a token was routed to
+    t = synth.make(small_workload(d=64, E=5, k=2, F=64, T=64, seed=23, act="bf16", wt="bf16"))
+    bias = np.zeros(5, np.float32)
+    bias[3] = -1e4
+    layer, ref, _ = check_backward(device, t, bias=bias)
+    assert not ref.grad_gate[3].any()
+    for which in (L.W_GATE, L.W_UP, L.W_DOWN):
+        assert not layer.weight_grad(which, 3).any()
+    layer.close()
+
+
+def test_large_auxiliary_loss_weights_reach_the_router(device):
+    # reference test src/moe.rs:969-1013: the balance and z losses are differentiated inside backward
+    t = synth.make(small_workload(d=64, E=8, k=2, F=64, T=256, seed=24, act="bf16", wt="bf16"))
+    layer, ref, _ = check_backward(device, t, aux_w=5.0, z_w=2.0)
+    layer.close()
+    # with a zero upstream gradient only the two losses drive the router
+    ref_layer = oracle_layer(t, aux_w=5.0, z_w=2.0)
+    zero = np.zeros_like(t.x)
+    want = ref_layer.backward(t.x, zero)
+    layer = gpu_layer(device, t, aux_w=5.0, z_w=2.0, training=True)
+    layer.forward_train(t.x)
+    gin = layer.backward(zero)
+    assert want.grad_router.any()
+    assert rel_l2(layer.weight_grad(L.W_ROUTER), want.grad_router) <= TOL
+    assert rel_l2(gin, want.grad_input) <= TOL
+    assert not layer.weight_grad(L.W_DOWN, 0).any()
+    layer.close()
+
+
+def test_weight_gradients_accumulate_until_zeroed(device):
+    # Param.grad accumulates across backward calls (src/param.rs:819-821) until zero_grad
+    t = synth.make(small_workload(d=64, E=4, k=2, F=64, T=40, seed=25, act="bf16", wt="bf16", shared=True))
+    layer, ref, gout = check_backward(device, t)
+    once = {w: layer.weight_grad(w, 1 if w in (L.W_GATE, L.W_UP, L.W_DOWN) else 0) for w in range(7)}
+    gin1 = layer.backward(gout)
+    for w, g in once.items():
+        twice = layer.weight_grad(w, 1 if w in (L.W_GATE, L.W_UP, L.W_DOWN) else 0)
+        assert rel_l2(twice, 2.0 * g) <= 1e-6, w
+    layer.zero_grads()
+    for w in range(7):
+        assert not layer.weight_grad(w, 1 if w in (L.W_GATE, L.W_UP, L.W_DOWN) else 0).any()
+    gin2 = layer.backward(gout)
+    assert np.array_equal(gin1, gin2)
+    for w, g in once.items():
+        again = layer.weight_grad(w, 1 if w in (L.W_GATE, L.W_UP, L.W_DOWN) else 0)
+        assert rel_l2(again, g) <= 1e-6, w
+    layer.close()
+
+
+def test_backward_follows_the_most_recent_forward(device):
+    t = synth.make(small_workload(d=64, E=4, k=2, F=64, T=120, seed=26, act="bf16", wt="bf16"))
+    layer = gpu_layer(device, t, training=True)
+    ref_layer = oracle_layer(t)
+    for rows in (120, 33, 1):
+        x = t.x[:rows]
+        gout = grad_output_for(t, rows)[:rows]
+        layer.zero_grads()
+        layer.forward_train(x)
+        gin = layer.backward(gout)
+        want = ref_layer.backward(x, gout)
+        assert rel_l2(gin, want.grad_input) <= TOL
+        assert rel_l2(layer.weight_grad(L.W_ROUTER), want.grad_router) <= TOL
+        for e in range(4):
+            if want.grad_down[e].any():
+                assert rel_l2(layer.weight_grad(L.W_DOWN, e), want.grad_down[e]) <= TOL
+    layer.close()
+
+
+def test_training_mode_errors(device):
+    cfg = rb.MoeConfig(4, 2, 64)
+    t = synth.make(small_workload(d=64, E=4, k=2, F=64, T=8, seed=27, act="bf16", wt="bf16"))
+    late = gpu_layer(device, t)
+    with pytest.raises(rb.InvalidConfig):
+        late.enable_training()         # the transposed copies are made when a weight is set
+    with pytest.raises(rb.InvalidConfig):
+        late.backward(np.zeros((8, 64), np.float32))
+    with pytest.raises(rb.InvalidConfig):
+        late.weight_grad(L.W_ROUTER)
+    late.close()
+    f32 = rb.MoeLayer(64, cfg, device, act_dtype="f32", weight_dtype="f32", max_tokens=8)
+    with pytest.raises(rb.Unsupported):
+        f32.enable_training()
+    f32.close()
+    fresh = rb.MoeLayer(64, cfg, device, act_dtype="bf16", weight_dtype="bf16", max_tokens=8)
+    fresh.enable_training()
+    fresh.enable_training()            # idempotent
+    with pytest.raises(rb.InvalidInput):
+        fresh.backward(np.zeros((8, 64), np.float32))   # no forward yet
+    fresh.load_tensors(t)
+    fresh.forward_train(t.x)
+    with pytest.raises(rb.InvalidInput):
+        fresh.backward(np.zeros((8, 32), np.float32))
+    assert fresh.kernel_name().startswith("mfma_bf16")
+    fresh.close()
+
+
+def test_c3_backward_at_full_size(device):
+    # the configuration the headline metric is quoted on; the oracle's f32 backward takes a few seconds here
+    t = synth.make(synth.WORKLOADS["c3_prefill_d768_e16"])
+    layer, ref, _ = check_backward(device, t)
+    layer.close()
