@@ -148,6 +148,8 @@ struct rbmoe_layer {
     Buf dhs, dgus, dxs;                   // shared: [T, Fs], [T, 2Fs], [T, d]
     Buf grad_gates, ones, dlogits, dxr, rpartial;
     Buf g_router, g_gu, g_down, g_sgu, g_sdown;   // f32 weight gradients, accumulated
+    Buf wg_chunks;                        // chunk table of the weight-gradient products
+    bool wgrad_generic = false, wgrad_split = true;
     Buf wdT, wguT, swdT, swguT;           // transposed packed weights: [E][F, d], [E][d, 2F], [Fs, d], [d, 2Fs]
     Buf st_gout, st_gin;
     // staging for the host entry point
@@ -158,6 +160,11 @@ struct rbmoe_layer {
 };
 
 namespace {
+
+int env_int(const char* name, int fallback) {
+    const char* v = std::getenv(name);
+    return v && v[0] ? std::atoi(v) : fallback;
+}
 
 struct Plan {
     std::vector<std::pair<Buf*, size_t>> items;
@@ -364,10 +371,6 @@ int rbmoe_layer_create(rbmoe_ctx* ctx, const rbmoe_config* cfg, rbmoe_layer** ou
     L->max_S = cfg->max_tokens * cfg->experts_per_token;
     L->max_nb = (cfg->max_tokens + kRouterTokens - 1) / kRouterTokens;
     L->max_tiles = L->max_S / kGenericTileM + cfg->num_experts + 1;
-    auto env_int = [](const char* name, int fallback) {
-        const char* v = std::getenv(name);
-        return v && v[0] ? std::atoi(v) : fallback;
-    };
     L->force_generic = env_int("RBMOE_FORCE_GENERIC", 0) == 1;
     L->explicit_gather = env_int("RBMOE_EXPLICIT_GATHER", 0) == 1;
     L->group_m = std::max(1, env_int("RBMOE_GROUP_M", 4));
@@ -645,7 +648,8 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     const int tile_m0 = mfma ? stream_tile_m() : (f32mc ? f32_tile_m() : kGenericTileM);
     L->kernel_name = mfma ? (wk == WeightKind::I8 ? "mfma_bf16_stream_int8w" : "mfma_bf16_stream")
                           : (f32mc ? "mfma_f32" : "generic");
-    const bool gather_in_product = (mfma || f32mc) && !L->explicit_gather;
+    // a training layer keeps the gathered rows: the weight gradients of gate and up multiply by them
+    const bool gather_in_product = (mfma || f32mc) && !L->explicit_gather && !L->training;
 
     // ---- a few tokens: route in one workgroup, then stream the touched weights once -------
     if (mfma && L->decode_path && !L->training && small_route_ok(T, E, k) && decode_shape_ok(F, d) && decode_shape_ok(d, F) &&
@@ -905,6 +909,7 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
     p.add(&L->g_down, E * d * F * 4);
     p.add(&L->wdT, E * F * d * 2);
     p.add(&L->wguT, E * d * 2 * F * 2);
+    p.add(&L->wg_chunks, (size_t)(4 * std::max(weight_grad_max_chunks((int)E, (int)S), weight_grad_max_chunks(1, (int)T)) + 1) * 4);
     p.add(&L->st_gout, T * d * as);
     p.add(&L->st_gin, T * d * as);
     if (c.shared_expert) {
@@ -939,6 +944,8 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
     }
     HIP_TRY(ctx, launch_fill_f32((float*)L->ones.p, 1.0f, (long long)S, ctx->stream));
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    L->wgrad_generic = env_int("RBMOE_WGRAD_GENERIC", 0) == 1;
+    L->wgrad_split = env_int("RBMOE_DETERMINISTIC", 0) != 1;
     L->training = true;
     return RBMOE_OK;
 }
@@ -991,10 +998,15 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
     gx.a = L->dgu.p; gx.w = L->wguT.p; gx.w_expert_stride = (size_t)d * 2 * F; gx.N = d; gx.K = 2 * F; gx.out = L->dxg.p;
     HIP_TRY(ctx, launch_grouped_stream(gx, WeightKind::BF16, L->variant, s));
     // weight gradients (src/param.rs:819-821): down += dY^T . H; (gate | up) += (dG | dU)^T . X[token]
-    HIP_TRY(ctx, launch_grouped_tn(L->dy.p, d, L->h.p, nullptr, F, counts, offsets, E, -1, (float*)L->g_down.p,
-                                   (size_t)d * F, abf, s));
-    HIP_TRY(ctx, launch_grouped_tn(L->dgu.p, 2 * F, L->xc.p, (const int*)L->perm_token.p, d, counts, offsets, E, -1,
-                                   (float*)L->g_gu.p, (size_t)2 * F * d, abf, s));
+    auto wgrad = [&](const void* a, int M, const void* b, const int* b_rows, int N, int groups, int dense_rows,
+                     int total_rows, float* out, size_t stride) -> hipError_t {
+        if (!L->wgrad_generic && abf && !b_rows && weight_grad_shape_ok(M, N))
+            return launch_weight_grad(a, M, b, N, counts, offsets, groups, dense_rows, total_rows,
+                                      L->wgrad_split, (int*)L->wg_chunks.p, out, stride, s);
+        return launch_grouped_tn(a, M, b, b_rows, N, counts, offsets, groups, dense_rows, out, stride, abf, s);
+    };
+    HIP_TRY(ctx, wgrad(L->dy.p, d, L->h.p, nullptr, F, E, -1, S, (float*)L->g_down.p, (size_t)d * F));
+    HIP_TRY(ctx, wgrad(L->dgu.p, 2 * F, L->xg.p, nullptr, d, E, -1, S, (float*)L->g_gu.p, (size_t)2 * F * d));
     // shared expert over every row (src/moe.rs:356-361)
     if (c.shared_expert) {
         GroupedArgs sh = g;
@@ -1005,10 +1017,8 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
         GroupedArgs sx = sh;
         sx.a = L->dgus.p; sx.w = L->swguT.p; sx.N = d; sx.K = 2 * Fs; sx.out = L->dxs.p;
         HIP_TRY(ctx, launch_grouped_stream(sx, WeightKind::BF16, L->variant, s));
-        HIP_TRY(ctx, launch_grouped_tn(grad_output, d, L->hs.p, nullptr, Fs, nullptr, nullptr, 1, T,
-                                       (float*)L->g_sdown.p, 0, abf, s));
-        HIP_TRY(ctx, launch_grouped_tn(L->dgus.p, 2 * Fs, L->xc.p, nullptr, d, nullptr, nullptr, 1, T,
-                                       (float*)L->g_sgu.p, 0, abf, s));
+        HIP_TRY(ctx, wgrad(grad_output, d, L->hs.p, nullptr, Fs, 1, T, T, (float*)L->g_sdown.p, 0));
+        HIP_TRY(ctx, wgrad(L->dgus.p, 2 * Fs, L->xc.p, nullptr, d, 1, T, T, (float*)L->g_sgu.p, 0));
     }
     // gates -> probabilities -> logits, with the two auxiliary losses (src/moe.rs:421-478), then the router
     HIP_TRY(ctx, launch_route_backward((const float*)L->P.p, (const float*)L->lse.p, (const int*)L->expert_of.p,

@@ -1,0 +1,287 @@
+// Weight gradients of the expert matrices on the bf16 matrix cores of gfx950
+// (Linear::backward, src/param.rs:819-821: weight.grad += grad_output^T . input):
+//
+//   out[e][m][n] += sum over the rows r of expert e of  A[r][m] * B[r][n]
+//
+// Both operands are stored row by row (m and n contiguous), while the matrix cores want, per
+// lane, consecutive elements of the reduction dimension, here the ROW index.  The tiles go to
+// LDS as they are (16-byte pieces, rows padded so that the eight rows a wave reads at once
+// fall in distinct bank groups), and the fragment reads use the transposing LDS read
+// (ds_read_b64_tr_b16): in a group of 16 lanes, lane 4 j + q supplies the address of four
+// consecutive 16-bit elements and lane 4 q + e receives element e of the pieces of lanes
+// q, 4 + q, 8 + q, 12 + q - so pointing lane 4 j + q at (row r0 + j, columns c0 + 4 q ..) hands
+// lane i column c0 + i of rows r0 .. r0 + 3, four consecutive reduction elements.
+//
+// A workgroup of 8 waves (4 x 2) owns 256 (m) x 256 (n) outputs of one CHUNK of one expert's rows;
+// a wave owns 64 x 128 (2 x 4 accumulator blocks of 32 x 32).  Rows go through LDS 32 at a
+// time, double buffered; the global loads run three stages ahead in three register sets, so a
+// load has two full stages of products to arrive in.  An expert with many more rows than the
+// others is cut into several chunks so that the launch stays balanced; chunks of one expert add
+// into the same matrix with hardware f32 atomics (their order is not fixed; an expert with a
+// single chunk adds in place, in one fixed order).
+#include "rbmoe_kernels.h"
+
+namespace rbmoe {
+
+namespace {
+
+constexpr int GM = 256;            // outputs along m per workgroup
+constexpr int GN = 256;            // outputs along n per workgroup
+constexpr int GR = 32;             // rows per LDS stage
+constexpr int GT = 512;            // threads per workgroup
+constexpr int GAS = GM * 2 + 64;   // LDS row pitch of the A tile in bytes: 64 mod 256
+constexpr int GBS = GN * 2 + 64;   // same for the B tile
+constexpr int GSTAGE = GR * (GAS + GBS);
+constexpr int GDEPTH = 3;          // register sets of loads in flight
+
+typedef short v4i16 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) v4i16 lds_v4i16;
+
+__device__ __forceinline__ bf16x8 tr_fragment(const char* p, int pitch) {
+    union {
+        v4i16 h[2];
+        bf16x8 v;
+    } u;
+    u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16*)(p));
+    u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16*)(p + 4 * pitch));
+    return u.v;
+}
+
+// chunk table: expert e with c rows gets ceil(c / limit) chunks of equal size (a multiple of 32)
+__global__ __launch_bounds__(256) void chunk_table_kernel(const int* __restrict__ counts,
+                                                          const int* __restrict__ offsets, int groups,
+                                                          int dense_rows, int limit, int max_chunks,
+                                                          int* __restrict__ chunk_expert, int* __restrict__ chunk_row0,
+                                                          int* __restrict__ chunk_rows, int* __restrict__ chunk_split,
+                                                          int* __restrict__ nchunks) {
+    __shared__ int scan[256];
+    __shared__ int base;
+    const int tid = threadIdx.x;
+    if (tid == 0) base = 0;
+    __syncthreads();
+    for (int e0 = 0; e0 < groups; e0 += 256) {
+        const int e = e0 + tid;
+        int rows = 0, row0 = 0;
+        if (e < groups) {
+            rows = dense_rows >= 0 ? dense_rows : counts[e];
+            row0 = dense_rows >= 0 ? 0 : offsets[e];
+        }
+        const int n = rows > 0 ? (rows + limit - 1) / limit : 0;
+        scan[tid] = n;
+        __syncthreads();
+        for (int o = 1; o < 256; o <<= 1) {
+            const int v = tid >= o ? scan[tid - o] : 0;
+            __syncthreads();
+            scan[tid] += v;
+            __syncthreads();
+        }
+        const int first = base + scan[tid] - n;
+        if (n > 0) {
+            const int per = (((rows + n - 1) / n) + 31) & ~31;
+            for (int c = 0; c < n; ++c) {
+                const int r0 = c * per;
+                const int r = min(per, rows - r0);
+                if (first + c < max_chunks && r > 0) {
+                    chunk_expert[first + c] = e;
+                    chunk_row0[first + c] = row0 + r0;
+                    chunk_rows[first + c] = r;
+                    chunk_split[first + c] = n > 1;
+                } else if (first + c < max_chunks) {
+                    chunk_expert[first + c] = e;
+                    chunk_row0[first + c] = row0;
+                    chunk_rows[first + c] = 0;
+                    chunk_split[first + c] = 1;
+                }
+            }
+        }
+        __syncthreads();
+        if (tid == 255) base += scan[255];
+        __syncthreads();
+    }
+    if (tid == 0) *nchunks = min(base, max_chunks);
+}
+
+__global__ __launch_bounds__(GT) void weight_grad_kernel(
+    const bf16_t* __restrict__ a, int M, const bf16_t* __restrict__ b, int N, int tiles_m, int tiles_n,
+    const int* __restrict__ chunk_expert, const int* __restrict__ chunk_row0, const int* __restrict__ chunk_rows,
+    const int* __restrict__ chunk_split, const int* __restrict__ nchunks, float* __restrict__ out,
+    size_t out_expert_stride) {
+    extern __shared__ __attribute__((aligned(16))) char lds[];  // 2 * GSTAGE
+
+    // Workgroup i runs on XCD i % 8.  A unit is one chunk's row of tiles (same m, every n): its
+    // workgroups share the A columns, so they go to one XCD and its L2; units go to the XCDs in
+    // turn, which spreads the long chunks of a cut expert (neighbours in the table) evenly.
+    const int idx = (int)(blockIdx.x >> 3);
+    const int unit = (int)(blockIdx.x & 7) + 8 * (idx / tiles_n);
+    const int ch = unit / tiles_m;
+    if (ch >= *nchunks) return;
+    const int tile = (unit - ch * tiles_m) * tiles_n + idx % tiles_n;
+    const int m0 = (tile / tiles_n) * GM, n0 = (tile % tiles_n) * GN;
+    const int rows = chunk_rows[ch];
+    if (rows <= 0) return;
+    const int row0 = chunk_row0[ch];
+    const bool split = chunk_split[ch] != 0;
+    float* const o = out + (size_t)chunk_expert[ch] * out_expert_stride;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    // ---- global -> register -> LDS staging: 16-byte pieces ---------------------
+    // each tile: 32 rows x 32 pieces; a thread moves piece tid % 32 of rows tid / 32 and tid / 32 + 16
+    const int pc = tid & 31, tr = tid >> 5;
+    // columns past the edge: loaded from a valid place, never stored
+    const bf16_t* const a_src = a + (size_t)row0 * M + (m0 + 8 * pc < M ? m0 + 8 * pc : 0);
+    const bf16_t* const b_src = b + (size_t)row0 * N + (n0 + 8 * pc < N ? n0 + 8 * pc : 0);
+    struct Set {
+        uint4 a[2], b[2];
+    } sets[GDEPTH];
+    auto fetch = [&](auto kc, int r0) {
+        constexpr int k = decltype(kc)::value;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int r = min(r0 + tr + 16 * i, rows - 1);  // past the end: a valid row, zeroed when staged
+            sets[k].a[i] = *reinterpret_cast<const uint4*>(a_src + (size_t)r * M);
+            sets[k].b[i] = *reinterpret_cast<const uint4*>(b_src + (size_t)r * N);
+        }
+    };
+    auto stage = [&](auto kc, int buf, int r0) {
+        constexpr int k = decltype(kc)::value;
+        char* const A = lds + buf * GSTAGE;
+        char* const B = A + GR * GAS;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const bool in = r0 + tr + 16 * i < rows;  // rows past the end of the chunk contribute nothing
+            *reinterpret_cast<uint4*>(A + (tr + 16 * i) * GAS + pc * 16) = in ? sets[k].a[i] : make_uint4(0, 0, 0, 0);
+            *reinterpret_cast<uint4*>(B + (tr + 16 * i) * GBS + pc * 16) = in ? sets[k].b[i] : make_uint4(0, 0, 0, 0);
+        }
+    };
+
+    floatx16 acc[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    // lane's share of a fragment read: group of 16 lanes gi covers columns 16 (gi % 2) .. and rows
+    // 8 (gi / 2) ..; inside the group lane s points at row s / 4, columns 4 (s % 4) ..
+    const int gi = lane >> 4, sl = lane & 15;
+    const int frow = 8 * (gi >> 1) + (sl >> 2);
+    const int fcol = 16 * (gi & 1) + 4 * (sl & 3);
+    const int a_lane = frow * GAS + (wm * 64 + fcol) * 2;
+    const int b_lane = frow * GBS + (wn * 128 + fcol) * 2;
+
+    const int nstages = (rows + GR - 1) / GR;
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    fetch(I0{}, 0);
+    fetch(I1{}, GR);
+    fetch(I2{}, 2 * GR);
+    stage(I0{}, 0, 0);
+    __syncthreads();
+    // stage s: its rows are in LDS buffer s % 2; register set s % 3 is free and takes stage s + 3;
+    // set (s + 1) % 3 holds stage s + 1, which goes to the other LDS buffer after the products
+    auto step = [&](auto kc, int s) {
+        constexpr int k = decltype(kc)::value;
+        const int buf = s & 1;
+        fetch(kc, (s + GDEPTH) * GR);
+        const char* const A = lds + buf * GSTAGE;
+        const char* const B = A + GR * GAS;
+#pragma unroll
+        for (int ks = 0; ks < GR / 16; ++ks) {
+            bf16x8 af[2], bf[4];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) af[i] = tr_fragment(A + a_lane + ks * 16 * GAS + i * 64, GAS);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) bf[j] = tr_fragment(B + b_lane + ks * 16 * GBS + j * 64, GBS);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        }
+        stage(std::integral_constant<int, (k + 1) % GDEPTH>{}, buf ^ 1, (s + 1) * GR);
+        __syncthreads();
+    };
+    // The stage count is rounded up to the number of register sets, so that every trip runs the
+    // same straight-line code (a stage past the end holds zeros: staged rows past the chunk are
+    // zeroed, and its loads re-read the last row).
+    for (int s = 0; s < nstages; s += GDEPTH) {
+        step(I0{}, s);
+        step(I1{}, s + 1);
+        step(I2{}, s + 2);
+    }
+
+    // accumulator element v of lane l: m = 8 (v / 4) + 4 (l / 32) + v % 4, n = l % 32 of the block.
+    // The only chunk of an expert owns its elements: it reads the 16 values of a block, adds, and
+    // stores (M is a multiple of 8, so a group of 8 rows is inside or outside as a whole).  The
+    // chunks of a cut expert meet on the same elements and add with no-return f32 atomics.
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int mb = m0 + wm * 64 + i * 32;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + wn * 128 + j * 32 + (lane & 31);
+            if (n >= N) continue;
+            float* const base = o + (size_t)(mb + 4 * (lane >> 5)) * N + n;
+            if (split) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    if (mb + 8 * (v >> 2) < M) unsafeAtomicAdd(base + (size_t)(8 * (v >> 2) + (v & 3)) * N, acc[i][j][v]);
+            } else {
+                float old[16];
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    if (mb + 8 * (v >> 2) < M) old[v] = base[(size_t)(8 * (v >> 2) + (v & 3)) * N];
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    if (mb + 8 * (v >> 2) < M) base[(size_t)(8 * (v >> 2) + (v & 3)) * N] = old[v] + acc[i][j][v];
+            }
+        }
+    }
+}
+
+}  // namespace
+
+bool weight_grad_shape_ok(int M, int N) { return M % 8 == 0 && N % 8 == 0 && M >= 8 && N >= 8; }
+
+// Upper bound of the number of chunks of one launch; `chunks` needs 4 * bound + 1 ints.
+int weight_grad_max_chunks(int groups, int total_rows) { return groups + total_rows / 256 + 1; }
+
+hipError_t launch_weight_grad(const void* a, int M, const void* b, int N, const int* counts, const int* offsets,
+                              int groups, int dense_rows, int total_rows, bool allow_split, int* chunks, float* out,
+                              size_t out_expert_stride, hipStream_t s) {
+    if (groups <= 0 || total_rows <= 0) return hipSuccess;
+    if (!weight_grad_shape_ok(M, N)) return hipErrorInvalidValue;
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(weight_grad_kernel),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 2 * GSTAGE);
+    if (attr != hipSuccess) return attr;
+    const int tiles_m = (M + GM - 1) / GM, tiles_n = (N + GN - 1) / GN;
+    const int tiles = tiles_m * tiles_n;
+    // Enough (chunk, tile) pairs to fill the chip twice, and no chunk longer than twice the average
+    // expert's share: an expert above that is cut into equal pieces (the cut costs atomics, which
+    // are several times slower than the read-add-store of an expert's only chunk).
+    int limit = 1 << 30;
+    if (allow_split) {
+        const int want = std::max(groups, (512 + tiles - 1) / tiles);
+        const int share = (total_rows + want - 1) / want;
+        limit = std::max(256, ((dense_rows >= 0 ? share : 2 * share) + 31) & ~31);
+    }
+    const int max_chunks = weight_grad_max_chunks(groups, total_rows);
+    int* const chunk_expert = chunks;
+    int* const chunk_row0 = chunks + max_chunks;
+    int* const chunk_rows = chunks + 2 * max_chunks;
+    int* const chunk_split = chunks + 3 * max_chunks;
+    int* const nchunks = chunks + 4 * max_chunks;
+    hipLaunchKernelGGL(chunk_table_kernel, dim3(1), dim3(256), 0, s, counts, offsets, groups, dense_rows, limit,
+                       max_chunks, chunk_expert, chunk_row0, chunk_rows, chunk_split, nchunks);
+    const int grid = ((max_chunks * tiles_m + 7) / 8) * 8 * tiles_n;
+    hipLaunchKernelGGL(weight_grad_kernel, dim3(grid), dim3(GT), 2 * GSTAGE, s, static_cast<const bf16_t*>(a), M,
+                       static_cast<const bf16_t*>(b), N, tiles_m, tiles_n, chunk_expert, chunk_row0, chunk_rows,
+                       chunk_split, nchunks, out, out_expert_stride);
+    return hipGetLastError();
+}
+
+}  // namespace rbmoe
