@@ -2,19 +2,19 @@
 // src/ffn.rs:87-120): the small kernels around the matrix products.
 //
 //   scale_rows_kernel      dY[pos] = gate * dOut[token]; dgate[slot] = dOut[token] . Y[pos]
-//   swiglu_grad_kernel     dG = dH * U * silu'(G),  dU = dH * silu(G)
-//   grouped_tn_kernel      dW[e] += A_e^T . B_e   (weight.grad += grad_output^T . input)
+//   grouped_tn_kernel      dW[e] += A_e^T . B_e   (weight.grad += grad_output^T . input), plain f32
+//                          arithmetic: the path for shapes the matrix-core kernel does not take
 //   route_backward_kernel  dgate -> dP (renormalisation, balancing loss) -> dlogits (softmax, z loss)
 //   router_grad_*          dWr += dlogits^T . X (two stages, fixed order), dX_router = dlogits . Wr
 //
 // The row products (dH = dY . Wd, dX = dG . Wg + dU . Wu) run on the forward pass's streaming
-// kernel with transposed packed copies of the weights.  No floating-point atomics anywhere:
-// every sum has one fixed order.
+// kernel with transposed packed copies of the weights (SwiGLU's backward is applied where the
+// first of them stores its rows); the weight gradients have a matrix-core kernel of their own.
+// Every sum in this file has one fixed order.  Rows are moved in 16-byte pieces: the row width
+// must be a multiple of 8 (bf16) or 4 (f32) elements.
 #include "rbmoe_kernels.h"
 
 namespace rbmoe {
-
-__device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + __expf(-x)); }
 
 // ---------------------------------------------------------------------------
 // One wave per routed row (src/moe.rs:374-385 and :404-416).
@@ -26,6 +26,7 @@ __global__ __launch_bounds__(256) void scale_rows_kernel(const XT* __restrict__ 
                                                          const float* __restrict__ gate_of,
                                                          const int* __restrict__ offsets, int E, int d,
                                                          XT* __restrict__ dy, float* __restrict__ grad_gates) {
+    constexpr int VN = Vec16<XT>::N;
     const int lane = threadIdx.x & 63;
     const int pos = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (pos >= offsets[E]) return;
@@ -35,31 +36,20 @@ __global__ __launch_bounds__(256) void scale_rows_kernel(const XT* __restrict__ 
     const XT* yr = y + (size_t)pos * d;
     XT* dr = dy + (size_t)pos * d;
     float dot = 0.0f;
-    for (int c = lane; c < d; c += 64) {
-        const float v = to_f32(go[c]);
-        dr[c] = from_f32<XT>(g * v);
-        dot += v * to_f32(yr[c]);
+    for (int c = lane * VN; c < d; c += 64 * VN) {
+        float v[VN], w[VN], o[VN];
+        Vec16<XT>::load(go + c, v);
+        Vec16<XT>::load(yr + c, w);
+#pragma unroll
+        for (int i = 0; i < VN; ++i) {
+            o[i] = g * v[i];
+            dot = fmaf(v[i], w[i], dot);
+        }
+        Vec16<XT>::store(dr + c, o);
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) dot += __shfl_xor(dot, o);
     if (lane == 0) grad_gates[slot] = dot;
-}
-
-// gu, dgu: [rows, 2F] with the gate half in columns [0, F) and the up half in [F, 2F)
-template <typename XT>
-__global__ __launch_bounds__(256) void swiglu_grad_kernel(const XT* __restrict__ dh, const XT* __restrict__ gu,
-                                                          const int* __restrict__ row_limit, int limit_index,
-                                                          int rows, int F, XT* __restrict__ dgu) {
-    const int nrows = row_limit ? row_limit[limit_index] : rows;
-    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (long long)nrows * F) return;
-    const int r = (int)(idx / F), f = (int)(idx - (long long)r * F);
-    const float g = to_f32(gu[(size_t)r * 2 * F + f]);
-    const float u = to_f32(gu[(size_t)r * 2 * F + F + f]);
-    const float up = to_f32(dh[(size_t)r * F + f]);
-    const float s = sigmoid_f32(g);
-    dgu[(size_t)r * 2 * F + f] = from_f32<XT>(up * u * (s * (1.0f + g * (1.0f - s))));  // silu'(g), src/ffn.rs:235-238
-    dgu[(size_t)r * 2 * F + F + f] = from_f32<XT>(up * (g * s));
 }
 
 // ---------------------------------------------------------------------------
@@ -133,20 +123,25 @@ __global__ __launch_bounds__(256) void grouped_tn_kernel(const XT* __restrict__ 
 }
 
 // ---------------------------------------------------------------------------
-// One token per thread (src/moe.rs:421-478).  V = routed slots / k.
+// Gates -> probabilities -> logits (src/moe.rs:421-478).  V = routed slots / k.  A group of G
+// lanes (16, 32 or 64: the smallest that covers E, or 64) owns one token; lane j owns experts
+// j, j + G, ...: a token's row of probabilities is read and its row of logit gradients written
+// by neighbouring lanes.  The sum over the experts (the softmax's dot product) is a butterfly
+// inside the group, so every lane of the group holds the same value in the same order.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void route_backward_kernel(const float* __restrict__ P, const float* __restrict__ lse,
-                                                             const int* __restrict__ expert_of,
-                                                             const float* __restrict__ grad_gates,
-                                                             const int* __restrict__ counts,
-                                                             const int* __restrict__ offsets, int T, int E, int k,
-                                                             float w_aux, float w_z, float* __restrict__ dlogits) {
-    const int t = blockIdx.x * 256 + threadIdx.x;
+template <int G>
+__global__ __launch_bounds__(256) void route_backward_kernel(
+    const float* __restrict__ P, const float* __restrict__ lse, const int* __restrict__ expert_of,
+    const float* __restrict__ grad_gates, const int* __restrict__ counts, const int* __restrict__ offsets, int T, int E,
+    int k, float w_aux, float w_z, float* __restrict__ dlogits) {
+    const int t = (blockIdx.x * 256 + threadIdx.x) / G;
+    const int j = threadIdx.x % G;
+    // a whole group leaves together: the shuffles below stay inside groups that are all there
     if (t >= T) return;
     float* row = dlogits + (size_t)t * E;
     const int* sel = expert_of + (size_t)t * k;
     if (sel[0] < 0) {  // padding row: nothing flows
-        for (int e = 0; e < E; ++e) row[e] = 0.0f;
+        for (int e = j; e < E; e += G) row[e] = 0.0f;
         return;
     }
     const float* p = P + (size_t)t * E;
@@ -158,77 +153,152 @@ __global__ __launch_bounds__(256) void route_backward_kernel(const float* __rest
     for (int r = 0; r < k; ++r) weighted += grad_gates[(size_t)t * k + r] * p[sel[r]];
     const float aux_scale = (w_aux != 0.0f && V > 0) ? w_aux * (float)E / (float)V : 0.0f;
     const float slots = (float)(V * k);
-    // first pass: dot = sum_e p_e * dP_e, with dP assembled on the fly
-    float dot = 0.0f;
-    for (int e = 0; e < E; ++e) {
+    const float inv_total = total > 0.0f ? 1.0f / total : 0.0f;
+    const float renorm = weighted * inv_total * inv_total;
+    // dP of expert e, assembled on the fly (twice: once for the softmax's dot product, once for
+    // the result - cheaper than a trip through memory)
+    auto grad_p = [&](int e) {
         float gp = 0.0f;
         if (total > 0.0f)
             for (int r = 0; r < k; ++r)
-                if (sel[r] == e) gp += grad_gates[(size_t)t * k + r] / total - weighted / (total * total);
+                if (sel[r] == e) gp += grad_gates[(size_t)t * k + r] * inv_total - renorm;
         if (aux_scale != 0.0f) gp += aux_scale * ((float)counts[e] / slots);
-        row[e] = gp;
-        dot += p[e] * gp;
-    }
+        return gp;
+    };
+    float dot = 0.0f;
+    for (int e = j; e < E; e += G) dot += p[e] * grad_p(e);
+#pragma unroll
+    for (int o = G / 2; o > 0; o >>= 1) dot += __shfl_xor(dot, o);
     const float zf = (w_z != 0.0f) ? 2.0f * w_z * lse[t] / (float)(V > 0 ? V : 1) : 0.0f;
-    for (int e = 0; e < E; ++e) row[e] = p[e] * (row[e] - dot) + zf * p[e];
+    for (int e = j; e < E; e += G) row[e] = p[e] * (grad_p(e) - dot) + zf * p[e];
 }
 
 // ---------------------------------------------------------------------------
-// dWr[e][c] += sum_t dlogits[t][e] * x[t][c]: stage 1 sums chunks of 128 tokens into
-// partial[chunk][e][c] (one thread per column, experts in batches of 8); stage 2 adds the
-// chunks in order.  dxr[t][c] = sum_e dlogits[t][e] * wr[e][c].
+// Router weight gradient dWr[e][c] += sum_t dlogits[t][e] * x[t][c] in two stages with one
+// fixed order of additions.  Stage 1: a block of 128 threads owns 256 columns (a thread: two
+// neighbours, one 4-byte or 8-byte load per token), one chunk of tokens and a batch of 16
+// experts, with the chunk's dlogits in LDS; it writes partial[chunk][e][c].  Stage 2 adds the
+// chunks in order.  At most kRouterGradMaxChunks chunks, of a multiple of 32 tokens each.
 // ---------------------------------------------------------------------------
-constexpr int kRouterGradChunk = 128;
+constexpr int kRouterGradMaxChunks = 256;
+constexpr int kRouterGradExperts = 16;
+
+__host__ __device__ inline int router_grad_chunk_tokens(int T) {
+    const int per = (T + kRouterGradMaxChunks - 1) / kRouterGradMaxChunks;
+    return ((per > 0 ? per : 1) + 31) & ~31;
+}
+
+__device__ __forceinline__ float2 load_pair(const float* p) { return *reinterpret_cast<const float2*>(p); }
+__device__ __forceinline__ float2 load_pair(const bf16_t* p) {
+    const uint32_t w = *reinterpret_cast<const uint32_t*>(p);
+    return make_float2(__uint_as_float(w << 16), __uint_as_float(w & 0xffff0000u));
+}
 
 template <typename XT>
-__global__ __launch_bounds__(256) void router_grad_partial_kernel(const float* __restrict__ dlogits,
+__global__ __launch_bounds__(128) void router_grad_partial_kernel(const float* __restrict__ dlogits,
                                                                   const XT* __restrict__ x, int T, int d, int E,
-                                                                  float* __restrict__ partial) {
-    const int c = blockIdx.x * 256 + threadIdx.x;
+                                                                  int chunk_tokens, float* __restrict__ partial) {
+    extern __shared__ float dl[];  // [chunk_tokens][16]
+    const int c = (blockIdx.x * 128 + threadIdx.x) * 2;
     const int chunk = blockIdx.y;
-    const int t0 = chunk * kRouterGradChunk, t1 = min(T, t0 + kRouterGradChunk);
-    __shared__ float dl[kRouterGradChunk][8];
-    for (int e0 = 0; e0 < E; e0 += 8) {
-        __syncthreads();
-        for (int i = threadIdx.x; i < (t1 - t0) * 8; i += 256) {
-            const int tt = i >> 3, j = i & 7;
-            dl[tt][j] = e0 + j < E ? dlogits[(size_t)(t0 + tt) * E + e0 + j] : 0.0f;
-        }
-        __syncthreads();
-        if (c < d) {
-            float acc[8];
+    const int e0 = blockIdx.z * kRouterGradExperts;
+    const int t0 = chunk * chunk_tokens, t1 = min(T, t0 + chunk_tokens);
+    for (int i = threadIdx.x; i < (t1 - t0) * kRouterGradExperts; i += 128) {
+        const int tt = i / kRouterGradExperts, j = i % kRouterGradExperts;
+        dl[i] = e0 + j < E ? dlogits[(size_t)(t0 + tt) * E + e0 + j] : 0.0f;
+    }
+    __syncthreads();
+    if (c >= d) return;  // d is even
+    float acc0[kRouterGradExperts], acc1[kRouterGradExperts];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
-            for (int t = t0; t < t1; ++t) {
-                const float xv = to_f32(x[(size_t)t * d + c]);
+    for (int j = 0; j < kRouterGradExperts; ++j) acc0[j] = acc1[j] = 0.0f;
+#pragma unroll 4
+    for (int t = t0; t < t1; ++t) {
+        const float2 xp = load_pair(x + (size_t)t * d + c);
+        const float x0 = xp.x, x1 = xp.y;
+        const float4* row = reinterpret_cast<const float4*>(dl + (t - t0) * kRouterGradExperts);
 #pragma unroll
-                for (int j = 0; j < 8; ++j) acc[j] = fmaf(dl[t - t0][j], xv, acc[j]);
-            }
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-                if (e0 + j < E) partial[((size_t)chunk * E + e0 + j) * d + c] = acc[j];
+        for (int q = 0; q < kRouterGradExperts / 4; ++q) {
+            const float4 v = row[q];
+            acc0[4 * q + 0] = fmaf(v.x, x0, acc0[4 * q + 0]); acc1[4 * q + 0] = fmaf(v.x, x1, acc1[4 * q + 0]);
+            acc0[4 * q + 1] = fmaf(v.y, x0, acc0[4 * q + 1]); acc1[4 * q + 1] = fmaf(v.y, x1, acc1[4 * q + 1]);
+            acc0[4 * q + 2] = fmaf(v.z, x0, acc0[4 * q + 2]); acc1[4 * q + 2] = fmaf(v.z, x1, acc1[4 * q + 2]);
+            acc0[4 * q + 3] = fmaf(v.w, x0, acc0[4 * q + 3]); acc1[4 * q + 3] = fmaf(v.w, x1, acc1[4 * q + 3]);
         }
     }
+#pragma unroll
+    for (int j = 0; j < kRouterGradExperts; ++j)
+        if (e0 + j < E)
+            *reinterpret_cast<float2*>(partial + ((size_t)chunk * E + e0 + j) * d + c) = make_float2(acc0[j], acc1[j]);
 }
 
+// 64 outputs per block of 256 threads; thread (q, i) adds every fourth chunk starting at q for
+// output i, then the four sums are added in order.
 __global__ __launch_bounds__(256) void router_grad_reduce_kernel(const float* __restrict__ partial, int chunks, int n,
                                                                  float* __restrict__ grad) {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
+    __shared__ float part[4][64];
+    const int i = blockIdx.x * 64 + (threadIdx.x & 63);
+    const int q = threadIdx.x >> 6;
     float s = 0.0f;
-    for (int ch = 0; ch < chunks; ++ch) s += partial[(size_t)ch * n + i];
-    grad[i] += s;
+    if (i < n) {
+#pragma unroll 8
+        for (int ch = q; ch < chunks; ch += 4) s += partial[(size_t)ch * n + i];
+    }
+    part[q][threadIdx.x & 63] = s;
+    __syncthreads();
+    if (q == 0 && i < n) grad[i] += ((part[0][threadIdx.x] + part[1][threadIdx.x]) + part[2][threadIdx.x]) + part[3][threadIdx.x];
 }
+
+// dxr[t][c] = sum_e dlogits[t][e] * wr[e][c].  A thread owns one 16-byte piece of the output
+// rows of kDxTokens consecutive tokens, so a piece of a router row fetched once serves them all.
+constexpr int kDxTokens = 4;
 
 template <typename XT>
 __global__ __launch_bounds__(256) void router_dx_kernel(const float* __restrict__ dlogits, const float* __restrict__ wr,
                                                         int T, int d, int E, XT* __restrict__ dxr) {
+    constexpr int VN = Vec16<XT>::N;
+    const int pieces = d / VN;
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (long long)T * d) return;
-    const int t = (int)(idx / d), c = (int)(idx - (long long)t * d);
-    float s = 0.0f;
-    for (int e = 0; e < E; ++e) s = fmaf(dlogits[(size_t)t * E + e], wr[(size_t)e * d + c], s);
-    dxr[idx] = from_f32<XT>(s);
+    const int groups = (T + kDxTokens - 1) / kDxTokens;
+    if (idx >= (long long)groups * pieces) return;
+    const int tg = (int)(idx / pieces), c = (int)(idx - (long long)tg * pieces) * VN;
+    const int t0 = tg * kDxTokens;
+    float s[kDxTokens][VN];
+#pragma unroll
+    for (int u = 0; u < kDxTokens; ++u)
+#pragma unroll
+        for (int i = 0; i < VN; ++i) s[u][i] = 0.0f;
+    for (int e0 = 0; e0 < E; e0 += 4) {
+        // a batch of 4 experts: every load is issued before the first product (experts past E and
+        // tokens past T re-read the last one; the former with a zero factor, the latter unstored)
+        float g[kDxTokens][4];
+        float4 w[4][VN / 4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int e = min(e0 + j, E - 1);
+#pragma unroll
+            for (int q = 0; q < VN / 4; ++q) w[j][q] = *reinterpret_cast<const float4*>(wr + (size_t)e * d + c + 4 * q);
+#pragma unroll
+            for (int u = 0; u < kDxTokens; ++u) {
+                const float v = dlogits[(size_t)min(t0 + u, T - 1) * E + e];
+                g[u][j] = e0 + j < E ? v : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int u = 0; u < kDxTokens; ++u)
+#pragma unroll
+                for (int q = 0; q < VN / 4; ++q) {
+                    s[u][4 * q + 0] = fmaf(g[u][j], w[j][q].x, s[u][4 * q + 0]);
+                    s[u][4 * q + 1] = fmaf(g[u][j], w[j][q].y, s[u][4 * q + 1]);
+                    s[u][4 * q + 2] = fmaf(g[u][j], w[j][q].z, s[u][4 * q + 2]);
+                    s[u][4 * q + 3] = fmaf(g[u][j], w[j][q].w, s[u][4 * q + 3]);
+                }
+    }
+#pragma unroll
+    for (int u = 0; u < kDxTokens; ++u)
+        if (t0 + u < T) Vec16<XT>::store(dxr + (size_t)(t0 + u) * d + c, s[u]);
 }
 
 __global__ __launch_bounds__(256) void fill_f32_kernel(float* p, float v, long long n) {
@@ -239,10 +309,13 @@ __global__ __launch_bounds__(256) void fill_f32_kernel(float* p, float v, long l
 // ---------------------------------------------------------------------------
 // launchers
 // ---------------------------------------------------------------------------
+bool backward_width_ok(int d, bool bf16) { return d > 0 && d % (bf16 ? 8 : 4) == 0; }
+
 hipError_t launch_scale_rows(const void* gout, const void* y, const int* perm_slot, const int* perm_token,
                              const float* gate_of, const int* offsets, int E, int d, int max_rows, void* dy,
                              float* grad_gates, bool bf16, hipStream_t s) {
     if (max_rows <= 0) return hipSuccess;
+    if (!backward_width_ok(d, bf16)) return hipErrorInvalidValue;
     const dim3 grid((max_rows + 3) / 4), block(256);
     if (bf16)
         hipLaunchKernelGGL(scale_rows_kernel<bf16_t>, grid, block, 0, s, static_cast<const bf16_t*>(gout),
@@ -252,20 +325,6 @@ hipError_t launch_scale_rows(const void* gout, const void* y, const int* perm_sl
         hipLaunchKernelGGL(scale_rows_kernel<float>, grid, block, 0, s, static_cast<const float*>(gout),
                            static_cast<const float*>(y), perm_slot, perm_token, gate_of, offsets, E, d,
                            static_cast<float*>(dy), grad_gates);
-    return hipGetLastError();
-}
-
-hipError_t launch_swiglu_grad(const void* dh, const void* gu, const int* row_limit, int limit_index, int rows, int F,
-                              void* dgu, bool bf16, hipStream_t s) {
-    if (rows <= 0) return hipSuccess;
-    const long long total = (long long)rows * F;
-    const dim3 grid((unsigned)((total + 255) / 256)), block(256);
-    if (bf16)
-        hipLaunchKernelGGL(swiglu_grad_kernel<bf16_t>, grid, block, 0, s, static_cast<const bf16_t*>(dh),
-                           static_cast<const bf16_t*>(gu), row_limit, limit_index, rows, F, static_cast<bf16_t*>(dgu));
-    else
-        hipLaunchKernelGGL(swiglu_grad_kernel<float>, grid, block, 0, s, static_cast<const float*>(dh),
-                           static_cast<const float*>(gu), row_limit, limit_index, rows, F, static_cast<float*>(dgu));
     return hipGetLastError();
 }
 
@@ -289,31 +348,44 @@ hipError_t launch_route_backward(const float* P, const float* lse, const int* ex
                                  const int* counts, const int* offsets, int T, int E, int k, float w_aux, float w_z,
                                  float* dlogits, hipStream_t s) {
     if (T <= 0) return hipSuccess;
-    hipLaunchKernelGGL(route_backward_kernel, dim3((T + 255) / 256), dim3(256), 0, s, P, lse, expert_of, grad_gates,
-                       counts, offsets, T, E, k, w_aux, w_z, dlogits);
+    const float* const cP = P;
+    auto go = [&](auto gc) {
+        constexpr int G = decltype(gc)::value;
+        const long long threads = (long long)T * G;
+        hipLaunchKernelGGL(route_backward_kernel<G>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, cP, lse,
+                           expert_of, grad_gates, counts, offsets, T, E, k, w_aux, w_z, dlogits);
+    };
+    if (E <= 16) go(std::integral_constant<int, 16>{});
+    else if (E <= 32) go(std::integral_constant<int, 32>{});
+    else go(std::integral_constant<int, 64>{});
     return hipGetLastError();
 }
 
-int router_grad_chunks(int T) { return (T + kRouterGradChunk - 1) / kRouterGradChunk; }
+// chunks of partial sums a layer of up to `max_tokens` rows needs room for
+int router_grad_chunks(int max_tokens) { return std::min(kRouterGradMaxChunks, (std::max(max_tokens, 1) + 31) / 32); }
 
 hipError_t launch_router_grad(const float* dlogits, const void* x, const float* wr, int T, int d, int E,
                               float* partial, float* grad_router, void* dxr, bool bf16, hipStream_t s) {
     if (T <= 0) return hipSuccess;
-    const int chunks = router_grad_chunks(T);
-    const dim3 g1((d + 255) / 256, chunks), block(256);
-    const long long td = (long long)T * d;
+    if (!backward_width_ok(d, bf16)) return hipErrorInvalidValue;
+    const int ct = router_grad_chunk_tokens(T);
+    const int chunks = (T + ct - 1) / ct;
+    const dim3 g1((d / 2 + 127) / 128, chunks, (E + kRouterGradExperts - 1) / kRouterGradExperts), b1(128);
+    const size_t lds = (size_t)ct * kRouterGradExperts * sizeof(float);
+    if (lds > 48 * 1024) return hipErrorInvalidValue;  // 768 tokens a chunk: beyond 196608 tokens a launch
+    const long long pieces = (long long)((T + kDxTokens - 1) / kDxTokens) * (d / (bf16 ? 8 : 4));
     if (bf16) {
-        hipLaunchKernelGGL(router_grad_partial_kernel<bf16_t>, g1, block, 0, s, dlogits,
-                           static_cast<const bf16_t*>(x), T, d, E, partial);
-        hipLaunchKernelGGL(router_dx_kernel<bf16_t>, dim3((unsigned)((td + 255) / 256)), block, 0, s, dlogits, wr, T, d,
-                           E, static_cast<bf16_t*>(dxr));
+        hipLaunchKernelGGL(router_grad_partial_kernel<bf16_t>, g1, b1, lds, s, dlogits,
+                           static_cast<const bf16_t*>(x), T, d, E, ct, partial);
+        hipLaunchKernelGGL(router_dx_kernel<bf16_t>, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, s, dlogits,
+                           wr, T, d, E, static_cast<bf16_t*>(dxr));
     } else {
-        hipLaunchKernelGGL(router_grad_partial_kernel<float>, g1, block, 0, s, dlogits, static_cast<const float*>(x),
-                           T, d, E, partial);
-        hipLaunchKernelGGL(router_dx_kernel<float>, dim3((unsigned)((td + 255) / 256)), block, 0, s, dlogits, wr, T, d,
-                           E, static_cast<float*>(dxr));
+        hipLaunchKernelGGL(router_grad_partial_kernel<float>, g1, b1, lds, s, dlogits, static_cast<const float*>(x),
+                           T, d, E, ct, partial);
+        hipLaunchKernelGGL(router_dx_kernel<float>, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, s, dlogits,
+                           wr, T, d, E, static_cast<float*>(dxr));
     }
-    hipLaunchKernelGGL(router_grad_reduce_kernel, dim3((E * d + 255) / 256), block, 0, s, partial, chunks, E * d,
+    hipLaunchKernelGGL(router_grad_reduce_kernel, dim3((E * d + 63) / 64), dim3(256), 0, s, partial, chunks, E * d,
                        grad_router);
     return hipGetLastError();
 }

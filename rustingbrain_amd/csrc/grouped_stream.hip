@@ -124,6 +124,7 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
     size_t w_expert_stride_bytes, const float* __restrict__ scales, size_t s_expert_stride, int N, int K,
     const int* __restrict__ tile_expert, const int* __restrict__ tile_row0, const int* __restrict__ tile_rows,
     const int* __restrict__ ntiles, int dense_rows, bf16_t* __restrict__ out, bf16_t* __restrict__ gu_out,
+    const bf16_t* __restrict__ bw_gu,
     int group_m) {
     constexpr int BN = SWIGLU ? NW * 32 : NW * 64;  // output features per workgroup
     // Two LDS stages of one activation slice each; the epilogue reuses both as one
@@ -418,6 +419,39 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
             const int r = idx >> 4, p = idx & 15;
             if (r < rows && col0 + 8 * p < N) {
                 const uint4 v = *reinterpret_cast<const uint4*>(stage + r * 256 + ((p ^ (r & 15)) * 16));
+                if constexpr (!SWIGLU) {
+                    if (bw_gu != nullptr) {  // uniform over the launch
+                        // SwiGlu::backward (src/ffn.rs:87-120) on the way out: the product rows are the
+                        // gradient of the hidden rows; with the gate and up pre-activations G | U of
+                        // the forward pass, dG = dH * U * silu'(G) and dU = dH * silu(G) go to `gu_out`
+                        // (both [rows, 2 N]) and the hidden gradient itself is never stored.
+                        const size_t off = (size_t)(row0 + r) * 2 * N + col0 + 8 * p;
+                        const uint4 g8 = *reinterpret_cast<const uint4*>(bw_gu + off);
+                        const uint4 u8 = *reinterpret_cast<const uint4*>(bw_gu + off + N);
+                        const uint32_t hw[4] = {v.x, v.y, v.z, v.w}, gw[4] = {g8.x, g8.y, g8.z, g8.w},
+                                       uw[4] = {u8.x, u8.y, u8.z, u8.w};
+                        uint32_t dg[4], du[4];
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            float dgv[2], duv[2];
+#pragma unroll
+                            for (int h = 0; h < 2; ++h) {
+                                const float dh = __uint_as_float(h ? hw[q] & 0xffff0000u : hw[q] << 16);
+                                const float gv = __uint_as_float(h ? gw[q] & 0xffff0000u : gw[q] << 16);
+                                const float uv = __uint_as_float(h ? uw[q] & 0xffff0000u : uw[q] << 16);
+                                const float sg = __builtin_amdgcn_rcpf(
+                                    1.0f + __builtin_amdgcn_exp2f(gv * -1.44269504088896340736f));
+                                dgv[h] = dh * uv * (sg * (1.0f + gv * (1.0f - sg)));  // silu', src/ffn.rs:235-238
+                                duv[h] = dh * (gv * sg);
+                            }
+                            dg[q] = pack2(dgv[0], dgv[1]);
+                            du[q] = pack2(duv[0], duv[1]);
+                        }
+                        *reinterpret_cast<uint4*>(gu_out + off) = make_uint4(dg[0], dg[1], dg[2], dg[3]);
+                        *reinterpret_cast<uint4*>(gu_out + off + N) = make_uint4(du[0], du[1], du[2], du[3]);
+                        continue;
+                    }
+                }
                 *reinterpret_cast<uint4*>(dst + (size_t)(row0 + r) * dstride + col0 + 8 * p) = v;
             }
         }
@@ -435,7 +469,8 @@ hipError_t launch_t(const GroupedArgs& g, hipStream_t s) {
     hipLaunchKernelGGL((grouped_stream_kernel<SWIGLU, I8, RING, TFBUF, AREG>), dim3(grid), dim3(NT), 0, s,
                        static_cast<const bf16_t*>(g.a), g.row_index, g.w, g.w_expert_stride * (I8 ? 1 : 2), g.scales,
                        g.s_expert_stride, g.N, g.K, g.tile_expert, g.tile_row0, g.tile_rows, g.ntiles, g.dense_rows,
-                       static_cast<bf16_t*>(g.out), static_cast<bf16_t*>(g.gu_out), g.group_m > 0 ? g.group_m : 4);
+                       static_cast<bf16_t*>(g.out), static_cast<bf16_t*>(g.gu_out), static_cast<const bf16_t*>(g.swiglu_grad_gu),
+                       g.group_m > 0 ? g.group_m : 4);
     return hipGetLastError();
 }
 

@@ -144,8 +144,8 @@ struct rbmoe_layer {
     bool weights_set = false;
     Buf xc;                               // copy of the last input [T, d]
     Buf gu, gus;                          // pre-activations (gate | up): [S, 2F], shared [T, 2Fs]
-    Buf dy, dh, dgu, dxg;                 // [S, d], [S, F], [S, 2F], [S, d]
-    Buf dhs, dgus, dxs;                   // shared: [T, Fs], [T, 2Fs], [T, d]
+    Buf dy, dgu, dxg;                     // [S, d], [S, 2F], [S, d]
+    Buf dgus, dxs;                        // shared: [T, 2Fs], [T, d]
     Buf grad_gates, ones, dlogits, dxr, rpartial;
     Buf g_router, g_gu, g_down, g_sgu, g_sdown;   // f32 weight gradients, accumulated
     Buf wg_chunks;                        // chunk table of the weight-gradient products
@@ -896,7 +896,6 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
     p.add(&L->xc, T * d * as);
     p.add(&L->gu, S * 2 * F * as);
     p.add(&L->dy, S * d * as);
-    p.add(&L->dh, S * F * as);
     p.add(&L->dgu, S * 2 * F * as);
     p.add(&L->dxg, S * d * as);
     p.add(&L->grad_gates, S * 4);
@@ -914,7 +913,6 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
     p.add(&L->st_gin, T * d * as);
     if (c.shared_expert) {
         p.add(&L->gus, T * 2 * Fs * as);
-        p.add(&L->dhs, T * Fs * as);
         p.add(&L->dgus, T * 2 * Fs * as);
         p.add(&L->dxs, T * d * as);
         p.add(&L->g_sgu, 2 * Fs * d * 4);
@@ -976,7 +974,7 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
     const int* counts = (const int*)L->counts.p;
 
     // upstream of every expert: gate * dOut[token]; gate gradient: dOut[token] . Y[row]
-    HIP_TRY(ctx, hipMemsetAsync(L->grad_gates.p, 0, (size_t)S * 4, s));
+    // (grad_gates of unrouted slots stays unwritten: the only reader skips padding rows)
     HIP_TRY(ctx, launch_scale_rows(grad_output, L->y.p, (const int*)L->perm_slot.p, (const int*)L->perm_token.p,
                                    (const float*)L->gate_of.p, offsets, E, d, S, L->dy.p, (float*)L->grad_gates.p, abf,
                                    s));
@@ -991,9 +989,9 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
     g.swiglu = false;
     g.group_m = L->group_m;
     GroupedArgs gh = g;  // grad_hidden = dY . Wdown
-    gh.a = L->dy.p; gh.w = L->wdT.p; gh.w_expert_stride = (size_t)F * d; gh.N = F; gh.K = d; gh.out = L->dh.p;
+    gh.a = L->dy.p; gh.w = L->wdT.p; gh.w_expert_stride = (size_t)F * d; gh.N = F; gh.K = d;
+    gh.swiglu_grad_gu = L->gu.p; gh.gu_out = L->dgu.p;  // the hidden gradient goes straight through SwiGLU's backward
     HIP_TRY(ctx, launch_grouped_stream(gh, WeightKind::BF16, L->variant, s));
-    HIP_TRY(ctx, launch_swiglu_grad(L->dh.p, L->gu.p, offsets, E, S, F, L->dgu.p, abf, s));
     GroupedArgs gx = g;  // grad_input rows = dG . Wgate + dU . Wup
     gx.a = L->dgu.p; gx.w = L->wguT.p; gx.w_expert_stride = (size_t)d * 2 * F; gx.N = d; gx.K = 2 * F; gx.out = L->dxg.p;
     HIP_TRY(ctx, launch_grouped_stream(gx, WeightKind::BF16, L->variant, s));
@@ -1011,10 +1009,11 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
     if (c.shared_expert) {
         GroupedArgs sh = g;
         sh.dense_rows = T;
-        sh.a = grad_output; sh.w = L->swdT.p; sh.w_expert_stride = 0; sh.N = Fs; sh.K = d; sh.out = L->dhs.p;
+        sh.a = grad_output; sh.w = L->swdT.p; sh.w_expert_stride = 0; sh.N = Fs; sh.K = d;
+        sh.swiglu_grad_gu = L->gus.p; sh.gu_out = L->dgus.p;
         HIP_TRY(ctx, launch_grouped_stream(sh, WeightKind::BF16, L->variant, s));
-        HIP_TRY(ctx, launch_swiglu_grad(L->dhs.p, L->gus.p, nullptr, 0, T, Fs, L->dgus.p, abf, s));
-        GroupedArgs sx = sh;
+        GroupedArgs sx = g;
+        sx.dense_rows = T; sx.w_expert_stride = 0;
         sx.a = L->dgus.p; sx.w = L->swguT.p; sx.N = d; sx.K = 2 * Fs; sx.out = L->dxs.p;
         HIP_TRY(ctx, launch_grouped_stream(sx, WeightKind::BF16, L->variant, s));
         HIP_TRY(ctx, wgrad(grad_output, d, L->hs.p, nullptr, Fs, 1, T, T, (float*)L->g_sdown.p, 0));

@@ -102,6 +102,10 @@ struct GroupedArgs {
     int dense_rows;         // >= 0: one group of this many rows, no tile table (shared expert)
     void* out;              // [rows, N] activation dtype
     void* gu_out = nullptr; // streaming gate/up kernel only: [rows, 2N] pre-activations (gate | up) kept for a backward pass
+    // streaming down-shaped kernel only: [rows, 2N] pre-activations of the forward pass.  The product rows are
+    // then taken as the gradient of the hidden rows and SwiGLU's backward is applied on the way out: the
+    // gradients of the pre-activations go to `gu_out` [rows, 2N] and `out` is not written.
+    const void* swiglu_grad_gu = nullptr;
     bool swiglu;
     int group_m;            // MFMA path: M-tiles per scheduling group (0 = default)
 };
@@ -124,11 +128,10 @@ bool f32_shape_ok(int N, int K);
 hipError_t launch_grouped_f32(const GroupedArgs& a, hipStream_t s);
 
 // ---- backward pass: the kernels around the matrix products (backward_kernels.hip) --------
+// dy[pos] = gate * gout[token(pos)], grad_gates[slot] = gout[token] . y[pos]; row widths: multiples of 16 bytes
 hipError_t launch_scale_rows(const void* gout, const void* y, const int* perm_slot, const int* perm_token,
                              const float* gate_of, const int* offsets, int E, int d, int max_rows, void* dy,
                              float* grad_gates, bool bf16, hipStream_t s);
-hipError_t launch_swiglu_grad(const void* dh, const void* gu, const int* row_limit, int limit_index, int rows, int F,
-                              void* dgu, bool bf16, hipStream_t s);
 // out[e][M][N] += A_e^T . B_e over the rows of group e (counts/offsets), or over dense_rows rows when >= 0
 hipError_t launch_grouped_tn(const void* a, int M, const void* b, const int* b_row_index, int N, const int* counts,
                              const int* offsets, int groups, int dense_rows, float* out, size_t out_expert_stride,
@@ -142,10 +145,14 @@ int weight_grad_max_chunks(int groups, int total_rows);
 hipError_t launch_weight_grad(const void* a, int M, const void* b, int N, const int* counts, const int* offsets,
                               int groups, int dense_rows, int total_rows, bool allow_split, int* chunks, float* out,
                               size_t out_expert_stride, hipStream_t s);
+
+// gates -> probabilities -> logits, with the gradients of the two auxiliary losses
 hipError_t launch_route_backward(const float* P, const float* lse, const int* expert_of, const float* grad_gates,
                                  const int* counts, const int* offsets, int T, int E, int k, float w_aux, float w_z,
                                  float* dlogits, hipStream_t s);
-int router_grad_chunks(int T);
+// grad_router += dlogits^T . x (through `partial`, router_grad_chunks(max_tokens) * E * d floats) and
+// dxr = dlogits . wr
+int router_grad_chunks(int max_tokens);
 hipError_t launch_router_grad(const float* dlogits, const void* x, const float* wr, int T, int d, int E,
                               float* partial, float* grad_router, void* dxr, bool bf16, hipStream_t s);
 hipError_t launch_fill_f32(float* p, float v, long long n, hipStream_t s);

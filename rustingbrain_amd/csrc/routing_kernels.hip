@@ -846,50 +846,6 @@ __global__ __launch_bounds__(256) void dispatch_kernel(
 // One thread per (token, 16-byte column piece); the token's slots are sorted
 // by position in registers when k <= KMAX, otherwise found by repeated search.
 // ---------------------------------------------------------------------------
-template <typename T>
-struct Vec16;
-template <>
-struct Vec16<float> {
-    static constexpr int N = 4;
-    static __device__ __forceinline__ uint4 load_raw(const float* p) { return *reinterpret_cast<const uint4*>(p); }
-    static __device__ __forceinline__ void widen(const uint4& a, float (&v)[4]) {
-        v[0] = __uint_as_float(a.x); v[1] = __uint_as_float(a.y); v[2] = __uint_as_float(a.z); v[3] = __uint_as_float(a.w);
-    }
-    static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
-        const float4 a = *reinterpret_cast<const float4*>(p);
-        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
-    }
-    static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
-        *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
-    }
-};
-template <>
-struct Vec16<bf16_t> {
-    static constexpr int N = 8;
-    static __device__ __forceinline__ uint4 load_raw(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
-    static __device__ __forceinline__ void widen(const uint4& a, float (&v)[8]) {
-        v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xffff0000u);
-        v[2] = __uint_as_float(a.y << 16); v[3] = __uint_as_float(a.y & 0xffff0000u);
-        v[4] = __uint_as_float(a.z << 16); v[5] = __uint_as_float(a.z & 0xffff0000u);
-        v[6] = __uint_as_float(a.w << 16); v[7] = __uint_as_float(a.w & 0xffff0000u);
-    }
-    static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[8]) {
-        const uint4 a = *reinterpret_cast<const uint4*>(p);
-        v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xffff0000u);
-        v[2] = __uint_as_float(a.y << 16); v[3] = __uint_as_float(a.y & 0xffff0000u);
-        v[4] = __uint_as_float(a.z << 16); v[5] = __uint_as_float(a.z & 0xffff0000u);
-        v[6] = __uint_as_float(a.w << 16); v[7] = __uint_as_float(a.w & 0xffff0000u);
-    }
-    static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[8]) {
-        uint4 o;
-        o.x = f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16);
-        o.y = f32_to_bf16_bits(v[2]) | ((uint32_t)f32_to_bf16_bits(v[3]) << 16);
-        o.z = f32_to_bf16_bits(v[4]) | ((uint32_t)f32_to_bf16_bits(v[5]) << 16);
-        o.w = f32_to_bf16_bits(v[6]) | ((uint32_t)f32_to_bf16_bits(v[7]) << 16);
-        *reinterpret_cast<uint4*>(p) = o;
-    }
-};
-
 template <typename XT, int KMAX>
 __global__ __launch_bounds__(256) void combine_vec_kernel(
     const XT* __restrict__ y, const XT* __restrict__ yshared, const XT* __restrict__ residual,
