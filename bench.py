@@ -1,14 +1,16 @@
 #!/usr/bin/env python3
 """Benchmark of the mixture-of-experts layer forward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--backward]
 
 A step is one forward pass of the layer (router, dispatch, grouped SwiGLU expert
 products, combine, auxiliary losses) over one batch of seeded synthetic tokens
 already resident in HBM.  Prints ONE JSON line: tokens/s for the whole layer, the
 roofline of the dominant kernel (the grouped gate/up product) measured with HIP
 events on the library's stream, per-stage figures, and the CPU restatement of
-the reference's rayon path timed on this machine's host cores.
+the reference's rayon path timed on this machine's host cores.  With --backward
+a second layer in training mode is also timed: forward with the backward pass's
+state kept, the backward pass, and both (a "backward" object in the same line).
 """
 from __future__ import annotations
 
@@ -112,6 +114,72 @@ def cpu_baseline(t: synth.Tensors, budget_s: float = 20.0) -> dict:
             "ms_per_forward": best * 1e3}
 
 
+def cpu_baseline_backward(t: synth.Tensors, grad_output: np.ndarray) -> dict:
+    """The CPU restatement's forward + backward (oracle/, C++, one thread), one call.  With cpu_baseline, the
+    only code of this file that touches oracle/."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from helpers import oracle_layer
+    layer = oracle_layer(t)
+    t0 = time.perf_counter()
+    layer.backward(t.x, grad_output, router_bias=t.router_bias)
+    ms = (time.perf_counter() - t0) * 1e3
+    return {"value": t.x.shape[0] / (ms * 1e-3), "unit": "tokens/s", "cores": 1, "kind": "port",
+            "sample": "whole workload, one forward + backward call of the C++ restatement", "ms": ms}
+
+
+def backward_leg(dev, w, t, x, out, bp, args, alg, with_cpu: bool) -> dict:
+    """Times MoeLayer::backward (reference src/moe.rs:348-489) on a second layer in training mode: K forwards
+    that keep the backward pass's state, K backward passes of the last forward (weight gradients accumulate, as
+    Param.grad does), and K forward + backward pairs."""
+    if w.act_dtype != "bf16" or w.weight_dtype != "bf16":
+        return {"skipped": "the backward pass needs bf16 activations and weights"}
+    T = w.tokens
+    cfg = rb.MoeConfig(w.num_experts, w.experts_per_token, w.d_ff, w.shared_expert)
+    layer = rb.MoeLayer(w.d_model, cfg, dev, act_dtype=w.act_dtype, weight_dtype=w.weight_dtype, max_tokens=T,
+                        shared_d_ff=w.shared_d_ff if w.shared_expert else 0)
+    layer.enable_training()
+    layer.load_tensors(t)
+    rng = np.random.default_rng(w.seed + 1000)
+    gh = synth.round_bf16(rng.standard_normal(t.x.shape).astype(np.float32))
+    g = DeviceBuffer(dev, x.nbytes).upload(synth.f32_to_bf16_bits(gh))
+    gin = DeviceBuffer(dev, x.nbytes)
+
+    def fwd():
+        layer.forward_device(x.ptr, T, out.ptr, bias_ptr=bp)
+
+    def bwd():
+        layer.backward_device(g.ptr, gin.ptr)
+
+    def timed(fn, n):
+        dev.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        dev.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / n
+
+    for _ in range(max(3, args.warmup // 4)):
+        fwd()
+        bwd()
+    n = max(5, args.steps // 4)
+    ms_f = timed(fwd, n)
+    ms_b = timed(bwd, n)
+    ms_fb = timed(lambda: (fwd(), bwd()), n)
+    # products of the backward pass: twice the forward's (grad_input and weight gradients)
+    flops = 2 * alg["gemm_flops"]
+    res = {"ms_forward_training": ms_f, "ms_backward": ms_b, "ms_forward_backward": ms_fb,
+           "tokens_per_s_forward_backward": T / (ms_fb * 1e-3), "steps": n,
+           "backward_product_flops": flops, "backward_tflops": flops / (ms_b * 1e-3) / 1e12,
+           "backward_frac_of_peak": flops / (ms_b * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+           "note": "weight gradients are f32 accumulators: every backward pass reads and writes all of them"}
+    if with_cpu:
+        res["cpu_baseline"] = cpu_baseline_backward(t, gh)
+    layer.close()
+    g.free()
+    gin.free()
+    return res
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -119,6 +187,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="c3_prefill_d768_e16", choices=list(synth.WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--backward", action="store_true",
+                    help="also time the backward pass (bf16 activations and weights only)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (the plain copy that FETCH_SIZE / "
                          "WRITE_SIZE readings are scaled by when this command runs under rocprofv3 --pmc)")
@@ -260,6 +330,8 @@ def main() -> int:
         assert dev._lib.rbmoe_copy_device(dev.handle, C.c_void_p(b.ptr), C.c_void_p(a.ptr), n) == L.OK
         a.free()
         b.free()
+    if args.backward:
+        result["backward"] = backward_leg(dev, w, t, x, out, bp, args, alg, with_cpu=not args.no_cpu)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(t)
     print(json.dumps(result))

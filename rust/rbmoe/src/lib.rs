@@ -235,6 +235,39 @@ impl MoeLayer {
         self.set(sys::RBMOE_W_SHARED_DOWN, 0, down, d, f)
     }
 
+    /// Makes the forward pass keep what `backward` needs and allocates the f32 gradient accumulators (the
+    /// role of `Param.grad`).  Call before the weights are set.  The library runs the backward pass for
+    /// layers with bf16 activations and weights; on this f32-boundary layer it reports `UnsupportedCuda`.
+    pub fn enable_training(&mut self) -> Result<(), NetworkError> {
+        check(unsafe { sys::rbmoe_layer_enable_training(self.layer) }, self.device.raw(), 0, 0)
+    }
+
+    /// `MoeLayer::backward` (src/moe.rs:348-489) for the last `forward_train`: `grad_output` and the
+    /// returned gradient of the input are `[rows, d_model]` in the layer's activation type (raw bytes of
+    /// f32 or bf16 values); weight gradients accumulate until `zero_grads`.
+    pub fn backward_raw(&mut self, grad_output: &[u8]) -> Result<Vec<u8>, NetworkError> {
+        let mut grad_input = vec![0u8; grad_output.len()];
+        check(unsafe {
+            sys::rbmoe_backward_host(self.layer, grad_output.as_ptr() as *const c_void,
+                                     grad_input.as_mut_ptr() as *mut c_void)
+        }, self.device.raw(), 0, 0)?;
+        Ok(grad_input)
+    }
+
+    /// `Param::zero_grad` over every weight of the layer.
+    pub fn zero_grads(&mut self) -> Result<(), NetworkError> {
+        check(unsafe { sys::rbmoe_zero_grads(self.layer) }, self.device.raw(), 0, 0)
+    }
+
+    /// The accumulated gradient of one weight matrix (`which`: `sys::RBMOE_W_*`), `[rows, cols]` as the weight.
+    pub fn weight_grad(&self, which: i32, expert: usize, rows: usize, cols: usize) -> Result<Vec<f32>, NetworkError> {
+        let mut g = vec![0f32; rows * cols];
+        check(unsafe {
+            sys::rbmoe_get_weight_grad(self.layer, which, expert as i32, g.as_mut_ptr(), rows as i32, cols as i32)
+        }, self.device.raw(), 0, 0)?;
+        Ok(g)
+    }
+
     /// `MoeLayer::forward` (src/moe.rs:237-241).
     pub fn forward(&self, input: &[f32], rows: usize, cols: usize) -> Result<Vec<f32>, NetworkError> {
         self.forward_train(input, rows, cols, Layout::default()).map(|(out, _)| out)

@@ -89,6 +89,13 @@ extern "C" {
     pub fn rbmoe_get_losses(layer: *mut rbmoe_layer, aux_loss: *mut f32, z_loss: *mut f32) -> c_int;
     pub fn rbmoe_get_routing(layer: *mut rbmoe_layer, routing: *mut rbmoe_routing) -> c_int;
     pub fn rbmoe_get_expert_rows(layer: *mut rbmoe_layer, hidden: *mut f32, expert_out: *mut f32) -> c_int;
+    // backward pass (MoeLayer::backward, src/moe.rs:348-489)
+    pub fn rbmoe_layer_enable_training(layer: *mut rbmoe_layer) -> c_int;
+    pub fn rbmoe_backward(layer: *mut rbmoe_layer, grad_output: *const c_void, grad_input: *mut c_void) -> c_int;
+    pub fn rbmoe_backward_host(layer: *mut rbmoe_layer, grad_output: *const c_void, grad_input: *mut c_void) -> c_int;
+    pub fn rbmoe_zero_grads(layer: *mut rbmoe_layer) -> c_int;
+    pub fn rbmoe_get_weight_grad(layer: *mut rbmoe_layer, which: i32, expert: i32, host: *mut f32, rows: i32,
+                                 cols: i32) -> c_int;
     pub fn rbmoe_expert_kernel_name(layer: *const rbmoe_layer) -> *const c_char;
     pub fn rbmoe_device_alloc(ctx: *mut rbmoe_ctx, bytes: usize, out: *mut *mut c_void) -> c_int;
     pub fn rbmoe_device_free(ctx: *mut rbmoe_ctx, ptr: *mut c_void) -> c_int;

@@ -5,7 +5,7 @@
 //   Matrix        reference src/matrix.rs:13-18          (row-major f32)
 //   Layout        reference src/batch.rs:224-269
 //   MoeConfig     reference src/moe.rs:25-87
-//   MoeLayer      reference src/moe.rs:203-341            (forward, forward_train)
+//   MoeLayer      reference src/moe.rs:203-341, :348-489   (forward, forward_train, backward)
 //   MoeCache      reference src/moe.rs:131-188
 //   NetworkError  reference src/network.rs:19-83          (the variants this path raises)
 //   TransformerBuilder (the methods that size the sparse layers) reference src/transformer.rs:278-447
@@ -172,7 +172,7 @@ class MoeLayer {
     // MoeLayer::new: validates, then creates the device layer (weights start at zero).
     MoeLayer(size_t d_model, const MoeConfig& cfg, std::shared_ptr<Device> device, size_t max_tokens = 1024,
              int act_dtype = RBMOE_F32, int weight_dtype = RBMOE_F32, size_t shared_d_ff = 0)
-        : config(cfg), d_model_(d_model), device_(std::move(device)), act_(act_dtype) {
+        : config(cfg), d_model_(d_model), device_(std::move(device)), act_(act_dtype), shared_d_ff_(shared_d_ff) {
         cfg.validate();
         const rbmoe_config c = cfg.raw(d_model, act_dtype, weight_dtype, max_tokens, shared_d_ff);
         check(rbmoe_layer_create(device_->raw(), &c, &layer_), device_->raw());
@@ -245,6 +245,48 @@ class MoeLayer {
         return {std::move(out), std::move(cache)};
     }
 
+    // ---- training (MoeLayer::backward, src/moe.rs:348-489).  The reference takes the cache of the forward pass
+    // as an argument; the device layer keeps that state itself, so backward differentiates the last forward.
+    void enable_training() { check(rbmoe_layer_enable_training(layer_), device_->raw()); }
+
+    Matrix backward(const Matrix& grad_output) {
+        if (grad_output.cols != d_model_)
+            throw InvalidInput("grad_output length " + std::to_string(grad_output.cols) +
+                                   " does not match expected length " + std::to_string(d_model_),
+                               d_model_, grad_output.cols);
+        Matrix grad_input(grad_output.rows, d_model_);
+        if (act_ == RBMOE_F32) {
+            check(rbmoe_backward_host(layer_, grad_output.data.data(), grad_input.data.data()), device_->raw());
+        } else {
+            std::vector<uint16_t> gin(grad_output.data.size()), gout(grad_output.data.size());
+            for (size_t i = 0; i < gin.size(); ++i) gin[i] = to_bf16(grad_output.data[i]);
+            check(rbmoe_backward_host(layer_, gin.data(), gout.data()), device_->raw());
+            for (size_t i = 0; i < gout.size(); ++i) grad_input.data[i] = from_bf16(gout[i]);
+        }
+        return grad_input;
+    }
+
+    // Param::zero_grad over the layer's parameters (src/param.rs)
+    void zero_grads() { check(rbmoe_zero_grads(layer_), device_->raw()); }
+
+    // accumulated gradient of one weight matrix (`which`: RBMOE_W_*), shaped like the weight
+    Matrix weight_grad(int which, size_t expert = 0) {
+        const size_t E = config.num_experts, F = config.d_ff, Fs = shared_d_ff_ ? shared_d_ff_ : config.d_ff;
+        size_t rows = 0, cols = 0;
+        switch (which) {
+            case RBMOE_W_ROUTER: rows = E; cols = d_model_; break;
+            case RBMOE_W_GATE: case RBMOE_W_UP: rows = F; cols = d_model_; break;
+            case RBMOE_W_DOWN: rows = d_model_; cols = F; break;
+            case RBMOE_W_SHARED_GATE: case RBMOE_W_SHARED_UP: rows = Fs; cols = d_model_; break;
+            case RBMOE_W_SHARED_DOWN: rows = d_model_; cols = Fs; break;
+            default: throw InvalidConfig("unknown weight id");
+        }
+        Matrix g(rows, cols);
+        check(rbmoe_get_weight_grad(layer_, which, (int32_t)expert, g.data.data(), (int32_t)rows, (int32_t)cols),
+              device_->raw());
+        return g;
+    }
+
     uint64_t num_parameters() const { return counts().first; }
     uint64_t active_parameters() const { return counts().second; }
     std::string kernel_name() const { return rbmoe_expert_kernel_name(layer_); }
@@ -278,6 +320,7 @@ class MoeLayer {
     size_t d_model_;
     std::shared_ptr<Device> device_;
     int act_;
+    size_t shared_d_ff_ = 0;
     rbmoe_layer* layer_ = nullptr;
 };
 
