@@ -171,6 +171,24 @@ int rbmoe_get_routing(rbmoe_layer* layer, rbmoe_routing* routing);
  * (src/moe.rs:150-152, src/ffn.rs:27-33).  Synchronises. */
 int rbmoe_get_expert_rows(rbmoe_layer* layer, float* hidden, float* expert_out);
 
+/* ---- the block's steps either side of the layer ------------------------------------------
+ * TransformerBlock::forward_train's feed-forward half (src/transformer_block.rs:216-222):
+ *   normed = feed_forward_norm.forward(residual)   RmsNorm::forward, src/norm.rs:41-61
+ *   output = moe.forward_train(normed) + residual  add_in_place, src/transformer_block.rs:310-323
+ * rbmoe_set_feed_forward_norm uploads the norm's weight [d_model] (f32, host) and eps
+ * (TransformerConfig::rmsnorm_eps, src/transformer.rs:42); the first call allocates the normed rows. */
+int rbmoe_set_feed_forward_norm(rbmoe_layer* layer, const float* weight, int32_t cols, float eps);
+/* out = x + layer(rmsnorm(x)) on DEVICE pointers ([T, d] act_dtype; `out` may be `x` itself).  The norm
+ * runs as a prologue kernel with the reference's sequential sum of squares, so routing is decided on the
+ * same normed rows as on the CPU; the residual add is part of the combine kernel.  Routing, losses and
+ * the backward pass's state refer to the NORMED rows (rbmoe_backward then returns the gradient with
+ * respect to them).  Other arguments as rbmoe_forward. */
+int rbmoe_forward_block(rbmoe_layer* layer, const void* x, int32_t tokens, int32_t cols, const uint8_t* valid,
+                        const float* router_bias, void* out);
+/* Same on HOST pointers; synchronises. */
+int rbmoe_forward_block_host(rbmoe_layer* layer, const void* x, int32_t tokens, int32_t cols,
+                             const uint8_t* valid, const float* router_bias, void* out);
+
 /* ---- backward pass (MoeLayer::backward, src/moe.rs:348-489) ------------------------------
  * Training mode makes the forward keep what MoeCache keeps for the backward pass (the input,
  * src/moe.rs:133-135; gate and up pre-activations, src/ffn.rs:27-33) and allocates f32 gradient

@@ -2,7 +2,9 @@
 //
 // This file restates, on the CPU and in plain C++, the algorithm of
 // RustingBrain's `MoeLayer::forward_train` (reference src/moe.rs:243-341), of
-// `MoeLayer::backward` (src/moe.rs:348-489) and of the helpers under them.  It is NOT the Rust binary: no Rust toolchain exists
+// `MoeLayer::backward` (src/moe.rs:348-489), of the helpers under them, and of the block's
+// steps either side of the layer (RmsNorm::forward, src/norm.rs:41-61; the residual add,
+// src/transformer_block.rs:221-222).  It is NOT the Rust binary: no Rust toolchain exists
 // where this is built, so every function below follows the reference source
 // text line by line and cites the lines it follows.  Nothing in the shipped
 // library links, loads or calls this file; only tests, the smoke check and
@@ -694,6 +696,22 @@ int rbo_moe_forward(const rbo_layer* L, const float* x, int T, int cols, const u
 // `ulps` units in the last place.  Such tokens may route differently under
 // another summation order or libm; every other token cannot.
 // ---------------------------------------------------------------------------
+// RmsNorm::forward (reference src/norm.rs:41-61 with inverse_rms, :128-131), the step in front of
+// the layer in a decoder block (feed_forward_norm, src/transformer_block.rs:216): per row
+// mean_square = (sum of value * value, in index order) / cols; inverse_rms = 1 / sqrt(mean_square + eps);
+// out = (value * inverse_rms) * weight.  Pinned by the reference's three forward tests
+// (src/norm.rs:138-170) and a float64 closed form (tests/test_oracle_norm.py).
+void rbo_rmsnorm_rows(const float* x, int T, int d, const float* weight, float eps, float* out) {
+    for (int t = 0; t < T; ++t) {
+        const float* row = x + (size_t)t * d;
+        float sum = 0.0f;
+        for (int c = 0; c < d; ++c) sum = sum + row[c] * row[c];
+        const float mean_square = sum / (float)d;
+        const float inverse_rms = 1.0f / std::sqrt(mean_square + eps);
+        for (int c = 0; c < d; ++c) out[(size_t)t * d + c] = (row[c] * inverse_rms) * weight[c];
+    }
+}
+
 int rbo_near_ties(const float* P, int T, int E, int k, int ulps) {
     if (k >= E) return 0;
     int n = 0;

@@ -292,6 +292,21 @@ _lib.rbo_moe_backward.restype = C.c_int
 _lib.rbo_moe_backward.argtypes = [C.POINTER(_Layer), _f32p, C.c_int, C.c_int, _u8p, _f32p, _f32p, C.POINTER(_Grads)]
 
 
+_lib.rbo_rmsnorm_rows.restype = None
+_lib.rbo_rmsnorm_rows.argtypes = [_f32p, C.c_int, C.c_int, _f32p, C.c_float, _f32p]
+
+
+def rmsnorm(x: np.ndarray, weight: np.ndarray, eps: float) -> np.ndarray:
+    """RmsNorm::forward (src/norm.rs:41-61): rows of ``x`` times ``1 / sqrt(mean(x^2) + eps)`` times ``weight``."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    weight = np.ascontiguousarray(weight, dtype=np.float32)
+    T, d = x.shape
+    assert weight.shape == (d,)
+    out = np.empty_like(x)
+    _lib.rbo_rmsnorm_rows(_fp(x), T, d, _fp(weight), C.c_float(eps), _fp(out))
+    return out
+
+
 @dataclass
 class BackwardResult:
     """Gradients of MoeLayer::backward (src/moe.rs:348-489); the weight gradients start from zero here."""
@@ -365,6 +380,20 @@ class OracleLayer:
         res["hidden"] = res["hidden"][:R]
         res["expert_out"] = res["expert_out"][:R]
         return ForwardResult(aux_loss=float(outs.aux_loss), z_loss=float(outs.z_loss), **res)
+
+    def forward_block(self, residual: np.ndarray, norm_weight: np.ndarray, eps: float,
+                      valid: Optional[np.ndarray] = None, router_bias: Optional[np.ndarray] = None,
+                      threads: int = 1, round_normed=None):
+        """The feed-forward half of TransformerBlock::forward_train (src/transformer_block.rs:216-222):
+        ``normed = feed_forward_norm.forward(residual)``, ``projected = moe.forward_train(normed)``,
+        ``output = projected + residual``.  ``round_normed`` (e.g. rounding to bf16) is applied to the normed rows
+        when the layer's activations are narrower than f32.  Returns (output, normed, ForwardResult)."""
+        residual = np.ascontiguousarray(residual, dtype=np.float32)
+        normed = rmsnorm(residual, norm_weight, eps)
+        if round_normed is not None:
+            normed = np.ascontiguousarray(round_normed(normed), dtype=np.float32)
+        res = self.forward(normed, valid=valid, router_bias=router_bias, threads=threads)
+        return res.out + residual, normed, res
 
     def backward(self, x: np.ndarray, grad_output: np.ndarray, valid: Optional[np.ndarray] = None,
                  router_bias: Optional[np.ndarray] = None) -> BackwardResult:

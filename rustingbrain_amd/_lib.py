@@ -67,6 +67,10 @@ SIGNATURES = {
     "rbmoe_copy_to_device": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
     "rbmoe_copy_to_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
     "rbmoe_copy_device": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
+    "rbmoe_set_feed_forward_norm": (C.c_int, [C.c_void_p, C.POINTER(C.c_float), C.c_int32, C.c_float]),
+    "rbmoe_forward_block": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "rbmoe_forward_block_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p,
+                                           C.c_void_p]),
     "rbmoe_layer_enable_training": (C.c_int, [C.c_void_p]),
     "rbmoe_backward": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
     "rbmoe_backward_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),

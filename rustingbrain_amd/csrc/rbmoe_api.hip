@@ -139,6 +139,10 @@ struct rbmoe_layer {
     Buf counts, offsets, tile_expert, tile_row0, tile_rows, ntiles, losses;
     Buf perm_slot, perm_token, inv_pos;
     Buf xg, h, y, hs, ys;
+    // feed-forward norm in front of the layer (allocated by rbmoe_set_feed_forward_norm)
+    Buf xn, norm_w;  // [max_T, d] activation dtype, [d] f32
+    float norm_eps = 0.0f;
+    bool norm_set = false;
     // training (allocated by rbmoe_layer_enable_training)
     bool training = false;
     bool weights_set = false;
@@ -866,6 +870,99 @@ int rbmoe_forward_host(rbmoe_layer* L, const void* x, int32_t T, int32_t cols, c
     int rc = forward_impl(L, L->st_x.p, T, cols, valid ? (const uint8_t*)L->st_valid.p : nullptr,
                           router_bias ? (const float*)L->st_bias.p : nullptr, residual ? L->st_res.p : nullptr,
                           L->st_out.p, false);
+    if (rc != RBMOE_OK) return rc;
+    if (T > 0) HIP_TRY(ctx, hipMemcpyAsync(out, L->st_out.p, nbytes, hipMemcpyDeviceToHost, s));
+    HIP_TRY(ctx, hipStreamSynchronize(s));
+    return RBMOE_OK;
+}
+
+// ---------------------------------------------------------------------------
+// The block's steps either side of the layer: RmsNorm::forward in front
+// (src/norm.rs:41-61, src/transformer_block.rs:216), the residual add behind
+// (src/transformer_block.rs:221-222).
+// ---------------------------------------------------------------------------
+int rbmoe_set_feed_forward_norm(rbmoe_layer* L, const float* weight, int32_t cols, float eps) {
+    if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
+    rbmoe_ctx* ctx = L->ctx;
+    const rbmoe_config& c = L->cfg;
+    if (!weight) return fail(ctx, RBMOE_NULL_POINTER, "weight is NULL");
+    if (cols != c.d_model) {
+        char buf[120];
+        std::snprintf(buf, sizeof buf, "norm weight length %d does not match expected length %d", cols, c.d_model);
+        return fail(ctx, RBMOE_INVALID_INPUT, buf);
+    }
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    if (!L->norm_w.p) {
+        Plan p;
+        p.add(&L->xn, (size_t)L->max_T * c.d_model * dtype_size(c.act_dtype));
+        p.add(&L->norm_w, (size_t)c.d_model * 4);
+        if (ctx->budget_bytes && ctx->allocated + p.total > ctx->budget_bytes) {
+            char buf[200];
+            std::snprintf(buf, sizeof buf, "memory budget exceeded: estimated %zu MiB exceeds budget %zu MiB",
+                          (ctx->allocated + p.total + (1 << 20) - 1) >> 20, ctx->budget_bytes >> 20);
+            return fail(ctx, RBMOE_MEMORY_BUDGET, buf);
+        }
+        for (auto& it : p.items) {
+            void* q = nullptr;
+            if (hipMalloc(&q, it.second) != hipSuccess) {
+                (void)hipGetLastError();
+                return fail(ctx, RBMOE_OUT_OF_MEMORY, "out of memory while allocating the normed rows");
+            }
+            it.first->p = q;
+            it.first->bytes = it.second;
+            ctx->allocated += it.second;
+            L->all.push_back(it.first);
+        }
+    }
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));  // no forward may still read the old weight
+    HIP_TRY(ctx, hipMemcpy(L->norm_w.p, weight, (size_t)c.d_model * 4, hipMemcpyHostToDevice));
+    L->norm_eps = eps;
+    L->norm_set = true;
+    return RBMOE_OK;
+}
+
+int rbmoe_forward_block(rbmoe_layer* L, const void* x, int32_t T, int32_t cols, const uint8_t* valid,
+                        const float* router_bias, void* out) {
+    if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
+    rbmoe_ctx* ctx = L->ctx;
+    if (!L->norm_set) return fail(ctx, RBMOE_INVALID_CONFIG, "the feed-forward norm has not been set");
+    if (cols != L->cfg.d_model) {
+        char buf[120];
+        std::snprintf(buf, sizeof buf, "input length %d does not match expected length %d", cols, L->cfg.d_model);
+        return fail(ctx, RBMOE_INVALID_INPUT, buf);
+    }
+    if (T < 0 || T > L->max_T) return fail(ctx, RBMOE_INVALID_INPUT, "token count outside [0, max_tokens]");
+    if (T > 0 && (!x || !out)) return fail(ctx, RBMOE_NULL_POINTER, "x or out is NULL");
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    HIP_TRY(ctx, launch_rmsnorm(x, (const float*)L->norm_w.p, L->norm_eps, T, cols, L->xn.p,
+                                L->cfg.act_dtype == RBMOE_BF16, ctx->stream));
+    return forward_impl(L, L->xn.p, T, cols, valid, router_bias, x, out, false);
+}
+
+int rbmoe_forward_block_host(rbmoe_layer* L, const void* x, int32_t T, int32_t cols, const uint8_t* valid,
+                             const float* router_bias, void* out) {
+    if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
+    rbmoe_ctx* ctx = L->ctx;
+    const rbmoe_config& c = L->cfg;
+    if (!L->norm_set) return fail(ctx, RBMOE_INVALID_CONFIG, "the feed-forward norm has not been set");
+    if (cols != c.d_model) {
+        char buf[120];
+        std::snprintf(buf, sizeof buf, "input length %d does not match expected length %d", cols, c.d_model);
+        return fail(ctx, RBMOE_INVALID_INPUT, buf);
+    }
+    if (T < 0 || T > L->max_T) return fail(ctx, RBMOE_INVALID_INPUT, "token count outside [0, max_tokens]");
+    if (T > 0 && (!x || !out)) return fail(ctx, RBMOE_NULL_POINTER, "x or out is NULL");
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    const size_t nbytes = (size_t)T * c.d_model * dtype_size(c.act_dtype);
+    hipStream_t s = ctx->stream;
+    if (T > 0) {
+        HIP_TRY(ctx, hipMemcpyAsync(L->st_x.p, x, nbytes, hipMemcpyHostToDevice, s));
+        if (valid) HIP_TRY(ctx, hipMemcpyAsync(L->st_valid.p, valid, (size_t)T, hipMemcpyHostToDevice, s));
+    }
+    if (router_bias)
+        HIP_TRY(ctx, hipMemcpyAsync(L->st_bias.p, router_bias, (size_t)c.num_experts * 4, hipMemcpyHostToDevice, s));
+    int rc = rbmoe_forward_block(L, L->st_x.p, T, cols, valid ? (const uint8_t*)L->st_valid.p : nullptr,
+                                 router_bias ? (const float*)L->st_bias.p : nullptr, L->st_out.p);
     if (rc != RBMOE_OK) return rc;
     if (T > 0) HIP_TRY(ctx, hipMemcpyAsync(out, L->st_out.p, nbytes, hipMemcpyDeviceToHost, s));
     HIP_TRY(ctx, hipStreamSynchronize(s));

@@ -74,6 +74,11 @@ struct CombineArgs {
 };
 hipError_t launch_combine(const CombineArgs& a, bool bf16, hipStream_t s);
 
+// RmsNorm::forward (src/norm.rs:41-61) over rows: out = (x * inverse_rms(row)) * weight, the sum of squares in
+// index order
+hipError_t launch_rmsnorm(const void* x, const float* weight, float eps, int T, int d, void* out, bool bf16,
+                          hipStream_t s);
+
 // ---------------------------------------------------------------------------
 // Grouped expert products.  Rows of `a` are grouped by expert through the tile
 // table written by the scan kernel; a tile never spans two experts.

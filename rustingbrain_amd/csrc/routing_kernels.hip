@@ -1051,6 +1051,78 @@ static hipError_t launch_combine_t(const CombineArgs& a, hipStream_t s) {
     return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// RmsNorm::forward (src/norm.rs:41-61, inverse_rms :128-131) in front of the layer
+// (feed_forward_norm, src/transformer_block.rs:216).  A block of 64 threads owns 64 rows.
+// First every thread adds up the squares of ITS row in index order - the reference's
+// sequential f32 sum, so the normed rows (and with them the routing) come out identical - then
+// the block walks its rows with neighbouring lanes on neighbouring 16-byte pieces and writes
+// (value * inverse_rms) * weight, two separately rounded products as in the reference.
+// ---------------------------------------------------------------------------
+template <typename XT>
+__global__ __launch_bounds__(64) void rmsnorm_rows_kernel(const XT* __restrict__ x, const float* __restrict__ weight,
+                                                          float eps, int T, int d, XT* __restrict__ out) {
+    constexpr int VN = Vec16<XT>::N;
+    __shared__ float inv[64];
+    const int lane = threadIdx.x;
+    const int row0 = blockIdx.x * 64;
+    const int my = min(row0 + lane, T - 1);  // rows past the end: a valid row, result unused
+    const XT* xr = x + (size_t)my * d;
+    const bool vec = d % VN == 0;  // uniform
+    float sum = 0.0f;
+    if (vec) {
+        for (int c = 0; c < d; c += VN) {
+            float v[VN];
+            Vec16<XT>::load(xr + c, v);
+#pragma unroll
+            for (int i = 0; i < VN; ++i) sum = __fadd_rn(sum, __fmul_rn(v[i], v[i]));
+        }
+    } else {
+        for (int c = 0; c < d; ++c) {
+            const float v = to_f32(xr[c]);
+            sum = __fadd_rn(sum, __fmul_rn(v, v));
+        }
+    }
+    const float mean_square = __fdiv_rn(sum, (float)d);
+    // The root must be the correctly rounded one (the reference's f32::sqrt): taken in double and rounded once,
+    // which is exact for a square root; the single-precision root instruction alone is not.
+    const float root = (float)sqrt((double)__fadd_rn(mean_square, eps));
+    inv[lane] = __fdiv_rn(1.0f, root);
+    __syncthreads();
+    const int nrows = min(64, T - row0);
+    if (vec) {
+        const int pieces = d / VN;
+        for (int idx = lane; idx < nrows * pieces; idx += 64) {
+            const int r = idx / pieces, c = (idx - r * pieces) * VN;
+            float v[VN], o[VN];
+            Vec16<XT>::load(x + (size_t)(row0 + r) * d + c, v);
+            const float s = inv[r];
+#pragma unroll
+            for (int i = 0; i < VN; ++i) o[i] = __fmul_rn(__fmul_rn(v[i], s), weight[c + i]);
+            Vec16<XT>::store(out + (size_t)(row0 + r) * d + c, o);
+        }
+    } else {
+        for (int idx = lane; idx < nrows * d; idx += 64) {
+            const int r = idx / d, c = idx - r * d;
+            const float v = to_f32(x[(size_t)(row0 + r) * d + c]);
+            out[(size_t)(row0 + r) * d + c] = from_f32<XT>(__fmul_rn(__fmul_rn(v, inv[r]), weight[c]));
+        }
+    }
+}
+
+hipError_t launch_rmsnorm(const void* x, const float* weight, float eps, int T, int d, void* out, bool bf16,
+                          hipStream_t s) {
+    if (T <= 0) return hipSuccess;
+    const dim3 grid((T + 63) / 64), block(64);
+    if (bf16)
+        hipLaunchKernelGGL(rmsnorm_rows_kernel<bf16_t>, grid, block, 0, s, static_cast<const bf16_t*>(x), weight, eps,
+                           T, d, static_cast<bf16_t*>(out));
+    else
+        hipLaunchKernelGGL(rmsnorm_rows_kernel<float>, grid, block, 0, s, static_cast<const float*>(x), weight, eps, T,
+                           d, static_cast<float*>(out));
+    return hipGetLastError();
+}
+
 hipError_t launch_combine(const CombineArgs& a, bool bf16, hipStream_t s) {
     if (a.T <= 0) return hipSuccess;
     return bf16 ? launch_combine_t<bf16_t>(a, s) : launch_combine_t<float>(a, s);

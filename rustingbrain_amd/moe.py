@@ -396,6 +396,48 @@ class MoeLayer:
                self.device.handle)
         return h[:routed], y[:routed]
 
+    # ---- the block's steps either side of the layer (reference src/transformer_block.rs:216-222)
+    def set_feed_forward_norm(self, weight: np.ndarray, eps: float = 1e-6) -> None:
+        """Weight ``[d_model]`` and eps of the block's ``feed_forward_norm`` (RmsNorm, src/norm.rs:23-37)."""
+        w = np.ascontiguousarray(np.asarray(weight, dtype=np.float32).reshape(-1))
+        _check(self._lib.rbmoe_set_feed_forward_norm(self.handle, w.ctypes.data_as(C.POINTER(C.c_float)), w.size,
+                                                     C.c_float(eps)), self.device.handle)
+
+    def forward_block(self, residual: np.ndarray, layout: Layout = Layout(),
+                      router_bias: Optional[np.ndarray] = None) -> Tuple[np.ndarray, MoeCache]:
+        """``residual + forward_train(feed_forward_norm(residual))``; the cache describes the normed rows."""
+        residual = np.asarray(residual)
+        if residual.ndim != 2:
+            raise InvalidInput("input must be a [tokens, d_model] matrix")
+        rows, cols = residual.shape
+        if cols != self._d_model:
+            raise InvalidInput(f"input length {cols} does not match expected length {self._d_model}",
+                               expected=self._d_model, actual=cols)
+        layout.check(rows)
+        x = self._to_act(residual)
+        out = np.empty_like(x)
+        vp = bp = None
+        valid = None
+        if layout.valid is not None:
+            valid = np.ascontiguousarray(np.asarray(layout.valid, dtype=bool).astype(np.uint8))
+            vp = valid.ctypes.data_as(C.c_void_p)
+        if router_bias is not None:
+            router_bias = np.ascontiguousarray(router_bias, dtype=np.float32)
+            bp = router_bias.ctypes.data_as(C.c_void_p)
+        _check(self._lib.rbmoe_forward_block_host(self.handle, x.ctypes.data_as(C.c_void_p), rows, cols, vp, bp,
+                                                  out.ctypes.data_as(C.c_void_p)), self.device.handle)
+        if self.act_dtype == "bf16":
+            out = bf16_bits_to_f32(out).reshape(rows, cols)
+        valid_tokens = rows if valid is None else int(valid.sum())
+        return out, self.cache(rows, valid_tokens)
+
+    def forward_block_device(self, x_ptr: int, tokens: int, out_ptr: int, valid_ptr: int = 0,
+                             bias_ptr: int = 0) -> None:
+        """Enqueue one block step on device pointers (no synchronisation); ``out_ptr`` may equal ``x_ptr``."""
+        _check(self._lib.rbmoe_forward_block(self.handle, C.c_void_p(x_ptr), tokens, self._d_model,
+                                             C.c_void_p(valid_ptr or None), C.c_void_p(bias_ptr or None),
+                                             C.c_void_p(out_ptr)), self.device.handle)
+
     # ---- backward (reference MoeLayer::backward, src/moe.rs:348-489)
     def enable_training(self) -> None:
         """Makes the forward keep what the backward pass needs and allocates the gradient accumulators.

@@ -158,6 +158,7 @@ def write(path: str, config: dict, params: List[np.ndarray], precision: str = "F
 class MoeBlockParams:
     """The parameters of one sparse block's feed-forward, in the reference's order (src/moe.rs:516-525)."""
     block: int
+    norm: RbwParam          # feed_forward_norm.weight, 1 x d_model (src/norm.rs:30-35)
     router: RbwParam
     experts: List[Dict[str, RbwParam]]
     shared: Optional[Dict[str, RbwParam]]
@@ -202,12 +203,13 @@ def moe_blocks(snapshot: RbwFile) -> List[MoeBlockParams]:
         take(kv_heads * head_dim, d, f"block {b} key")
         take(kv_heads * head_dim, d, f"block {b} value")
         take(d, heads * head_dim, f"block {b} output")
+        ff_norm = params[pos] if pos < len(params) else None
         pos += 1  # feed_forward_norm
         if b in sparse:
             router = take(E, d, f"block {b} router")
             experts = [take_swiglu(moe_d_ff, f"block {b} expert {e}") for e in range(E)]
             sh = take_swiglu(moe_d_ff, f"block {b} shared expert") if shared else None
-            out.append(MoeBlockParams(b, router, experts, sh))
+            out.append(MoeBlockParams(b, ff_norm, router, experts, sh))
         else:
             take_swiglu(d_ff, f"block {b} feed-forward")
     pos += 1  # final_norm
@@ -235,6 +237,9 @@ def load_moe_layers(path: str, device, max_tokens: int, act_dtype: str = "bf16",
         layer = MoeLayer(int(c["d_model"]), cfg, device, act_dtype=act_dtype, weight_dtype=weight_dtype,
                          max_tokens=max_tokens)
         layer.set_router(blk.router.dequantized())
+        if blk.norm is not None and blk.norm.rows * blk.norm.cols == int(c["d_model"]):
+            # the norm in front of the layer, for MoeLayer.forward_block
+            layer.set_feed_forward_norm(blk.norm.dequantized().reshape(-1), float(c.get("rmsnorm_eps", 1e-6)))
 
         def put(setter_f32, setter_q8, ex):
             if snap.precision == "Q8" and weight_dtype == "int8":

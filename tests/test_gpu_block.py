@@ -1,0 +1,131 @@
+"""GPU parity of the block step around the layer (src/transformer_block.rs:216-222): RmsNorm::forward in front
+(src/norm.rs:41-61), the residual add behind.  The norm's sum of squares runs in the reference's order on both
+sides, so the normed rows - and with them every routing table - must be identical in every bit; outputs within
+rel-L2 1e-5 (all-f32 layers) or 2e-2 (bf16 / int8).
+"""
+import numpy as np
+import pytest
+
+import rustingbrain_amd as rb
+from conftest import rel_l2
+from helpers import assert_routing_identical, gpu_layer, oracle_layer, small_workload, tolerance
+from rustingbrain_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def norm_weight(d, seed):
+    return np.random.default_rng(seed).uniform(0.5, 1.5, d).astype(np.float32)
+
+
+def check_block(device, t, eps=1e-6, valid=None, bias=None, seed=3, scale=1.0):
+    w = t.workload
+    nw = norm_weight(w.d_model, seed)
+    x = t.x * np.float32(scale)
+    if w.act_dtype == "bf16":
+        x = synth.round_bf16(x)
+    rounder = synth.round_bf16 if w.act_dtype == "bf16" else None
+    want, normed, ref = oracle_layer(t).forward_block(x, nw, eps, valid=valid, router_bias=bias, round_normed=rounder)
+    layer = gpu_layer(device, t)
+    layer.set_feed_forward_norm(nw, eps)
+    layout = rb.Layout(valid=None if valid is None else [bool(v) for v in valid])
+    out, cache = layer.forward_block(x, layout, router_bias=bias)
+    assert_routing_identical(cache, ref)
+    tol = tolerance(w)
+    assert rel_l2(out, want) <= tol
+    # the layer's own share, without the residual that dominates the sum; a bf16 output carries the rounding
+    # of the SUM (2^-9 of its size), which weighs more the larger the residual is against the share
+    share = float(np.linalg.norm(want - x))
+    rounding = 2.0 ** -8 * float(np.linalg.norm(want)) / max(share, 1e-30) if w.act_dtype == "bf16" else 0.0
+    assert rel_l2(out - x, want - x) <= 2 * tol + rounding
+    layer.close()
+    return out, cache, ref
+
+
+SHAPES = [
+    dict(d=8, E=4, k=2, F=6, T=7),
+    dict(d=33, E=7, k=3, F=19, T=65),
+    dict(d=64, E=8, k=2, F=64, T=200, shared=True),
+    dict(d=128, E=16, k=2, F=64, T=513),
+    dict(d=768, E=8, k=2, F=128, T=130, shared=True),
+]
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "d{d}_E{E}_k{k}_F{F}_T{T}".format(**s))
+@pytest.mark.parametrize("act,wt", [("f32", "f32"), ("bf16", "bf16"), ("bf16", "int8")])
+def test_block_step_matches_the_oracle(device, shape, act, wt):
+    t = synth.make(small_workload(seed=41, act=act, wt=wt, **shape))
+    check_block(device, t)
+
+
+def test_block_step_with_padding_rows_bias_and_large_inputs(device):
+    t = synth.make(small_workload(d=64, E=6, k=2, F=64, T=90, seed=42, act="bf16", wt="bf16", shared=True))
+    valid = (np.arange(90) % 4 != 3).astype(np.uint8)
+    bias = np.linspace(-0.3, 0.3, 6).astype(np.float32)
+    out, cache, ref = check_block(device, t, eps=1e-5, valid=valid, bias=bias, scale=37.0)
+    assert cache.valid_tokens == int(valid.sum())
+
+
+def test_a_few_tokens_take_the_decode_kernels(device):
+    t = synth.make(small_workload(d=128, E=8, k=2, F=128, T=5, seed=43, act="bf16", wt="bf16", shared=True))
+    nw = norm_weight(128, 1)
+    layer = gpu_layer(device, t, max_tokens=8)
+    layer.set_feed_forward_norm(nw, 1e-6)
+    want, _, ref = oracle_layer(t).forward_block(t.x, nw, 1e-6, round_normed=synth.round_bf16)
+    out, cache = layer.forward_block(t.x)
+    assert layer.kernel_name().startswith("mfma_bf16_decode")
+    assert_routing_identical(cache, ref)
+    assert rel_l2(out, want) <= 2e-2
+    layer.close()
+
+
+def test_in_place_and_device_pointers(device):
+    from bench import DeviceBuffer
+    t = synth.make(small_workload(d=64, E=4, k=2, F=64, T=300, seed=44, act="bf16", wt="bf16"))
+    nw = norm_weight(64, 2)
+    layer = gpu_layer(device, t)
+    layer.set_feed_forward_norm(nw, 1e-6)
+    want, _ = layer.forward_block(t.x)
+    bits = synth.f32_to_bf16_bits(t.x)
+    buf = DeviceBuffer(device, bits.nbytes).upload(bits)
+    layer.forward_block_device(buf.ptr, 300, buf.ptr)     # out == x
+    device.synchronize()
+    got = synth.bf16_bits_to_f32(buf.download(np.empty_like(bits))).reshape(300, 64)
+    assert np.array_equal(got, want)
+    buf.free()
+    layer.close()
+
+
+def test_norm_errors(device):
+    t = synth.make(small_workload(d=8, E=4, k=2, F=6, T=4, seed=45))
+    layer = gpu_layer(device, t)
+    with pytest.raises(rb.InvalidConfig):
+        layer.forward_block(t.x)                           # norm not set
+    with pytest.raises(rb.InvalidInput):
+        layer.set_feed_forward_norm(np.ones(7, np.float32))
+    layer.set_feed_forward_norm(np.ones(8, np.float32), 1e-6)
+    layer.set_feed_forward_norm(np.full(8, 2.0, np.float32), 1e-6)   # replacing it is allowed
+    with pytest.raises(rb.InvalidInput):
+        layer.forward_block(np.zeros((4, 9), np.float32))
+    out, _ = layer.forward_block(np.zeros((4, 8), np.float32))       # zero rows stay finite (eps under the root)
+    assert np.isfinite(out).all()
+    layer.close()
+
+
+def test_c3_block_step_at_full_size(device):
+    t = synth.make(synth.WORKLOADS["c3_prefill_d768_e16"])
+    w = t.workload
+    nw = norm_weight(w.d_model, 9)
+    # a residual stream with rows of very different size, as after a few blocks
+    rng = np.random.default_rng(10)
+    x = synth.round_bf16(t.x * rng.uniform(0.25, 8.0, (w.tokens, 1)).astype(np.float32))
+    want, normed, ref = oracle_layer(t).forward_block(x, nw, 1e-6, router_bias=t.router_bias, threads=8,
+                                                      round_normed=synth.round_bf16)
+    layer = gpu_layer(device, t)
+    layer.set_feed_forward_norm(nw, 1e-6)
+    out, cache = layer.forward_block(x, router_bias=t.router_bias)
+    assert_routing_identical(cache, ref)
+    assert rel_l2(out, want) <= 2e-2
+    share = float(np.linalg.norm(want - x))
+    assert rel_l2(out - x, want - x) <= 4e-2 + 2.0 ** -8 * float(np.linalg.norm(want)) / share
+    layer.close()

@@ -28,7 +28,8 @@ def model_params(c, seed=3):
     params, moe = [m(c["vocab_size"], d)], {}
     for b in range(c["n_layers"]):
         params += [np.ones((1, d), np.float32), m(c["n_heads"] * hd, d), m(c["n_kv_heads"] * hd, d),
-                   m(c["n_kv_heads"] * hd, d), m(d, c["n_heads"] * hd), np.ones((1, d), np.float32)]
+                   m(c["n_kv_heads"] * hd, d), m(d, c["n_heads"] * hd),
+                   (np.float32(1.0) + m(1, d, 0.1)).astype(np.float32)]  # feed_forward_norm: not all ones
         if b in c["moe_layers"]:
             start = len(params)
             params.append(m(c["num_experts"], d, 0.5))
@@ -143,4 +144,10 @@ def test_sparse_blocks_of_a_snapshot_run_on_the_device(tmp_path, device, precisi
         assert layer.kernel_name().startswith("mfma_bf16")
         assert_routing_identical(cache, ref)
         assert rel_l2(out, ref.out) <= 2e-2
+        # the block step with the snapshot's own feed_forward_norm and rmsnorm_eps
+        nw = blk.norm.dequantized().reshape(-1)
+        want, _, ref_b = ref_layer.forward_block(x, nw, c["rmsnorm_eps"], round_normed=synth.round_bf16)
+        out_b, cache_b = layer.forward_block(x)
+        assert_routing_identical(cache_b, ref_b)
+        assert rel_l2(out_b, want) <= 2e-2
         layer.close()
