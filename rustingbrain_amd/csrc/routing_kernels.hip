@@ -1053,74 +1053,123 @@ static hipError_t launch_combine_t(const CombineArgs& a, hipStream_t s) {
 
 // ---------------------------------------------------------------------------
 // RmsNorm::forward (src/norm.rs:41-61, inverse_rms :128-131) in front of the layer
-// (feed_forward_norm, src/transformer_block.rs:216).  A block of 64 threads owns 64 rows.
-// First every thread adds up the squares of ITS row in index order - the reference's
-// sequential f32 sum, so the normed rows (and with them the routing) come out identical - then
-// the block walks its rows with neighbouring lanes on neighbouring 16-byte pieces and writes
-// (value * inverse_rms) * weight, two separately rounded products as in the reference.
+// (feed_forward_norm, src/transformer_block.rs:216).  The sum of squares of a row is the
+// reference's sequential f32 sum in index order, so the normed rows (and with them the routing)
+// come out identical; the output is (value * inverse_rms) * weight, two separately rounded
+// products as in the reference.
+//
+// The chain of d dependent additions per row is the floor of this kernel.  To keep memory
+// latency off that chain, a block first copies its R rows into LDS with every lane's loads in
+// flight at once (the rows of a block are one contiguous range), then lane r of the first wave
+// walks row r in LDS (pitch padded by 16 bytes: lanes fall into different banks), then the whole
+// block writes the normed rows from the LDS copy - the input is read from memory once.
 // ---------------------------------------------------------------------------
+__device__ __forceinline__ float inverse_rms_of(float sum, int d, float eps) {
+    const float mean_square = __fdiv_rn(sum, (float)d);
+    // The root must be the correctly rounded one (the reference's f32::sqrt): taken in double and rounded once,
+    // which is exact for a square root; the single-precision root instruction alone is not.
+    const float root = (float)sqrt((double)__fadd_rn(mean_square, eps));
+    return __fdiv_rn(1.0f, root);
+}
+
 template <typename XT>
-__global__ __launch_bounds__(64) void rmsnorm_rows_kernel(const XT* __restrict__ x, const float* __restrict__ weight,
-                                                          float eps, int T, int d, XT* __restrict__ out) {
+__global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const XT* __restrict__ x, const float* __restrict__ weight,
+                                                           float eps, int T, int d, int R, int pitch,
+                                                           XT* __restrict__ out) {
     constexpr int VN = Vec16<XT>::N;
+    extern __shared__ __attribute__((aligned(16))) char smem[];  // R rows of `pitch` bytes, then R floats
+    float* const inv = reinterpret_cast<float*>(smem + (size_t)R * pitch);
+    const int tid = threadIdx.x;
+    const int row0 = blockIdx.x * R;
+    const int nrows = min(R, T - row0);
+    const int pieces = d / VN;  // d is a multiple of VN (checked by the launcher)
+    const XT* const src = x + (size_t)row0 * d;
+    for (int idx = tid; idx < nrows * pieces; idx += 256) {
+        const int r = idx / pieces, p = idx - r * pieces;
+        *reinterpret_cast<uint4*>(smem + (size_t)r * pitch + p * 16) =
+            *reinterpret_cast<const uint4*>(src + (size_t)idx * VN);
+    }
+    __syncthreads();
+    if (tid < nrows) {
+        const XT* const row = reinterpret_cast<const XT*>(smem + (size_t)tid * pitch);
+        float sum = 0.0f;
+#pragma unroll 4
+        for (int c = 0; c < d; c += VN) {
+            float v[VN];
+            Vec16<XT>::load(row + c, v);
+#pragma unroll
+            for (int i = 0; i < VN; ++i) sum = __fadd_rn(sum, __fmul_rn(v[i], v[i]));
+        }
+        inv[tid] = inverse_rms_of(sum, d, eps);
+    }
+    __syncthreads();
+    XT* const dst = out + (size_t)row0 * d;
+    for (int idx = tid; idx < nrows * pieces; idx += 256) {
+        const int r = idx / pieces, p = idx - r * pieces;
+        float v[VN], o[VN];
+        Vec16<XT>::load(reinterpret_cast<const XT*>(smem + (size_t)r * pitch + p * 16), v);
+        const float s = inv[r];
+        const float4* w = reinterpret_cast<const float4*>(weight + p * VN);
+#pragma unroll
+        for (int q = 0; q < VN / 4; ++q) {
+            const float4 wv = w[q];
+            o[4 * q + 0] = __fmul_rn(__fmul_rn(v[4 * q + 0], s), wv.x);
+            o[4 * q + 1] = __fmul_rn(__fmul_rn(v[4 * q + 1], s), wv.y);
+            o[4 * q + 2] = __fmul_rn(__fmul_rn(v[4 * q + 2], s), wv.z);
+            o[4 * q + 3] = __fmul_rn(__fmul_rn(v[4 * q + 3], s), wv.w);
+        }
+        Vec16<XT>::store(dst + (size_t)idx * VN, o);
+    }
+}
+
+// Any width, rows straight from memory: one thread per row for the sum, then the block walks its 64 rows.
+template <typename XT>
+__global__ __launch_bounds__(64) void rmsnorm_rows_direct_kernel(const XT* __restrict__ x,
+                                                                 const float* __restrict__ weight, float eps, int T,
+                                                                 int d, XT* __restrict__ out) {
     __shared__ float inv[64];
     const int lane = threadIdx.x;
     const int row0 = blockIdx.x * 64;
     const int my = min(row0 + lane, T - 1);  // rows past the end: a valid row, result unused
     const XT* xr = x + (size_t)my * d;
-    const bool vec = d % VN == 0;  // uniform
     float sum = 0.0f;
-    if (vec) {
-        for (int c = 0; c < d; c += VN) {
-            float v[VN];
-            Vec16<XT>::load(xr + c, v);
-#pragma unroll
-            for (int i = 0; i < VN; ++i) sum = __fadd_rn(sum, __fmul_rn(v[i], v[i]));
-        }
-    } else {
-        for (int c = 0; c < d; ++c) {
-            const float v = to_f32(xr[c]);
-            sum = __fadd_rn(sum, __fmul_rn(v, v));
-        }
+    for (int c = 0; c < d; ++c) {
+        const float v = to_f32(xr[c]);
+        sum = __fadd_rn(sum, __fmul_rn(v, v));
     }
-    const float mean_square = __fdiv_rn(sum, (float)d);
-    // The root must be the correctly rounded one (the reference's f32::sqrt): taken in double and rounded once,
-    // which is exact for a square root; the single-precision root instruction alone is not.
-    const float root = (float)sqrt((double)__fadd_rn(mean_square, eps));
-    inv[lane] = __fdiv_rn(1.0f, root);
+    inv[lane] = inverse_rms_of(sum, d, eps);
     __syncthreads();
     const int nrows = min(64, T - row0);
-    if (vec) {
-        const int pieces = d / VN;
-        for (int idx = lane; idx < nrows * pieces; idx += 64) {
-            const int r = idx / pieces, c = (idx - r * pieces) * VN;
-            float v[VN], o[VN];
-            Vec16<XT>::load(x + (size_t)(row0 + r) * d + c, v);
-            const float s = inv[r];
-#pragma unroll
-            for (int i = 0; i < VN; ++i) o[i] = __fmul_rn(__fmul_rn(v[i], s), weight[c + i]);
-            Vec16<XT>::store(out + (size_t)(row0 + r) * d + c, o);
-        }
-    } else {
-        for (int idx = lane; idx < nrows * d; idx += 64) {
-            const int r = idx / d, c = idx - r * d;
-            const float v = to_f32(x[(size_t)(row0 + r) * d + c]);
-            out[(size_t)(row0 + r) * d + c] = from_f32<XT>(__fmul_rn(__fmul_rn(v, inv[r]), weight[c]));
-        }
+    for (int idx = lane; idx < nrows * d; idx += 64) {
+        const int r = idx / d, c = idx - r * d;
+        const float v = to_f32(x[(size_t)(row0 + r) * d + c]);
+        out[(size_t)(row0 + r) * d + c] = from_f32<XT>(__fmul_rn(__fmul_rn(v, inv[r]), weight[c]));
     }
+}
+
+template <typename XT>
+hipError_t launch_rmsnorm_t(const XT* x, const float* weight, float eps, int T, int d, XT* out, hipStream_t s) {
+    constexpr int VN = Vec16<XT>::N;
+    const int pitch = d * (int)sizeof(XT) + 16;
+    const bool pieces_ok = d % VN == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+                           (reinterpret_cast<uintptr_t>(out) & 15) == 0 && (reinterpret_cast<uintptr_t>(weight) & 15) == 0;
+    if (pieces_ok && pitch + 4 <= 40 * 1024) {
+        const int R = std::max(1, std::min(64, (32 * 1024) / pitch));
+        const size_t lds = (size_t)R * pitch + (size_t)R * 4;
+        hipLaunchKernelGGL(rmsnorm_rows_kernel<XT>, dim3((T + R - 1) / R), dim3(256), lds, s, x, weight, eps, T, d, R,
+                           pitch, out);
+    } else {
+        hipLaunchKernelGGL(rmsnorm_rows_direct_kernel<XT>, dim3((T + 63) / 64), dim3(64), 0, s, x, weight, eps, T, d,
+                           out);
+    }
+    return hipGetLastError();
 }
 
 hipError_t launch_rmsnorm(const void* x, const float* weight, float eps, int T, int d, void* out, bool bf16,
                           hipStream_t s) {
     if (T <= 0) return hipSuccess;
-    const dim3 grid((T + 63) / 64), block(64);
-    if (bf16)
-        hipLaunchKernelGGL(rmsnorm_rows_kernel<bf16_t>, grid, block, 0, s, static_cast<const bf16_t*>(x), weight, eps,
-                           T, d, static_cast<bf16_t*>(out));
-    else
-        hipLaunchKernelGGL(rmsnorm_rows_kernel<float>, grid, block, 0, s, static_cast<const float*>(x), weight, eps, T,
-                           d, static_cast<float*>(out));
-    return hipGetLastError();
+    return bf16 ? launch_rmsnorm_t(static_cast<const bf16_t*>(x), weight, eps, T, d, static_cast<bf16_t*>(out), s)
+                : launch_rmsnorm_t(static_cast<const float*>(x), weight, eps, T, d, static_cast<float*>(out), s);
 }
 
 hipError_t launch_combine(const CombineArgs& a, bool bf16, hipStream_t s) {
