@@ -129,8 +129,8 @@ def cpu_baseline_backward(t: synth.Tensors, grad_output: np.ndarray) -> dict:
 
 def backward_leg(dev, w, t, x, out, bp, args, alg, with_cpu: bool) -> dict:
     """Times MoeLayer::backward (reference src/moe.rs:348-489) on a second layer in training mode: K forwards
-    that keep the backward pass's state, K backward passes of the last forward (weight gradients accumulate, as
-    Param.grad does), and K forward + backward pairs."""
+    that keep the backward pass's state, K backward passes of the last forward (accumulating, as Param.grad does,
+    and after zero_grads), and K training steps (zero_grads, forward, backward)."""
     if w.act_dtype != "bf16" or w.weight_dtype != "bf16":
         return {"skipped": "the backward pass needs bf16 activations and weights"}
     T = w.tokens
@@ -163,15 +163,18 @@ def backward_leg(dev, w, t, x, out, bp, args, alg, with_cpu: bool) -> dict:
         bwd()
     n = max(5, args.steps // 4)
     ms_f = timed(fwd, n)
-    ms_b = timed(bwd, n)
-    ms_fb = timed(lambda: (fwd(), bwd()), n)
+    ms_b_acc = timed(bwd, n)                                     # every pass adds to the gradients
+    ms_b = timed(lambda: (layer.zero_grads(), bwd()), n)         # as in a training loop: cleared, then written
+    ms_fb = timed(lambda: (layer.zero_grads(), fwd(), bwd()), n)
     # products of the backward pass: twice the forward's (grad_input and weight gradients)
     flops = 2 * alg["gemm_flops"]
-    res = {"ms_forward_training": ms_f, "ms_backward": ms_b, "ms_forward_backward": ms_fb,
+    res = {"ms_forward_training": ms_f, "ms_backward": ms_b, "ms_backward_accumulating": ms_b_acc,
+           "ms_forward_backward": ms_fb,
            "tokens_per_s_forward_backward": T / (ms_fb * 1e-3), "steps": n,
            "backward_product_flops": flops, "backward_tflops": flops / (ms_b * 1e-3) / 1e12,
            "backward_frac_of_peak": flops / (ms_b * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
-           "note": "weight gradients are f32 accumulators: every backward pass reads and writes all of them"}
+           "note": "ms_backward and ms_forward_backward include zero_grads, as a training step does (the expert "
+                   "gradients, f32, are then written once); ms_backward_accumulating adds to them (read and write)"}
     if with_cpu:
         res["cpu_baseline"] = cpu_baseline_backward(t, gh)
     layer.close()

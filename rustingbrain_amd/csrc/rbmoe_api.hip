@@ -154,6 +154,9 @@ struct rbmoe_layer {
     Buf g_router, g_gu, g_down, g_sgu, g_sdown;   // f32 weight gradients, accumulated
     Buf wg_chunks;                        // chunk table of the weight-gradient products
     bool wgrad_generic = false, wgrad_split = true;
+    // The expert gradients count as zero without having been cleared (set by rbmoe_zero_grads): the next
+    // backward pass overwrites them.
+    bool grads_clear = false;
     Buf wdT, wguT, swdT, swguT;           // transposed packed weights: [E][F, d], [E][d, 2F], [Fs, d], [d, 2Fs]
     Buf st_gout, st_gin;
     // staging for the host entry point
@@ -1042,6 +1045,7 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
     L->wgrad_generic = env_int("RBMOE_WGRAD_GENERIC", 0) == 1;
     L->wgrad_split = env_int("RBMOE_DETERMINISTIC", 0) != 1;
     L->training = true;
+    L->grads_clear = true;
     return RBMOE_OK;
 }
 
@@ -1049,8 +1053,11 @@ int rbmoe_zero_grads(rbmoe_layer* L) {
     if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
     rbmoe_ctx* ctx = L->ctx;
     if (!L->training) return fail(ctx, RBMOE_INVALID_CONFIG, "training is not enabled on this layer");
-    for (Buf* b : {&L->g_router, &L->g_gu, &L->g_down, &L->g_sgu, &L->g_sdown})
-        if (b->p) HIP_TRY(ctx, hipMemsetAsync(b->p, 0, b->bytes, ctx->stream));
+    // The expert matrices (hundreds of MB) are not touched: they count as zero from here on, and the next
+    // backward pass writes them instead of adding to them.  The router's gradient is small and is cleared.
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    HIP_TRY(ctx, hipMemsetAsync(L->g_router.p, 0, L->g_router.bytes, ctx->stream));
+    L->grads_clear = true;
     return RBMOE_OK;
 }
 
@@ -1097,7 +1104,11 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
                      int total_rows, float* out, size_t stride) -> hipError_t {
         if (!L->wgrad_generic && abf && !b_rows && weight_grad_shape_ok(M, N))
             return launch_weight_grad(a, M, b, N, counts, offsets, groups, dense_rows, total_rows,
-                                      L->wgrad_split, (int*)L->wg_chunks.p, out, stride, s);
+                                      L->wgrad_split, L->grads_clear, (int*)L->wg_chunks.p, out, stride, s);
+        if (L->grads_clear) {
+            const hipError_t e = hipMemsetAsync(out, 0, (size_t)groups * (stride ? stride : (size_t)M * N) * 4, s);
+            if (e != hipSuccess) return e;
+        }
         return launch_grouped_tn(a, M, b, b_rows, N, counts, offsets, groups, dense_rows, out, stride, abf, s);
     };
     HIP_TRY(ctx, wgrad(L->dy.p, d, L->h.p, nullptr, F, E, -1, S, (float*)L->g_down.p, (size_t)d * F));
@@ -1126,6 +1137,7 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
     CombineArgs ca{L->dxg.p, c.shared_expert ? L->dxs.p : nullptr, L->dxr.p, (const int*)L->inv_pos.p,
                    (const float*)L->ones.p, T, d, k, grad_input};
     HIP_TRY(ctx, launch_combine(ca, abf, s));
+    L->grads_clear = false;
     return RBMOE_OK;
 }
 
@@ -1186,6 +1198,10 @@ int rbmoe_get_weight_grad(rbmoe_layer* L, int32_t which, int32_t expert, float* 
     }
     if ((size_t)rows != want_rows || (size_t)cols != want_cols)
         return fail(ctx, RBMOE_INVALID_INPUT, "gradient shape does not match the weight");
+    if (L->grads_clear && which != RBMOE_W_ROUTER) {  // cleared and not written since
+        std::memset(host, 0, want_rows * want_cols * 4);
+        return RBMOE_OK;
+    }
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
     HIP_TRY(ctx, hipMemcpy(host, src, want_rows * want_cols * 4, hipMemcpyDeviceToHost));
     return RBMOE_OK;

@@ -18,7 +18,9 @@
 // load has two full stages of products to arrive in.  An expert with many more rows than the
 // others is cut into several chunks so that the launch stays balanced; chunks of one expert add
 // into the same matrix with hardware f32 atomics (their order is not fixed; an expert with a
-// single chunk adds in place, in one fixed order).
+// single chunk adds in place, in one fixed order).  When the caller knows that the gradient is
+// zero (first backward pass after it was cleared), a single chunk stores instead of adding, and
+// only the experts that have no chunk or several are cleared beforehand.
 #include "rbmoe_kernels.h"
 
 namespace rbmoe {
@@ -105,7 +107,7 @@ __global__ __launch_bounds__(GT) void weight_grad_kernel(
     const bf16_t* __restrict__ a, int M, const bf16_t* __restrict__ b, int N, int tiles_m, int tiles_n,
     const int* __restrict__ chunk_expert, const int* __restrict__ chunk_row0, const int* __restrict__ chunk_rows,
     const int* __restrict__ chunk_split, const int* __restrict__ nchunks, float* __restrict__ out,
-    size_t out_expert_stride) {
+    size_t out_expert_stride, int overwrite) {
     extern __shared__ __attribute__((aligned(16))) char lds[];  // 2 * GSTAGE
 
     // Workgroup i runs on XCD i % 8.  A unit is one chunk's row of tiles (same m, every n): its
@@ -189,19 +191,23 @@ __global__ __launch_bounds__(GT) void weight_grad_kernel(
         fetch(kc, (s + GDEPTH) * GR);
         const char* const A = lds + buf * GSTAGE;
         const char* const B = A + GR * GAS;
+        // both 16-row steps' fragments are requested before the first product: the second step's reads
+        // are in flight during the first step's products
+        bf16x8 af[GR / 16][2], bf[GR / 16][4];
 #pragma unroll
         for (int ks = 0; ks < GR / 16; ++ks) {
-            bf16x8 af[2], bf[4];
 #pragma unroll
-            for (int i = 0; i < 2; ++i) af[i] = tr_fragment(A + a_lane + ks * 16 * GAS + i * 64, GAS);
+            for (int i = 0; i < 2; ++i) af[ks][i] = tr_fragment(A + a_lane + ks * 16 * GAS + i * 64, GAS);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) bf[j] = tr_fragment(B + b_lane + ks * 16 * GBS + j * 64, GBS);
+            for (int j = 0; j < 4; ++j) bf[ks][j] = tr_fragment(B + b_lane + ks * 16 * GBS + j * 64, GBS);
+        }
+#pragma unroll
+        for (int ks = 0; ks < GR / 16; ++ks)
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
-        }
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks][i], bf[ks][j], acc[i][j], 0, 0, 0);
         stage(std::integral_constant<int, (k + 1) % GDEPTH>{}, buf ^ 1, (s + 1) * GR);
         __syncthreads();
     };
@@ -230,6 +236,10 @@ __global__ __launch_bounds__(GT) void weight_grad_kernel(
 #pragma unroll
                 for (int v = 0; v < 16; ++v)
                     if (mb + 8 * (v >> 2) < M) unsafeAtomicAdd(base + (size_t)(8 * (v >> 2) + (v & 3)) * N, acc[i][j][v]);
+            } else if (overwrite) {  // the gradient is known to be zero: nothing to read
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    if (mb + 8 * (v >> 2) < M) base[(size_t)(8 * (v >> 2) + (v & 3)) * N] = acc[i][j][v];
             } else {
                 float old[16];
 #pragma unroll
@@ -243,6 +253,20 @@ __global__ __launch_bounds__(GT) void weight_grad_kernel(
     }
 }
 
+// Overwrite mode: an expert with exactly one chunk is written in full by that chunk's tiles; every
+// other expert (no rows, or cut into chunks that add atomically) is cleared here first.
+__global__ __launch_bounds__(256) void clear_other_experts_kernel(const int* __restrict__ counts, int dense_rows,
+                                                                  int limit, float* __restrict__ out,
+                                                                  size_t out_expert_stride, size_t elems) {
+    const int e = blockIdx.y;
+    const int rows = dense_rows >= 0 ? dense_rows : counts[e];
+    if (rows > 0 && rows <= limit) return;  // exactly one chunk
+    float4* const o = reinterpret_cast<float4*>(out + (size_t)e * out_expert_stride);
+    const size_t n4 = elems / 4;  // M and N are multiples of 8
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (size_t)gridDim.x * 256)
+        o[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+}
+
 }  // namespace
 
 bool weight_grad_shape_ok(int M, int N) { return M % 8 == 0 && N % 8 == 0 && M >= 8 && N >= 8; }
@@ -251,8 +275,8 @@ bool weight_grad_shape_ok(int M, int N) { return M % 8 == 0 && N % 8 == 0 && M >
 int weight_grad_max_chunks(int groups, int total_rows) { return groups + total_rows / 256 + 1; }
 
 hipError_t launch_weight_grad(const void* a, int M, const void* b, int N, const int* counts, const int* offsets,
-                              int groups, int dense_rows, int total_rows, bool allow_split, int* chunks, float* out,
-                              size_t out_expert_stride, hipStream_t s) {
+                              int groups, int dense_rows, int total_rows, bool allow_split, bool overwrite, int* chunks,
+                              float* out, size_t out_expert_stride, hipStream_t s) {
     if (groups <= 0 || total_rows <= 0) return hipSuccess;
     if (!weight_grad_shape_ok(M, N)) return hipErrorInvalidValue;
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(weight_grad_kernel),
@@ -277,10 +301,13 @@ hipError_t launch_weight_grad(const void* a, int M, const void* b, int N, const 
     int* const nchunks = chunks + 4 * max_chunks;
     hipLaunchKernelGGL(chunk_table_kernel, dim3(1), dim3(256), 0, s, counts, offsets, groups, dense_rows, limit,
                        max_chunks, chunk_expert, chunk_row0, chunk_rows, chunk_split, nchunks);
+    if (overwrite)
+        hipLaunchKernelGGL(clear_other_experts_kernel, dim3(64, groups), dim3(256), 0, s, counts, dense_rows, limit, out,
+                           out_expert_stride, (size_t)M * N);
     const int grid = ((max_chunks * tiles_m + 7) / 8) * 8 * tiles_n;
     hipLaunchKernelGGL(weight_grad_kernel, dim3(grid), dim3(GT), 2 * GSTAGE, s, static_cast<const bf16_t*>(a), M,
                        static_cast<const bf16_t*>(b), N, tiles_m, tiles_n, chunk_expert, chunk_row0, chunk_rows,
-                       chunk_split, nchunks, out, out_expert_stride);
+                       chunk_split, nchunks, out, out_expert_stride, overwrite ? 1 : 0);
     return hipGetLastError();
 }
 

@@ -133,6 +133,45 @@ def test_weight_gradients_accumulate_until_zeroed(device):
     layer.close()
 
 
+def test_cleared_gradients_are_overwritten_not_added_to(device):
+    # zero_grads leaves the expert matrices as they are and marks them clear; the next backward pass must not
+    # see the stale values, also for an expert that then gets no rows and for one that is cut into chunks
+    t = synth.make(small_workload(d=64, E=5, k=2, F=64, T=600, seed=28, act="bf16", wt="bf16", shared=True))
+    layer, ref, gout = check_backward(device, t)               # fills every gradient
+    layer.zero_grads()
+    for which in (L.W_GATE, L.W_UP, L.W_DOWN):
+        assert not layer.weight_grad(which, 2).any()
+    bias = np.zeros(5, np.float32)
+    bias[3] = -1e4                                             # expert 3 gets nothing ...
+    bias[1] = 3.0                                              # ... and expert 1 most rows (cut into chunks)
+    ref_layer = oracle_layer(t)
+    want = ref_layer.backward(t.x, gout, router_bias=bias)
+    layer.forward_train(t.x, router_bias=bias)
+    layer.backward(gout)
+    for which, w in ((L.W_GATE, want.grad_gate), (L.W_UP, want.grad_up), (L.W_DOWN, want.grad_down)):
+        assert not layer.weight_grad(which, 3).any()
+        for e in (0, 1, 2, 4):
+            assert rel_l2(layer.weight_grad(which, e), w[e]) <= TOL, (which, e)
+    assert rel_l2(layer.weight_grad(L.W_SHARED_DOWN), want.grad_shared[2]) <= TOL
+    assert rel_l2(layer.weight_grad(L.W_ROUTER), want.grad_router) <= TOL
+    layer.close()
+
+
+def test_deterministic_mode_gives_identical_bits(device, monkeypatch):
+    # RBMOE_DETERMINISTIC=1: no expert is cut into chunks, so no sum depends on the order of atomics
+    monkeypatch.setenv("RBMOE_DETERMINISTIC", "1")
+    t = synth.make(small_workload(d=64, E=4, k=2, F=128, T=900, seed=29, act="bf16", wt="bf16"))
+    bias = np.array([2.5, 0.0, 0.0, 0.0], np.float32)          # one expert far above its share
+    runs = []
+    for _ in range(2):
+        layer, ref, gout = check_backward(device, t, bias=bias)
+        runs.append([layer.weight_grad(w, e) for w in (L.W_GATE, L.W_UP, L.W_DOWN) for e in range(4)] +
+                    [layer.weight_grad(L.W_ROUTER)])
+        layer.close()
+    for a, b in zip(*runs):
+        assert np.array_equal(a, b)
+
+
 def test_backward_follows_the_most_recent_forward(device):
     t = synth.make(small_workload(d=64, E=4, k=2, F=64, T=120, seed=26, act="bf16", wt="bf16"))
     layer = gpu_layer(device, t, training=True)
