@@ -62,6 +62,10 @@ SHAPES = [
     dict(d=128, E=8, k=3, F=192, T=300, shared=True, shared_d_ff=128),
     dict(d=192, E=16, k=2, F=64, T=1000, shared=True),
     dict(d=64, E=3, k=3, F=64, T=129),
+    dict(d=64, E=24, k=4, F=64, T=333),                                   # 32 lanes per token, two expert batches
+    dict(d=256, E=64, k=6, F=128, T=2048, shared=True, shared_d_ff=256),  # C4's proportions, scaled down
+    dict(d=64, E=70, k=8, F=64, T=77),                                    # more experts than lanes, ragged batches
+    dict(d=320, E=5, k=2, F=192, T=3000),                                 # widths that are not multiples of 256
 ]
 
 
