@@ -131,7 +131,7 @@ __global__ __launch_bounds__(kSmallThreads) void route_small_kernel(
     int* __restrict__ counts, int* __restrict__ offsets, int* __restrict__ tile_expert,
     int* __restrict__ tile_row0, int* __restrict__ tile_rows, int* __restrict__ ntiles,
     float* __restrict__ losses, int* __restrict__ perm_slot, int* __restrict__ perm_token,
-    int* __restrict__ inv_pos) {
+    int* __restrict__ inv_pos, const float* __restrict__ norm_w, float norm_eps, XT* __restrict__ xn_out) {
     __shared__ __align__(16) unsigned char stage[kStageBytes];
     __shared__ float prob[kSmallRouteMaxPairs];
     __shared__ float lsev[kSmallRouteMaxTokens];
@@ -178,6 +178,41 @@ __global__ __launch_bounds__(kSmallThreads) void route_small_kernel(
             }
         }
         __syncthreads();
+        if (norm_w != nullptr) {
+            // RmsNorm::forward (src/norm.rs:41-61) on the staged rows, in place: thread t adds up the squares
+            // of row t in index order (the reference's sequential sum), then the block scales the rows with two
+            // separately rounded products, rounds them to the activation type, and writes them out for the
+            // kernels that follow.  (The launcher passes the norm only when the rows are staged.)
+            float* const inv = lsev;  // free until the token phase
+            constexpr int VN = Vec16<XT>::N;  // d is a multiple of 8 here, rows start on 16-byte boundaries
+            if (tid < T) {
+                const XT* row = xs + (size_t)tid * ds;
+                float sum = 0.0f;
+#pragma unroll 4
+                for (int c = 0; c < d; c += VN) {
+                    float v[VN];
+                    Vec16<XT>::load(row + c, v);
+#pragma unroll
+                    for (int i = 0; i < VN; ++i) sum = __fadd_rn(sum, __fmul_rn(v[i], v[i]));
+                }
+                const float mean_square = __fdiv_rn(sum, (float)d);
+                // correctly rounded root: in double, rounded once (the f32 root instruction is not)
+                inv[tid] = __fdiv_rn(1.0f, (float)sqrt((double)__fadd_rn(mean_square, norm_eps)));
+            }
+            __syncthreads();
+            const int pieces = d / VN;
+            for (int i = tid; i < T * pieces; i += kSmallThreads) {
+                const int t = i / pieces, c = (i - t * pieces) * VN;
+                float v[VN], o[VN];
+                Vec16<XT>::load(xs + (size_t)t * ds + c, v);
+                const float sc = inv[t];
+#pragma unroll
+                for (int q = 0; q < VN; ++q) o[q] = __fmul_rn(__fmul_rn(v[q], sc), norm_w[c + q]);
+                Vec16<XT>::store(xs + (size_t)t * ds + c, o);
+                Vec16<XT>::store(xn_out + (size_t)t * d + c, o);
+            }
+            __syncthreads();
+        }
         const int tasks = T * E * 8;
         for (int base = 0; base < tasks; base += kSmallThreads) {
             const int task = base + tid;
@@ -374,18 +409,29 @@ bool small_route_ok(int T, int E, int k) {
            T * E <= kSmallRouteMaxPairs;
 }
 
+// Whether route_small_kernel copies the router and the token rows into LDS for this call (the condition the
+// kernel itself evaluates); only then can it apply the norm in front of the layer.
+bool small_route_stages_rows(const void* x, const float* wr, int T, int d, int E, bool bf16) {
+    const size_t ds = (size_t)d + 8;
+    return d % 8 == 0 && (size_t)E * ds * 4 + (size_t)T * ds * (bf16 ? 2 : 4) <= (size_t)kStageBytes &&
+           reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(wr) % 16 == 0;
+}
+
 hipError_t launch_route_small(const SmallRouteArgs& a, bool bf16, hipStream_t s) {
     if (!small_route_ok(a.T, a.E, a.k)) return hipErrorInvalidValue;
+    if (a.norm_w && (!a.xn_out || !small_route_stages_rows(a.x, a.wr, a.T, a.d, a.E, bf16))) return hipErrorInvalidValue;
     if (bf16)
         hipLaunchKernelGGL(route_small_kernel<bf16_t>, dim3(1), dim3(kSmallThreads), 0, s,
                            static_cast<const bf16_t*>(a.x), a.wr, a.bias, a.valid, a.T, a.d, a.E, a.k, a.w_aux, a.w_z,
                            a.tile_m, a.P, a.lse, a.expert_of, a.gate_of, a.counts, a.offsets, a.tile_expert,
-                           a.tile_row0, a.tile_rows, a.ntiles, a.losses, a.perm_slot, a.perm_token, a.inv_pos);
+                           a.tile_row0, a.tile_rows, a.ntiles, a.losses, a.perm_slot, a.perm_token, a.inv_pos,
+                           a.norm_w, a.norm_eps, static_cast<bf16_t*>(a.xn_out));
     else
         hipLaunchKernelGGL(route_small_kernel<float>, dim3(1), dim3(kSmallThreads), 0, s,
                            static_cast<const float*>(a.x), a.wr, a.bias, a.valid, a.T, a.d, a.E, a.k, a.w_aux, a.w_z,
                            a.tile_m, a.P, a.lse, a.expert_of, a.gate_of, a.counts, a.offsets, a.tile_expert,
-                           a.tile_row0, a.tile_rows, a.ntiles, a.losses, a.perm_slot, a.perm_token, a.inv_pos);
+                           a.tile_row0, a.tile_rows, a.ntiles, a.losses, a.perm_slot, a.perm_token, a.inv_pos,
+                           a.norm_w, a.norm_eps, static_cast<float*>(a.xn_out));
     return hipGetLastError();
 }
 

@@ -619,8 +619,10 @@ int rbmoe_set_weight(rbmoe_layer* L, int32_t which, int32_t expert, const void* 
 
 namespace {
 
+// `norm_src` (block step): the raw rows; `x` is then the layer's buffer of normed rows, filled here - by the
+// small-route kernel itself for a few tokens, by the norm kernel otherwise - before anything reads it.
 int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* valid, const float* router_bias,
-                 const void* residual, void* out, bool timed) {
+                 const void* residual, void* out, bool timed, const void* norm_src = nullptr) {
     if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
     rbmoe_ctx* ctx = L->ctx;
     const rbmoe_config& c = L->cfg;
@@ -658,12 +660,22 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     // a training layer keeps the gathered rows: the weight gradients of gate and up multiply by them
     const bool gather_in_product = (mfma || f32mc) && !L->explicit_gather && !L->training;
 
+    const bool decode_ok = mfma && L->decode_path && !L->training && small_route_ok(T, E, k) && decode_shape_ok(F, d) &&
+                           decode_shape_ok(d, F) &&
+                           (!c.shared_expert || (decode_shape_ok(Fs, d) && decode_shape_ok(d, Fs)));
+    const bool norm_in_route = norm_src && decode_ok &&
+                               small_route_stages_rows(norm_src, (const float*)L->router.p, T, d, E, abf);
+    if (norm_src && !norm_in_route)
+        HIP_TRY(ctx, launch_rmsnorm(norm_src, (const float*)L->norm_w.p, L->norm_eps, T, d, L->xn.p, abf, s));
+
     // ---- a few tokens: route in one workgroup, then stream the touched weights once -------
-    if (mfma && L->decode_path && !L->training && small_route_ok(T, E, k) && decode_shape_ok(F, d) && decode_shape_ok(d, F) &&
-        (!c.shared_expert || (decode_shape_ok(Fs, d) && decode_shape_ok(d, Fs)))) {
+    if (decode_ok) {
         L->kernel_name = wk == WeightKind::I8 ? "mfma_bf16_decode_int8w" : "mfma_bf16_decode";
         SmallRouteArgs sr{};
         sr.x = x; sr.wr = (const float*)L->router.p; sr.bias = router_bias; sr.valid = valid;
+        if (norm_in_route) {
+            sr.x = norm_src; sr.norm_w = (const float*)L->norm_w.p; sr.norm_eps = L->norm_eps; sr.xn_out = L->xn.p;
+        }
         sr.T = T; sr.d = d; sr.E = E; sr.k = k;
         sr.w_aux = c.aux_loss_weight; sr.w_z = c.router_z_loss_weight;
         sr.tile_m = kDecodeTileM;
@@ -937,9 +949,7 @@ int rbmoe_forward_block(rbmoe_layer* L, const void* x, int32_t T, int32_t cols, 
     if (T < 0 || T > L->max_T) return fail(ctx, RBMOE_INVALID_INPUT, "token count outside [0, max_tokens]");
     if (T > 0 && (!x || !out)) return fail(ctx, RBMOE_NULL_POINTER, "x or out is NULL");
     HIP_TRY(ctx, hipSetDevice(ctx->device));
-    HIP_TRY(ctx, launch_rmsnorm(x, (const float*)L->norm_w.p, L->norm_eps, T, cols, L->xn.p,
-                                L->cfg.act_dtype == RBMOE_BF16, ctx->stream));
-    return forward_impl(L, L->xn.p, T, cols, valid, router_bias, x, out, false);
+    return forward_impl(L, L->xn.p, T, cols, valid, router_bias, x, out, false, x);
 }
 
 int rbmoe_forward_block_host(rbmoe_layer* L, const void* x, int32_t T, int32_t cols, const uint8_t* valid,

@@ -190,7 +190,14 @@ struct SmallRouteArgs {
     int* perm_slot;
     int* perm_token;
     int* inv_pos;
+    // Optional norm in front of the layer (RmsNorm::forward, src/norm.rs:41-61): `x` holds the raw rows, the
+    // kernel normalises them in LDS, routes on the normed rows and writes them to `xn_out` [T, d].  Only for
+    // calls whose rows are staged in LDS (small_route_stages_rows).
+    const float* norm_w = nullptr;
+    float norm_eps = 0.0f;
+    void* xn_out = nullptr;
 };
+bool small_route_stages_rows(const void* x, const float* wr, int T, int d, int E, bool bf16);
 bool small_route_ok(int T, int E, int k);
 hipError_t launch_route_small(const SmallRouteArgs& a, bool bf16, hipStream_t s);
 

@@ -79,6 +79,31 @@ def test_a_few_tokens_take_the_decode_kernels(device):
     layer.close()
 
 
+@pytest.mark.parametrize("T", [1, 2, 8, 32])
+@pytest.mark.parametrize("wt", ["bf16", "int8"])
+def test_decode_steps_normalise_inside_the_routing_kernel(device, T, wt):
+    # TransformerBlock::forward_cached (src/transformer_block.rs:236-250): norm, layer, residual add on the rows
+    # of one decode step.  With one row the reference's Linear takes its eight-lane dot for the router
+    # (src/matrix.rs:131-153), the order the oracle uses for every row count.
+    t = synth.make(small_workload(d=768, E=8, k=2, F=128, T=T, seed=46 + T, act="bf16", wt=wt, shared=True))
+    nw = norm_weight(768, 4)
+    x = synth.round_bf16(t.x * np.float32(5.0))
+    layer = gpu_layer(device, t, max_tokens=32)
+    layer.set_feed_forward_norm(nw, 1e-6)
+    want, normed, ref = oracle_layer(t).forward_block(x, nw, 1e-6, round_normed=synth.round_bf16)
+    out, cache = layer.forward_block(x)
+    assert layer.kernel_name().startswith("mfma_bf16_decode")
+    assert_routing_identical(cache, ref)
+    assert rel_l2(out, want) <= 2e-2
+    # the same call again (the normed rows are rewritten), then a plain forward on the normed rows
+    out2, _ = layer.forward_block(x)
+    assert np.array_equal(out, out2)
+    plain, cache_p = layer.forward_train(normed, residual=x)
+    assert_routing_identical(cache_p, ref)
+    assert np.array_equal(plain, out)
+    layer.close()
+
+
 def test_in_place_and_device_pointers(device):
     from bench import DeviceBuffer
     t = synth.make(small_workload(d=64, E=4, k=2, F=64, T=300, seed=44, act="bf16", wt="bf16"))
