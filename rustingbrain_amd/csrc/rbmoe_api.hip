@@ -1066,7 +1066,8 @@ int rbmoe_zero_grads(rbmoe_layer* L) {
     // The expert matrices (hundreds of MB) are not touched: they count as zero from here on, and the next
     // backward pass writes them instead of adding to them.  The router's gradient is small and is cleared.
     HIP_TRY(ctx, hipSetDevice(ctx->device));
-    HIP_TRY(ctx, hipMemsetAsync(L->g_router.p, 0, L->g_router.bytes, ctx->stream));
+    // (a fill kernel, not a memset: a caller may capture a training step in a graph)
+    HIP_TRY(ctx, launch_fill_f32((float*)L->g_router.p, 0.0f, (long long)(L->g_router.bytes / 4), ctx->stream));
     L->grads_clear = true;
     return RBMOE_OK;
 }
@@ -1116,7 +1117,7 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
             return launch_weight_grad(a, M, b, N, counts, offsets, groups, dense_rows, total_rows,
                                       L->wgrad_split, L->grads_clear, (int*)L->wg_chunks.p, out, stride, s);
         if (L->grads_clear) {
-            const hipError_t e = hipMemsetAsync(out, 0, (size_t)groups * (stride ? stride : (size_t)M * N) * 4, s);
+            const hipError_t e = launch_fill_f32(out, 0.0f, (long long)((size_t)groups * (stride ? stride : (size_t)M * N)), s);
             if (e != hipSuccess) return e;
         }
         return launch_grouped_tn(a, M, b, b_rows, N, counts, offsets, groups, dense_rows, out, stride, abf, s);
