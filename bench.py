@@ -133,8 +133,9 @@ def backward_leg(dev, w, t, x, out, bp, args, alg, with_cpu: bool) -> dict:
     """Times MoeLayer::backward (reference src/moe.rs:348-489) on a second layer in training mode: K forwards
     that keep the backward pass's state, K backward passes of the last forward (accumulating, as Param.grad does,
     and after zero_grads), and K training steps (zero_grads, forward, backward)."""
-    if w.act_dtype != "bf16" or w.weight_dtype != "bf16":
-        return {"skipped": "the backward pass needs bf16 activations and weights"}
+    if (w.act_dtype, w.weight_dtype) not in (("bf16", "bf16"), ("f32", "f32")):
+        return {"skipped": "the backward pass exists for bf16 layers and for all-f32 layers"}
+    bf16 = w.act_dtype == "bf16"
     T = w.tokens
     cfg = rb.MoeConfig(w.num_experts, w.experts_per_token, w.d_ff, w.shared_expert)
     layer = rb.MoeLayer(w.d_model, cfg, dev, act_dtype=w.act_dtype, weight_dtype=w.weight_dtype, max_tokens=T,
@@ -143,7 +144,7 @@ def backward_leg(dev, w, t, x, out, bp, args, alg, with_cpu: bool) -> dict:
     layer.load_tensors(t)
     rng = np.random.default_rng(w.seed + 1000)
     gh = synth.round_bf16(rng.standard_normal(t.x.shape).astype(np.float32))
-    g = DeviceBuffer(dev, x.nbytes).upload(synth.f32_to_bf16_bits(gh))
+    g = DeviceBuffer(dev, x.nbytes).upload(synth.f32_to_bf16_bits(gh) if bf16 else gh)
     gin = DeviceBuffer(dev, x.nbytes)
 
     def fwd():
@@ -174,7 +175,7 @@ def backward_leg(dev, w, t, x, out, bp, args, alg, with_cpu: bool) -> dict:
            "ms_forward_backward": ms_fb,
            "tokens_per_s_forward_backward": T / (ms_fb * 1e-3), "steps": n,
            "backward_product_flops": flops, "backward_tflops": flops / (ms_b * 1e-3) / 1e12,
-           "backward_frac_of_peak": flops / (ms_b * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+           "backward_frac_of_peak": flops / (ms_b * 1e-3) / 1e12 / (PEAK_BF16_TFLOPS if bf16 else PEAK_F32_TFLOPS),
            "note": "ms_backward and ms_forward_backward include zero_grads, as a training step does (the expert "
                    "gradients, f32, are then written once); ms_backward_accumulating adds to them (read and write)"}
     if with_cpu:
@@ -193,7 +194,7 @@ def main() -> int:
     ap.add_argument("--workload", default="c3_prefill_d768_e16", choices=list(synth.WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--backward", action="store_true",
-                    help="also time the backward pass (bf16 activations and weights only)")
+                    help="also time the backward pass (bf16 layers and all-f32 layers)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (the plain copy that FETCH_SIZE / "
                          "WRITE_SIZE readings are scaled by when this command runs under rocprofv3 --pmc)")

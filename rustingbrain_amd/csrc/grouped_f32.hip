@@ -11,7 +11,8 @@
 // the routed rows (gather_rows, src/moe.rs:658-664) never materialises.  The weight fragment
 // is the matrix-core A operand and the token fragment B, so a lane ends with 4 consecutive
 // features of one token (one 16-byte store).  SiLU uses the exact division: this path is held
-// to 1e-5.
+// to 1e-5.  For a backward pass the gate/up launch can also keep the pre-activations (`gu_out`),
+// and a plain launch can apply SwiGLU's backward where it stores its rows (`swiglu_grad_gu`).
 #include "rbmoe_kernels.h"
 
 namespace rbmoe {
@@ -27,7 +28,8 @@ template <bool SWIGLU>
 __global__ __launch_bounds__(256) void grouped_f32_kernel(
     const float* __restrict__ a, const int* __restrict__ row_index, const float* __restrict__ w,
     size_t w_expert_stride, int N, int K, const int* __restrict__ tile_expert, const int* __restrict__ tile_row0,
-    const int* __restrict__ tile_rows, const int* __restrict__ ntiles, int dense_rows, float* __restrict__ out) {
+    const int* __restrict__ tile_rows, const int* __restrict__ ntiles, int dense_rows, float* __restrict__ out,
+    float* __restrict__ gu_out, const float* __restrict__ bw_gu) {
     constexpr int WR = SWIGLU ? 2 * FN : FN;  // weight rows staged per slice
     __shared__ float As[FM * LS];
     __shared__ float Ws[WR * LS];
@@ -140,8 +142,33 @@ __global__ __launch_bounds__(256) void grouped_f32_kernel(
             y.y = silu_f32(acc0[4 * q + 1]) * acc1[4 * q + 1];
             y.z = silu_f32(acc0[4 * q + 2]) * acc1[4 * q + 2];
             y.w = silu_f32(acc0[4 * q + 3]) * acc1[4 * q + 3];
+            if (gu_out != nullptr) {  // uniform: the pre-activations G | U [rows, 2 N] kept for a backward pass
+                float* const grow = gu_out + (size_t)(row0 + tok) * 2 * N + n0 + wx * 32 + f;
+                *reinterpret_cast<float4*>(grow) =
+                    make_float4(acc0[4 * q + 0], acc0[4 * q + 1], acc0[4 * q + 2], acc0[4 * q + 3]);
+                *reinterpret_cast<float4*>(grow + N) =
+                    make_float4(acc1[4 * q + 0], acc1[4 * q + 1], acc1[4 * q + 2], acc1[4 * q + 3]);
+            }
         } else {
             y = make_float4(acc0[4 * q + 0], acc0[4 * q + 1], acc0[4 * q + 2], acc0[4 * q + 3]);
+            if (bw_gu != nullptr) {  // uniform
+                // SwiGlu::backward (src/ffn.rs:87-120) on the way out: the product row is the gradient of the
+                // hidden row; dG = dH * U * silu'(G), dU = dH * silu(G) go to `gu_out`, `out` is not written.
+                const size_t off = (size_t)(row0 + tok) * 2 * N + n0 + wx * 32 + f;
+                const float4 g4 = *reinterpret_cast<const float4*>(bw_gu + off);
+                const float4 u4 = *reinterpret_cast<const float4*>(bw_gu + off + N);
+                const float dh[4] = {y.x, y.y, y.z, y.w}, gv[4] = {g4.x, g4.y, g4.z, g4.w}, uv[4] = {u4.x, u4.y, u4.z, u4.w};
+                float dg[4], du[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float sg = 1.0f / (1.0f + __expf(-gv[i]));
+                    dg[i] = dh[i] * uv[i] * (sg * (1.0f + gv[i] * (1.0f - sg)));  // silu', src/ffn.rs:235-238
+                    du[i] = dh[i] * (gv[i] * sg);
+                }
+                *reinterpret_cast<float4*>(gu_out + off) = make_float4(dg[0], dg[1], dg[2], dg[3]);
+                *reinterpret_cast<float4*>(gu_out + off + N) = make_float4(du[0], du[1], du[2], du[3]);
+                continue;
+            }
         }
         *reinterpret_cast<float4*>(orow + f) = y;
     }
@@ -161,11 +188,13 @@ hipError_t launch_grouped_f32(const GroupedArgs& g, hipStream_t s) {
     if (g.swiglu)
         hipLaunchKernelGGL((grouped_f32_kernel<true>), grid, block, 0, s, static_cast<const float*>(g.a), g.row_index,
                            static_cast<const float*>(g.w), g.w_expert_stride, g.N, g.K, g.tile_expert, g.tile_row0,
-                           g.tile_rows, g.ntiles, g.dense_rows, static_cast<float*>(g.out));
+                           g.tile_rows, g.ntiles, g.dense_rows, static_cast<float*>(g.out), static_cast<float*>(g.gu_out),
+                           static_cast<const float*>(g.swiglu_grad_gu));
     else
         hipLaunchKernelGGL((grouped_f32_kernel<false>), grid, block, 0, s, static_cast<const float*>(g.a), g.row_index,
                            static_cast<const float*>(g.w), g.w_expert_stride, g.N, g.K, g.tile_expert, g.tile_row0,
-                           g.tile_rows, g.ntiles, g.dense_rows, static_cast<float*>(g.out));
+                           g.tile_rows, g.ntiles, g.dense_rows, static_cast<float*>(g.out), static_cast<float*>(g.gu_out),
+                           static_cast<const float*>(g.swiglu_grad_gu));
     return hipGetLastError();
 }
 

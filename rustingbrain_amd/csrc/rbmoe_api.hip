@@ -583,33 +583,52 @@ int rbmoe_set_weight(rbmoe_layer* L, int32_t which, int32_t expert, const void* 
     L->weights_set = true;
     if (L->training && !is_router) {
         // The backward products multiply by the weight itself, not by its transpose (grad_input =
-        // grad_output . W, src/param.rs:822-823): keep a transposed copy in the packed layout.  Gate and up
-        // share one matrix [d, 2F] (gate^T in columns [0, F), up^T in [F, 2F)) so that dX = dG . Wg + dU . Wu is
-        // one product; packed column steps of 16 never straddle the two halves.
-        std::vector<uint16_t> plain(n), tr(n), trp(n);
-        if (dtype == RBMOE_BF16) {
-            std::memcpy(plain.data(), data, n * 2);
-        } else {
-            const float* f = static_cast<const float*>(data);
-            for (size_t i = 0; i < n; ++i) plain[i] = host_f32_to_bf16(f[i]);
-        }
-        for (int r = 0; r < rows; ++r)
-            for (int cc = 0; cc < cols; ++cc) tr[(size_t)cc * rows + r] = plain[(size_t)r * cols + cc];
-        pack_weight_bf16(tr.data(), cols, rows, trp.data());  // [cols, rows] matrix
+        // grad_output . W, src/param.rs:822-823): keep a transposed copy in the layout the product kernels
+        // read.  Gate and up share one matrix [d, 2F] (gate^T in columns [0, F), up^T in [F, 2F)) so that
+        // dX = dG . Wg + dU . Wu is one product.
         const bool shared_w = which >= RBMOE_W_SHARED_GATE;
+        const bool is_down = which == RBMOE_W_DOWN || which == RBMOE_W_SHARED_DOWN;
+        const bool is_up = which == RBMOE_W_UP || which == RBMOE_W_SHARED_UP;
         const int Fw = shared_w ? Fs : F;
-        if (which == RBMOE_W_DOWN || which == RBMOE_W_SHARED_DOWN) {
-            char* tdst = static_cast<char*>(shared_w ? L->swdT.p : L->wdT.p) + (shared_w ? 0 : (size_t)expert * Fw * d * 2);
-            HIP_TRY(ctx, hipMemcpy(tdst, trp.data(), n * 2, hipMemcpyHostToDevice));
+        if (target == RBMOE_F32) {
+            // plain row-major f32, as the f32 product kernel reads its weights
+            const float* f = static_cast<const float*>(src);
+            std::vector<float> tr(n);
+            for (int r = 0; r < rows; ++r)
+                for (int cc = 0; cc < cols; ++cc) tr[(size_t)cc * rows + r] = f[(size_t)r * cols + cc];
+            if (is_down) {
+                float* tdst = static_cast<float*>(shared_w ? L->swdT.p : L->wdT.p) + (shared_w ? 0 : (size_t)expert * Fw * d);
+                HIP_TRY(ctx, hipMemcpy(tdst, tr.data(), n * 4, hipMemcpyHostToDevice));
+            } else {
+                float* base = static_cast<float*>(shared_w ? L->swguT.p : L->wguT.p) +
+                              (shared_w ? 0 : (size_t)expert * d * 2 * Fw) + (is_up ? Fw : 0);
+                HIP_TRY(ctx, hipMemcpy2D(base, (size_t)2 * Fw * 4, tr.data(), (size_t)Fw * 4, (size_t)Fw * 4, (size_t)d,
+                                         hipMemcpyHostToDevice));
+            }
         } else {
-            // [d, Fw] packed as [d/32][Fw/16][512]; destination [d/32][2Fw/16][512]
-            const bool is_up = which == RBMOE_W_UP || which == RBMOE_W_SHARED_UP;
-            char* base = static_cast<char*>(shared_w ? L->swguT.p : L->wguT.p) +
-                         (shared_w ? 0 : (size_t)expert * d * 2 * Fw * 2);
-            const size_t half = (size_t)(Fw / 16) * 512;  // elements per row block and half
-            for (int rb = 0; rb < d / 32; ++rb)
-                HIP_TRY(ctx, hipMemcpy(base + ((size_t)rb * 2 * half + (is_up ? half : 0)) * 2,
-                                       trp.data() + (size_t)rb * half, half * 2, hipMemcpyHostToDevice));
+            // packed bf16; column steps of 16 never straddle the two halves of [d, 2F]
+            std::vector<uint16_t> plain(n), tr(n), trp(n);
+            if (dtype == RBMOE_BF16) {
+                std::memcpy(plain.data(), data, n * 2);
+            } else {
+                const float* f = static_cast<const float*>(data);
+                for (size_t i = 0; i < n; ++i) plain[i] = host_f32_to_bf16(f[i]);
+            }
+            for (int r = 0; r < rows; ++r)
+                for (int cc = 0; cc < cols; ++cc) tr[(size_t)cc * rows + r] = plain[(size_t)r * cols + cc];
+            pack_weight_bf16(tr.data(), cols, rows, trp.data());  // [cols, rows] matrix
+            if (is_down) {
+                char* tdst = static_cast<char*>(shared_w ? L->swdT.p : L->wdT.p) + (shared_w ? 0 : (size_t)expert * Fw * d * 2);
+                HIP_TRY(ctx, hipMemcpy(tdst, trp.data(), n * 2, hipMemcpyHostToDevice));
+            } else {
+                // [d, Fw] packed as [d/32][Fw/16][512]; destination [d/32][2Fw/16][512]
+                char* base = static_cast<char*>(shared_w ? L->swguT.p : L->wguT.p) +
+                             (shared_w ? 0 : (size_t)expert * d * 2 * Fw * 2);
+                const size_t half = (size_t)(Fw / 16) * 512;  // elements per row block and half
+                for (int rb = 0; rb < d / 32; ++rb)
+                    HIP_TRY(ctx, hipMemcpy(base + ((size_t)rb * 2 * half + (is_up ? half : 0)) * 2,
+                                           trp.data() + (size_t)rb * half, half * 2, hipMemcpyHostToDevice));
+            }
         }
     }
     return RBMOE_OK;
@@ -990,17 +1009,23 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
     rbmoe_ctx* ctx = L->ctx;
     if (L->training) return RBMOE_OK;
     const rbmoe_config& c = L->cfg;
-    if (!L->use_stream || c.weight_dtype != RBMOE_BF16)
+    const bool bf16_layer = L->use_stream && c.weight_dtype == RBMOE_BF16;
+    if (!bf16_layer && !L->use_f32_mc)
         return fail(ctx, RBMOE_UNSUPPORTED,
-                    "the backward pass needs bf16 activations and weights with widths that are multiples of 64");
+                    "the backward pass needs a bf16 layer (widths multiples of 64) or an all-f32 layer (multiples of 32)");
     if (L->weights_set)
         return fail(ctx, RBMOE_INVALID_CONFIG, "enable training before the weights are set");
     const size_t E = c.num_experts, d = c.d_model, F = c.d_ff, Fs = L->Fs, T = L->max_T, S = L->max_S;
-    if (!stream_shape_ok((int)d, (int)(2 * F)) || (c.shared_expert && !stream_shape_ok((int)d, (int)(2 * Fs))))
+    if (bf16_layer) {
+        if (!stream_shape_ok((int)d, (int)(2 * F)) || (c.shared_expert && !stream_shape_ok((int)d, (int)(2 * Fs))))
+            return fail(ctx, RBMOE_UNSUPPORTED, "expert width not supported by the backward products");
+        // 32-bit byte offsets into the widest operand of the backward products: [S, 2F] bf16
+        if (std::max(S * 2 * F, T * 2 * Fs) * 2 >= ((size_t)1 << 32))
+            return fail(ctx, RBMOE_UNSUPPORTED, "max_tokens x expert width too large for the backward products");
+    } else if (!f32_shape_ok((int)d, (int)(2 * F)) || (c.shared_expert && !f32_shape_ok((int)d, (int)(2 * Fs)))) {
         return fail(ctx, RBMOE_UNSUPPORTED, "expert width not supported by the backward products");
-    // 32-bit byte offsets into the widest operand of the backward products: [S, 2F] bf16
-    if (std::max(S * 2 * F, T * 2 * Fs) * 2 >= ((size_t)1 << 32))
-        return fail(ctx, RBMOE_UNSUPPORTED, "max_tokens x expert width too large for the backward products");
+    }
+    const size_t ws = bf16_layer ? 2 : 4;  // bytes per element of the transposed weight copies
     const size_t as = dtype_size(c.act_dtype);
     Plan p;
     p.add(&L->xc, T * d * as);
@@ -1016,8 +1041,8 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
     p.add(&L->g_router, E * d * 4);
     p.add(&L->g_gu, E * 2 * F * d * 4);
     p.add(&L->g_down, E * d * F * 4);
-    p.add(&L->wdT, E * F * d * 2);
-    p.add(&L->wguT, E * d * 2 * F * 2);
+    p.add(&L->wdT, E * F * d * ws);
+    p.add(&L->wguT, E * d * 2 * F * ws);
     p.add(&L->wg_chunks, (size_t)(4 * std::max(weight_grad_max_chunks((int)E, (int)S), weight_grad_max_chunks(1, (int)T)) + 1) * 4);
     p.add(&L->st_gout, T * d * as);
     p.add(&L->st_gin, T * d * as);
@@ -1027,8 +1052,8 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
         p.add(&L->dxs, T * d * as);
         p.add(&L->g_sgu, 2 * Fs * d * 4);
         p.add(&L->g_sdown, d * Fs * 4);
-        p.add(&L->swdT, Fs * d * 2);
-        p.add(&L->swguT, d * 2 * Fs * 2);
+        p.add(&L->swdT, Fs * d * ws);
+        p.add(&L->swguT, d * 2 * Fs * ws);
     }
     if (ctx->budget_bytes && ctx->allocated + p.total > ctx->budget_bytes) {
         char buf[200];
@@ -1099,17 +1124,20 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
     g.tile_row0 = (const int*)L->tile_row0.p;
     g.tile_rows = (const int*)L->tile_rows.p;
     g.ntiles = (const int*)L->ntiles.p;
-    g.max_tiles = S / stream_tile_m() + E;
+    g.max_tiles = S / (L->use_stream ? stream_tile_m() : f32_tile_m()) + E;
     g.dense_rows = -1;
     g.swiglu = false;
     g.group_m = L->group_m;
     GroupedArgs gh = g;  // grad_hidden = dY . Wdown
     gh.a = L->dy.p; gh.w = L->wdT.p; gh.w_expert_stride = (size_t)F * d; gh.N = F; gh.K = d;
     gh.swiglu_grad_gu = L->gu.p; gh.gu_out = L->dgu.p;  // the hidden gradient goes straight through SwiGLU's backward
-    HIP_TRY(ctx, launch_grouped_stream(gh, WeightKind::BF16, L->variant, s));
+    auto prod = [&](const GroupedArgs& a) -> hipError_t {
+        return L->use_stream ? launch_grouped_stream(a, WeightKind::BF16, L->variant, s) : launch_grouped_f32(a, s);
+    };
+    HIP_TRY(ctx, prod(gh));
     GroupedArgs gx = g;  // grad_input rows = dG . Wgate + dU . Wup
     gx.a = L->dgu.p; gx.w = L->wguT.p; gx.w_expert_stride = (size_t)d * 2 * F; gx.N = d; gx.K = 2 * F; gx.out = L->dxg.p;
-    HIP_TRY(ctx, launch_grouped_stream(gx, WeightKind::BF16, L->variant, s));
+    HIP_TRY(ctx, prod(gx));
     // weight gradients (src/param.rs:819-821): down += dY^T . H; (gate | up) += (dG | dU)^T . X[token]
     auto wgrad = [&](const void* a, int M, const void* b, const int* b_rows, int N, int groups, int dense_rows,
                      int total_rows, float* out, size_t stride) -> hipError_t {
@@ -1130,11 +1158,11 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
         sh.dense_rows = T;
         sh.a = grad_output; sh.w = L->swdT.p; sh.w_expert_stride = 0; sh.N = Fs; sh.K = d;
         sh.swiglu_grad_gu = L->gus.p; sh.gu_out = L->dgus.p;
-        HIP_TRY(ctx, launch_grouped_stream(sh, WeightKind::BF16, L->variant, s));
+        HIP_TRY(ctx, prod(sh));
         GroupedArgs sx = g;
         sx.dense_rows = T; sx.w_expert_stride = 0;
         sx.a = L->dgus.p; sx.w = L->swguT.p; sx.N = d; sx.K = 2 * Fs; sx.out = L->dxs.p;
-        HIP_TRY(ctx, launch_grouped_stream(sx, WeightKind::BF16, L->variant, s));
+        HIP_TRY(ctx, prod(sx));
         HIP_TRY(ctx, wgrad(grad_output, d, L->hs.p, nullptr, Fs, 1, T, T, (float*)L->g_sdown.p, 0));
         HIP_TRY(ctx, wgrad(L->dgus.p, 2 * Fs, L->xc.p, nullptr, d, 1, T, T, (float*)L->g_sgu.p, 0));
     }

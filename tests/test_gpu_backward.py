@@ -1,7 +1,7 @@
 """GPU parity of the backward pass (MoeLayer::backward, src/moe.rs:348-489) through the C ABI against the CPU
 oracle's backward on the same seeded inputs.  The routing of the forward is bit-identical, so both sides
-differentiate the same selection; every gradient must agree within rel-L2 2e-2 (bf16 activations and weights; the
-oracle computes in f32 from the same bf16-representable values).
+differentiate the same selection; every gradient must agree within rel-L2 2e-2 for bf16 layers (the oracle
+computes in f32 from the same bf16-representable values) and 1e-5 for all-f32 layers.
 """
 import numpy as np
 import pytest
@@ -22,8 +22,10 @@ def grad_output_for(t, seed):
     return synth.round_bf16(rng.standard_normal(t.x.shape).astype(np.float32))
 
 
-def check_backward(device, t, valid=None, bias=None, aux_w=0.01, z_w=1e-3, seed=1, tol=TOL):
+def check_backward(device, t, valid=None, bias=None, aux_w=0.01, z_w=1e-3, seed=1, tol=None):
     w = t.workload
+    if tol is None:
+        tol = 1e-5 if w.act_dtype == "f32" else TOL
     E = w.num_experts
     gout = grad_output_for(t, seed)
     ref_layer = oracle_layer(t, aux_w=aux_w, z_w=z_w)
@@ -73,6 +75,30 @@ SHAPES = [
 def test_backward_matches_the_oracle(device, shape):
     t = synth.make(small_workload(seed=21, act="bf16", wt="bf16", **shape))
     layer, _, _ = check_backward(device, t)
+    layer.close()
+
+
+SHAPES_F32 = [
+    dict(d=32, E=4, k=2, F=32, T=50),
+    dict(d=64, E=8, k=3, F=96, T=300, shared=True, shared_d_ff=64),
+    dict(d=96, E=24, k=2, F=32, T=1000),
+    dict(d=512, E=8, k=2, F=1408, T=1024),          # the f32 configuration of the benchmark set (C1)
+]
+
+
+@pytest.mark.parametrize("shape", SHAPES_F32, ids=lambda s: "d{d}_E{E}_k{k}_F{F}_T{T}".format(**s))
+def test_backward_of_all_f32_layers(device, shape):
+    t = synth.make(small_workload(seed=31, act="f32", wt="f32", **shape))
+    valid = (np.arange(shape["T"]) % 7 != 3).astype(np.uint8) if shape["T"] == 300 else None
+    layer, ref, gout = check_backward(device, t, valid=valid)
+    assert layer.kernel_name() == "mfma_f32"
+    # accumulate, clear, overwrite
+    once = layer.weight_grad(L.W_DOWN, 1)
+    layer.backward(gout)
+    assert rel_l2(layer.weight_grad(L.W_DOWN, 1), 2.0 * once) <= 1e-6
+    layer.zero_grads()
+    layer.backward(gout)
+    assert rel_l2(layer.weight_grad(L.W_DOWN, 1), once) <= 1e-6
     layer.close()
 
 
@@ -206,10 +232,14 @@ def test_training_mode_errors(device):
     with pytest.raises(rb.InvalidConfig):
         late.weight_grad(L.W_ROUTER)
     late.close()
-    f32 = rb.MoeLayer(64, cfg, device, act_dtype="f32", weight_dtype="f32", max_tokens=8)
-    with pytest.raises(rb.Unsupported):
-        f32.enable_training()
-    f32.close()
+    q8 = rb.MoeLayer(64, cfg, device, act_dtype="bf16", weight_dtype="int8", max_tokens=8)
+    with pytest.raises(rb.Unsupported):          # quantized experts have no backward pass (src/ffn.rs:87-93)
+        q8.enable_training()
+    q8.close()
+    odd = rb.MoeLayer(40, rb.MoeConfig(4, 2, 24), device, act_dtype="f32", weight_dtype="f32", max_tokens=8)
+    with pytest.raises(rb.Unsupported):          # widths off the matrix-core kernels
+        odd.enable_training()
+    odd.close()
     fresh = rb.MoeLayer(64, cfg, device, act_dtype="bf16", weight_dtype="bf16", max_tokens=8)
     fresh.enable_training()
     fresh.enable_training()            # idempotent
