@@ -1141,9 +1141,9 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
     // weight gradients (src/param.rs:819-821): down += dY^T . H; (gate | up) += (dG | dU)^T . X[token]
     auto wgrad = [&](const void* a, int M, const void* b, const int* b_rows, int N, int groups, int dense_rows,
                      int total_rows, float* out, size_t stride) -> hipError_t {
-        if (!L->wgrad_generic && abf && !b_rows && weight_grad_shape_ok(M, N))
+        if (!L->wgrad_generic && !b_rows && weight_grad_shape_ok(M, N, abf))
             return launch_weight_grad(a, M, b, N, counts, offsets, groups, dense_rows, total_rows,
-                                      L->wgrad_split, L->grads_clear, (int*)L->wg_chunks.p, out, stride, s);
+                                      L->wgrad_split, L->grads_clear, (int*)L->wg_chunks.p, out, stride, abf, s);
         if (L->grads_clear) {
             const hipError_t e = launch_fill_f32(out, 0.0f, (long long)((size_t)groups * (stride ? stride : (size_t)M * N)), s);
             if (e != hipSuccess) return e;

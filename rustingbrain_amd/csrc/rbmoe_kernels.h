@@ -142,15 +142,15 @@ hipError_t launch_grouped_tn(const void* a, int M, const void* b, const int* b_r
                              const int* offsets, int groups, int dense_rows, float* out, size_t out_expert_stride,
                              bool bf16, hipStream_t s);
 
-// Weight gradients on the bf16 matrix cores: out[e] += A_e^T . B_e with the rows of a group cut into
+// Weight gradients on the matrix cores (bf16 or f32 operands): out[e] += A_e^T . B_e with the rows of a group cut into
 // chunks (`allow_split`: an expert far above the average share is cut into several chunks, which
 // then add with f32 atomics; `overwrite`: out is known to hold zeros, whatever its bytes are, and is
 // written instead of added to).  `chunks` is scratch of 4 * weight_grad_max_chunks(...) + 1 ints.
-bool weight_grad_shape_ok(int M, int N);
+bool weight_grad_shape_ok(int M, int N, bool bf16);
 int weight_grad_max_chunks(int groups, int total_rows);
 hipError_t launch_weight_grad(const void* a, int M, const void* b, int N, const int* counts, const int* offsets,
                               int groups, int dense_rows, int total_rows, bool allow_split, bool overwrite, int* chunks,
-                              float* out, size_t out_expert_stride, hipStream_t s);
+                              float* out, size_t out_expert_stride, bool bf16, hipStream_t s);
 
 // gates -> probabilities -> logits, with the gradients of the two auxiliary losses
 hipError_t launch_route_backward(const float* P, const float* lse, const int* expert_of, const float* grad_gates,

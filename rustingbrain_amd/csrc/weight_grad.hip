@@ -49,6 +49,43 @@ __device__ __forceinline__ bf16x8 tr_fragment(const char* p, int pitch) {
     return u.v;
 }
 
+// A wave's NI x NJ accumulator blocks of 32 x 32 go into the gradient.  Accumulator element v of lane
+// l: m = 8 (v / 4) + 4 (l / 32) + v % 4, n = l % 32 of the block.  The only chunk of an expert owns its
+// elements: it reads the 16 values of a block, adds, and stores (M is a multiple of 4, so a group of 4
+// rows is inside or outside as a whole) - or just stores when the gradient is known to be zero.  The chunks
+// of a cut expert meet on the same elements and add with no-return f32 atomics.
+template <int NI, int NJ>
+__device__ __forceinline__ void add_tiles(const floatx16 (&acc)[NI][NJ], float* __restrict__ o, int M, int N, int mw,
+                                          int nw, int lane, bool split, bool overwrite) {
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        const int mb = mw + i * 32 + 4 * (lane >> 5);
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const int n = nw + j * 32 + (lane & 31);
+            if (n >= N) continue;
+            float* const base = o + (size_t)mb * N + n;
+            if (split) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    if (mb + 8 * (v >> 2) < M) unsafeAtomicAdd(base + (size_t)(8 * (v >> 2) + (v & 3)) * N, acc[i][j][v]);
+            } else if (overwrite) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    if (mb + 8 * (v >> 2) < M) base[(size_t)(8 * (v >> 2) + (v & 3)) * N] = acc[i][j][v];
+            } else {
+                float old[16];
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    if (mb + 8 * (v >> 2) < M) old[v] = base[(size_t)(8 * (v >> 2) + (v & 3)) * N];
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    if (mb + 8 * (v >> 2) < M) base[(size_t)(8 * (v >> 2) + (v & 3)) * N] = old[v] + acc[i][j][v];
+            }
+        }
+    }
+}
+
 // chunk table: expert e with c rows gets ceil(c / limit) chunks of equal size (a multiple of 32)
 __global__ __launch_bounds__(256) void chunk_table_kernel(const int* __restrict__ counts,
                                                           const int* __restrict__ offsets, int groups,
@@ -220,37 +257,118 @@ __global__ __launch_bounds__(GT) void weight_grad_kernel(
         step(I2{}, s + 2);
     }
 
-    // accumulator element v of lane l: m = 8 (v / 4) + 4 (l / 32) + v % 4, n = l % 32 of the block.
-    // The only chunk of an expert owns its elements: it reads the 16 values of a block, adds, and
-    // stores (M is a multiple of 8, so a group of 8 rows is inside or outside as a whole).  The
-    // chunks of a cut expert meet on the same elements and add with no-return f32 atomics.
+    add_tiles<2, 4>(acc, o, M, N, m0 + wm * 64, n0 + wn * 128, lane, split, overwrite != 0);
+}
+
+// ---------------------------------------------------------------------------
+// The same product for all-f32 layers on the f32 matrix cores (v_mfma_f32_32x32x2_f32: one
+// reduction element per lane, so a fragment is read from the row-major LDS tile as it lies,
+// 32 neighbouring columns of two neighbouring rows).  4 waves (2 x 2) own 128 x 128 outputs, a
+// wave 64 x 64; 16 rows per LDS stage, double buffered, loads three stages ahead.  LDS rows are
+// padded to 160 floats: the two rows of a fragment read fall into different halves of the banks.
+// ---------------------------------------------------------------------------
+constexpr int FM = 128, FN = 128, FR = 16, FT = 256;
+constexpr int FP = FM + 32;                 // LDS row pitch in floats (FM == FN)
+constexpr int FSTAGE = FR * 2 * FP;         // floats per stage (A tile, then B tile)
+
+__global__ __launch_bounds__(FT, 2) void weight_grad_f32_kernel(
+    const float* __restrict__ a, int M, const float* __restrict__ b, int N, int tiles_m, int tiles_n,
+    const int* __restrict__ chunk_expert, const int* __restrict__ chunk_row0, const int* __restrict__ chunk_rows,
+    const int* __restrict__ chunk_split, const int* __restrict__ nchunks, float* __restrict__ out,
+    size_t out_expert_stride, int overwrite) {
+    __shared__ __attribute__((aligned(16))) float lds[2 * FSTAGE];  // 40 KB
+
+    const int idx = (int)(blockIdx.x >> 3);
+    const int unit = (int)(blockIdx.x & 7) + 8 * (idx / tiles_n);
+    const int ch = unit / tiles_m;
+    if (ch >= *nchunks) return;
+    const int m0 = (unit - ch * tiles_m) * FM, n0 = (idx % tiles_n) * FN;
+    const int rows = chunk_rows[ch];
+    if (rows <= 0) return;
+    const int row0 = chunk_row0[ch];
+    const bool split = chunk_split[ch] != 0;
+    float* const o = out + (size_t)chunk_expert[ch] * out_expert_stride;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    // each tile: 16 rows x 32 pieces of 4 floats; a thread moves piece tid % 32 of rows tid / 32 and tid / 32 + 8
+    const int pc = tid & 31, tr = tid >> 5;
+    const float* const a_src = a + (size_t)row0 * M + (m0 + 4 * pc < M ? m0 + 4 * pc : 0);
+    const float* const b_src = b + (size_t)row0 * N + (n0 + 4 * pc < N ? n0 + 4 * pc : 0);
+    struct Set {
+        float4 a[2], b[2];
+    } sets[GDEPTH];
+    auto fetch = [&](auto kc, int r0) {
+        constexpr int k = decltype(kc)::value;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int mb = m0 + wm * 64 + i * 32;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int n = n0 + wn * 128 + j * 32 + (lane & 31);
-            if (n >= N) continue;
-            float* const base = o + (size_t)(mb + 4 * (lane >> 5)) * N + n;
-            if (split) {
-#pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    if (mb + 8 * (v >> 2) < M) unsafeAtomicAdd(base + (size_t)(8 * (v >> 2) + (v & 3)) * N, acc[i][j][v]);
-            } else if (overwrite) {  // the gradient is known to be zero: nothing to read
-#pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    if (mb + 8 * (v >> 2) < M) base[(size_t)(8 * (v >> 2) + (v & 3)) * N] = acc[i][j][v];
-            } else {
-                float old[16];
-#pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    if (mb + 8 * (v >> 2) < M) old[v] = base[(size_t)(8 * (v >> 2) + (v & 3)) * N];
-#pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    if (mb + 8 * (v >> 2) < M) base[(size_t)(8 * (v >> 2) + (v & 3)) * N] = old[v] + acc[i][j][v];
-            }
+        for (int i = 0; i < 2; ++i) {
+            const int r = min(r0 + tr + 8 * i, rows - 1);
+            sets[k].a[i] = *reinterpret_cast<const float4*>(a_src + (size_t)r * M);
+            sets[k].b[i] = *reinterpret_cast<const float4*>(b_src + (size_t)r * N);
         }
+    };
+    auto stage = [&](auto kc, int buf, int r0) {
+        constexpr int k = decltype(kc)::value;
+        float* const A = lds + buf * FSTAGE;
+        float* const B = A + FR * FP;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const bool in = r0 + tr + 8 * i < rows;
+            const float4 z = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            *reinterpret_cast<float4*>(A + (tr + 8 * i) * FP + pc * 4) = in ? sets[k].a[i] : z;
+            *reinterpret_cast<float4*>(B + (tr + 8 * i) * FP + pc * 4) = in ? sets[k].b[i] : z;
+        }
+    };
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    const int a_lane = (lane >> 5) * FP + wm * 64 + (lane & 31);
+    const int b_lane = (lane >> 5) * FP + wn * 64 + (lane & 31);
+
+    const int nstages = (rows + FR - 1) / FR;
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    fetch(I0{}, 0);
+    fetch(I1{}, FR);
+    fetch(I2{}, 2 * FR);
+    stage(I0{}, 0, 0);
+    __syncthreads();
+    auto step = [&](auto kc, int s) {
+        constexpr int k = decltype(kc)::value;
+        const int buf = s & 1;
+        fetch(kc, (s + GDEPTH) * FR);
+        const float* const A = lds + buf * FSTAGE;
+        const float* const B = A + FR * FP;
+#pragma unroll
+        for (int kk = 0; kk < FR / 2; ++kk) {
+            float af[2], bf[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) af[i] = A[a_lane + 2 * kk * FP + i * 32];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) bf[j] = B[b_lane + 2 * kk * FP + j * 32];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[j], acc[i][j], 0, 0, 0);
+        }
+        stage(std::integral_constant<int, (k + 1) % GDEPTH>{}, buf ^ 1, (s + 1) * FR);
+        __syncthreads();
+    };
+    for (int s = 0; s < nstages; s += GDEPTH) {
+        step(I0{}, s);
+        step(I1{}, s + 1);
+        step(I2{}, s + 2);
     }
+    add_tiles<2, 2>(acc, o, M, N, m0 + wm * 64, n0 + wn * 64, lane, split, overwrite != 0);
 }
 
 // Overwrite mode: an expert with exactly one chunk is written in full by that chunk's tiles; every
@@ -262,27 +380,33 @@ __global__ __launch_bounds__(256) void clear_other_experts_kernel(const int* __r
     const int rows = dense_rows >= 0 ? dense_rows : counts[e];
     if (rows > 0 && rows <= limit) return;  // exactly one chunk
     float4* const o = reinterpret_cast<float4*>(out + (size_t)e * out_expert_stride);
-    const size_t n4 = elems / 4;  // M and N are multiples of 8
+    const size_t n4 = elems / 4;  // M and N are multiples of 4
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (size_t)gridDim.x * 256)
         o[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 }
 
 }  // namespace
 
-bool weight_grad_shape_ok(int M, int N) { return M % 8 == 0 && N % 8 == 0 && M >= 8 && N >= 8; }
+bool weight_grad_shape_ok(int M, int N, bool bf16) {
+    const int q = bf16 ? 8 : 4;  // 16-byte pieces
+    return M % q == 0 && N % q == 0 && M >= q && N >= q;
+}
 
 // Upper bound of the number of chunks of one launch; `chunks` needs 4 * bound + 1 ints.
 int weight_grad_max_chunks(int groups, int total_rows) { return groups + total_rows / 256 + 1; }
 
 hipError_t launch_weight_grad(const void* a, int M, const void* b, int N, const int* counts, const int* offsets,
                               int groups, int dense_rows, int total_rows, bool allow_split, bool overwrite, int* chunks,
-                              float* out, size_t out_expert_stride, hipStream_t s) {
+                              float* out, size_t out_expert_stride, bool bf16, hipStream_t s) {
     if (groups <= 0 || total_rows <= 0) return hipSuccess;
-    if (!weight_grad_shape_ok(M, N)) return hipErrorInvalidValue;
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(weight_grad_kernel),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 2 * GSTAGE);
-    if (attr != hipSuccess) return attr;
-    const int tiles_m = (M + GM - 1) / GM, tiles_n = (N + GN - 1) / GN;
+    if (!weight_grad_shape_ok(M, N, bf16)) return hipErrorInvalidValue;
+    if (bf16) {
+        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(weight_grad_kernel),
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, 2 * GSTAGE);
+        if (attr != hipSuccess) return attr;
+    }
+    const int tile_m = bf16 ? GM : FM, tile_n = bf16 ? GN : FN;
+    const int tiles_m = (M + tile_m - 1) / tile_m, tiles_n = (N + tile_n - 1) / tile_n;
     const int tiles = tiles_m * tiles_n;
     // Enough (chunk, tile) pairs to fill the chip twice, and no chunk longer than twice the average
     // expert's share: an expert above that is cut into equal pieces (the cut costs atomics, which
@@ -305,9 +429,14 @@ hipError_t launch_weight_grad(const void* a, int M, const void* b, int N, const 
         hipLaunchKernelGGL(clear_other_experts_kernel, dim3(64, groups), dim3(256), 0, s, counts, dense_rows, limit, out,
                            out_expert_stride, (size_t)M * N);
     const int grid = ((max_chunks * tiles_m + 7) / 8) * 8 * tiles_n;
-    hipLaunchKernelGGL(weight_grad_kernel, dim3(grid), dim3(GT), 2 * GSTAGE, s, static_cast<const bf16_t*>(a), M,
-                       static_cast<const bf16_t*>(b), N, tiles_m, tiles_n, chunk_expert, chunk_row0, chunk_rows,
-                       chunk_split, nchunks, out, out_expert_stride, overwrite ? 1 : 0);
+    if (bf16)
+        hipLaunchKernelGGL(weight_grad_kernel, dim3(grid), dim3(GT), 2 * GSTAGE, s, static_cast<const bf16_t*>(a), M,
+                           static_cast<const bf16_t*>(b), N, tiles_m, tiles_n, chunk_expert, chunk_row0, chunk_rows,
+                           chunk_split, nchunks, out, out_expert_stride, overwrite ? 1 : 0);
+    else
+        hipLaunchKernelGGL(weight_grad_f32_kernel, dim3(grid), dim3(FT), 0, s, static_cast<const float*>(a), M,
+                           static_cast<const float*>(b), N, tiles_m, tiles_n, chunk_expert, chunk_row0, chunk_rows,
+                           chunk_split, nchunks, out, out_expert_stride, overwrite ? 1 : 0);
     return hipGetLastError();
 }
 
