@@ -202,6 +202,18 @@ def test_deterministic_mode_gives_identical_bits(device, monkeypatch):
         assert np.array_equal(a, b)
 
 
+def test_plain_f32_weight_gradient_kernel_agrees(device, monkeypatch):
+    # RBMOE_WGRAD_GENERIC=1 swaps the matrix-core weight-gradient kernels for the plain f32 one (A/B switch)
+    monkeypatch.setenv("RBMOE_WGRAD_GENERIC", "1")
+    for act in ("bf16", "f32"):
+        t = synth.make(small_workload(d=64, E=4, k=2, F=64, T=150, seed=32, act=act, wt=act, shared=True))
+        layer, ref, gout = check_backward(device, t)
+        layer.zero_grads()
+        layer.backward(gout)             # cleared, then written through the plain kernel's path
+        assert rel_l2(layer.weight_grad(L.W_UP, 2), ref.grad_up[2]) <= (1e-5 if act == "f32" else TOL)
+        layer.close()
+
+
 def test_backward_follows_the_most_recent_forward(device):
     t = synth.make(small_workload(d=64, E=4, k=2, F=64, T=120, seed=26, act="bf16", wt="bf16"))
     layer = gpu_layer(device, t, training=True)
