@@ -712,6 +712,33 @@ void rbo_rmsnorm_rows(const float* x, int T, int d, const float* weight, float e
     }
 }
 
+// RmsNorm::backward (reference src/norm.rs:63-121): returns dL/dinput and ACCUMULATES the scale gradient into
+// grad_weight (tiles of 32 rows, per-tile partials added in tile order, src/norm.rs:8-14, :111-118).  The inverse
+// rms is recomputed per row.  Pinned by the reference's two finite-difference tests (src/norm.rs:172-216) and a
+// float64 differentiation (tests/test_oracle_norm.py).
+void rbo_rmsnorm_backward(const float* x, const float* grad_output, int T, int d, const float* weight, float eps,
+                          float* grad_input, float* grad_weight) {
+    const int ROWS_PER_TILE = 32;
+    std::vector<float> partial(d);
+    for (int tile0 = 0; tile0 < T; tile0 += ROWS_PER_TILE) {
+        std::fill(partial.begin(), partial.end(), 0.0f);
+        for (int t = tile0; t < std::min(T, tile0 + ROWS_PER_TILE); ++t) {
+            const float* source = x + (size_t)t * d;
+            const float* upstream = grad_output + (size_t)t * d;
+            float sum = 0.0f;
+            for (int c = 0; c < d; ++c) sum = sum + source[c] * source[c];
+            const float inverse_rms = 1.0f / std::sqrt(sum / (float)d + eps);
+            float projection = 0.0f;
+            for (int c = 0; c < d; ++c) projection += upstream[c] * weight[c] * source[c];
+            const float shared = projection * (inverse_rms * inverse_rms * inverse_rms) / (float)d;  // powi(3)
+            for (int c = 0; c < d; ++c)
+                grad_input[(size_t)t * d + c] = upstream[c] * weight[c] * inverse_rms - source[c] * shared;
+            for (int c = 0; c < d; ++c) partial[c] += upstream[c] * source[c] * inverse_rms;
+        }
+        for (int c = 0; c < d; ++c) grad_weight[c] += partial[c];
+    }
+}
+
 int rbo_near_ties(const float* P, int T, int E, int k, int ulps) {
     if (k >= E) return 0;
     int n = 0;

@@ -307,6 +307,22 @@ def rmsnorm(x: np.ndarray, weight: np.ndarray, eps: float) -> np.ndarray:
     return out
 
 
+_lib.rbo_rmsnorm_backward.restype = None
+_lib.rbo_rmsnorm_backward.argtypes = [_f32p, _f32p, C.c_int, C.c_int, _f32p, C.c_float, _f32p, _f32p]
+
+
+def rmsnorm_backward(x: np.ndarray, grad_output: np.ndarray, weight: np.ndarray, eps: float):
+    """RmsNorm::backward (src/norm.rs:63-121): (dL/dinput, dL/dweight); the weight gradient starts from zero."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    grad_output = np.ascontiguousarray(grad_output, dtype=np.float32)
+    weight = np.ascontiguousarray(weight, dtype=np.float32)
+    T, d = x.shape
+    gi = np.zeros_like(x)
+    gw = np.zeros(d, np.float32)
+    _lib.rbo_rmsnorm_backward(_fp(x), _fp(grad_output), T, d, _fp(weight), C.c_float(eps), _fp(gi), _fp(gw))
+    return gi, gw
+
+
 @dataclass
 class BackwardResult:
     """Gradients of MoeLayer::backward (src/moe.rs:348-489); the weight gradients start from zero here."""
@@ -394,6 +410,20 @@ class OracleLayer:
             normed = np.ascontiguousarray(round_normed(normed), dtype=np.float32)
         res = self.forward(normed, valid=valid, router_bias=router_bias, threads=threads)
         return res.out + residual, normed, res
+
+    def backward_block(self, residual: np.ndarray, norm_weight: np.ndarray, eps: float, grad_output: np.ndarray,
+                       valid: Optional[np.ndarray] = None, router_bias: Optional[np.ndarray] = None,
+                       round_normed=None):
+        """The feed-forward half of TransformerBlock::backward (src/transformer_block.rs:257-263):
+        ``grad_projected = moe.backward(cache, grad_output)``, ``grad_residual = feed_forward_norm.backward(residual,
+        grad_projected) + grad_output``.  Returns (grad_residual, grad_norm_weight, BackwardResult of the layer)."""
+        residual = np.ascontiguousarray(residual, dtype=np.float32)
+        normed = rmsnorm(residual, norm_weight, eps)
+        if round_normed is not None:
+            normed = np.ascontiguousarray(round_normed(normed), dtype=np.float32)
+        inner = self.backward(normed, grad_output, valid=valid, router_bias=router_bias)
+        gi, gw = rmsnorm_backward(residual, inner.grad_input, norm_weight, eps)
+        return gi + np.ascontiguousarray(grad_output, dtype=np.float32), gw, inner
 
     def backward(self, x: np.ndarray, grad_output: np.ndarray, valid: Optional[np.ndarray] = None,
                  router_bias: Optional[np.ndarray] = None) -> BackwardResult:

@@ -8,6 +8,8 @@
   reversed summation gives different bits);
 * the block step: output = moe(normed) + residual, checked against the oracle's own layer on the normed rows
   (composition only; the layer itself is pinned elsewhere).
+* RmsNorm::backward (src/norm.rs:63-121): the reference's two finite-difference tests (src/norm.rs:172-216, same
+  inputs, epsilon 1e-3, tolerance 1e-2) and a float64 differentiation of the closed form for both gradients.
 No GPU."""
 import numpy as np
 
@@ -84,3 +86,90 @@ def test_block_step_is_norm_then_layer_then_residual():
     outp, _, resp = layer.forward_block(t.x, w, 1e-6, valid=valid)
     assert np.all(resp.expert_of.reshape(9, 2)[valid == 0] == -1)
     assert np.array_equal(outp, resp.out + t.x)
+
+
+def test_backward_matches_finite_differences():
+    # src/norm.rs:172-196
+    w = np.array([1.5, 0.5, -2.0, 1.0], np.float32)
+    x = np.array([0.3, -1.2, 2.5, 0.1, -0.7, 0.4, 1.1, -1.9], np.float32).reshape(2, 4)
+    gi, _ = orc.rmsnorm_backward(x, np.ones((2, 4), np.float32), w, 1e-6)
+    eps = np.float32(1e-3)
+    for i in range(x.size):
+        hi, lo = x.copy(), x.copy()
+        hi.flat[i] += eps
+        lo.flat[i] -= eps
+        numeric = (orc.rmsnorm(hi, w, 1e-6).sum(dtype=np.float32) - orc.rmsnorm(lo, w, 1e-6).sum(dtype=np.float32)) / (2 * eps)
+        assert abs(gi.flat[i] - numeric) < 1e-2, (i, gi.flat[i], numeric)
+
+
+def test_weight_gradient_matches_finite_differences():
+    # src/norm.rs:198-216
+    x = np.array([0.5, -1.0, 2.0, 1.5, 0.25, -0.5], np.float32).reshape(2, 3)
+    _, gw = orc.rmsnorm_backward(x, np.ones((2, 3), np.float32), np.ones(3, np.float32), 1e-6)
+    eps = np.float32(1e-3)
+    for i in range(3):
+        hi, lo = np.ones(3, np.float32), np.ones(3, np.float32)
+        hi[i] += eps
+        lo[i] -= eps
+        numeric = (orc.rmsnorm(x, hi, 1e-6).sum(dtype=np.float32) - orc.rmsnorm(x, lo, 1e-6).sum(dtype=np.float32)) / (2 * eps)
+        assert abs(gw[i] - numeric) < 1e-2
+
+
+def test_backward_against_float64_differentiation():
+    rng = np.random.default_rng(8)
+    T, d, eps = 70, 48, 1e-5          # three tiles of 32 rows, the last one ragged
+    x = (rng.standard_normal((T, d)) * 2.0).astype(np.float32)
+    w = rng.uniform(-1.5, 1.5, d).astype(np.float32)
+    up = rng.standard_normal((T, d)).astype(np.float32)
+    gi, gw = orc.rmsnorm_backward(x, up, w, eps)
+    x64, w64, u64 = x.astype(np.float64), w.astype(np.float64), up.astype(np.float64)
+
+    def loss(xv, wv):
+        return float((u64 * (xv / np.sqrt((xv * xv).mean(axis=1, keepdims=True) + np.float64(np.float32(eps))) * wv)).sum())
+
+    h = 1e-6
+    for idx in rng.choice(T * d, 60, replace=False):
+        hi, lo = x64.copy(), x64.copy()
+        hi.flat[idx] += h
+        lo.flat[idx] -= h
+        want = (loss(hi, w64) - loss(lo, w64)) / (2 * h)
+        assert abs(gi.flat[idx] - want) <= 2e-5 * max(1.0, abs(want)), (idx, gi.flat[idx], want)
+    for c in range(d):
+        hi, lo = w64.copy(), w64.copy()
+        hi[c] += h
+        lo[c] -= h
+        want = (loss(x64, hi) - loss(x64, lo)) / (2 * h)
+        assert abs(gw[c] - want) <= 2e-5 * max(1.0, abs(want)), (c, gw[c], want)
+    # the weight gradient accumulates
+    gw2 = gw.copy()
+    orc._lib.rbo_rmsnorm_backward(orc._fp(x), orc._fp(up), T, d, orc._fp(w), orc.C.c_float(eps), orc._fp(gi.copy()), orc._fp(gw2))
+    assert np.allclose(gw2, 2 * gw, rtol=1e-6)
+
+
+def test_block_backward_is_layer_then_norm_then_residual():
+    t = synth.make(small_workload(d=16, E=4, k=2, F=12, T=9, seed=33, shared=True))
+    layer = oracle_layer(t, aux_w=0.0, z_w=0.0)   # the objective below has no loss terms
+    rng = np.random.default_rng(7)
+    w = rng.uniform(0.5, 1.5, 16).astype(np.float32)
+    up = rng.standard_normal(t.x.shape).astype(np.float32)
+    g, gw, inner = layer.backward_block(t.x, w, 1e-6, up)
+    normed = orc.rmsnorm(t.x, w, 1e-6)
+    again = layer.backward(normed, up)
+    assert np.array_equal(inner.grad_input, again.grad_input)
+    gi, gw2 = orc.rmsnorm_backward(t.x, again.grad_input, w, 1e-6)
+    assert np.array_equal(g, gi + up) and np.array_equal(gw, gw2)
+    # finite differences of the whole block step in the oracle's own f32 arithmetic (selection held fixed by
+    # bumps far smaller than the gaps between probabilities); objective: a weighted sum of the outputs
+    def objective(xv):
+        out, _, _ = layer.forward_block(xv, w, 1e-6)
+        return float((out.astype(np.float64) * up.astype(np.float64)).sum())
+    base_sel = layer.forward_block(t.x, w, 1e-6)[2].expert_of
+    for idx in rng.choice(t.x.size, 12, replace=False):
+        hi, lo = t.x.copy(), t.x.copy()
+        hi.flat[idx] += np.float32(2e-3)
+        lo.flat[idx] -= np.float32(2e-3)
+        if not (np.array_equal(layer.forward_block(hi, w, 1e-6)[2].expert_of, base_sel) and
+                np.array_equal(layer.forward_block(lo, w, 1e-6)[2].expert_of, base_sel)):
+            continue
+        numeric = (objective(hi) - objective(lo)) / (float(hi.flat[idx]) - float(lo.flat[idx]))
+        assert abs(g.flat[idx] - numeric) < 2e-2 * max(1.0, abs(numeric)), (idx, g.flat[idx], numeric)
