@@ -51,7 +51,8 @@ typedef enum rbmoe_weight {
     RBMOE_W_DOWN = 3,         /* [d, F]  per expert  SwiGlu.down                            */
     RBMOE_W_SHARED_GATE = 4,  /* [Fs, d]             MoeLayer.shared    (src/moe.rs:210)    */
     RBMOE_W_SHARED_UP = 5,    /* [Fs, d]                                                    */
-    RBMOE_W_SHARED_DOWN = 6   /* [d, Fs]                                                    */
+    RBMOE_W_SHARED_DOWN = 6,  /* [d, Fs]                                                    */
+    RBMOE_W_NORM = 7          /* [1, d]  feed_forward_norm.weight: rbmoe_get_weight_grad only  */
 } rbmoe_weight;
 
 /* `MoeConfig` (reference src/moe.rs:25-39) plus what a device layer must know
@@ -210,6 +211,17 @@ int rbmoe_zero_grads(rbmoe_layer* layer);
  * rbmoe_set_weight).  Synchronises. */
 int rbmoe_get_weight_grad(rbmoe_layer* layer, int32_t which, int32_t expert, float* host, int32_t rows,
                           int32_t cols);
+
+/* The feed-forward half of TransformerBlock::backward (src/transformer_block.rs:257-263) after
+ * rbmoe_forward_block, on DEVICE pointers:
+ *   grad_projected = moe.backward(cache, grad_output)
+ *   grad_input     = feed_forward_norm.backward(residual, grad_projected) + grad_output
+ * (RmsNorm::backward, src/norm.rs:63-121).  The norm's scale gradient accumulates like the other weight
+ * gradients and is read with rbmoe_get_weight_grad(layer, RBMOE_W_NORM, 0, host, 1, d_model).  `grad_input`
+ * may be `grad_output` itself.  Needs training mode and a norm (in either order). */
+int rbmoe_backward_block(rbmoe_layer* layer, const void* grad_output, void* grad_input);
+/* Same on HOST pointers; synchronises. */
+int rbmoe_backward_block_host(rbmoe_layer* layer, const void* grad_output, void* grad_input);
 
 /* Per-stage timing of one forward with HIP events on the context's stream.
  * `ms` receives RBMOE_NUM_STAGES durations in milliseconds.  Synchronises.

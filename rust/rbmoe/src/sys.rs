@@ -24,6 +24,7 @@ pub const RBMOE_W_DOWN: i32 = 3;
 pub const RBMOE_W_SHARED_GATE: i32 = 4;
 pub const RBMOE_W_SHARED_UP: i32 = 5;
 pub const RBMOE_W_SHARED_DOWN: i32 = 6;
+pub const RBMOE_W_NORM: i32 = 7;
 
 pub const RBMOE_NUM_STAGES: usize = 8;
 
@@ -89,10 +90,19 @@ extern "C" {
     pub fn rbmoe_get_losses(layer: *mut rbmoe_layer, aux_loss: *mut f32, z_loss: *mut f32) -> c_int;
     pub fn rbmoe_get_routing(layer: *mut rbmoe_layer, routing: *mut rbmoe_routing) -> c_int;
     pub fn rbmoe_get_expert_rows(layer: *mut rbmoe_layer, hidden: *mut f32, expert_out: *mut f32) -> c_int;
+    // the block's steps either side of the layer (src/transformer_block.rs:216-222)
+    pub fn rbmoe_set_feed_forward_norm(layer: *mut rbmoe_layer, weight: *const f32, cols: i32, eps: f32) -> c_int;
+    pub fn rbmoe_forward_block(layer: *mut rbmoe_layer, x: *const c_void, tokens: i32, cols: i32, valid: *const u8,
+                               router_bias: *const f32, out: *mut c_void) -> c_int;
+    pub fn rbmoe_forward_block_host(layer: *mut rbmoe_layer, x: *const c_void, tokens: i32, cols: i32,
+                                    valid: *const u8, router_bias: *const f32, out: *mut c_void) -> c_int;
     // backward pass (MoeLayer::backward, src/moe.rs:348-489)
     pub fn rbmoe_layer_enable_training(layer: *mut rbmoe_layer) -> c_int;
     pub fn rbmoe_backward(layer: *mut rbmoe_layer, grad_output: *const c_void, grad_input: *mut c_void) -> c_int;
     pub fn rbmoe_backward_host(layer: *mut rbmoe_layer, grad_output: *const c_void, grad_input: *mut c_void) -> c_int;
+    pub fn rbmoe_backward_block(layer: *mut rbmoe_layer, grad_output: *const c_void, grad_input: *mut c_void) -> c_int;
+    pub fn rbmoe_backward_block_host(layer: *mut rbmoe_layer, grad_output: *const c_void,
+                                     grad_input: *mut c_void) -> c_int;
     pub fn rbmoe_zero_grads(layer: *mut rbmoe_layer) -> c_int;
     pub fn rbmoe_get_weight_grad(layer: *mut rbmoe_layer, which: i32, expert: i32, host: *mut f32, rows: i32,
                                  cols: i32) -> c_int;

@@ -18,7 +18,7 @@ OK, INVALID_INPUT, INVALID_CONFIG, DEVICE_ERROR, BACKEND_UNAVAILABLE, MEMORY_BUD
 F32, BF16, I8 = 0, 1, 2
 DTYPES = {"f32": F32, "bf16": BF16, "int8": I8}
 # rbmoe_weight
-W_ROUTER, W_GATE, W_UP, W_DOWN, W_SHARED_GATE, W_SHARED_UP, W_SHARED_DOWN = range(7)
+W_ROUTER, W_GATE, W_UP, W_DOWN, W_SHARED_GATE, W_SHARED_UP, W_SHARED_DOWN, W_NORM = range(8)
 NUM_STAGES = 8
 STAGE_NAMES = ("router", "empty", "dispatch", "gate_up", "down", "shared", "combine", "total")
 
@@ -74,6 +74,8 @@ SIGNATURES = {
     "rbmoe_layer_enable_training": (C.c_int, [C.c_void_p]),
     "rbmoe_backward": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
     "rbmoe_backward_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
+    "rbmoe_backward_block": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
+    "rbmoe_backward_block_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
     "rbmoe_zero_grads": (C.c_int, [C.c_void_p]),
     "rbmoe_get_weight_grad": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_float), C.c_int32, C.c_int32]),
     "rbmoe_version": (C.c_char_p, []),

@@ -301,6 +301,82 @@ __global__ __launch_bounds__(256) void router_dx_kernel(const float* __restrict_
         if (t0 + u < T) Vec16<XT>::store(dxr + (size_t)(t0 + u) * d + c, s[u]);
 }
 
+// ---------------------------------------------------------------------------
+// RmsNorm::backward (src/norm.rs:63-121) behind the layer's own backward pass, with the block's residual
+// gradient added on the way out (src/transformer_block.rs:258-263): one wave per row,
+//   inverse_rms = 1 / sqrt(mean(x^2) + eps),  projection = sum_j up_j w_j x_j,
+//   dx_j = up_j w_j inverse_rms - x_j projection inverse_rms^3 / d  (+ residual_grad_j).
+// The inverse rms of every row is kept for the scale gradient, which is summed in the reference's tiles of 32
+// rows: partial[tile][c] = sum over the tile's rows of up * x * inverse_rms, tiles added in order afterwards.
+// ---------------------------------------------------------------------------
+template <typename XT>
+__global__ __launch_bounds__(256) void rmsnorm_backward_kernel(const XT* __restrict__ x, const XT* __restrict__ up,
+                                                               const float* __restrict__ weight, float eps,
+                                                               const XT* residual_grad, int T, int d,
+                                                               XT* grad_input, float* __restrict__ inv_rms) {
+    constexpr int VN = Vec16<XT>::N;
+    const int lane = threadIdx.x & 63;
+    const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= T) return;
+    const XT* xr = x + (size_t)t * d;
+    const XT* ur = up + (size_t)t * d;
+    float sumsq = 0.0f, proj = 0.0f;
+    for (int c = lane * VN; c < d; c += 64 * VN) {
+        float xv[VN], uv[VN];
+        Vec16<XT>::load(xr + c, xv);
+        Vec16<XT>::load(ur + c, uv);
+#pragma unroll
+        for (int i = 0; i < VN; ++i) {
+            sumsq = fmaf(xv[i], xv[i], sumsq);
+            proj = fmaf(uv[i] * weight[c + i], xv[i], proj);
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        sumsq += __shfl_xor(sumsq, o);
+        proj += __shfl_xor(proj, o);
+    }
+    const float inv = 1.0f / sqrtf(sumsq / (float)d + eps);
+    const float shared = proj * (inv * inv * inv) / (float)d;
+    if (lane == 0) inv_rms[t] = inv;
+    for (int c = lane * VN; c < d; c += 64 * VN) {
+        float xv[VN], uv[VN], o[VN];
+        Vec16<XT>::load(xr + c, xv);
+        Vec16<XT>::load(ur + c, uv);
+#pragma unroll
+        for (int i = 0; i < VN; ++i) o[i] = uv[i] * weight[c + i] * inv - xv[i] * shared;
+        if (residual_grad) {  // uniform
+            float rv[VN];
+            Vec16<XT>::load(residual_grad + (size_t)t * d + c, rv);
+#pragma unroll
+            for (int i = 0; i < VN; ++i) o[i] += rv[i];
+        }
+        Vec16<XT>::store(grad_input + (size_t)t * d + c, o);
+    }
+}
+
+constexpr int kNormTileRows = 32;  // ROWS_PER_TILE, src/norm.rs:14
+
+template <typename XT>
+__global__ __launch_bounds__(128) void rmsnorm_wgrad_partial_kernel(const XT* __restrict__ x, const XT* __restrict__ up,
+                                                                    const float* __restrict__ inv_rms, int T, int d,
+                                                                    float* __restrict__ partial) {
+    const int c = (blockIdx.x * 128 + threadIdx.x) * 2;
+    if (c >= d) return;  // d is even
+    const int tile = blockIdx.y;
+    const int t0 = tile * kNormTileRows, t1 = min(T, t0 + kNormTileRows);
+    float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll 4
+    for (int t = t0; t < t1; ++t) {
+        const float2 xp = load_pair(x + (size_t)t * d + c);
+        const float2 upv = load_pair(up + (size_t)t * d + c);
+        const float s = inv_rms[t];
+        a0 += upv.x * xp.x * s;
+        a1 += upv.y * xp.y * s;
+    }
+    *reinterpret_cast<float2*>(partial + (size_t)tile * d + c) = make_float2(a0, a1);
+}
+
 __global__ __launch_bounds__(256) void fill_f32_kernel(float* p, float v, long long n) {
     const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
     if (i < n) p[i] = v;
@@ -387,6 +463,33 @@ hipError_t launch_router_grad(const float* dlogits, const void* x, const float* 
     }
     hipLaunchKernelGGL(router_grad_reduce_kernel, dim3((E * d + 63) / 64), dim3(256), 0, s, partial, chunks, E * d,
                        grad_router);
+    return hipGetLastError();
+}
+
+int rmsnorm_grad_tiles(int T) { return (std::max(T, 1) + kNormTileRows - 1) / kNormTileRows; }
+
+hipError_t launch_rmsnorm_backward(const void* x, const void* up, const float* weight, float eps,
+                                   const void* residual_grad, int T, int d, void* grad_input, float* inv_rms,
+                                   float* partial, float* grad_weight, bool bf16, hipStream_t s) {
+    if (T <= 0) return hipSuccess;
+    if (!backward_width_ok(d, bf16)) return hipErrorInvalidValue;
+    const dim3 g1((T + 3) / 4), b1(256);
+    const int tiles = rmsnorm_grad_tiles(T);
+    const dim3 g2((d / 2 + 127) / 128, tiles), b2(128);
+    if (bf16) {
+        hipLaunchKernelGGL(rmsnorm_backward_kernel<bf16_t>, g1, b1, 0, s, static_cast<const bf16_t*>(x),
+                           static_cast<const bf16_t*>(up), weight, eps, static_cast<const bf16_t*>(residual_grad), T, d,
+                           static_cast<bf16_t*>(grad_input), inv_rms);
+        hipLaunchKernelGGL(rmsnorm_wgrad_partial_kernel<bf16_t>, g2, b2, 0, s, static_cast<const bf16_t*>(x),
+                           static_cast<const bf16_t*>(up), inv_rms, T, d, partial);
+    } else {
+        hipLaunchKernelGGL(rmsnorm_backward_kernel<float>, g1, b1, 0, s, static_cast<const float*>(x),
+                           static_cast<const float*>(up), weight, eps, static_cast<const float*>(residual_grad), T, d,
+                           static_cast<float*>(grad_input), inv_rms);
+        hipLaunchKernelGGL(rmsnorm_wgrad_partial_kernel<float>, g2, b2, 0, s, static_cast<const float*>(x),
+                           static_cast<const float*>(up), inv_rms, T, d, partial);
+    }
+    hipLaunchKernelGGL(router_grad_reduce_kernel, dim3((d + 63) / 64), dim3(256), 0, s, partial, tiles, d, grad_weight);
     return hipGetLastError();
 }
 

@@ -143,6 +143,9 @@ struct rbmoe_layer {
     Buf xn, norm_w;  // [max_T, d] activation dtype, [d] f32
     float norm_eps = 0.0f;
     bool norm_set = false;
+    // training through the block step (allocated once both the norm and training mode are there)
+    Buf xraw, dxn, inv_rms, norm_partial, g_norm;  // [T, d] x2 activation dtype, [T], [T/32][d], [d] f32
+    bool last_was_block = false;
     // training (allocated by rbmoe_layer_enable_training)
     bool training = false;
     bool weights_set = false;
@@ -661,6 +664,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     if (T > 0 && (!x || !out)) return fail(ctx, RBMOE_NULL_POINTER, "x or out is NULL");
     HIP_TRY(ctx, hipSetDevice(ctx->device));
     hipStream_t s = ctx->stream;
+    L->last_was_block = false;  // rbmoe_forward_block sets it once this call has succeeded
     const bool abf = c.act_dtype == RBMOE_BF16;
     const WeightKind wk = c.weight_dtype == RBMOE_F32 ? WeightKind::F32
                           : c.weight_dtype == RBMOE_BF16 ? WeightKind::BF16 : WeightKind::I8;
@@ -856,6 +860,41 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     return RBMOE_OK;
 }
 
+// Buffers of the backward pass through the norm: allocated by whichever of rbmoe_set_feed_forward_norm and
+// rbmoe_layer_enable_training comes second.
+int ensure_block_training_buffers(rbmoe_layer* L) {
+    rbmoe_ctx* ctx = L->ctx;
+    if (!L->training || !L->norm_w.p || L->xraw.p) return RBMOE_OK;
+    const rbmoe_config& c = L->cfg;
+    const size_t T = L->max_T, d = c.d_model, as = dtype_size(c.act_dtype);
+    Plan p;
+    p.add(&L->xraw, T * d * as);
+    p.add(&L->dxn, T * d * as);
+    p.add(&L->inv_rms, T * 4);
+    p.add(&L->norm_partial, (size_t)rmsnorm_grad_tiles((int)T) * d * 4);
+    p.add(&L->g_norm, d * 4);
+    if (ctx->budget_bytes && ctx->allocated + p.total > ctx->budget_bytes) {
+        char buf[200];
+        std::snprintf(buf, sizeof buf, "memory budget exceeded: estimated %zu MiB exceeds budget %zu MiB",
+                      (ctx->allocated + p.total + (1 << 20) - 1) >> 20, ctx->budget_bytes >> 20);
+        return fail(ctx, RBMOE_MEMORY_BUDGET, buf);
+    }
+    for (auto& it : p.items) {
+        void* q = nullptr;
+        if (hipMalloc(&q, it.second) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(ctx, RBMOE_OUT_OF_MEMORY, "out of memory while allocating the norm's backward buffers");
+        }
+        it.first->p = q;
+        it.first->bytes = it.second;
+        ctx->allocated += it.second;
+        L->all.push_back(it.first);
+        HIP_TRY(ctx, hipMemsetAsync(q, 0, it.second, ctx->stream));
+    }
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return RBMOE_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -952,7 +991,7 @@ int rbmoe_set_feed_forward_norm(rbmoe_layer* L, const float* weight, int32_t col
     HIP_TRY(ctx, hipMemcpy(L->norm_w.p, weight, (size_t)c.d_model * 4, hipMemcpyHostToDevice));
     L->norm_eps = eps;
     L->norm_set = true;
-    return RBMOE_OK;
+    return ensure_block_training_buffers(L);
 }
 
 int rbmoe_forward_block(rbmoe_layer* L, const void* x, int32_t T, int32_t cols, const uint8_t* valid,
@@ -968,7 +1007,12 @@ int rbmoe_forward_block(rbmoe_layer* L, const void* x, int32_t T, int32_t cols, 
     if (T < 0 || T > L->max_T) return fail(ctx, RBMOE_INVALID_INPUT, "token count outside [0, max_tokens]");
     if (T > 0 && (!x || !out)) return fail(ctx, RBMOE_NULL_POINTER, "x or out is NULL");
     HIP_TRY(ctx, hipSetDevice(ctx->device));
-    return forward_impl(L, L->xn.p, T, cols, valid, router_bias, x, out, false, x);
+    if (L->training && T > 0)  // TransformerBlockCache keeps the residual (src/transformer_block.rs:224-232)
+        HIP_TRY(ctx, hipMemcpyAsync(L->xraw.p, x, (size_t)T * cols * dtype_size(L->cfg.act_dtype),
+                                    hipMemcpyDeviceToDevice, ctx->stream));
+    const int rc = forward_impl(L, L->xn.p, T, cols, valid, router_bias, x, out, false, x);
+    if (rc == RBMOE_OK) L->last_was_block = true;
+    return rc;
 }
 
 int rbmoe_forward_block_host(rbmoe_layer* L, const void* x, int32_t T, int32_t cols, const uint8_t* valid,
@@ -1081,7 +1125,7 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
     L->wgrad_split = env_int("RBMOE_DETERMINISTIC", 0) != 1;
     L->training = true;
     L->grads_clear = true;
-    return RBMOE_OK;
+    return ensure_block_training_buffers(L);
 }
 
 int rbmoe_zero_grads(rbmoe_layer* L) {
@@ -1093,6 +1137,7 @@ int rbmoe_zero_grads(rbmoe_layer* L) {
     HIP_TRY(ctx, hipSetDevice(ctx->device));
     // (a fill kernel, not a memset: a caller may capture a training step in a graph)
     HIP_TRY(ctx, launch_fill_f32((float*)L->g_router.p, 0.0f, (long long)(L->g_router.bytes / 4), ctx->stream));
+    if (L->g_norm.p) HIP_TRY(ctx, launch_fill_f32((float*)L->g_norm.p, 0.0f, (long long)(L->g_norm.bytes / 4), ctx->stream));
     L->grads_clear = true;
     return RBMOE_OK;
 }
@@ -1198,6 +1243,46 @@ int rbmoe_backward_host(rbmoe_layer* L, const void* grad_output, void* grad_inpu
     return RBMOE_OK;
 }
 
+int rbmoe_backward_block(rbmoe_layer* L, const void* grad_output, void* grad_input) {
+    if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
+    rbmoe_ctx* ctx = L->ctx;
+    if (!L->training) return fail(ctx, RBMOE_INVALID_CONFIG, "training is not enabled on this layer");
+    if (!L->norm_set) return fail(ctx, RBMOE_INVALID_CONFIG, "the feed-forward norm has not been set");
+    if (L->last_T < 0 || !L->last_was_block)
+        return fail(ctx, RBMOE_INVALID_INPUT, "the last forward pass was not rbmoe_forward_block");
+    const int T = L->last_T, d = L->cfg.d_model;
+    if (T == 0) return RBMOE_OK;
+    if (!grad_output || !grad_input) return fail(ctx, RBMOE_NULL_POINTER, "grad_output or grad_input is NULL");
+    // grad_projected = feed_forward.backward(cache, grad_output)  (src/transformer_block.rs:257)
+    const int rc = rbmoe_backward(L, grad_output, L->dxn.p);
+    if (rc != RBMOE_OK) return rc;
+    // grad_residual = feed_forward_norm.backward(residual, grad_projected) + grad_output  (:258-263)
+    HIP_TRY(ctx, launch_rmsnorm_backward(L->xraw.p, L->dxn.p, (const float*)L->norm_w.p, L->norm_eps, grad_output, T, d,
+                                         grad_input, (float*)L->inv_rms.p, (float*)L->norm_partial.p,
+                                         (float*)L->g_norm.p, L->cfg.act_dtype == RBMOE_BF16, ctx->stream));
+    return RBMOE_OK;
+}
+
+int rbmoe_backward_block_host(rbmoe_layer* L, const void* grad_output, void* grad_input) {
+    if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
+    rbmoe_ctx* ctx = L->ctx;
+    if (!L->training) return fail(ctx, RBMOE_INVALID_CONFIG, "training is not enabled on this layer");
+    if (!L->norm_set) return fail(ctx, RBMOE_INVALID_CONFIG, "the feed-forward norm has not been set");
+    if (L->last_T < 0 || !L->last_was_block)
+        return fail(ctx, RBMOE_INVALID_INPUT, "the last forward pass was not rbmoe_forward_block");
+    const int T = L->last_T;
+    if (T == 0) return RBMOE_OK;
+    if (!grad_output || !grad_input) return fail(ctx, RBMOE_NULL_POINTER, "grad_output or grad_input is NULL");
+    const size_t nbytes = (size_t)T * L->cfg.d_model * dtype_size(L->cfg.act_dtype);
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    HIP_TRY(ctx, hipMemcpyAsync(L->st_gout.p, grad_output, nbytes, hipMemcpyHostToDevice, ctx->stream));
+    const int rc = rbmoe_backward_block(L, L->st_gout.p, L->st_gin.p);
+    if (rc != RBMOE_OK) return rc;
+    HIP_TRY(ctx, hipMemcpyAsync(grad_input, L->st_gin.p, nbytes, hipMemcpyDeviceToHost, ctx->stream));
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return RBMOE_OK;
+}
+
 int rbmoe_get_weight_grad(rbmoe_layer* L, int32_t which, int32_t expert, float* host, int32_t rows, int32_t cols) {
     if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
     rbmoe_ctx* ctx = L->ctx;
@@ -1232,12 +1317,17 @@ int rbmoe_get_weight_grad(rbmoe_layer* L, int32_t which, int32_t expert, float* 
             src = (const float*)L->g_sdown.p;
             want_rows = d; want_cols = Fs;
             break;
+        case RBMOE_W_NORM:
+            if (!L->g_norm.p) return fail(ctx, RBMOE_INVALID_CONFIG, "the feed-forward norm has not been set");
+            src = (const float*)L->g_norm.p;
+            want_rows = 1; want_cols = d;
+            break;
         default:
             return fail(ctx, RBMOE_INVALID_CONFIG, "unknown weight id");
     }
     if ((size_t)rows != want_rows || (size_t)cols != want_cols)
         return fail(ctx, RBMOE_INVALID_INPUT, "gradient shape does not match the weight");
-    if (L->grads_clear && which != RBMOE_W_ROUTER) {  // cleared and not written since
+    if (L->grads_clear && which != RBMOE_W_ROUTER && which != RBMOE_W_NORM) {  // cleared and not written since
         std::memset(host, 0, want_rows * want_cols * 4);
         return RBMOE_OK;
     }

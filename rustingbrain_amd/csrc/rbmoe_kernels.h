@@ -161,6 +161,12 @@ hipError_t launch_route_backward(const float* P, const float* lse, const int* ex
 int router_grad_chunks(int max_tokens);
 hipError_t launch_router_grad(const float* dlogits, const void* x, const float* wr, int T, int d, int E,
                               float* partial, float* grad_router, void* dxr, bool bf16, hipStream_t s);
+// RmsNorm::backward (src/norm.rs:63-121): grad_input = d(norm)/dx applied to `up` (+ residual_grad when given),
+// grad_weight += scale gradient (through `partial`, rmsnorm_grad_tiles(max_tokens) * d floats); `inv_rms` [T] scratch
+int rmsnorm_grad_tiles(int max_tokens);
+hipError_t launch_rmsnorm_backward(const void* x, const void* up, const float* weight, float eps,
+                                   const void* residual_grad, int T, int d, void* grad_input, float* inv_rms,
+                                   float* partial, float* grad_weight, bool bf16, hipStream_t s);
 hipError_t launch_fill_f32(float* p, float v, long long n, hipStream_t s);
 
 // ---- decode-shaped path (a few tokens) -------------------------------------------

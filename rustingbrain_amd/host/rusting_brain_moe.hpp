@@ -266,6 +266,47 @@ class MoeLayer {
         return grad_input;
     }
 
+    // ---- the block's steps either side of the layer (src/transformer_block.rs:216-222, :257-263)
+    void set_feed_forward_norm(const std::vector<float>& weight, float eps) {
+        check(rbmoe_set_feed_forward_norm(layer_, weight.data(), (int32_t)weight.size(), eps), device_->raw());
+    }
+
+    // input + forward(feed_forward_norm(input)); f32 boundary only (as forward_train's bf16 conversion is not repeated here)
+    Matrix forward_block(const Matrix& residual) {
+        if (residual.cols != d_model_)
+            throw InvalidInput("input length " + std::to_string(residual.cols) + " does not match expected length " +
+                                   std::to_string(d_model_),
+                               d_model_, residual.cols);
+        Matrix out(residual.rows, d_model_);
+        if (act_ == RBMOE_F32) {
+            check(rbmoe_forward_block_host(layer_, residual.data.data(), (int32_t)residual.rows, (int32_t)residual.cols,
+                                           nullptr, nullptr, out.data.data()),
+                  device_->raw());
+        } else {
+            std::vector<uint16_t> xin(residual.data.size()), xout(residual.data.size());
+            for (size_t i = 0; i < xin.size(); ++i) xin[i] = to_bf16(residual.data[i]);
+            check(rbmoe_forward_block_host(layer_, xin.data(), (int32_t)residual.rows, (int32_t)residual.cols, nullptr,
+                                           nullptr, xout.data()),
+                  device_->raw());
+            for (size_t i = 0; i < xout.size(); ++i) out.data[i] = from_bf16(xout[i]);
+        }
+        return out;
+    }
+
+    // gradient of forward_block's input: through the layer, the norm and the residual
+    Matrix backward_block(const Matrix& grad_output) {
+        Matrix grad_input(grad_output.rows, d_model_);
+        if (act_ == RBMOE_F32) {
+            check(rbmoe_backward_block_host(layer_, grad_output.data.data(), grad_input.data.data()), device_->raw());
+        } else {
+            std::vector<uint16_t> gin(grad_output.data.size()), gout(grad_output.data.size());
+            for (size_t i = 0; i < gin.size(); ++i) gin[i] = to_bf16(grad_output.data[i]);
+            check(rbmoe_backward_block_host(layer_, gin.data(), gout.data()), device_->raw());
+            for (size_t i = 0; i < gout.size(); ++i) grad_input.data[i] = from_bf16(gout[i]);
+        }
+        return grad_input;
+    }
+
     // Param::zero_grad over the layer's parameters (src/param.rs)
     void zero_grads() { check(rbmoe_zero_grads(layer_), device_->raw()); }
 
@@ -279,6 +320,7 @@ class MoeLayer {
             case RBMOE_W_DOWN: rows = d_model_; cols = F; break;
             case RBMOE_W_SHARED_GATE: case RBMOE_W_SHARED_UP: rows = Fs; cols = d_model_; break;
             case RBMOE_W_SHARED_DOWN: rows = d_model_; cols = Fs; break;
+            case RBMOE_W_NORM: rows = 1; cols = d_model_; break;
             default: throw InvalidConfig("unknown weight id");
         }
         Matrix g(rows, cols);

@@ -458,6 +458,26 @@ class MoeLayer:
             out = bf16_bits_to_f32(out).reshape(g.shape)
         return out
 
+    def backward_block(self, grad_output: np.ndarray) -> np.ndarray:
+        """Gradient of the last ``forward_block``'s input: through the layer, the norm and the residual
+        (reference TransformerBlock::backward, src/transformer_block.rs:257-263)."""
+        grad_output = np.asarray(grad_output)
+        if grad_output.ndim != 2 or grad_output.shape[1] != self._d_model:
+            raise InvalidInput(f"grad_output must be [tokens, {self._d_model}]", expected=self._d_model,
+                               actual=grad_output.shape[-1] if grad_output.ndim else 0)
+        g = self._to_act(grad_output)
+        out = np.empty_like(g)
+        _check(self._lib.rbmoe_backward_block_host(self.handle, g.ctypes.data_as(C.c_void_p),
+                                                   out.ctypes.data_as(C.c_void_p)), self.device.handle)
+        if self.act_dtype == "bf16":
+            out = bf16_bits_to_f32(out).reshape(g.shape)
+        return out
+
+    def backward_block_device(self, grad_output_ptr: int, grad_input_ptr: int) -> None:
+        """Enqueue the block step's backward pass on device pointers (no synchronisation)."""
+        _check(self._lib.rbmoe_backward_block(self.handle, C.c_void_p(grad_output_ptr), C.c_void_p(grad_input_ptr)),
+               self.device.handle)
+
     def backward_device(self, grad_output_ptr: int, grad_input_ptr: int) -> None:
         """Enqueue the backward pass on device pointers (no synchronisation)."""
         _check(self._lib.rbmoe_backward(self.handle, C.c_void_p(grad_output_ptr), C.c_void_p(grad_input_ptr)),
@@ -470,7 +490,7 @@ class MoeLayer:
         """Accumulated gradient (f32) of one weight matrix: ``which`` is one of ``_lib.W_*``."""
         F, d, Fs = self.config.d_ff, self._d_model, self.shared_d_ff
         shape = {L.W_ROUTER: (self.config.num_experts, d), L.W_GATE: (F, d), L.W_UP: (F, d), L.W_DOWN: (d, F),
-                 L.W_SHARED_GATE: (Fs, d), L.W_SHARED_UP: (Fs, d), L.W_SHARED_DOWN: (d, Fs)}[which]
+                 L.W_SHARED_GATE: (Fs, d), L.W_SHARED_UP: (Fs, d), L.W_SHARED_DOWN: (d, Fs), L.W_NORM: (1, d)}[which]
         g = np.zeros(shape, np.float32)
         _check(self._lib.rbmoe_get_weight_grad(self.handle, which, expert, g.ctypes.data_as(C.POINTER(C.c_float)),
                                                shape[0], shape[1]), self.device.handle)

@@ -9,6 +9,7 @@ import pytest
 import rustingbrain_amd as rb
 from conftest import rel_l2
 from helpers import assert_routing_identical, gpu_layer, oracle_layer, small_workload, tolerance
+from rustingbrain_amd import _lib as L
 from rustingbrain_amd import synth
 
 pytestmark = pytest.mark.gpu
@@ -153,4 +154,78 @@ def test_c3_block_step_at_full_size(device):
     assert rel_l2(out, want) <= 2e-2
     share = float(np.linalg.norm(want - x))
     assert rel_l2(out - x, want - x) <= 4e-2 + 2.0 ** -8 * float(np.linalg.norm(want)) / share
+    layer.close()
+
+
+# ------------------------------------------------------------------ backward through the block step
+def check_block_backward(device, t, valid=None, bias=None, seed=5, norm_first=True):
+    w = t.workload
+    bf16 = w.act_dtype == "bf16"
+    tol = 2e-2 if bf16 else 1e-5
+    nw = norm_weight(w.d_model, seed)
+    rng = np.random.default_rng(seed + 1)
+    gout = synth.round_bf16(rng.standard_normal(t.x.shape).astype(np.float32))
+    rounder = synth.round_bf16 if bf16 else None
+    ref_layer = oracle_layer(t)
+    want_out, _, ref_f = ref_layer.forward_block(t.x, nw, 1e-6, valid=valid, router_bias=bias, round_normed=rounder)
+    want_g, want_gw, inner = ref_layer.backward_block(t.x, nw, 1e-6, gout, valid=valid, router_bias=bias,
+                                                      round_normed=rounder)
+    cfg = rb.MoeConfig(w.num_experts, w.experts_per_token, w.d_ff, w.shared_expert)
+    layer = rb.MoeLayer(w.d_model, cfg, device, act_dtype=w.act_dtype, weight_dtype=w.weight_dtype,
+                        max_tokens=t.x.shape[0], shared_d_ff=w.shared_d_ff if w.shared_expert else 0)
+    if norm_first:                       # the two set-up calls in either order
+        layer.set_feed_forward_norm(nw, 1e-6)
+        layer.enable_training()
+    else:
+        layer.enable_training()
+        layer.set_feed_forward_norm(nw, 1e-6)
+    layer.load_tensors(t)
+    layout = rb.Layout(valid=None if valid is None else [bool(v) for v in valid])
+    out, cache = layer.forward_block(t.x, layout, router_bias=bias)
+    assert_routing_identical(cache, ref_f)
+    assert rel_l2(out, want_out) <= tol
+    g = layer.backward_block(gout)
+    assert rel_l2(g, want_g) <= tol
+    # the branch's share alone (the residual passes grad_output through, which dominates the sum)
+    share = float(np.linalg.norm(want_g - gout))
+    rounding = 2.0 ** -8 * float(np.linalg.norm(want_g)) / max(share, 1e-30) if bf16 else 0.0
+    assert rel_l2(g - gout, want_g - gout) <= 2 * tol + rounding
+    assert rel_l2(layer.weight_grad(L.W_NORM).reshape(-1), want_gw) <= tol
+    assert rel_l2(layer.weight_grad(L.W_ROUTER), inner.grad_router) <= tol
+    assert rel_l2(layer.weight_grad(L.W_DOWN, 0), inner.grad_down[0]) <= tol
+    return layer, gout, want_gw
+
+
+@pytest.mark.parametrize("act", ["bf16", "f32"])
+@pytest.mark.parametrize("shape", [dict(d=64, E=4, k=2, F=64, T=70), dict(d=128, E=8, k=2, F=64, T=300, shared=True)],
+                         ids=lambda s: "d{d}_E{E}_T{T}".format(**s))
+def test_block_backward_matches_the_oracle(device, act, shape):
+    t = synth.make(small_workload(seed=51, act=act, wt=act, **shape))
+    layer, _, _ = check_block_backward(device, t, norm_first=shape["T"] == 70)
+    layer.close()
+
+
+def test_block_backward_with_padding_accumulation_and_errors(device):
+    t = synth.make(small_workload(d=64, E=6, k=2, F=64, T=100, seed=52, act="bf16", wt="bf16", shared=True))
+    valid = (np.arange(100) % 6 != 1).astype(np.uint8)
+    bias = np.linspace(-0.4, 0.4, 6).astype(np.float32)
+    layer, gout, want_gw = check_block_backward(device, t, valid=valid, bias=bias)
+    layer.backward_block(gout)                              # the norm's scale gradient accumulates ...
+    assert rel_l2(layer.weight_grad(L.W_NORM).reshape(-1), 2.0 * want_gw) <= 2e-2
+    layer.zero_grads()                                      # ... until cleared
+    assert not layer.weight_grad(L.W_NORM).any()
+    layer.forward_train(synth.round_bf16(t.x))              # a plain forward is not a block step
+    with pytest.raises(rb.InvalidInput):
+        layer.backward_block(gout)
+    layer.close()
+    plain = gpu_layer(device, t, training=True)             # no norm set
+    plain.forward_train(t.x)
+    with pytest.raises(rb.InvalidConfig):
+        plain.backward_block(gout)
+    plain.close()
+
+
+def test_c3_block_training_step_at_full_size(device):
+    t = synth.make(synth.WORKLOADS["c3_prefill_d768_e16"])
+    layer, _, _ = check_block_backward(device, t, bias=t.router_bias)
     layer.close()
