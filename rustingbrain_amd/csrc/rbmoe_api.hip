@@ -78,6 +78,10 @@ struct rbmoe_ctx {
     int device = 0;
     hipStream_t own_stream = nullptr;
     hipStream_t stream = nullptr;
+    // The backward pass runs the router's branch beside the weight gradients: a second stream (default
+    // priority, like the first) forked from and joined to `stream` with two events.  Created on first use.
+    hipStream_t side_stream = nullptr;
+    hipEvent_t ev_fork = nullptr, ev_join = nullptr;
     size_t budget_bytes = 0;
     size_t allocated = 0;
     std::string last_error;
@@ -156,7 +160,7 @@ struct rbmoe_layer {
     Buf grad_gates, ones, dlogits, dxr, rpartial;
     Buf g_router, g_gu, g_down, g_sgu, g_sdown;   // f32 weight gradients, accumulated
     Buf wg_chunks;                        // chunk table of the weight-gradient products
-    bool wgrad_generic = false, wgrad_split = true;
+    bool wgrad_generic = false, wgrad_split = true, side_branch = true;
     // The expert gradients count as zero without having been cleared (set by rbmoe_zero_grads): the next
     // backward pass overwrites them.
     bool grads_clear = false;
@@ -336,6 +340,12 @@ int rbmoe_ctx_create(int32_t device, size_t budget_mib, rbmoe_ctx** out) {
 
 static void ctx_release(rbmoe_ctx* ctx) {
     if (!ctx || --ctx->refs > 0) return;
+    if (ctx->side_stream) {
+        (void)hipStreamSynchronize(ctx->side_stream);
+        (void)hipStreamDestroy(ctx->side_stream);
+    }
+    if (ctx->ev_fork) (void)hipEventDestroy(ctx->ev_fork);
+    if (ctx->ev_join) (void)hipEventDestroy(ctx->ev_join);
     if (ctx->own_stream) {
         (void)hipStreamSynchronize(ctx->own_stream);
         (void)hipStreamDestroy(ctx->own_stream);
@@ -1123,6 +1133,12 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
     L->wgrad_generic = env_int("RBMOE_WGRAD_GENERIC", 0) == 1;
     L->wgrad_split = env_int("RBMOE_DETERMINISTIC", 0) != 1;
+    L->side_branch = env_int("RBMOE_NO_SIDE_STREAM", 0) != 1;
+    if (L->side_branch && !ctx->side_stream) {
+        HIP_TRY(ctx, hipStreamCreateWithFlags(&ctx->side_stream, hipStreamNonBlocking));
+        HIP_TRY(ctx, hipEventCreateWithFlags(&ctx->ev_fork, hipEventDisableTiming));
+        HIP_TRY(ctx, hipEventCreateWithFlags(&ctx->ev_join, hipEventDisableTiming));
+    }
     L->training = true;
     L->grads_clear = true;
     return ensure_block_training_buffers(L);
@@ -1163,6 +1179,22 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
     HIP_TRY(ctx, launch_scale_rows(grad_output, L->y.p, (const int*)L->perm_slot.p, (const int*)L->perm_token.p,
                                    (const float*)L->gate_of.p, offsets, E, d, S, L->dy.p, (float*)L->grad_gates.p, abf,
                                    s));
+    // The router's branch needs nothing but the gate gradients from here on and is a handful of small launches
+    // that leave most of the chip idle: it runs on the side stream, beside the products below, and meets
+    // them again at the final sum.  Gates -> probabilities -> logits with the two auxiliary losses
+    // (src/moe.rs:421-478), then the router's weight and input gradients.
+    const bool side = L->side_branch && ctx->side_stream != nullptr;
+    const hipStream_t rs = side ? ctx->side_stream : s;
+    if (side) {
+        HIP_TRY(ctx, hipEventRecord(ctx->ev_fork, s));
+        HIP_TRY(ctx, hipStreamWaitEvent(rs, ctx->ev_fork, 0));
+    }
+    HIP_TRY(ctx, launch_route_backward((const float*)L->P.p, (const float*)L->lse.p, (const int*)L->expert_of.p,
+                                       (const float*)L->grad_gates.p, counts, offsets, T, E, k, c.aux_loss_weight,
+                                       c.router_z_loss_weight, (float*)L->dlogits.p, rs));
+    HIP_TRY(ctx, launch_router_grad((const float*)L->dlogits.p, L->xc.p, (const float*)L->router.p, T, d, E,
+                                    (float*)L->rpartial.p, (float*)L->g_router.p, L->dxr.p, abf, rs));
+    if (side) HIP_TRY(ctx, hipEventRecord(ctx->ev_join, rs));
     // SwiGlu::backward over the routed rows (src/ffn.rs:87-120)
     GroupedArgs g{};
     g.tile_expert = (const int*)L->tile_expert.p;
@@ -1211,13 +1243,8 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
         HIP_TRY(ctx, wgrad(grad_output, d, L->hs.p, nullptr, Fs, 1, T, T, (float*)L->g_sdown.p, 0));
         HIP_TRY(ctx, wgrad(L->dgus.p, 2 * Fs, L->xc.p, nullptr, d, 1, T, T, (float*)L->g_sgu.p, 0));
     }
-    // gates -> probabilities -> logits, with the two auxiliary losses (src/moe.rs:421-478), then the router
-    HIP_TRY(ctx, launch_route_backward((const float*)L->P.p, (const float*)L->lse.p, (const int*)L->expert_of.p,
-                                       (const float*)L->grad_gates.p, counts, offsets, T, E, k, c.aux_loss_weight,
-                                       c.router_z_loss_weight, (float*)L->dlogits.p, s));
-    HIP_TRY(ctx, launch_router_grad((const float*)L->dlogits.p, L->xc.p, (const float*)L->router.p, T, d, E,
-                                    (float*)L->rpartial.p, (float*)L->g_router.p, L->dxr.p, abf, s));
     // grad_input = sum over a token's slots of its expert rows + shared + router
+    if (side) HIP_TRY(ctx, hipStreamWaitEvent(s, ctx->ev_join, 0));
     CombineArgs ca{L->dxg.p, c.shared_expert ? L->dxs.p : nullptr, L->dxr.p, (const int*)L->inv_pos.p,
                    (const float*)L->ones.p, T, d, k, grad_input};
     HIP_TRY(ctx, launch_combine(ca, abf, s));
