@@ -81,7 +81,7 @@ struct rbmoe_ctx {
     // The backward pass runs the router's branch beside the weight gradients: a second stream (default
     // priority, like the first) forked from and joined to `stream` with two events.  Created on first use.
     hipStream_t side_stream = nullptr;
-    hipEvent_t ev_fork = nullptr, ev_join = nullptr;
+    hipEvent_t ev_fork = nullptr, ev_fork2 = nullptr, ev_join = nullptr;
     size_t budget_bytes = 0;
     size_t allocated = 0;
     std::string last_error;
@@ -345,6 +345,7 @@ static void ctx_release(rbmoe_ctx* ctx) {
         (void)hipStreamDestroy(ctx->side_stream);
     }
     if (ctx->ev_fork) (void)hipEventDestroy(ctx->ev_fork);
+    if (ctx->ev_fork2) (void)hipEventDestroy(ctx->ev_fork2);
     if (ctx->ev_join) (void)hipEventDestroy(ctx->ev_join);
     if (ctx->own_stream) {
         (void)hipStreamSynchronize(ctx->own_stream);
@@ -1137,6 +1138,7 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
     if (L->side_branch && !ctx->side_stream) {
         HIP_TRY(ctx, hipStreamCreateWithFlags(&ctx->side_stream, hipStreamNonBlocking));
         HIP_TRY(ctx, hipEventCreateWithFlags(&ctx->ev_fork, hipEventDisableTiming));
+        HIP_TRY(ctx, hipEventCreateWithFlags(&ctx->ev_fork2, hipEventDisableTiming));
         HIP_TRY(ctx, hipEventCreateWithFlags(&ctx->ev_join, hipEventDisableTiming));
     }
     L->training = true;
@@ -1180,8 +1182,8 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
                                    (const float*)L->gate_of.p, offsets, E, d, S, L->dy.p, (float*)L->grad_gates.p, abf,
                                    s));
     // The router's branch needs nothing but the gate gradients from here on and is a handful of small launches
-    // that leave most of the chip idle: it runs on the side stream, beside the products below, and meets
-    // them again at the final sum.  Gates -> probabilities -> logits with the two auxiliary losses
+    // that leave most of the chip idle: it runs on the side stream, beside the products below, which meet
+    // again at the final sum.  Gates -> probabilities -> logits with the two auxiliary losses
     // (src/moe.rs:421-478), then the router's weight and input gradients.
     const bool side = L->side_branch && ctx->side_stream != nullptr;
     const hipStream_t rs = side ? ctx->side_stream : s;
@@ -1194,7 +1196,7 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
                                        c.router_z_loss_weight, (float*)L->dlogits.p, rs));
     HIP_TRY(ctx, launch_router_grad((const float*)L->dlogits.p, L->xc.p, (const float*)L->router.p, T, d, E,
                                     (float*)L->rpartial.p, (float*)L->g_router.p, L->dxr.p, abf, rs));
-    if (side) HIP_TRY(ctx, hipEventRecord(ctx->ev_join, rs));
+
     // SwiGlu::backward over the routed rows (src/ffn.rs:87-120)
     GroupedArgs g{};
     g.tile_expert = (const int*)L->tile_expert.p;
@@ -1214,7 +1216,16 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
     HIP_TRY(ctx, prod(gh));
     GroupedArgs gx = g;  // grad_input rows = dG . Wgate + dU . Wup
     gx.a = L->dgu.p; gx.w = L->wguT.p; gx.w_expert_stride = (size_t)d * 2 * F; gx.N = d; gx.K = 2 * F; gx.out = L->dxg.p;
-    HIP_TRY(ctx, prod(gx));
+    if (side) {
+        // the input-gradient product follows the router's branch on the side stream, beside the weight gradients
+        // (it needs dG | dU, which the launch above has just written)
+        HIP_TRY(ctx, hipEventRecord(ctx->ev_fork2, s));
+        HIP_TRY(ctx, hipStreamWaitEvent(rs, ctx->ev_fork2, 0));
+        HIP_TRY(ctx, L->use_stream ? launch_grouped_stream(gx, WeightKind::BF16, L->variant, rs) : launch_grouped_f32(gx, rs));
+        HIP_TRY(ctx, hipEventRecord(ctx->ev_join, rs));
+    } else {
+        HIP_TRY(ctx, prod(gx));
+    }
     // weight gradients (src/param.rs:819-821): down += dY^T . H; (gate | up) += (dG | dU)^T . X[token]
     auto wgrad = [&](const void* a, int M, const void* b, const int* b_rows, int N, int groups, int dense_rows,
                      int total_rows, float* out, size_t stride) -> hipError_t {
