@@ -26,48 +26,25 @@ constexpr int kSmallThreads = 512;
 constexpr int kStageBytes = 44 * 1024;  // LDS for the staged router and token rows
 
 // softmax_rows (src/moe.rs, softmax over one row) and route (src/moe.rs:553-593) of one token, by one
-// thread.  EMAX > 0: the row is copied into EMAX registers and every loop over the experts is
-// unrolled with the tail predicated off; EMAX == 0: the row is used where it lies (LDS).
-template <int EMAX>
-__device__ __forceinline__ void token_phase(float* row_lds, int t, int E, int k, const uint8_t* valid, float* P,
-                                            float* lse, float* lsev, int* sexp, int* expert_of, float* gate_of) {
-    constexpr int N = EMAX > 0 ? EMAX : 1;
-    float reg[N];
-    auto get = [&](int e) -> float {
-        if constexpr (EMAX > 0) return reg[e];
-        else return row_lds[e];
-    };
-    auto set = [&](int e, float v) {
-        if constexpr (EMAX > 0) reg[e] = v;
-        else row_lds[e] = v;
-    };
-    const int EB = EMAX > 0 ? EMAX : E;  // loop bound (a compile-time constant when EMAX > 0)
-    if constexpr (EMAX > 0) {
-#pragma unroll
-        for (int e = 0; e < EMAX; ++e) reg[e] = e < E ? row_lds[e] : 0.0f;
-    }
+// thread, the row used where it lies in LDS: the path for more experts than a wave has lanes.
+__device__ __forceinline__ void token_phase_serial(float* row, int t, int E, int k, const uint8_t* valid, float* P,
+                                                   float* lse, float* lsev, int* sexp, int* expert_of, float* gate_of) {
     const float neg_inf = __uint_as_float(0xff800000u);
     float mx = neg_inf;
-#pragma unroll
-    for (int e = 0; e < EB; ++e)
-        if (e < E && get(e) > mx) mx = get(e);  // a NaN never replaces the maximum
+    for (int e = 0; e < E; ++e)
+        if (row[e] > mx) mx = row[e];  // a NaN never replaces the maximum
     float sum = 0.0f;
-#pragma unroll
-    for (int e = 0; e < EB; ++e)
-        if (e < E) {
-            set(e, rb_expf(__fadd_rn(get(e), -mx)));
-            sum = __fadd_rn(sum, get(e));
-        }
+    for (int e = 0; e < E; ++e) {
+        row[e] = rb_expf(__fadd_rn(row[e], -mx));
+        sum = __fadd_rn(sum, row[e]);
+    }
     const float l = __fadd_rn(mx, rb_logf(sum));
     lsev[t] = l;
     lse[t] = l;
-#pragma unroll
-    for (int e = 0; e < EB; ++e)
-        if (e < E) {
-            if (sum > 0.0f) set(e, __fdiv_rn(get(e), sum));
-            P[(size_t)t * E + e] = get(e);
-            if constexpr (EMAX > 0) row_lds[e] = get(e);  // the loss phase reads the probabilities from LDS
-        }
+    for (int e = 0; e < E; ++e) {
+        if (sum > 0.0f) row[e] = __fdiv_rn(row[e], sum);
+        P[(size_t)t * E + e] = row[e];
+    }
 
     int* eo = sexp + t * k;
     const bool ok = (valid == nullptr) || (valid[t] != 0);
@@ -79,48 +56,98 @@ __device__ __forceinline__ void token_phase(float* row_lds, int t, int E, int k,
         }
         return;
     }
-    // taken experts as a bit set when they fit one (EMAX <= 64), else through the slot list
-    unsigned long long taken_bits = 0ull;
     float total = 0.0f;
     for (int r = 0; r < k; ++r) {
         int best = -1;
         float bestv = 0.0f;
-#pragma unroll
-        for (int e = 0; e < EB; ++e) {
-            if (e >= E) continue;
-            bool taken;
-            if constexpr (EMAX > 0) {
-                taken = (taken_bits >> e) & 1ull;
-            } else {
-                taken = false;
-                for (int q = 0; q < r; ++q) taken = taken || (eo[q] == e);
-            }
+        for (int e = 0; e < E; ++e) {
+            bool taken = false;
+            for (int q = 0; q < r; ++q) taken = taken || (eo[q] == e);
             if (taken) continue;
-            const float v = get(e);
+            const float v = row[e];
             if (best < 0 || v > bestv) {
                 best = e;
                 bestv = v;
             }
         }
         eo[r] = best;
-        if constexpr (EMAX > 0) taken_bits |= 1ull << best;
         total = __fadd_rn(total, bestv);
         gate_of[t * k + r] = bestv;  // rewritten below once the sum is known
         expert_of[t * k + r] = best;
     }
     if (total > 0.0f)
-        for (int r = 0; r < k; ++r) {
-            float g;
-            if constexpr (EMAX > 0) {
-                g = 0.0f;
+        for (int r = 0; r < k; ++r) gate_of[t * k + r] = __fdiv_rn(row[eo[r]], total);
+}
+
+// The same two steps with G lanes per token (G = 16 or 64, E <= G), lane j holding expert j: the
+// exponentials, divisions and the argmax of every round run side by side, and only what the reference
+// does in sequence stays a sequence - the sum of the exponentials in index order (every lane of the group
+// adds the E values up in the same order, fetching them with shuffles) and the running sum of the selected
+// probabilities.  A round's winner is the largest 64-bit key (probability bits above the inverted index:
+// probabilities are >= +0, so their bit patterns order like their values, and among equal ones the lower
+// index wins, as the reference's strict `>` scan does); a taken expert's key is 0.
+template <int G>
+__device__ __forceinline__ void token_phase_lanes(float* row_lds, int t, int j, int E, int k, const uint8_t* valid,
+                                                  float* P, float* lse, float* lsev, int* sexp, int* expert_of,
+                                                  float* gate_of) {
+    const int lane = threadIdx.x & 63;
+    const int base = lane - j;  // first lane of the group
+    const bool mine = j < E;
+    const float neg_inf = __uint_as_float(0xff800000u);
+    const float v = mine ? row_lds[j] : neg_inf;
+    float mx = (v == v) ? v : neg_inf;  // a NaN never replaces the maximum
 #pragma unroll
-                for (int e = 0; e < EMAX; ++e)
-                    if (e == eo[r]) g = reg[e];
-            } else {
-                g = row_lds[eo[r]];
-            }
-            gate_of[t * k + r] = __fdiv_rn(g, total);
+    for (int o = G / 2; o > 0; o >>= 1) {
+        const float other = __shfl_xor(mx, o);
+        mx = other > mx ? other : mx;
+    }
+    const float ex = mine ? rb_expf(__fadd_rn(v, -mx)) : 0.0f;
+    float sum = 0.0f;
+    for (int e = 0; e < E; ++e) sum = __fadd_rn(sum, __shfl(ex, base + e));
+    const float l = __fadd_rn(mx, rb_logf(sum));
+    const float p = sum > 0.0f ? __fdiv_rn(ex, sum) : ex;
+    if (mine) {
+        P[(size_t)t * E + j] = p;
+        row_lds[j] = p;  // the loss phase reads the probabilities from LDS
+    }
+    if (j == 0) {
+        lsev[t] = l;
+        lse[t] = l;
+    }
+    const bool ok = (valid == nullptr) || (valid[t] != 0);
+    if (!ok) {
+        if (j < k) {
+            sexp[t * k + j] = -1;
+            expert_of[t * k + j] = -1;
+            gate_of[t * k + j] = 0.0f;
         }
+        return;
+    }
+    unsigned long long key = mine ? (((unsigned long long)__float_as_uint(p) << 32) | (0xffffffffu - (unsigned)j)) : 0ull;
+    float total = 0.0f;
+    float my_p = 0.0f;  // lane r keeps round r's probability
+    int my_e = -1;
+    for (int r = 0; r < k; ++r) {
+        unsigned long long best = key;
+#pragma unroll
+        for (int o = G / 2; o > 0; o >>= 1) {
+            const unsigned long long other = __shfl_xor(best, o);
+            best = other > best ? other : best;
+        }
+        const int be = (int)(0xffffffffu - (unsigned)(best & 0xffffffffull));
+        const float bv = __uint_as_float((unsigned)(best >> 32));
+        total = __fadd_rn(total, bv);
+        if (j == be) key = 0ull;
+        if (j == r) {
+            my_p = bv;
+            my_e = be;
+        }
+    }
+    if (j < k) {
+        sexp[t * k + j] = my_e;
+        expert_of[t * k + j] = my_e;
+        gate_of[t * k + j] = total > 0.0f ? __fdiv_rn(my_p, total) : my_p;
+    }
 }
 
 template <typename XT>
@@ -285,15 +312,17 @@ __global__ __launch_bounds__(kSmallThreads) void route_small_kernel(
     __syncthreads();
 
     // ---- softmax_rows and route: one token per thread --------------------------
-    // With few experts the token's row lives in registers (every loop fully unrolled, the
-    // same operations in the same order); otherwise it stays in LDS.
-    if (tid < T) {
-        if (E <= 16)
-            token_phase<16>(prob + tid * E, tid, E, k, valid, P, lse, lsev, sexp, expert_of, gate_of);
-        else if (E <= 64)
-            token_phase<64>(prob + tid * E, tid, E, k, valid, P, lse, lsev, sexp, expert_of, gate_of);
-        else
-            token_phase<0>(prob + tid * E, tid, E, k, valid, P, lse, lsev, sexp, expert_of, gate_of);
+    // Up to 64 experts: a group of lanes per token; more: one thread per token.
+    if (E <= 16 && k <= 16) {
+        // 16 lanes per token, 32 tokens per pass of the block
+        for (int t = tid >> 4; t < T; t += kSmallThreads / 16)
+            token_phase_lanes<16>(prob + t * E, t, tid & 15, E, k, valid, P, lse, lsev, sexp, expert_of, gate_of);
+    } else if (E <= 64) {
+        // a wave per token (k <= 32 < 64 always)
+        for (int t = tid >> 6; t < T; t += kSmallThreads / 64)
+            token_phase_lanes<64>(prob + t * E, t, tid & 63, E, k, valid, P, lse, lsev, sexp, expert_of, gate_of);
+    } else if (tid < T) {
+        token_phase_serial(prob + tid * E, tid, E, k, valid, P, lse, lsev, sexp, expert_of, gate_of);
     }
     __syncthreads();
 

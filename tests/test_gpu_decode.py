@@ -45,7 +45,10 @@ def run(device, t, valid=None, bias=None, residual=None):
 
 # widths are multiples of 64: the packed-weight kernels need that in both directions
 SHAPES = [dict(d=64, E=4, k=1, F=64, T=1), dict(d=128, E=8, k=2, F=128, T=8), dict(d=192, E=6, k=3, F=192, T=7),
-          dict(d=256, E=64, k=6, F=64, T=32), dict(d=128, E=5, k=2, F=320, T=19)]
+          dict(d=256, E=64, k=6, F=64, T=32), dict(d=128, E=5, k=2, F=320, T=19),
+          dict(d=64, E=24, k=5, F=64, T=20),     # a wave per token, 40 lanes idle
+          dict(d=64, E=16, k=16, F=64, T=9),     # every expert selected, 16 lanes per token
+          dict(d=64, E=100, k=4, F=64, T=16)]    # more experts than lanes: one thread per token
 
 
 @pytest.mark.parametrize("wt", ["bf16", "int8"])
