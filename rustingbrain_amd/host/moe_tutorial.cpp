@@ -161,6 +161,60 @@ static void gpu_checks() {
         EXPECT(layers.size() == 2 && layers.count(1) && layers.count(3));
         EXPECT(layers[1]->num_parameters() == 4 * 16 + 5 * 3 * 16 * 12);
     }
+    // training through the C++ mirror: the block step (norm, layer, residual) forward and backward on an all-f32 layer
+    {
+        const size_t TD = 64, TE = 4, TF = 32, TR = 48;
+        MoeLayer train(TD, MoeConfig(TE, 2, TF).with_aux_loss_weight(0.0f).with_router_z_loss_weight(0.0f), device, TR);
+        train.enable_training();
+        std::vector<float> norm_w(TD);
+        for (size_t c = 0; c < TD; ++c) norm_w[c] = 0.75f + 0.01f * (float)c;
+        train.set_feed_forward_norm(norm_w, 1e-6f);
+        const float tb = std::sqrt(6.0f / (float)(TD + TF));
+        train.set_router(random_matrix(TE, TD, 0.5f, 21));
+        for (size_t e = 0; e < TE; ++e)
+            train.set_expert(e, random_matrix(TF, TD, tb, 200 + 3 * e), random_matrix(TF, TD, tb, 201 + 3 * e),
+                             random_matrix(TD, TF, tb, 202 + 3 * e));
+        const Matrix x = random_matrix(TR, TD, 1.0f, 23);
+        Matrix ones(TR, TD);
+        for (float& v : ones.data) v = 1.0f;
+        const Matrix out = train.forward_block(x);
+        const Matrix grad = train.backward_block(ones);
+        EXPECT(grad.rows == TR && grad.cols == TD);
+        // finite differences of sum(out) in a few coordinates (reference src/moe.rs:895-925: epsilon 1e-3, 2e-2)
+        double sum0 = 0.0;
+        for (float v : out.data) sum0 += v;
+        (void)sum0;
+        bool fd_ok = true;
+        for (size_t idx : {size_t(0), size_t(7 * TD + 3), size_t(40 * TD + 60)}) {
+            Matrix hi = x, lo = x;
+            hi.data[idx] += 1e-3f;
+            lo.data[idx] -= 1e-3f;
+            double sh = 0.0, sl = 0.0;
+            for (float v : train.forward_block(hi).data) sh += v;
+            for (float v : train.forward_block(lo).data) sl += v;
+            const double numeric = (sh - sl) / (double)(hi.data[idx] - lo.data[idx]);
+            fd_ok = fd_ok && std::fabs(numeric - grad.data[idx]) < 2e-2 * std::fmax(1.0, std::fabs(numeric));
+        }
+        EXPECT(fd_ok);
+        // gradients accumulate until cleared (Param.grad), and the norm's scale has one too
+        train.forward_block(x);
+        const Matrix g1 = train.weight_grad(RBMOE_W_DOWN, 1);
+        train.backward_block(ones);
+        const Matrix g2 = train.weight_grad(RBMOE_W_DOWN, 1);
+        bool doubled = true, any = false;
+        for (size_t i = 0; i < g1.data.size(); ++i) {
+            doubled = doubled && std::fabs(g2.data[i] - 2.0f * g1.data[i]) <= 1e-5f * (1.0f + std::fabs(g2.data[i]));
+            any = any || g1.data[i] != 0.0f;
+        }
+        EXPECT(doubled && any);
+        EXPECT(train.weight_grad(RBMOE_W_NORM).cols == TD);
+        train.zero_grads();
+        bool cleared = true;
+        for (float v : train.weight_grad(RBMOE_W_DOWN, 1).data) cleared = cleared && v == 0.0f;
+        EXPECT(cleared);
+        // no backward pass for a layer that is not in training mode
+        EXPECT(throws<InvalidConfig>([&] { layer.backward(Matrix(ROWS, D)); }));
+    }
     // a budget that cannot hold the layer is refused before anything is allocated
     EXPECT(throws<MemoryBudget>([&] {
         auto small = Device::open(0, 1);
