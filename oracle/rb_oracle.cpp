@@ -831,8 +831,11 @@ static void swiglu_backward(const rbo_expert_weights* w, const float* x, const f
 }
 
 // Returns 0; 1 when cols != d_model; 2 when an expert is quantized.
-int rbo_moe_backward(const rbo_layer* L, const float* x, int T, int cols, const uint8_t* valid,
-                     const float* router_bias, const float* grad_output, rbo_grads* G) {
+// `threads` > 1: experts are independent tasks (their forward rows, then their backward); everything that adds
+// into rows shared between experts runs afterwards on one thread, in the same order as with one thread, so the
+// results do not depend on the thread count.
+int rbo_moe_backward_mt(const rbo_layer* L, const float* x, int T, int cols, const uint8_t* valid,
+                        const float* router_bias, const float* grad_output, rbo_grads* G, int threads) {
     const int d = L->d_model, E = L->num_experts, k = L->experts_per_token, F = L->d_ff;
     if (cols != d) return 1;
     for (int e = 0; e < E; ++e)
@@ -856,10 +859,29 @@ int rbo_moe_backward(const rbo_layer* L, const float* x, int T, int cols, const 
     std::vector<float> xg(Rn * d), gate(Rn * F), up(Rn * F), hidden(Rn * F), eout(Rn * d);
     for (int i = 0; i < R; ++i)
         std::memcpy(xg.data() + (int64_t)i * d, x + (int64_t)perm_token[i] * d, sizeof(float) * d);
-    for (int e = 0; e < E; ++e)
+    auto for_each_expert = [&](auto&& body) {
+        std::atomic<int> next{0};
+        auto worker = [&]() {
+            for (;;) {
+                const int e = next.fetch_add(1);
+                if (e >= E) break;
+                body(e);
+            }
+        };
+        const int nthreads = std::max(1, std::min(threads, E));
+        if (nthreads == 1) {
+            worker();
+        } else {
+            std::vector<std::thread> pool;
+            for (int i = 0; i < nthreads; ++i) pool.emplace_back(worker);
+            for (auto& th : pool) th.join();
+        }
+    };
+    for_each_expert([&](int e) {
         swiglu_rows(&L->experts[e], xg.data() + (int64_t)offsets[e] * d, 0, counts[e], d, F,
                     gate.data() + (int64_t)offsets[e] * F, up.data() + (int64_t)offsets[e] * F,
                     hidden.data() + (int64_t)offsets[e] * F, eout.data() + (int64_t)offsets[e] * d);
+    });
 
     float* gin = G->grad_input;
     std::memset(gin, 0, sizeof(float) * (size_t)T * d);
@@ -876,11 +898,12 @@ int rbo_moe_backward(const rbo_layer* L, const float* x, int T, int cols, const 
 
     // ---- routed experts (src/moe.rs:366-399) -----------------------------------------
     std::vector<float> grad_gates((size_t)std::max(S, 1), 0.0f);
-    for (int e = 0; e < E; ++e) {
+    std::vector<float> gx_rows(Rn * d);  // every expert's input-gradient rows, permuted order
+    for_each_expert([&](int e) {
         const int rows = counts[e];
-        if (rows == 0) continue;
+        if (rows == 0) return;
         const int64_t base = offsets[e];
-        std::vector<float> scaled((size_t)rows * d), gx((size_t)rows * d);
+        std::vector<float> scaled((size_t)rows * d);
         for (int i = 0; i < rows; ++i) {
             const float g = gate_of[perm_slot[base + i]];
             const float* upstream = grad_output + (int64_t)perm_token[base + i] * d;
@@ -888,10 +911,14 @@ int rbo_moe_backward(const rbo_layer* L, const float* x, int T, int cols, const 
         }
         swiglu_backward(&L->experts[e], xg.data() + base * d, gate.data() + base * F, up.data() + base * F,
                         hidden.data() + base * F, scaled.data(), rows, d, F, G->grad_gate + (int64_t)e * F * d,
-                        G->grad_up + (int64_t)e * F * d, G->grad_down + (int64_t)e * d * F, gx.data());
-        for (int i = 0; i < rows; ++i) {
+                        G->grad_up + (int64_t)e * F * d, G->grad_down + (int64_t)e * d * F, gx_rows.data() + base * d);
+    });
+    for (int e = 0; e < E; ++e) {  // scatter-add in expert order, rows ascending (src/moe.rs:392-398)
+        const int64_t base = offsets[e];
+        for (int i = 0; i < counts[e]; ++i) {
             float* dst = gin + (int64_t)perm_token[base + i] * d;
-            for (int c = 0; c < d; ++c) dst[c] = dst[c] + gx[(int64_t)i * d + c];
+            const float* src = gx_rows.data() + (base + i) * d;
+            for (int c = 0; c < d; ++c) dst[c] = dst[c] + src[c];
         }
     }
     // gate gradients: one dot product per routed slot (src/moe.rs:404-416)
@@ -953,6 +980,11 @@ int rbo_moe_backward(const rbo_layer* L, const float* x, int T, int cols, const 
     if (G->grad_gates && S > 0) std::memcpy(G->grad_gates, grad_gates.data(), sizeof(float) * (size_t)S);
     if (G->grad_logits) std::memcpy(G->grad_logits, gl.data(), sizeof(float) * (size_t)T * E);
     return 0;
+}
+
+int rbo_moe_backward(const rbo_layer* L, const float* x, int T, int cols, const uint8_t* valid,
+                     const float* router_bias, const float* grad_output, rbo_grads* G) {
+    return rbo_moe_backward_mt(L, x, T, cols, valid, router_bias, grad_output, G, 1);
 }
 
 }  // extern "C"

@@ -288,6 +288,8 @@ class _Grads(C.Structure):
                 ("grad_gates", _f32p), ("grad_logits", _f32p)]
 
 
+_lib.rbo_moe_backward_mt.restype = C.c_int
+_lib.rbo_moe_backward_mt.argtypes = [C.POINTER(_Layer), _f32p, C.c_int, C.c_int, _u8p, _f32p, _f32p, C.POINTER(_Grads), C.c_int]
 _lib.rbo_moe_backward.restype = C.c_int
 _lib.rbo_moe_backward.argtypes = [C.POINTER(_Layer), _f32p, C.c_int, C.c_int, _u8p, _f32p, _f32p, C.POINTER(_Grads)]
 
@@ -413,7 +415,7 @@ class OracleLayer:
 
     def backward_block(self, residual: np.ndarray, norm_weight: np.ndarray, eps: float, grad_output: np.ndarray,
                        valid: Optional[np.ndarray] = None, router_bias: Optional[np.ndarray] = None,
-                       round_normed=None):
+                       round_normed=None, threads: int = 1):
         """The feed-forward half of TransformerBlock::backward (src/transformer_block.rs:257-263):
         ``grad_projected = moe.backward(cache, grad_output)``, ``grad_residual = feed_forward_norm.backward(residual,
         grad_projected) + grad_output``.  Returns (grad_residual, grad_norm_weight, BackwardResult of the layer)."""
@@ -421,12 +423,12 @@ class OracleLayer:
         normed = rmsnorm(residual, norm_weight, eps)
         if round_normed is not None:
             normed = np.ascontiguousarray(round_normed(normed), dtype=np.float32)
-        inner = self.backward(normed, grad_output, valid=valid, router_bias=router_bias)
+        inner = self.backward(normed, grad_output, valid=valid, router_bias=router_bias, threads=threads)
         gi, gw = rmsnorm_backward(residual, inner.grad_input, norm_weight, eps)
         return gi + np.ascontiguousarray(grad_output, dtype=np.float32), gw, inner
 
     def backward(self, x: np.ndarray, grad_output: np.ndarray, valid: Optional[np.ndarray] = None,
-                 router_bias: Optional[np.ndarray] = None) -> BackwardResult:
+                 router_bias: Optional[np.ndarray] = None, threads: int = 1) -> BackwardResult:
         x = np.ascontiguousarray(x, dtype=np.float32)
         grad_output = np.ascontiguousarray(grad_output, dtype=np.float32)
         T, cols = x.shape
@@ -453,8 +455,8 @@ class OracleLayer:
             valid = np.ascontiguousarray(valid, dtype=np.uint8)
         if router_bias is not None:
             router_bias = np.ascontiguousarray(router_bias, dtype=np.float32)
-        rc = _lib.rbo_moe_backward(C.byref(layer), _fp(x), T, cols, _up(valid), _fp(router_bias), _fp(grad_output),
-                                   C.byref(grads))
+        rc = _lib.rbo_moe_backward_mt(C.byref(layer), _fp(x), T, cols, _up(valid), _fp(router_bias),
+                                      _fp(grad_output), C.byref(grads), threads)
         if rc == 1:
             raise ValueError(f"InvalidInput: expected {d} columns, got {cols}")
         if rc == 2:

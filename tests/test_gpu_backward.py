@@ -29,8 +29,8 @@ def check_backward(device, t, valid=None, bias=None, aux_w=0.01, z_w=1e-3, seed=
     E = w.num_experts
     gout = grad_output_for(t, seed)
     ref_layer = oracle_layer(t, aux_w=aux_w, z_w=z_w)
-    ref_fwd = ref_layer.forward(t.x, valid=valid, router_bias=bias)
-    ref = ref_layer.backward(t.x, gout, valid=valid, router_bias=bias)
+    ref_fwd = ref_layer.forward(t.x, valid=valid, router_bias=bias, threads=8)
+    ref = ref_layer.backward(t.x, gout, valid=valid, router_bias=bias, threads=8)
     layer = gpu_layer(device, t, aux_w=aux_w, z_w=z_w, training=True)
     layout = rb.Layout(valid=None if valid is None else [bool(v) for v in valid])
     out, cache = layer.forward_train(t.x, layout, router_bias=bias)

@@ -167,9 +167,10 @@ def check_block_backward(device, t, valid=None, bias=None, seed=5, norm_first=Tr
     gout = synth.round_bf16(rng.standard_normal(t.x.shape).astype(np.float32))
     rounder = synth.round_bf16 if bf16 else None
     ref_layer = oracle_layer(t)
-    want_out, _, ref_f = ref_layer.forward_block(t.x, nw, 1e-6, valid=valid, router_bias=bias, round_normed=rounder)
+    want_out, _, ref_f = ref_layer.forward_block(t.x, nw, 1e-6, valid=valid, router_bias=bias, round_normed=rounder,
+                                                 threads=8)
     want_g, want_gw, inner = ref_layer.backward_block(t.x, nw, 1e-6, gout, valid=valid, router_bias=bias,
-                                                      round_normed=rounder)
+                                                      round_normed=rounder, threads=8)
     cfg = rb.MoeConfig(w.num_experts, w.experts_per_token, w.d_ff, w.shared_expert)
     layer = rb.MoeLayer(w.d_model, cfg, device, act_dtype=w.act_dtype, weight_dtype=w.weight_dtype,
                         max_tokens=t.x.shape[0], shared_d_ff=w.shared_d_ff if w.shared_expert else 0)
