@@ -125,17 +125,17 @@ __device__ __forceinline__ float silu_bf16_grade(float x) {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 
-// two int8 values of `word` (bytes shift/8 and shift/8 + 1) as a pair of bf16
-__device__ __forceinline__ uint32_t widen2(uint32_t word, int shift) {
-    const float lo = (float)(int)(int8_t)(word >> shift);
-    const float hi = (float)(int)(int8_t)(word >> (shift + 8));
-    return (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xffff0000u);  // small integers are exact in bf16
-}
-
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
     typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
     bf16x2 v = {(__bf16)lo, (__bf16)hi};
     return __builtin_bit_cast(uint32_t, v);
+}
+
+// two int8 values of `word` (bytes shift/8 and shift/8 + 1) as a pair of bf16
+__device__ __forceinline__ uint32_t widen2(uint32_t word, int shift) {
+    const float lo = (float)(int)(int8_t)(word >> shift);
+    const float hi = (float)(int)(int8_t)(word >> (shift + 8));
+    return pack2(lo, hi);  // small integers are exact in bf16; one packed conversion instead of shift + and-or
 }
 
 __device__ __forceinline__ bf16x8 widen_i8(uint2 q) {
