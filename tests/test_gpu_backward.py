@@ -214,6 +214,26 @@ def test_plain_f32_weight_gradient_kernel_agrees(device, monkeypatch):
         layer.close()
 
 
+def test_backward_of_degenerate_batches(device):
+    # every row padding (nothing routed; only the shared expert sees the rows), then a single row
+    t = synth.make(small_workload(d=64, E=4, k=2, F=64, T=40, seed=34, act="bf16", wt="bf16", shared=True))
+    layer, ref, gout = check_backward(device, t, valid=np.zeros(40, np.uint8))
+    for which in (L.W_GATE, L.W_UP, L.W_DOWN):
+        for e in range(4):
+            assert not layer.weight_grad(which, e).any()
+    assert not layer.weight_grad(L.W_ROUTER).any()
+    assert layer.weight_grad(L.W_SHARED_DOWN).any()
+    layer.close()
+    one = synth.make(small_workload(d=64, E=4, k=2, F=64, T=1, seed=35, act="bf16", wt="bf16"))
+    layer, ref, gout = check_backward(device, one)
+    assert int((np.abs(ref.grad_down).sum(axis=(1, 2)) > 0).sum()) == 2     # exactly the two selected experts
+    layer.close()
+    plain = synth.make(small_workload(d=64, E=4, k=2, F=64, T=40, seed=36, act="f32", wt="f32"))
+    layer, _, _ = check_backward(device, plain, valid=np.zeros(40, np.uint8))  # no shared expert: all gradients zero
+    assert not layer.weight_grad(L.W_DOWN, 0).any()
+    layer.close()
+
+
 def test_backward_follows_the_most_recent_forward(device):
     t = synth.make(small_workload(d=64, E=4, k=2, F=64, T=120, seed=26, act="bf16", wt="bf16"))
     layer = gpu_layer(device, t, training=True)
