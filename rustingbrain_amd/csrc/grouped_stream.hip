@@ -452,7 +452,15 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
                         continue;
                     }
                 }
-                *reinterpret_cast<uint4*>(dst + (size_t)(row0 + r) * dstride + col0 + 8 * p) = v;
+                uint4* const where = reinterpret_cast<uint4*>(dst + (size_t)(row0 + r) * dstride + col0 + 8 * p);
+                if (SWIGLU && b > 0) {
+                    // the pre-activations are not read again before the backward pass: stored past the caches,
+                    // so that they do not push the hidden rows out before the down product reads them
+                    typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+                    __builtin_nontemporal_store(u32x4_t{v.x, v.y, v.z, v.w}, reinterpret_cast<u32x4_t*>(where));
+                } else {
+                    *where = v;
+                }
             }
         }
     }
