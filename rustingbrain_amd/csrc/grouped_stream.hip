@@ -426,8 +426,10 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
                         // the forward pass, dG = dH * U * silu'(G) and dU = dH * silu(G) go to `gu_out`
                         // (both [rows, 2 N]) and the hidden gradient itself is never stored.
                         const size_t off = (size_t)(row0 + r) * 2 * N + col0 + 8 * p;
-                        const uint4 g8 = *reinterpret_cast<const uint4*>(bw_gu + off);
-                        const uint4 u8 = *reinterpret_cast<const uint4*>(bw_gu + off + N);
+                        // (read once: fetched past the caches)
+                        typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+                        const u32x4_t g8 = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(bw_gu + off));
+                        const u32x4_t u8 = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(bw_gu + off + N));
                         const uint32_t hw[4] = {v.x, v.y, v.z, v.w}, gw[4] = {g8.x, g8.y, g8.z, g8.w},
                                        uw[4] = {u8.x, u8.y, u8.z, u8.w};
                         uint32_t dg[4], du[4];

@@ -70,17 +70,22 @@ __device__ __forceinline__ void add_tiles(const floatx16 (&acc)[NI][NJ], float* 
                 for (int v = 0; v < 16; ++v)
                     if (mb + 8 * (v >> 2) < M) unsafeAtomicAdd(base + (size_t)(8 * (v >> 2) + (v & 3)) * N, acc[i][j][v]);
             } else if (overwrite) {
+                // (the gradient is read again only by the optimiser: stored past the caches, which hold the
+                // operand rows that other workgroups are still reading)
 #pragma unroll
                 for (int v = 0; v < 16; ++v)
-                    if (mb + 8 * (v >> 2) < M) base[(size_t)(8 * (v >> 2) + (v & 3)) * N] = acc[i][j][v];
+                    if (mb + 8 * (v >> 2) < M)
+                        __builtin_nontemporal_store(acc[i][j][v], base + (size_t)(8 * (v >> 2) + (v & 3)) * N);
             } else {
                 float old[16];
 #pragma unroll
                 for (int v = 0; v < 16; ++v)
-                    if (mb + 8 * (v >> 2) < M) old[v] = base[(size_t)(8 * (v >> 2) + (v & 3)) * N];
+                    if (mb + 8 * (v >> 2) < M)
+                        old[v] = __builtin_nontemporal_load(base + (size_t)(8 * (v >> 2) + (v & 3)) * N);
 #pragma unroll
                 for (int v = 0; v < 16; ++v)
-                    if (mb + 8 * (v >> 2) < M) base[(size_t)(8 * (v >> 2) + (v & 3)) * N] = old[v] + acc[i][j][v];
+                    if (mb + 8 * (v >> 2) < M)
+                        __builtin_nontemporal_store(old[v] + acc[i][j][v], base + (size_t)(8 * (v >> 2) + (v & 3)) * N);
             }
         }
     }
