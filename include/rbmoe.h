@@ -1,8 +1,10 @@
 /*
  * rbmoe.h — C ABI of the MI355X (gfx950) mixture-of-experts layer.
  *
- * Drop-in boundary for the forward pass of RustingBrain's `MoeLayer`
- * (reference src/moe.rs:203-341) and the two auxiliary losses.  The reference
+ * Drop-in boundary for RustingBrain's `MoeLayer`: the forward pass with the two
+ * auxiliary losses (reference src/moe.rs:203-341), the backward pass
+ * (src/moe.rs:348-489) and the block's RMSNorm and residual add either side of
+ * the layer (src/transformer_block.rs:216-222, 257-263).  The reference
  * has no FFI seam for this layer; each entry point below names the reference
  * interface it stands in for, so that a Rust `extern "C"` block can bind them
  * one to one.  Plain pointers and sizes only.  Every function returns an
