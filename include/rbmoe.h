@@ -195,8 +195,10 @@ int rbmoe_forward_block_host(rbmoe_layer* layer, const void* x, int32_t tokens, 
 /* ---- backward pass (MoeLayer::backward, src/moe.rs:348-489) ------------------------------
  * Training mode makes the forward keep what MoeCache keeps for the backward pass (the input,
  * src/moe.rs:133-135; gate and up pre-activations, src/ffn.rs:27-33) and allocates f32 gradient
- * accumulators, the role of Param.grad (src/param.rs).  For bf16 layers on the matrix-core path
- * (widths multiples of 64) and all-f32 layers (multiples of 32); RBMOE_UNSUPPORTED otherwise.
+ * accumulators, the role of Param.grad (src/param.rs).  For every f32 / bf16 layer: bf16 layers with
+ * widths that are multiples of 64 and all-f32 layers (multiples of 32) differentiate on the matrix
+ * cores, any other shape or dtype mix on plain kernels; int8 layers report RBMOE_UNSUPPORTED, as the
+ * reference has no backward for quantized experts (src/ffn.rs:87-93).
  * Call it before the weights are set.  A training layer always takes the large-batch kernels. */
 int rbmoe_layer_enable_training(rbmoe_layer* layer);
 

@@ -236,8 +236,8 @@ impl MoeLayer {
     }
 
     /// Makes the forward pass keep what `backward` needs and allocates the f32 gradient accumulators (the
-    /// role of `Param.grad`).  Call before the weights are set.  The library runs the backward pass for
-    /// layers with bf16 activations and weights; on this f32-boundary layer it reports `UnsupportedCuda`.
+    /// role of `Param.grad`).  Call before the weights are set.  Every f32 and bf16 layer has a backward pass
+    /// (matrix-core kernels where the widths fit them, plain ones otherwise); int8 layers report `UnsupportedCuda`.
     pub fn enable_training(&mut self) -> Result<(), NetworkError> {
         check(unsafe { sys::rbmoe_layer_enable_training(self.layer) }, self.device.raw(), 0, 0)
     }

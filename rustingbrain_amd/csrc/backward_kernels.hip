@@ -10,8 +10,9 @@
 // The row products (dH = dY . Wd, dX = dG . Wg + dU . Wu) run on the forward pass's streaming
 // kernel with transposed packed copies of the weights (SwiGLU's backward is applied where the
 // first of them stores its rows); the weight gradients have a matrix-core kernel of their own.
-// Every sum in this file has one fixed order.  Rows are moved in 16-byte pieces: the row width
-// must be a multiple of 8 (bf16) or 4 (f32) elements.
+// Every sum in this file has one fixed order.  Rows are moved in 16-byte pieces when the row
+// width is a multiple of 8 (bf16) or 4 (f32) elements; any other width takes the same kernels
+// one element at a time (`Vec1`) or the plain `*_any_kernel` versions further down.
 #include "rbmoe_kernels.h"
 
 namespace rbmoe {
@@ -19,14 +20,22 @@ namespace rbmoe {
 // ---------------------------------------------------------------------------
 // One wave per routed row (src/moe.rs:374-385 and :404-416).
 // ---------------------------------------------------------------------------
+// One element of a row, with the interface of Vec16: rows of any width.
 template <typename XT>
+struct Vec1 {
+    static constexpr int N = 1;
+    static __device__ __forceinline__ void load(const XT* p, float (&v)[1]) { v[0] = to_f32(*p); }
+    static __device__ __forceinline__ void store(XT* p, const float (&v)[1]) { *p = from_f32<XT>(v[0]); }
+};
+
+template <typename XT, typename V>
 __global__ __launch_bounds__(256) void scale_rows_kernel(const XT* __restrict__ gout, const XT* __restrict__ y,
                                                          const int* __restrict__ perm_slot,
                                                          const int* __restrict__ perm_token,
                                                          const float* __restrict__ gate_of,
                                                          const int* __restrict__ offsets, int E, int d,
                                                          XT* __restrict__ dy, float* __restrict__ grad_gates) {
-    constexpr int VN = Vec16<XT>::N;
+    constexpr int VN = V::N;
     const int lane = threadIdx.x & 63;
     const int pos = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (pos >= offsets[E]) return;
@@ -38,14 +47,14 @@ __global__ __launch_bounds__(256) void scale_rows_kernel(const XT* __restrict__ 
     float dot = 0.0f;
     for (int c = lane * VN; c < d; c += 64 * VN) {
         float v[VN], w[VN], o[VN];
-        Vec16<XT>::load(go + c, v);
-        Vec16<XT>::load(yr + c, w);
+        V::load(go + c, v);
+        V::load(yr + c, w);
 #pragma unroll
         for (int i = 0; i < VN; ++i) {
             o[i] = g * v[i];
             dot = fmaf(v[i], w[i], dot);
         }
-        Vec16<XT>::store(dr + c, o);
+        V::store(dr + c, o);
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) dot += __shfl_xor(dot, o);
@@ -309,12 +318,12 @@ __global__ __launch_bounds__(256) void router_dx_kernel(const float* __restrict_
 // The inverse rms of every row is kept for the scale gradient, which is summed in the reference's tiles of 32
 // rows: partial[tile][c] = sum over the tile's rows of up * x * inverse_rms, tiles added in order afterwards.
 // ---------------------------------------------------------------------------
-template <typename XT>
+template <typename XT, typename V>
 __global__ __launch_bounds__(256) void rmsnorm_backward_kernel(const XT* __restrict__ x, const XT* __restrict__ up,
                                                                const float* __restrict__ weight, float eps,
                                                                const XT* residual_grad, int T, int d,
                                                                XT* grad_input, float* __restrict__ inv_rms) {
-    constexpr int VN = Vec16<XT>::N;
+    constexpr int VN = V::N;
     const int lane = threadIdx.x & 63;
     const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (t >= T) return;
@@ -323,8 +332,8 @@ __global__ __launch_bounds__(256) void rmsnorm_backward_kernel(const XT* __restr
     float sumsq = 0.0f, proj = 0.0f;
     for (int c = lane * VN; c < d; c += 64 * VN) {
         float xv[VN], uv[VN];
-        Vec16<XT>::load(xr + c, xv);
-        Vec16<XT>::load(ur + c, uv);
+        V::load(xr + c, xv);
+        V::load(ur + c, uv);
 #pragma unroll
         for (int i = 0; i < VN; ++i) {
             sumsq = fmaf(xv[i], xv[i], sumsq);
@@ -341,17 +350,17 @@ __global__ __launch_bounds__(256) void rmsnorm_backward_kernel(const XT* __restr
     if (lane == 0) inv_rms[t] = inv;
     for (int c = lane * VN; c < d; c += 64 * VN) {
         float xv[VN], uv[VN], o[VN];
-        Vec16<XT>::load(xr + c, xv);
-        Vec16<XT>::load(ur + c, uv);
+        V::load(xr + c, xv);
+        V::load(ur + c, uv);
 #pragma unroll
         for (int i = 0; i < VN; ++i) o[i] = uv[i] * weight[c + i] * inv - xv[i] * shared;
         if (residual_grad) {  // uniform
             float rv[VN];
-            Vec16<XT>::load(residual_grad + (size_t)t * d + c, rv);
+            V::load(residual_grad + (size_t)t * d + c, rv);
 #pragma unroll
             for (int i = 0; i < VN; ++i) o[i] += rv[i];
         }
-        Vec16<XT>::store(grad_input + (size_t)t * d + c, o);
+        V::store(grad_input + (size_t)t * d + c, o);
     }
 }
 
@@ -377,6 +386,49 @@ __global__ __launch_bounds__(128) void rmsnorm_wgrad_partial_kernel(const XT* __
     *reinterpret_cast<float2*>(partial + (size_t)tile * d + c) = make_float2(a0, a1);
 }
 
+// ---------------------------------------------------------------------------
+// The same three sums for rows of any width, one output element per thread (the order of the
+// additions inside an element is the one of the kernels above: tokens, experts, rows in sequence).
+// ---------------------------------------------------------------------------
+template <typename XT>
+__global__ __launch_bounds__(256) void router_grad_partial_any_kernel(const float* __restrict__ dlogits,
+                                                                      const XT* __restrict__ x, int T, int d, int E,
+                                                                      int chunk_tokens, float* __restrict__ partial) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= d) return;
+    const int chunk = blockIdx.y, e = blockIdx.z;
+    const int t0 = chunk * chunk_tokens, t1 = min(T, t0 + chunk_tokens);
+    float acc = 0.0f;
+    for (int t = t0; t < t1; ++t) acc = fmaf(dlogits[(size_t)t * E + e], to_f32(x[(size_t)t * d + c]), acc);
+    partial[((size_t)chunk * E + e) * d + c] = acc;
+}
+
+template <typename XT>
+__global__ __launch_bounds__(256) void router_dx_any_kernel(const float* __restrict__ dlogits,
+                                                            const float* __restrict__ wr, int T, int d, int E,
+                                                            XT* __restrict__ dxr) {
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (long long)T * d) return;
+    const int t = (int)(idx / d), c = (int)(idx - (long long)t * d);
+    float acc = 0.0f;
+    for (int e = 0; e < E; ++e) acc = fmaf(dlogits[(size_t)t * E + e], wr[(size_t)e * d + c], acc);
+    dxr[idx] = from_f32<XT>(acc);
+}
+
+template <typename XT>
+__global__ __launch_bounds__(256) void rmsnorm_wgrad_partial_any_kernel(const XT* __restrict__ x,
+                                                                        const XT* __restrict__ up,
+                                                                        const float* __restrict__ inv_rms, int T, int d,
+                                                                        float* __restrict__ partial) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= d) return;
+    const int tile = blockIdx.y;
+    const int t0 = tile * kNormTileRows, t1 = min(T, t0 + kNormTileRows);
+    float a = 0.0f;
+    for (int t = t0; t < t1; ++t) a += to_f32(up[(size_t)t * d + c]) * to_f32(x[(size_t)t * d + c]) * inv_rms[t];
+    partial[(size_t)tile * d + c] = a;
+}
+
 __global__ __launch_bounds__(256) void fill_f32_kernel(float* p, float v, long long n) {
     const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
     if (i < n) p[i] = v;
@@ -391,16 +443,17 @@ hipError_t launch_scale_rows(const void* gout, const void* y, const int* perm_sl
                              const float* gate_of, const int* offsets, int E, int d, int max_rows, void* dy,
                              float* grad_gates, bool bf16, hipStream_t s) {
     if (max_rows <= 0) return hipSuccess;
-    if (!backward_width_ok(d, bf16)) return hipErrorInvalidValue;
     const dim3 grid((max_rows + 3) / 4), block(256);
-    if (bf16)
-        hipLaunchKernelGGL(scale_rows_kernel<bf16_t>, grid, block, 0, s, static_cast<const bf16_t*>(gout),
-                           static_cast<const bf16_t*>(y), perm_slot, perm_token, gate_of, offsets, E, d,
-                           static_cast<bf16_t*>(dy), grad_gates);
-    else
-        hipLaunchKernelGGL(scale_rows_kernel<float>, grid, block, 0, s, static_cast<const float*>(gout),
-                           static_cast<const float*>(y), perm_slot, perm_token, gate_of, offsets, E, d,
-                           static_cast<float*>(dy), grad_gates);
+    auto go = [&](auto tag, auto piece) {
+        using XT = decltype(tag);
+        using V = decltype(piece);
+        hipLaunchKernelGGL((scale_rows_kernel<XT, V>), grid, block, 0, s, static_cast<const XT*>(gout),
+                           static_cast<const XT*>(y), perm_slot, perm_token, gate_of, offsets, E, d,
+                           static_cast<XT*>(dy), grad_gates);
+    };
+    const bool wide = backward_width_ok(d, bf16);
+    if (bf16) { if (wide) go(bf16_t{}, Vec16<bf16_t>{}); else go(bf16_t{}, Vec1<bf16_t>{}); }
+    else { if (wide) go(float{}, Vec16<float>{}); else go(float{}, Vec1<float>{}); }
     return hipGetLastError();
 }
 
@@ -443,9 +496,25 @@ int router_grad_chunks(int max_tokens) { return std::min(kRouterGradMaxChunks, (
 hipError_t launch_router_grad(const float* dlogits, const void* x, const float* wr, int T, int d, int E,
                               float* partial, float* grad_router, void* dxr, bool bf16, hipStream_t s) {
     if (T <= 0) return hipSuccess;
-    if (!backward_width_ok(d, bf16)) return hipErrorInvalidValue;
     const int ct = router_grad_chunk_tokens(T);
     const int chunks = (T + ct - 1) / ct;
+    if (!backward_width_ok(d, bf16)) {
+        const dim3 ga((d + 255) / 256, chunks, E), gd((unsigned)(((long long)T * d + 255) / 256));
+        if (bf16) {
+            hipLaunchKernelGGL(router_grad_partial_any_kernel<bf16_t>, ga, dim3(256), 0, s, dlogits,
+                               static_cast<const bf16_t*>(x), T, d, E, ct, partial);
+            hipLaunchKernelGGL(router_dx_any_kernel<bf16_t>, gd, dim3(256), 0, s, dlogits, wr, T, d, E,
+                               static_cast<bf16_t*>(dxr));
+        } else {
+            hipLaunchKernelGGL(router_grad_partial_any_kernel<float>, ga, dim3(256), 0, s, dlogits,
+                               static_cast<const float*>(x), T, d, E, ct, partial);
+            hipLaunchKernelGGL(router_dx_any_kernel<float>, gd, dim3(256), 0, s, dlogits, wr, T, d, E,
+                               static_cast<float*>(dxr));
+        }
+        hipLaunchKernelGGL(router_grad_reduce_kernel, dim3((E * d + 63) / 64), dim3(256), 0, s, partial, chunks, E * d,
+                           grad_router);
+        return hipGetLastError();
+    }
     const dim3 g1((d / 2 + 127) / 128, chunks, (E + kRouterGradExperts - 1) / kRouterGradExperts), b1(128);
     const size_t lds = (size_t)ct * kRouterGradExperts * sizeof(float);
     if (lds > 48 * 1024) return hipErrorInvalidValue;  // 768 tokens a chunk: beyond 196608 tokens a launch
@@ -472,23 +541,24 @@ hipError_t launch_rmsnorm_backward(const void* x, const void* up, const float* w
                                    const void* residual_grad, int T, int d, void* grad_input, float* inv_rms,
                                    float* partial, float* grad_weight, bool bf16, hipStream_t s) {
     if (T <= 0) return hipSuccess;
-    if (!backward_width_ok(d, bf16)) return hipErrorInvalidValue;
     const dim3 g1((T + 3) / 4), b1(256);
     const int tiles = rmsnorm_grad_tiles(T);
-    const dim3 g2((d / 2 + 127) / 128, tiles), b2(128);
-    if (bf16) {
-        hipLaunchKernelGGL(rmsnorm_backward_kernel<bf16_t>, g1, b1, 0, s, static_cast<const bf16_t*>(x),
-                           static_cast<const bf16_t*>(up), weight, eps, static_cast<const bf16_t*>(residual_grad), T, d,
-                           static_cast<bf16_t*>(grad_input), inv_rms);
-        hipLaunchKernelGGL(rmsnorm_wgrad_partial_kernel<bf16_t>, g2, b2, 0, s, static_cast<const bf16_t*>(x),
-                           static_cast<const bf16_t*>(up), inv_rms, T, d, partial);
-    } else {
-        hipLaunchKernelGGL(rmsnorm_backward_kernel<float>, g1, b1, 0, s, static_cast<const float*>(x),
-                           static_cast<const float*>(up), weight, eps, static_cast<const float*>(residual_grad), T, d,
-                           static_cast<float*>(grad_input), inv_rms);
-        hipLaunchKernelGGL(rmsnorm_wgrad_partial_kernel<float>, g2, b2, 0, s, static_cast<const float*>(x),
-                           static_cast<const float*>(up), inv_rms, T, d, partial);
-    }
+    const bool wide = backward_width_ok(d, bf16);
+    auto go = [&](auto tag, auto piece) {
+        using XT = decltype(tag);
+        using V = decltype(piece);
+        hipLaunchKernelGGL((rmsnorm_backward_kernel<XT, V>), g1, b1, 0, s, static_cast<const XT*>(x),
+                           static_cast<const XT*>(up), weight, eps, static_cast<const XT*>(residual_grad), T, d,
+                           static_cast<XT*>(grad_input), inv_rms);
+        if (V::N > 1)
+            hipLaunchKernelGGL(rmsnorm_wgrad_partial_kernel<XT>, dim3((d / 2 + 127) / 128, tiles), dim3(128), 0, s,
+                               static_cast<const XT*>(x), static_cast<const XT*>(up), inv_rms, T, d, partial);
+        else
+            hipLaunchKernelGGL(rmsnorm_wgrad_partial_any_kernel<XT>, dim3((d + 255) / 256, tiles), dim3(256), 0, s,
+                               static_cast<const XT*>(x), static_cast<const XT*>(up), inv_rms, T, d, partial);
+    };
+    if (bf16) { if (wide) go(bf16_t{}, Vec16<bf16_t>{}); else go(bf16_t{}, Vec1<bf16_t>{}); }
+    else { if (wide) go(float{}, Vec16<float>{}); else go(float{}, Vec1<float>{}); }
     hipLaunchKernelGGL(router_grad_reduce_kernel, dim3((d + 63) / 64), dim3(256), 0, s, partial, tiles, d, grad_weight);
     return hipGetLastError();
 }

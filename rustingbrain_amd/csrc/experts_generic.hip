@@ -1,7 +1,9 @@
 // Grouped expert products for any shape and dtype: the fallback when a shape
 // does not fit the MFMA kernels (tiny widths, odd sizes) and the path for f32
 // and f32-activation layers.  A 16x16 thread block computes a 16x16 output tile
-// from 16-wide K slices staged in LDS; accumulation is f32 in index order.
+// from 16-wide K slices staged in LDS; accumulation is f32 in index order.  Like the matrix-core
+// kernels, the gate/up launch can keep the pre-activations for a backward pass (`gu_out`), and a
+// down-shaped launch can apply SwiGLU's backward to its rows on the way out (`bw_gu`).
 #include "rbmoe_kernels.h"
 
 namespace rbmoe {
@@ -16,7 +18,7 @@ __global__ __launch_bounds__(256) void grouped_generic_kernel(
     size_t w_expert_stride, const float* __restrict__ scales, size_t s_expert_stride, int N, int K,
     const int* __restrict__ tile_expert, const int* __restrict__ tile_row0,
     const int* __restrict__ tile_rows, const int* __restrict__ ntiles, int dense_rows,
-    AT* __restrict__ out) {
+    AT* __restrict__ out, AT* __restrict__ gu_out, const AT* __restrict__ bw_gu) {
     constexpr int TM = kGenericTileM, TN = 16, TK = 16;
     __shared__ float As[TM][TK + 1];
     __shared__ float Wg[TN][TK + 1];
@@ -66,8 +68,23 @@ __global__ __launch_bounds__(256) void grouped_generic_kernel(
             accg *= sc[n];
             if (SWIGLU) accu *= sc[N + n];
         }
-        const float v = SWIGLU ? silu_f32(accg) * accu : accg;
-        out[(size_t)(row0 + ty) * N + n] = from_f32<AT>(v);
+        const size_t row = (size_t)(row0 + ty);
+        if (SWIGLU) {
+            if (gu_out != nullptr) {  // pre-activations G | U [rows, 2 N]
+                gu_out[row * 2 * N + n] = from_f32<AT>(accg);
+                gu_out[row * 2 * N + N + n] = from_f32<AT>(accu);
+            }
+            out[row * N + n] = from_f32<AT>(silu_f32(accg) * accu);
+        } else if (bw_gu != nullptr) {
+            // SwiGlu::backward (src/ffn.rs:87-120): the product row is the gradient of the hidden row;
+            // dG = dH * U * silu'(G), dU = dH * silu(G) go to `gu_out`, `out` is not written.
+            const float gv = to_f32(bw_gu[row * 2 * N + n]), uv = to_f32(bw_gu[row * 2 * N + N + n]);
+            const float sg = 1.0f / (1.0f + __expf(-gv));
+            gu_out[row * 2 * N + n] = from_f32<AT>(accg * uv * (sg * (1.0f + gv * (1.0f - sg))));  // silu', src/ffn.rs:235-238
+            gu_out[row * 2 * N + N + n] = from_f32<AT>(accg * (gv * sg));
+        } else {
+            out[row * N + n] = from_f32<AT>(accg);
+        }
     }
 }
 
@@ -80,12 +97,14 @@ static hipError_t launch_t(const GroupedArgs& g, hipStream_t s) {
         hipLaunchKernelGGL((grouped_generic_kernel<AT, WT, true>), grid, block, 0, s,
                            static_cast<const AT*>(g.a), g.row_index, static_cast<const WT*>(g.w),
                            g.w_expert_stride, g.scales, g.s_expert_stride, g.N, g.K, g.tile_expert,
-                           g.tile_row0, g.tile_rows, g.ntiles, g.dense_rows, static_cast<AT*>(g.out));
+                           g.tile_row0, g.tile_rows, g.ntiles, g.dense_rows, static_cast<AT*>(g.out),
+                           static_cast<AT*>(g.gu_out), static_cast<const AT*>(g.swiglu_grad_gu));
     else
         hipLaunchKernelGGL((grouped_generic_kernel<AT, WT, false>), grid, block, 0, s,
                            static_cast<const AT*>(g.a), g.row_index, static_cast<const WT*>(g.w),
                            g.w_expert_stride, g.scales, g.s_expert_stride, g.N, g.K, g.tile_expert,
-                           g.tile_row0, g.tile_rows, g.ntiles, g.dense_rows, static_cast<AT*>(g.out));
+                           g.tile_row0, g.tile_rows, g.ntiles, g.dense_rows, static_cast<AT*>(g.out),
+                           static_cast<AT*>(g.gu_out), static_cast<const AT*>(g.swiglu_grad_gu));
     return hipGetLastError();
 }
 

@@ -619,6 +619,21 @@ int rbmoe_set_weight(rbmoe_layer* L, int32_t which, int32_t expert, const void* 
                 HIP_TRY(ctx, hipMemcpy2D(base, (size_t)2 * Fw * 4, tr.data(), (size_t)Fw * 4, (size_t)Fw * 4, (size_t)d,
                                          hipMemcpyHostToDevice));
             }
+        } else if (!L->use_stream) {
+            // plain row-major bf16, as the any-shape product kernel reads its weights
+            const uint16_t* h = static_cast<const uint16_t*>(src);
+            std::vector<uint16_t> tr(n);
+            for (int r = 0; r < rows; ++r)
+                for (int cc = 0; cc < cols; ++cc) tr[(size_t)cc * rows + r] = h[(size_t)r * cols + cc];
+            if (is_down) {
+                uint16_t* tdst = static_cast<uint16_t*>(shared_w ? L->swdT.p : L->wdT.p) + (shared_w ? 0 : (size_t)expert * Fw * d);
+                HIP_TRY(ctx, hipMemcpy(tdst, tr.data(), n * 2, hipMemcpyHostToDevice));
+            } else {
+                uint16_t* base = static_cast<uint16_t*>(shared_w ? L->swguT.p : L->wguT.p) +
+                                 (shared_w ? 0 : (size_t)expert * d * 2 * Fw) + (is_up ? Fw : 0);
+                HIP_TRY(ctx, hipMemcpy2D(base, (size_t)2 * Fw * 2, tr.data(), (size_t)Fw * 2, (size_t)Fw * 2, (size_t)d,
+                                         hipMemcpyHostToDevice));
+            }
         } else {
             // packed bf16; column steps of 16 never straddle the two halves of [d, 2F]
             std::vector<uint16_t> plain(n), tr(n), trp(n);
@@ -1065,9 +1080,8 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
     if (L->training) return RBMOE_OK;
     const rbmoe_config& c = L->cfg;
     const bool bf16_layer = L->use_stream && c.weight_dtype == RBMOE_BF16;
-    if (!bf16_layer && !L->use_f32_mc)
-        return fail(ctx, RBMOE_UNSUPPORTED,
-                    "the backward pass needs a bf16 layer (widths multiples of 64) or an all-f32 layer (multiples of 32)");
+    if (c.weight_dtype == RBMOE_I8)  // as in the reference: quantized experts are inference-only (src/ffn.rs:87-93)
+        return fail(ctx, RBMOE_UNSUPPORTED, "the backward pass is not defined for int8 weights");
     if (L->weights_set)
         return fail(ctx, RBMOE_INVALID_CONFIG, "enable training before the weights are set");
     const size_t E = c.num_experts, d = c.d_model, F = c.d_ff, Fs = L->Fs, T = L->max_T, S = L->max_S;
@@ -1077,10 +1091,12 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
         // 32-bit byte offsets into the widest operand of the backward products: [S, 2F] bf16
         if (std::max(S * 2 * F, T * 2 * Fs) * 2 >= ((size_t)1 << 32))
             return fail(ctx, RBMOE_UNSUPPORTED, "max_tokens x expert width too large for the backward products");
-    } else if (!f32_shape_ok((int)d, (int)(2 * F)) || (c.shared_expert && !f32_shape_ok((int)d, (int)(2 * Fs)))) {
+    } else if (L->use_f32_mc &&
+               (!f32_shape_ok((int)d, (int)(2 * F)) || (c.shared_expert && !f32_shape_ok((int)d, (int)(2 * Fs))))) {
         return fail(ctx, RBMOE_UNSUPPORTED, "expert width not supported by the backward products");
     }
-    const size_t ws = bf16_layer ? 2 : 4;  // bytes per element of the transposed weight copies
+    // (any other layer - odd widths, mixed dtypes - takes the any-shape kernels in both directions)
+    const size_t ws = dtype_size(c.weight_dtype);  // bytes per element of the transposed weight copies
     const size_t as = dtype_size(c.act_dtype);
     Plan p;
     p.add(&L->xc, T * d * as);
@@ -1203,16 +1219,20 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
     g.tile_row0 = (const int*)L->tile_row0.p;
     g.tile_rows = (const int*)L->tile_rows.p;
     g.ntiles = (const int*)L->ntiles.p;
-    g.max_tiles = S / (L->use_stream ? stream_tile_m() : f32_tile_m()) + E;
+    g.max_tiles = S / (L->use_stream ? stream_tile_m() : (L->use_f32_mc ? f32_tile_m() : kGenericTileM)) + E;
     g.dense_rows = -1;
     g.swiglu = false;
     g.group_m = L->group_m;
     GroupedArgs gh = g;  // grad_hidden = dY . Wdown
     gh.a = L->dy.p; gh.w = L->wdT.p; gh.w_expert_stride = (size_t)F * d; gh.N = F; gh.K = d;
     gh.swiglu_grad_gu = L->gu.p; gh.gu_out = L->dgu.p;  // the hidden gradient goes straight through SwiGLU's backward
-    auto prod = [&](const GroupedArgs& a) -> hipError_t {
-        return L->use_stream ? launch_grouped_stream(a, WeightKind::BF16, L->variant, s) : launch_grouped_f32(a, s);
+    const WeightKind wk = c.weight_dtype == RBMOE_F32 ? WeightKind::F32 : WeightKind::BF16;
+    auto prod_on = [&](const GroupedArgs& a, hipStream_t st) -> hipError_t {
+        if (L->use_stream) return launch_grouped_stream(a, WeightKind::BF16, L->variant, st);
+        if (L->use_f32_mc) return launch_grouped_f32(a, st);
+        return launch_grouped_generic(a, abf, wk, kGenericTileM, st);
     };
+    auto prod = [&](const GroupedArgs& a) -> hipError_t { return prod_on(a, s); };
     HIP_TRY(ctx, prod(gh));
     GroupedArgs gx = g;  // grad_input rows = dG . Wgate + dU . Wup
     gx.a = L->dgu.p; gx.w = L->wguT.p; gx.w_expert_stride = (size_t)d * 2 * F; gx.N = d; gx.K = 2 * F; gx.out = L->dxg.p;
@@ -1221,7 +1241,7 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
         // (it needs dG | dU, which the launch above has just written)
         HIP_TRY(ctx, hipEventRecord(ctx->ev_fork2, s));
         HIP_TRY(ctx, hipStreamWaitEvent(rs, ctx->ev_fork2, 0));
-        HIP_TRY(ctx, L->use_stream ? launch_grouped_stream(gx, WeightKind::BF16, L->variant, rs) : launch_grouped_f32(gx, rs));
+        HIP_TRY(ctx, prod_on(gx, rs));
         HIP_TRY(ctx, hipEventRecord(ctx->ev_join, rs));
     } else {
         HIP_TRY(ctx, prod(gx));

@@ -106,8 +106,8 @@ struct GroupedArgs {
     int max_tiles;
     int dense_rows;         // >= 0: one group of this many rows, no tile table (shared expert)
     void* out;              // [rows, N] activation dtype
-    void* gu_out = nullptr; // matrix-core gate/up kernels only (bf16 streaming, f32): [rows, 2N] pre-activations (gate | up) kept for a backward pass
-    // matrix-core down-shaped kernels only (bf16 streaming, f32): [rows, 2N] pre-activations of the forward pass.  The product rows are
+    void* gu_out = nullptr; // gate/up launches: [rows, 2N] pre-activations (gate | up) kept for a backward pass
+    // down-shaped launches: [rows, 2N] pre-activations of the forward pass.  The product rows are
     // then taken as the gradient of the hidden rows and SwiGLU's backward is applied on the way out: the
     // gradients of the pre-activations go to `gu_out` [rows, 2N] and `out` is not written.
     const void* swiglu_grad_gu = nullptr;
