@@ -98,13 +98,18 @@ __global__ __launch_bounds__(NE * 64) void logits_kernel(const XT* __restrict__ 
 #pragma unroll
     for (int l = 0; l < 8; ++l) la[l] = 0.0f;
     const bool vec = d % 8 == 0;
-    for (int c0 = 0; c0 < tail; c0 += kLogitChunk) {
-        const int np = min(PIECES, (tail - c0) / 8);  // pieces in this slice
-        __syncthreads();
-        for (int idx = tid; idx < kLogitTokens * np; idx += kLogitThreads) {
+    // A slice's pieces travel global -> registers -> LDS; the loads of the next slice are issued before the
+    // products of the current one, so their latency is covered by arithmetic.
+    constexpr int MAXP = (kLogitTokens * PIECES + kLogitThreads - 1) / kLogitThreads;
+    piece_t pre[MAXP];
+    auto fetch = [&](int c0) {
+        const int np = min(PIECES, (tail - c0) / 8);
+#pragma unroll
+        for (int u = 0; u < MAXP; ++u) {
+            const int idx = tid + u * kLogitThreads;
             const int r = idx / np, q = idx - r * np;
             piece_t v = {};
-            if (r < nt) {
+            if (idx < kLogitTokens * np && r < nt) {
                 const XT* src = x + (size_t)(t0 + r) * d + c0 + 8 * q;
                 if (vec) {
                     v = *reinterpret_cast<const piece_t*>(src);
@@ -115,9 +120,23 @@ __global__ __launch_bounds__(NE * 64) void logits_kernel(const XT* __restrict__ 
                     v = *reinterpret_cast<const piece_t*>(tmp);
                 }
             }
-            xs[r * STRIDE + q] = v;
+            pre[u] = v;
+        }
+    };
+    if (tail > 0) fetch(0);
+    for (int c0 = 0; c0 < tail; c0 += kLogitChunk) {
+        const int np = min(PIECES, (tail - c0) / 8);  // pieces in this slice
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < MAXP; ++u) {
+            const int idx = tid + u * kLogitThreads;
+            if (idx < kLogitTokens * np) {
+                const int r = idx / np, q = idx - r * np;
+                xs[r * STRIDE + q] = pre[u];
+            }
         }
         __syncthreads();
+        if (c0 + kLogitChunk < tail) fetch(c0 + kLogitChunk);
         if (has) {
             const float* wa = w0 + c0;
             int q = 0;
