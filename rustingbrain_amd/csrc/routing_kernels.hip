@@ -75,8 +75,10 @@ struct XPiece<float> {
 };
 
 // NE = experts (= waves) per workgroup.
-template <typename XT, int NE>
-__global__ __launch_bounds__(NE * 64) void logits_kernel(const XT* __restrict__ x,
+// (bf16 without AHEAD: 6 waves per SIMD, i.e. three workgroups on a compute unit, is what the launches of many
+// workgroups are tuned for - the bound keeps a later edit from quietly costing one of them)
+template <typename XT, int NE, bool AHEAD>
+__global__ __launch_bounds__(NE * 64, (!AHEAD && sizeof(XT) == 2) ? 6 : 2) void logits_kernel(const XT* __restrict__ x,
                                                                 const float* __restrict__ wr,
                                                                 const float* __restrict__ bias, int T, int d, int E,
                                                                 float* __restrict__ logits) {
@@ -98,45 +100,55 @@ __global__ __launch_bounds__(NE * 64) void logits_kernel(const XT* __restrict__ 
 #pragma unroll
     for (int l = 0; l < 8; ++l) la[l] = 0.0f;
     const bool vec = d % 8 == 0;
-    // A slice's pieces travel global -> registers -> LDS; the loads of the next slice are issued before the
-    // products of the current one, so their latency is covered by arithmetic.
+    // A slice's pieces travel global -> registers -> LDS.  AHEAD: the loads of the next slice are issued
+    // before the products of the current one, so their latency is covered by arithmetic - for launches of few
+    // workgroups; with several workgroups on a compute unit they cover for each other, and the registers the
+    // pieces in flight occupy would cost one of them.
     constexpr int MAXP = (kLogitTokens * PIECES + kLogitThreads - 1) / kLogitThreads;
     piece_t pre[MAXP];
+    auto load_piece = [&](int r, int c) {  // eight elements of row r from column c (zeros past the last row)
+        piece_t v = {};
+        if (r < nt) {
+            const XT* src = x + (size_t)(t0 + r) * d + c;
+            if (vec) {
+                v = *reinterpret_cast<const piece_t*>(src);
+            } else {  // rows are not 16-byte aligned: gather the eight elements
+                XT tmp[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) tmp[j] = src[j];
+                v = *reinterpret_cast<const piece_t*>(tmp);
+            }
+        }
+        return v;
+    };
     auto fetch = [&](int c0) {
         const int np = min(PIECES, (tail - c0) / 8);
 #pragma unroll
         for (int u = 0; u < MAXP; ++u) {
-            const int idx = tid + u * kLogitThreads;
-            const int r = idx / np, q = idx - r * np;
-            piece_t v = {};
-            if (idx < kLogitTokens * np && r < nt) {
-                const XT* src = x + (size_t)(t0 + r) * d + c0 + 8 * q;
-                if (vec) {
-                    v = *reinterpret_cast<const piece_t*>(src);
-                } else {  // rows are not 16-byte aligned: gather the eight elements
-                    XT tmp[8];
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) tmp[j] = src[j];
-                    v = *reinterpret_cast<const piece_t*>(tmp);
-                }
-            }
-            pre[u] = v;
+            const int idx = tid + u * kLogitThreads;  // over the full 64 x PIECES grid: no division by np
+            const int r = idx / PIECES, q = idx % PIECES;
+            pre[u] = (r < kLogitTokens && q < np) ? load_piece(r, c0 + 8 * q) : piece_t{};
         }
     };
-    if (tail > 0) fetch(0);
+    if (AHEAD && tail > 0) fetch(0);
     for (int c0 = 0; c0 < tail; c0 += kLogitChunk) {
         const int np = min(PIECES, (tail - c0) / 8);  // pieces in this slice
         __syncthreads();
+        if (AHEAD) {
 #pragma unroll
-        for (int u = 0; u < MAXP; ++u) {
-            const int idx = tid + u * kLogitThreads;
-            if (idx < kLogitTokens * np) {
+            for (int u = 0; u < MAXP; ++u) {
+                const int idx = tid + u * kLogitThreads;
+                const int r = idx / PIECES, q = idx % PIECES;
+                if (r < kLogitTokens && q < np) xs[r * STRIDE + q] = pre[u];
+            }
+        } else {
+            for (int idx = tid; idx < kLogitTokens * np; idx += kLogitThreads) {
                 const int r = idx / np, q = idx - r * np;
-                xs[r * STRIDE + q] = pre[u];
+                xs[r * STRIDE + q] = load_piece(r, c0 + 8 * q);
             }
         }
         __syncthreads();
-        if (c0 + kLogitChunk < tail) fetch(c0 + kLogitChunk);
+        if (AHEAD && c0 + kLogitChunk < tail) fetch(c0 + kLogitChunk);
         if (has) {
             const float* wa = w0 + c0;
             int q = 0;
@@ -993,8 +1005,13 @@ static hipError_t launch_router_t(const RouterArgs& a, hipStream_t s) {
     // eight experts (waves) per workgroup share one staged slice of 64 token rows
     constexpr int NE = 8;
     const int tiles_t = (a.T + kLogitTokens - 1) / kLogitTokens;
-    hipLaunchKernelGGL((logits_kernel<XT, NE>), dim3(tiles_t, (a.E + NE - 1) / NE), dim3(NE * 64), 0, s,
-                       static_cast<const XT*>(a.x), a.wr, a.bias, a.T, a.d, a.E, a.P);
+    const dim3 lgrid(tiles_t, (a.E + NE - 1) / NE);
+    if ((long long)lgrid.x * lgrid.y <= 512)  // at most two workgroups on a compute unit
+        hipLaunchKernelGGL((logits_kernel<XT, NE, true>), lgrid, dim3(NE * 64), 0, s, static_cast<const XT*>(a.x),
+                           a.wr, a.bias, a.T, a.d, a.E, a.P);
+    else
+        hipLaunchKernelGGL((logits_kernel<XT, NE, false>), lgrid, dim3(NE * 64), 0, s, static_cast<const XT*>(a.x),
+                           a.wr, a.bias, a.T, a.d, a.E, a.P);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     if (a.E <= 64)
