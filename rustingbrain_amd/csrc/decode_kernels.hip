@@ -467,7 +467,7 @@ hipError_t launch_route_small(const SmallRouteArgs& a, bool bf16, hipStream_t s)
 // ---------------------------------------------------------------------------
 // decode_gemm_kernel: out[row, n] for one tile of at most 32 rows and one block of 32
 // output features (gate/up: 32 gate rows and the matching 32 up rows of the packed weights).
-// The four waves of a workgroup take a quarter of the reduction steps each; a wave fetches
+// The waves of a workgroup take an equal share of the reduction steps each; a wave fetches
 // its weight fragments (1 KB per step and row block, straight from the packed layout) in
 // batches of kBatch steps so that tens of kilobytes are in flight, multiplies them on the
 // matrix cores against token fragments read from global memory (32 rows x K: they stay in
@@ -486,15 +486,26 @@ struct DecodeSide {
     int N, K, row0, rows;
 };
 
-template <bool SWIGLU, bool I8>
-__global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs g) {
-    __shared__ float red[4][2][16][64];
+// NW = waves of a workgroup, each with 1 / NW of the reduction steps: 4 for the gate/up product, 8 for the
+// down product (a third of the workgroups and twice the reduction length: with 8 waves every weight byte of
+// the launch is requested before the first multiply there as well).
+template <bool SWIGLU, bool I8, int NW>
+__global__ __launch_bounds__(NW * 64) void decode_gemm_kernel(DecodeGemmArgs g) {
+    __shared__ float red[NW][SWIGLU ? 2 : 1][16][64];
     const int fb = blockIdx.x;
     const int ty = blockIdx.y;
     DecodeSide sd;
-    if (ty < g.max_tiles) {
-        if (ty >= *g.ntiles) return;
-        const int expert = g.tile_expert[ty];
+    // One round trip for the whole tile table: the four entries are fetched side by side (a stale entry past
+    // *ntiles is read and dropped), not one after the other - with cold caches every dependent scalar load in
+    // front of the first weight load is a few hundred nanoseconds of a launch that lasts ten microseconds.
+    const bool routed = ty < g.max_tiles;
+    const int tix = routed ? ty : 0;
+    const int live_tiles = *g.ntiles;
+    const int t_expert = g.tile_expert[tix], t_row0 = g.tile_row0[tix], t_rows = g.tile_rows[tix];
+    asm volatile("" ::"s"(live_tiles), "s"(t_expert), "s"(t_row0), "s"(t_rows));  // all four here, not sunk into the branches
+    if (routed) {
+        if (ty >= live_tiles) return;
+        const int expert = t_expert;
         sd.a = static_cast<const bf16_t*>(g.a);
         sd.row_index = g.row_index;
         sd.w = static_cast<const char*>(g.w) + (size_t)expert * g.w_expert_stride * (I8 ? 1 : 2);
@@ -502,8 +513,8 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs g) {
         sd.out = static_cast<bf16_t*>(g.out);
         sd.N = g.N;
         sd.K = g.K;
-        sd.row0 = g.tile_row0[ty];
-        sd.rows = g.tile_rows[ty];
+        sd.row0 = t_row0;
+        sd.rows = t_rows;
     } else {
         const int st = ty - g.max_tiles;
         sd.a = static_cast<const bf16_t*>(g.a_shared);
@@ -523,7 +534,7 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs g) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int K = sd.K;
     const int steps = K / 16;
-    const int chunk = (steps + 3) / 4;
+    const int chunk = (steps + NW - 1) / NW;
     const int g0 = min(steps, wave * chunk), g1 = min(steps, g0 + chunk);
 
     // packed weights: row block rb starts at rb * K * 32 elements; step s, lane l at (s * 64 + l) * 16 bytes
@@ -542,8 +553,7 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs g) {
     };
     // token fragment: lane -> token lane % 32, columns 16 s + 8 (lane / 32) .. + 7
     const int trow = (lane & 31) < sd.rows ? (lane & 31) : 0;
-    const int grow = sd.row_index ? sd.row_index[sd.row0 + trow] : sd.row0 + trow;
-    const bf16_t* arow = sd.a + (size_t)grow * K + 8 * (lane >> 5);
+    int grow = sd.row_index ? sd.row_index[sd.row0 + trow] : sd.row0 + trow;  // awaited after the weight loads
 
     floatx16 acc0, acc1;
 #pragma unroll
@@ -551,13 +561,25 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs g) {
 
     for (int s0 = g0; s0 < g1; s0 += kBatch) {
         bf16x8 wa[kBatch], wb[kBatch], tf[kBatch];
+        // the weights first: the address of a token row depends on a load of its own (the row index), and
+        // loads are issued in order - nothing of the stream may queue up behind that wait
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) {
             const int s = min(s0 + u, g1 - 1);
             wa[u] = wfrag(w0, s);
             if constexpr (SWIGLU) wb[u] = wfrag(w1, s);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // (the empty statement pins the first use of the row index, and with it the wait for it, below the
+        // weight loads; the barriers keep every load of the batch ahead of the first multiply)
+        asm volatile("" : "+v"(grow));
+        const bf16_t* arow = sd.a + (size_t)grow * K + 8 * (lane >> 5);
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const int s = min(s0 + u, g1 - 1);
             tf[u] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(arow + 16 * s));
         }
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) {
             if (s0 + u < g1) {
@@ -572,17 +594,22 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs g) {
         if constexpr (SWIGLU) red[wave][1][v][lane] = acc1[v];
     }
     __syncthreads();
-    // accumulator element v of lane l: feature 8 (v / 4) + 4 (l / 32) + v % 4, token l % 32
+    // accumulator element v of lane l: feature 8 (v / 4) + 4 (l / 32) + v % 4, token l % 32;
+    // the partial sums of the waves are added in wave order
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int idx = i * 256 + tid;
+    for (int i = 0; i < 1024 / (NW * 64); ++i) {
+        const int idx = i * (NW * 64) + tid;
         const int v = idx >> 6, l = idx & 63;
         const int token = l & 31;
         const int f = 8 * (v >> 2) + 4 * (l >> 5) + (v & 3);
-        float y = ((red[0][0][v][l] + red[1][0][v][l]) + red[2][0][v][l]) + red[3][0][v][l];
+        float y = red[0][0][v][l];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) y += red[w][0][v][l];
         if constexpr (I8) y *= sd.scales[fb * 32 + f];
         if constexpr (SWIGLU) {
-            float u = ((red[0][1][v][l] + red[1][1][v][l]) + red[2][1][v][l]) + red[3][1][v][l];
+            float u = red[0][1][v][l];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) u += red[w][1][v][l];
             if constexpr (I8) u *= sd.scales[sd.N + fb * 32 + f];
             y = silu_bf16_grade(y) * u;
         }
@@ -597,13 +624,13 @@ hipError_t launch_decode_gemm(const DecodeGemmArgs& g, WeightKind wk, hipStream_
     const int tiles = g.max_tiles + shared_tiles;
     if (tiles <= 0) return hipSuccess;
     const int widest = g.a_shared ? (g.N > g.N_shared ? g.N : g.N_shared) : g.N;
-    const dim3 grid(widest / 32, tiles), block(256);
+    const dim3 grid(widest / 32, tiles);
     if (wk == WeightKind::BF16) {
-        if (g.swiglu) hipLaunchKernelGGL((decode_gemm_kernel<true, false>), grid, block, 0, s, g);
-        else hipLaunchKernelGGL((decode_gemm_kernel<false, false>), grid, block, 0, s, g);
+        if (g.swiglu) hipLaunchKernelGGL((decode_gemm_kernel<true, false, 4>), grid, dim3(256), 0, s, g);
+        else hipLaunchKernelGGL((decode_gemm_kernel<false, false, 8>), grid, dim3(512), 0, s, g);
     } else if (wk == WeightKind::I8) {
-        if (g.swiglu) hipLaunchKernelGGL((decode_gemm_kernel<true, true>), grid, block, 0, s, g);
-        else hipLaunchKernelGGL((decode_gemm_kernel<false, true>), grid, block, 0, s, g);
+        if (g.swiglu) hipLaunchKernelGGL((decode_gemm_kernel<true, true, 4>), grid, dim3(256), 0, s, g);
+        else hipLaunchKernelGGL((decode_gemm_kernel<false, true, 8>), grid, dim3(512), 0, s, g);
     } else {
         return hipErrorInvalidValue;
     }
