@@ -6,10 +6,16 @@
 //
 //   moe_tutorial --cpu-checks   configuration, accounting and error paths only (no GPU)
 //   moe_tutorial                everything, on GPU 0
+//   moe_tutorial --rbw FILE     parses a `.rbw` weight snapshot and prints what it holds (no GPU)
+//   moe_tutorial --rbw FILE ROWS.f32 TOKENS OUT
+//                               also loads its sparse blocks onto GPU 0 and runs the block step
+//                               x + layer(rmsnorm(x)) on the rows of ROWS.f32 ([TOKENS, d_model] f32),
+//                               writing each block's output to OUT.<block> (f32)
 #include <cmath>
 #include <cstdio>
 #include <cstring>
 
+#include "rbw.hpp"
 #include "rusting_brain_moe.hpp"
 
 using namespace rusting_brain;
@@ -222,8 +228,65 @@ static void gpu_checks() {
     }));
 }
 
+// sum of the values `load_bin` would restore, in double: a checksum that the Python reader can reproduce
+static double checksum(const rbw::Param& p) {
+    double s = 0.0;
+    if (p.q.empty()) {
+        for (float v : p.values) s += (double)v;
+    } else {
+        for (size_t r = 0; r < p.rows; ++r)
+            for (size_t c = 0; c < p.cols; ++c) s += (double)((float)p.q[r * p.cols + c] * p.scales[r]);
+    }
+    return s;
+}
+
+static int rbw_mode(int argc, char** argv) {
+    const std::string path = argv[2];
+    const rbw::Snapshot snap = rbw::read(path);
+    std::printf("precision %s parameters %zu optimizer_step %llu\n", snap.precision.c_str(), snap.params.size(),
+                (unsigned long long)snap.optimizer_step);
+    const std::vector<rbw::MoeBlock> blocks = rbw::moe_blocks(snap);
+    for (const rbw::MoeBlock& b : blocks) {
+        std::printf("block %zu experts %zu shared %d norm %.9g router %.9g gate0 %.9g down_last %.9g\n", b.block,
+                    b.experts.size(), b.has_shared ? 1 : 0, b.norm ? checksum(*b.norm) : 0.0, checksum(*b.router),
+                    checksum(*b.experts.front().gate),
+                    checksum(b.has_shared ? *b.shared.down : *b.experts.back().down));
+    }
+    if (argc < 6) return 0;
+    const size_t tokens = (size_t)std::atol(argv[4]);
+    const size_t d = snap.config.at("d_model").as_size("d_model");
+    Matrix x(tokens, d);
+    std::FILE* f = std::fopen(argv[3], "rb");
+    if (!f || std::fread(x.data.data(), 4, x.data.size(), f) != x.data.size()) {
+        std::printf("FAILED: cannot read %zu x %zu f32 from %s\n", tokens, d, argv[3]);
+        return 2;
+    }
+    std::fclose(f);
+    auto layers = rbw::load_moe_layers(path, Device::open(0), tokens);
+    for (size_t i = 0; i < layers.size(); ++i) {
+        const Matrix out = layers[i]->forward_block(x);
+        const std::string name = std::string(argv[5]) + "." + std::to_string(blocks[i].block);
+        std::FILE* o = std::fopen(name.c_str(), "wb");
+        if (!o || std::fwrite(out.data.data(), 4, out.data.size(), o) != out.data.size()) {
+            std::printf("FAILED: cannot write %s\n", name.c_str());
+            return 2;
+        }
+        std::fclose(o);
+        std::printf("block %zu ran on %s\n", blocks[i].block, layers[i]->kernel_name().c_str());
+    }
+    return 0;
+}
+
 int main(int argc, char** argv) {
     const bool cpu_only = argc > 1 && std::strcmp(argv[1], "--cpu-checks") == 0;
+    if (argc > 2 && std::strcmp(argv[1], "--rbw") == 0) {
+        try {
+            return rbw_mode(argc, argv);
+        } catch (const std::exception& e) {
+            std::printf("FAILED with exception: %s\n", e.what());
+            return 2;
+        }
+    }
     try {
         cpu_checks();
         if (!cpu_only) gpu_checks();

@@ -195,6 +195,13 @@ class MoeLayer {
         set(RBMOE_W_SHARED_DOWN, 0, down);
     }
 
+    // One weight matrix by its id (RBMOE_W_*): f32 values, or the int8 values and per-row scales of a quantized
+    // checkpoint as they are stored (DeviceParam::new, src/gpu_transformer.rs:471-490).
+    void set_weight(int which, int expert, const Matrix& w) { set(which, expert, w); }
+    void set_weight_q8(int which, int expert, const int8_t* q, const float* scales, size_t rows, size_t cols) {
+        check(rbmoe_set_weight(layer_, which, expert, q, RBMOE_I8, scales, (int32_t)rows, (int32_t)cols), device_->raw());
+    }
+
     Matrix forward(const Matrix& input) { return forward_train(input, Layout{}).first; }
 
     std::pair<Matrix, MoeCache> forward_train(const Matrix& input, const Layout& layout) {

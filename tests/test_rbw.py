@@ -151,3 +151,89 @@ def test_sparse_blocks_of_a_snapshot_run_on_the_device(tmp_path, device, precisi
         assert_routing_identical(cache_b, ref_b)
         assert rel_l2(out_b, want) <= 2e-2
         layer.close()
+
+
+# ------------------------------------------------------------------ the C++ host mirror's reader (host/rbw.hpp)
+def _cpp(*args):
+    import os
+    import subprocess
+    from conftest import ROOT
+    exe = os.path.join(ROOT, "rustingbrain_amd", "host", "moe_tutorial")
+    if not os.path.exists(exe):
+        from rustingbrain_amd import build
+        build.build_host()
+    return subprocess.run([exe, "--rbw", *args], capture_output=True, text=True, timeout=120)
+
+
+def _checksum(p):
+    return float(p.dequantized().astype(np.float64).sum())
+
+
+@pytest.mark.parametrize("precision", ["F32", "Q8"])
+def test_cpp_reader_sees_what_the_python_reader_sees(tmp_path, precision):
+    c = dict(CONFIG)
+    params, _ = model_params(c)
+    path = str(tmp_path / "model.rbw")
+    rbw.write(path, c, params, precision, optimizer_step=11)
+    res = _cpp(path)
+    assert res.returncode == 0, res.stdout + res.stderr
+    lines = res.stdout.strip().splitlines()
+    assert lines[0] == f"precision {precision} parameters {len(params)} optimizer_step 11"
+    blocks = rbw.moe_blocks(rbw.read(path))
+    assert len(lines) == 1 + len(blocks)
+    for line, b in zip(lines[1:], blocks):
+        f = line.split()
+        assert f[:6] == ["block", str(b.block), "experts", str(len(b.experts)), "shared", "1"]
+        got = dict(zip(f[6::2], (float(v) for v in f[7::2])))
+        want = {"norm": _checksum(b.norm), "router": _checksum(b.router), "gate0": _checksum(b.experts[0]["gate"]),
+                "down_last": _checksum(b.shared["down"])}
+        for name, v in want.items():
+            assert abs(got[name] - v) <= 1e-7 * max(1.0, abs(v)), (name, got[name], v)
+
+
+def test_cpp_reader_rejects_what_the_reference_rejects(tmp_path):
+    c = dict(CONFIG)
+    params, _ = model_params(c)
+    good = str(tmp_path / "model.rbw")
+    rbw.write(good, c, params, "F32")
+    blob = open(good, "rb").read()
+    bad = str(tmp_path / "bad.rbw")
+    for data, message in ((b"RBOPT001" + blob[8:], "not a RustingBrain weight file"), (blob[:-5], "truncated"),
+                          (blob + b"\0\0", "bytes follow the last parameter")):
+        open(bad, "wb").write(data)
+        res = _cpp(bad)
+        assert res.returncode == 2 and message in res.stdout, res.stdout
+    rbw.write(bad, c, params[:-1], "F32")
+    res = _cpp(bad)
+    assert res.returncode == 2 and "parameters" in res.stdout
+    wrong = list(params)
+    wrong[1 + 6] = np.zeros((5, 5), np.float32)
+    rbw.write(bad, c, wrong, "F32")
+    res = _cpp(bad)
+    assert res.returncode == 2 and "5x5 parameter where the model has 96x64" in res.stdout
+    rbw.write(bad, dict(c, lora={"rank": 4, "alpha": 8.0, "seed": 1}), params, "F32")
+    res = _cpp(bad)
+    assert res.returncode == 2 and "LoRA" in res.stdout
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("precision", ["Q8", "F32"])
+def test_cpp_host_loads_a_snapshot_and_runs_the_block_step(tmp_path, device, precision):
+    """Both hosts load the same file onto the device and run the same block step: identical bits."""
+    c = dict(CONFIG)
+    params, _ = model_params(c)
+    path = str(tmp_path / "model.rbw")
+    rbw.write(path, c, params, precision)
+    x = synth.round_bf16(synth.normal((40, c["d_model"]), 1.0, 9, 1))
+    rows = str(tmp_path / "rows.f32")
+    x.astype("<f4").tofile(rows)
+    out = str(tmp_path / "out")
+    res = _cpp(path, rows, "40", out)
+    assert res.returncode == 0, res.stdout + res.stderr
+    layers = rbw.load_moe_layers(path, device, max_tokens=40)
+    for layer, blk in zip(layers, rbw.moe_blocks(rbw.read(path))):
+        want, _ = layer.forward_block(x)
+        got = np.fromfile(f"{out}.{blk.block}", dtype="<f4").reshape(40, c["d_model"])
+        assert np.array_equal(got, want)
+        assert f"block {blk.block} ran on mfma_bf16" in res.stdout
+        layer.close()
