@@ -85,7 +85,8 @@ __device__ __forceinline__ void token_phase_serial(float* row, int t, int E, int
 // adds the E values up in the same order, fetching them with shuffles) and the running sum of the selected
 // probabilities.  A round's winner is the largest 64-bit key (probability bits above the inverted index:
 // probabilities are >= +0, so their bit patterns order like their values, and among equal ones the lower
-// index wins, as the reference's strict `>` scan does); a taken expert's key is 0.
+// index wins, as the reference's strict `>` scan does); a taken expert's key is 0, and so is a NaN's, which the
+// scan never prefers to anything and never replaces once it is the candidate.
 template <int G>
 __device__ __forceinline__ void token_phase_lanes(float* row_lds, int t, int j, int E, int k, const uint8_t* valid,
                                                   float* P, float* lse, float* lsev, int* sexp, int* expert_of,
@@ -123,7 +124,14 @@ __device__ __forceinline__ void token_phase_lanes(float* row_lds, int t, int j, 
         }
         return;
     }
-    unsigned long long key = mine ? (((unsigned long long)__float_as_uint(p) << 32) | (0xffffffffu - (unsigned)j)) : 0ull;
+    // A NaN is never greater than anything and nothing is greater than a NaN (src/moe.rs:566-581): a NaN takes
+    // part in no comparison - it is selected only when it is the first expert not yet taken, and then nothing
+    // replaces it.
+    const bool is_nan = p != p;
+    unsigned long long key =
+        (mine && !is_nan) ? (((unsigned long long)__float_as_uint(p) << 32) | (0xffffffffu - (unsigned)j)) : 0ull;
+    bool taken = !mine;
+    const unsigned long long gmask = G == 64 ? ~0ull : ((1ull << G) - 1ull);
     float total = 0.0f;
     float my_p = 0.0f;  // lane r keeps round r's probability
     int my_e = -1;
@@ -134,10 +142,17 @@ __device__ __forceinline__ void token_phase_lanes(float* row_lds, int t, int j, 
             const unsigned long long other = __shfl_xor(best, o);
             best = other > best ? other : best;
         }
-        const int be = (int)(0xffffffffu - (unsigned)(best & 0xffffffffull));
-        const float bv = __uint_as_float((unsigned)(best >> 32));
+        const unsigned long long untaken = (__ballot(!taken) >> base) & gmask;
+        const unsigned long long nans = (__ballot(!taken && is_nan) >> base) & gmask;
+        const int first = __ffsll((long long)untaken) - 1;  // k <= E: some expert is always left
+        const bool first_nan = ((nans >> first) & 1ull) != 0ull;
+        const int be = (first_nan || best == 0ull) ? first : (int)(0xffffffffu - (unsigned)(best & 0xffffffffull));
+        const float bv = __shfl(p, base + be);
         total = __fadd_rn(total, bv);
-        if (j == be) key = 0ull;
+        if (j == be) {
+            key = 0ull;
+            taken = true;
+        }
         if (j == r) {
             my_p = bv;
             my_e = be;

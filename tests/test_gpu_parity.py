@@ -137,6 +137,35 @@ def test_nan_row_routes_in_index_order(device):
     layer.close()
 
 
+@pytest.mark.parametrize("T,act", [(40, "f32"), (40, "bf16"), (3, "bf16")])   # (3, bf16): the single-workgroup routing
+def test_rows_whose_logits_overflow_route_like_the_cpu_path(device, T, act):
+    """A row of huge values gives infinite logits: `v - max` is inf - inf = NaN for the winners and -inf for the
+    rest, the sum of exponentials is NaN, `sum > 0` is false and the row is left un-normalised
+    (src/activations.rs:56-70); no NaN is ever 'greater', so the row routes to experts 0..k-1
+    (src/moe.rs:566-581).  A row of zeros beside it is the plain uniform case."""
+    d = 16 if act == "f32" else 64
+    t = synth.make(small_workload(d=d, E=6, k=2, F=8 if act == "f32" else 64, T=T, seed=4, act=act, wt=act))
+    t.x[1, :] = synth.round_bf16(np.float32(3.0e38))
+    t.x[2, :] = 0.0
+    t.router[0, :] = 2.0                                  # +inf
+    t.router[1, :] = -2.0                                 # -inf
+    t.router[2, :] = np.where(np.arange(d) % 2, 2.0, -2.0)  # inf - inf = NaN
+    t.router[3, :] = 2.0                                  # +inf again
+    ref = oracle_layer(t).forward(t.x)
+    layer = gpu_layer(device, t)
+    out, cache = layer.forward_train(t.x)
+    assert np.array_equal(cache.expert_of, ref.expert_of)
+    assert np.array_equal(cache.probabilities.view(np.uint32) & 0x7fffffff == 0x7f800000,
+                          ref.probabilities.view(np.uint32) & 0x7fffffff == 0x7f800000)
+    assert np.array_equal(np.isnan(cache.probabilities), np.isnan(ref.probabilities))
+    finite = ~np.isnan(ref.probabilities)
+    assert np.array_equal(cache.probabilities[finite], ref.probabilities[finite])
+    assert cache.expert_of.reshape(T, 2)[2].tolist() == [0, 1]          # all-equal probabilities: lowest indices
+    assert np.array_equal(cache.counts, ref.counts) and np.array_equal(cache.perm_slot, ref.perm_slot)
+    assert layer.kernel_name() == {"f32": "generic", "bf16": "mfma_bf16_decode" if T <= 32 else "mfma_bf16_stream"}[act]
+    layer.close()
+
+
 # ------------------------------------------------------------------ the reference's own MoE tests, on the GPU
 def one_hot_router(E, d, strength):
     w = np.zeros((E, d), np.float32)

@@ -119,6 +119,25 @@ def test_router_logits_shape_and_bias():
             assert base[t, e] == np.float32(orc.dot8(x[t], w[e]))
 
 
+def test_route_never_compares_a_nan():
+    # reference src/moe.rs:566-581: `best` starts as the first expert not yet taken and is replaced only when
+    # `p[e] > p[best]`, which is false whenever either side is NaN.  Worked by hand from that loop:
+    nan = np.float32(np.nan)
+    cases = [
+        ([nan, 0.0, nan, nan, 0.0, 0.0], 2, [0, 1]),   # a NaN in front is kept; then 0.0 is kept against NaN and 0.0
+        ([0.2, nan, 0.5, 0.3], 2, [2, 3]),             # a NaN further on is never preferred
+        ([nan, 0.9, 0.1], 2, [0, 1]),
+        ([0.1, nan, nan], 3, [0, 1, 2]),               # once the numbers are used up the NaNs come in index order
+        ([nan, nan, 0.7, 0.2], 3, [0, 1, 2]),
+    ]
+    for probs, k, want in cases:
+        experts, gates = orc.route(np.array([probs], np.float32), k)
+        assert experts.tolist() == want, (probs, experts.tolist())
+    # the sum of the selected probabilities is NaN there, `total > 0` is false and the gates stay un-normalised
+    experts, gates = orc.route(np.array([[nan, 0.9, 0.1]], np.float32), 2)
+    assert np.isnan(gates[0]) and gates[1] == np.float32(0.9)
+
+
 # ------------------------------------------------------------------ softmax
 def ramp(n):  # reference src/gpu_model.rs:3775-3779
     return np.array([((i * 37) % 23) / 11.0 - 1.0 for i in range(n)], np.float32)
