@@ -162,3 +162,47 @@ def test_backward_sweep(device, first):
             close("shared gate", layer.weight_grad(L.W_SHARED_GATE), ref.grad_shared[0])
             close("shared down", layer.weight_grad(L.W_SHARED_DOWN), ref.grad_shared[2])
         layer.close()
+
+
+@pytest.mark.parametrize("first", range(0, 120, 40))
+def test_block_step_sweep(device, first):
+    """x + layer(rmsnorm(x)): the norm in front (its own kernel, or inside the routing kernel of a few tokens) must
+    hand the router the very rows the CPU path normalises, whatever the rows hold."""
+    for seed in range(first, first + 40):
+        rng = np.random.default_rng(5000 + seed)
+        t, valid, bias, what = draw_layer(rng, 5000 + seed, FORWARD_MODES, [1, 2, 5, 31, 32, 33, 70])
+        w = t.workload
+        T, d = w.tokens, w.d_model
+        bf16 = w.act_dtype == "bf16"
+        rounder = synth.round_bf16 if bf16 else None
+        norm_weight = (np.float32(1) + synth.normal((d,), 0.2, seed, 77)).astype(np.float32)
+        eps = float(rng.choice([1e-6, 1e-5, 1e-2]))
+        x = (t.x * np.float32(rng.choice([1.0, 1e-3, 50.0]))).astype(np.float32)
+        if bf16:
+            x = synth.round_bf16(x)
+        special = str(rng.choice(["none", "nan", "huge", "zeros", "tiny"]))
+        if special == "nan":
+            x[rng.integers(0, T), rng.integers(0, d)] = np.nan
+        elif special == "huge":      # the sum of squares overflows: inverse rms 0, normed row 0
+            x[rng.integers(0, T), :] = synth.round_bf16(np.float32(3e38))
+        elif special == "zeros":     # eps alone under the root
+            x[::2, :] = 0
+        elif special == "tiny":      # squares underflow
+            x[rng.integers(0, T), :] = synth.round_bf16(np.float32(1e-30))
+        what += f" rows {special} eps {eps}"
+        want, _, ref = oracle_layer(t).forward_block(x, norm_weight, eps, valid=valid, router_bias=bias, threads=4,
+                                                     round_normed=rounder)
+        cfg = rb.MoeConfig(w.num_experts, w.experts_per_token, w.d_ff, w.shared_expert)
+        layer = rb.MoeLayer(d, cfg, device, act_dtype=w.act_dtype, weight_dtype=w.weight_dtype, max_tokens=T,
+                            shared_d_ff=w.shared_d_ff if w.shared_expert else 0)
+        layer.set_feed_forward_norm(norm_weight, eps)
+        layer.load_tensors(t)
+        layout = rb.Layout(valid=None if valid is None else [bool(v) for v in valid])
+        out, cache = layer.forward_block(x, layout, router_bias=bias)
+        for name in ("expert_of", "counts", "offsets"):
+            assert np.array_equal(getattr(cache, name), getattr(ref, name)), f"{what}: {name}"
+        assert same_bits_or_same_nans(cache.probabilities, ref.probabilities), f"{what}: probabilities"
+        assert same_bits_or_same_nans(cache.gate_of, ref.gate_of), f"{what}: gates"
+        tol = 1e-5 if (w.act_dtype == "f32" and w.weight_dtype == "f32") else 2e-2
+        assert rel_finite(out, want) <= tol, f"{what}: output"
+        layer.close()
