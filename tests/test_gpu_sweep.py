@@ -206,3 +206,72 @@ def test_block_step_sweep(device, first):
         tol = 1e-5 if (w.act_dtype == "f32" and w.weight_dtype == "f32") else 2e-2
         assert rel_finite(out, want) <= tol, f"{what}: output"
         layer.close()
+
+
+@pytest.mark.parametrize("first", range(0, 60, 20))
+def test_call_sequences_on_one_layer(device, first):
+    """One layer sized for 300 rows, seven calls of other sizes in a row (no rows, a few rows on the decode-shaped
+    path, hundreds on the large-batch path, the full size), with and without padding masks and bias, a backward
+    pass after some of them with the gradients cleared or accumulating: no call may see what an earlier one left
+    behind."""
+    for seed in range(first, first + 20):
+        rng = np.random.default_rng(9000 + seed)
+        mode = str(rng.choice(["stream", "stream_i8", "f32mc", "generic_f32", "generic_bf16"]))
+        training = bool(rng.integers(0, 2)) and mode != "stream_i8"
+        if mode.startswith("stream"):
+            d, F, act = int(rng.choice([64, 128])), int(rng.choice([64, 128])), "bf16"
+            wt = "int8" if mode.endswith("i8") else "bf16"
+        elif mode == "f32mc":
+            d, F, act, wt = int(rng.choice([32, 64])), int(rng.choice([32, 96])), "f32", "f32"
+        else:
+            d, F = int(rng.integers(1, 40)), int(rng.integers(1, 40))
+            act = wt = "f32" if mode == "generic_f32" else "bf16"
+        E = int(rng.choice([1, 3, 8, 17, 64]))
+        k = int(rng.integers(1, min(E, 6) + 1))
+        shared = bool(rng.integers(0, 2))
+        sdf = (int(rng.integers(1, 40)) if mode.startswith("generic") else (64 if act == "bf16" else 32)) if shared else 0
+        rows = 300
+        t = synth.make(small_workload(d=d, E=E, k=k, F=F, T=rows, seed=9000 + seed, act=act, wt=wt, shared=shared,
+                                      shared_d_ff=sdf))
+        about = f"seed {seed}: {mode} training {training} d{d} F{F} E{E} k{k} shared {sdf}"
+        oracle = oracle_layer(t)
+        layer = gpu_layer(device, t, max_tokens=rows, training=training)
+        tol = 1e-5 if (act == "f32" and wt == "f32") else 2e-2
+        for call in range(7):
+            T = int(rng.choice([0, 1, 3, 8, 32, 33, 100, 257, 300]))
+            x = t.x[rng.permutation(rows)[:T]].copy()
+            valid = None if rng.integers(0, 2) else rng.integers(0, 2, T).astype(np.uint8)
+            bias = synth.normal((E,), 0.5, seed, call) if rng.integers(0, 3) == 0 else None
+            what = f"{about} call {call} T{T} mask {valid is not None} bias {bias is not None}"
+            layout = rb.Layout(valid=None if valid is None else [bool(v) for v in valid])
+            out, cache = layer.forward_train(x, layout, router_bias=bias)
+            if T == 0:
+                assert out.shape == (0, d), what
+                continue
+            ref = oracle.forward(x, valid=valid, router_bias=bias, threads=4)
+            for name in ("expert_of", "counts", "offsets"):
+                assert np.array_equal(getattr(cache, name), getattr(ref, name)), f"{what}: {name}"
+            assert same_bits_or_same_nans(cache.probabilities, ref.probabilities), f"{what}: probabilities"
+            assert rel_finite(out, ref.out) <= tol, f"{what}: output"
+            assert abs(cache.aux_loss() - ref.aux_loss) <= tol * max(abs(ref.aux_loss), 1e-6), f"{what}: aux"
+            if not (training and rng.integers(0, 2)):
+                continue
+            gout = synth.round_bf16(rng.standard_normal(x.shape).astype(np.float32))
+            watched = ((L.W_ROUTER, 0), (L.W_DOWN, 0), (L.W_GATE, E - 1))
+            if rng.integers(0, 2):
+                layer.zero_grads()
+                before = [0.0, 0.0, 0.0]
+            else:
+                before = [layer.weight_grad(which, e) for which, e in watched]
+            gin = layer.backward(gout)
+            want = oracle.backward(x, gout, valid=valid, router_bias=bias, threads=4)
+            floor = (1e-7 if act == "f32" else 1e-3) * float(np.linalg.norm(gout)) * float(np.linalg.norm(x))
+
+            def close(name, got, wanted):
+                err = float(np.linalg.norm((got - wanted).astype(np.float64)))
+                assert err <= tol * float(np.linalg.norm(wanted.astype(np.float64))) + floor, f"{what}: {name} off by {err}"
+
+            close("grad_input", gin, want.grad_input)
+            for (which, e), old, wanted in zip(watched, before, (want.grad_router, want.grad_down[0], want.grad_gate[E - 1])):
+                close(f"weight {which}/{e}", layer.weight_grad(which, e) - old, wanted)
+        layer.close()
