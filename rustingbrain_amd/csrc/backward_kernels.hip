@@ -162,15 +162,16 @@ __global__ __launch_bounds__(256) void route_backward_kernel(
     for (int r = 0; r < k; ++r) weighted += grad_gates[(size_t)t * k + r] * p[sel[r]];
     const float aux_scale = (w_aux != 0.0f && V > 0) ? w_aux * (float)E / (float)V : 0.0f;
     const float slots = (float)(V * k);
-    const float inv_total = total > 0.0f ? 1.0f / total : 0.0f;
-    const float renorm = weighted * inv_total * inv_total;
+    // the reference's own two quotients (src/moe.rs:438-441): with one expert per token they cancel to rounding
+    // noise, and the noise should at least be the same kind of noise
+    const float renorm = total > 0.0f ? __fdiv_rn(weighted, __fmul_rn(total, total)) : 0.0f;
     // dP of expert e, assembled on the fly (twice: once for the softmax's dot product, once for
     // the result - cheaper than a trip through memory)
     auto grad_p = [&](int e) {
         float gp = 0.0f;
         if (total > 0.0f)
             for (int r = 0; r < k; ++r)
-                if (sel[r] == e) gp += grad_gates[(size_t)t * k + r] * inv_total - renorm;
+                if (sel[r] == e) gp += __fdiv_rn(grad_gates[(size_t)t * k + r], total) - renorm;
         if (aux_scale != 0.0f) gp += aux_scale * ((float)counts[e] / slots);
         return gp;
     };
