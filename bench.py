@@ -37,7 +37,9 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM-side bytes per launch of the gate/up kernel, measured with rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (each scaled by the reading of a 256 MiB copy; profiles/c3_prefill_hbm_traffic.txt).
 # Valid only for the workload and kernel it was measured on.
-MEASURED_TRAFFIC = {("c3_prefill_d768_e16", "mfma_bf16_stream"): 301.3e6}
+MEASURED_TRAFFIC = {("c3_prefill_d768_e16", "mfma_bf16_stream"): 301.3e6,
+                    # decode gate/up launch (profiles/c2_decode_hbm_traffic.txt): every weight byte once
+                    ("c2_decode_d768_e8", "mfma_bf16_decode"): 39.18e6}
 
 
 class DeviceBuffer:
@@ -284,7 +286,8 @@ def main() -> int:
         roofline = {"bound": "hbm", "kernel": "decode gate/up product + SwiGLU, routed and shared (" +
                                               layer.kernel_name() + "), caches flushed before every forward",
                     "achieved": gu_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gu_gbs / PEAK_HBM_GBS,
-                    "traffic": None, "bytes_per_launch": alg["decode_gate_up_bytes"],
+                    "traffic": MEASURED_TRAFFIC.get((w.name, layer.kernel_name())),
+                    "bytes_per_launch": alg["decode_gate_up_bytes"],
                     "avg_launch_ms": cold_ms["gate_up"], "touched_experts": touched,
                     "cache_resident_gbs": gbs(alg["decode_gate_up_bytes"], stage_ms["gate_up"])}
     else:
