@@ -230,3 +230,43 @@ def test_c3_block_training_step_at_full_size(device):
     t = synth.make(synth.WORKLOADS["c3_prefill_d768_e16"])
     layer, _, _ = check_block_backward(device, t, bias=t.router_bias)
     layer.close()
+
+
+# ------------------------------------------------------------------ the reference's cached-decode tests, feed-forward half
+@pytest.mark.parametrize("act,wt,d,F", [("f32", "f32", 64, 96), ("bf16", "bf16", 128, 192), ("bf16", "int8", 128, 192),
+                                        ("f32", "f32", 24, 10)])
+def test_a_cached_decode_reproduces_the_full_sequence_forward(device, act, wt, d, F):
+    """reference src/transformer.rs:2422-2454: feeding a sequence one token at a time (`forward_cached`), or a
+    prefill and then single tokens, must give what the whole sequence gives at once, within 1e-3.  For the
+    feed-forward half of the block that is: the block step on one row (the decode-shaped kernels where the layer
+    has them) against the same row inside a batch of 70 (the large-batch kernels) - the same experts and
+    probabilities in every bit, the same output within 1e-3 for f32 and within the bf16 bar otherwise."""
+    T = 70
+    t = synth.make(small_workload(d=d, E=8, k=2, F=F, T=T, seed=51, act=act, wt=wt, shared=True))
+    nw = norm_weight(d, 51)
+    cfg = rb.MoeConfig(8, 2, F, True)
+    layer = rb.MoeLayer(d, cfg, device, act_dtype=act, weight_dtype=wt, max_tokens=T)
+    layer.set_feed_forward_norm(nw, 1e-5)
+    layer.load_tensors(t)
+    full, cache_full = layer.forward_block(t.x)
+    big_kernels = layer.kernel_name()
+
+    def same_as_full(rows, out, cache):
+        k = 2
+        assert np.array_equal(cache.expert_of.reshape(-1, k), cache_full.expert_of.reshape(T, k)[rows])
+        assert np.array_equal(cache.probabilities.view(np.uint32), cache_full.probabilities[rows].view(np.uint32))
+        if act == "f32":
+            assert np.max(np.abs(out - full[rows])) < 1e-3
+        else:
+            assert rel_l2(out, full[rows]) <= 5e-3
+
+    for position in (0, 1, 2, 17, 69):                      # one token at a time
+        out, cache = layer.forward_block(t.x[position:position + 1])
+        same_as_full(slice(position, position + 1), out, cache)
+    if act == "bf16":
+        assert layer.kernel_name().startswith("mfma_bf16_decode") and big_kernels.startswith("mfma_bf16_stream")
+    out, cache = layer.forward_block(t.x[:40])              # a prefill, then the next token
+    same_as_full(slice(0, 40), out, cache)
+    out, cache = layer.forward_block(t.x[40:41])
+    same_as_full(slice(40, 41), out, cache)
+    layer.close()
