@@ -4,6 +4,7 @@
   5), inputs, epsilon and tolerances, run on the device layer: the finite differences are taken through the
   device's forward pass, the analytic side is `rbmoe_backward`.  The weights are this build's seeded ones (the
   reference draws its own from `StdRng`, which cannot be replayed here).
+* `SwiGlu`'s own two gradient tests (src/ffn.rs:274-322) on a layer with one expert, where the gate is exactly 1.
 * The same gradients against the CPU oracle at odd shapes, for f32, bf16 and mixed layers, with a shared expert
   of another width, padding rows, an expert without rows, accumulation and the block step's norm.
 """
@@ -152,4 +153,48 @@ def test_block_step_of_any_width(device, act):
     valid = (np.arange(50) % 6 != 1).astype(np.uint8)
     layer, _, _ = check_block_backward(device, t, valid=valid)
     assert layer.kernel_name() == "generic"
+    layer.close()
+
+
+# ------------------------------------------------------------------ SwiGlu's own gradient tests (src/ffn.rs:274-322)
+def single_expert_layer(device, d, F, T, seed):
+    """One expert, one expert per token: the gate is exactly 1, so the layer is that expert's SwiGLU."""
+    t = synth.make(small_workload(d=d, E=1, k=1, F=F, T=T, seed=seed))
+    return t, gpu_layer(device, t, aux_w=0.0, z_w=0.0, training=True)
+
+
+def test_swiglu_backward_matches_finite_differences(device):
+    t, layer = single_expert_layer(device, 4, 6, 2, seed=2)
+    x = np.array([0.5, -1.0, 2.0, 0.25, -0.75, 1.5, 0.1, -0.3], np.float32).reshape(2, 4)
+    out, cache = layer.forward_train(x)
+    assert np.all(cache.gate_of == 1.0)
+    gin = layer.backward(np.ones((2, 4), np.float32))
+    eps = np.float32(1e-3)
+    for i in range(x.size):
+        hi, lo = x.copy(), x.copy()
+        hi.flat[i] += eps
+        lo.flat[i] -= eps
+        numeric = (layer.forward(hi).sum(dtype=np.float32) - layer.forward(lo).sum(dtype=np.float32)) / (2 * eps)
+        assert abs(gin.flat[i] - numeric) < 1e-2, (i, gin.flat[i], numeric)
+    layer.close()
+
+
+def test_swiglu_gate_weight_gradient_matches_finite_differences(device):
+    t, layer = single_expert_layer(device, 3, 4, 2, seed=3)
+    x = np.array([0.4, -0.8, 1.2, 0.9, 0.3, -1.1], np.float32).reshape(2, 3)
+    layer.forward_train(x)
+    layer.backward(np.ones((2, 3), np.float32))
+    analytic = layer.weight_grad(L.W_GATE, 0)
+    assert np.any(analytic != 0.0)
+    w = t.experts[0]
+    eps = np.float32(1e-3)
+    for i in range(analytic.size):
+        sums = []
+        for sgn in (+1, -1):
+            gate = w["gate"].copy()
+            gate.flat[i] += sgn * eps
+            layer.set_expert(0, gate, w["up"], w["down"])
+            sums.append(layer.forward(x).sum(dtype=np.float32))
+        numeric = (sums[0] - sums[1]) / (2 * eps)
+        assert abs(analytic.flat[i] - numeric) < 1e-2, (i, analytic.flat[i], numeric)
     layer.close()
