@@ -155,7 +155,7 @@ def backward_leg(dev, w, t, x, out, bp, args, alg, with_cpu: bool) -> dict:
         layer.forward_device(x.ptr, T, out.ptr, bias_ptr=bp)
 
     def bwd():
-        layer.backward_device(g.ptr, gin.ptr)
+        layer.backward_device(g.ptr, T, gin.ptr)
 
     def timed(fn, n):
         dev.synchronize()

@@ -202,13 +202,16 @@ int rbmoe_forward_block_host(rbmoe_layer* layer, const void* x, int32_t tokens, 
  * Call it before the weights are set.  A training layer always takes the large-batch kernels. */
 int rbmoe_layer_enable_training(rbmoe_layer* layer);
 
-/* MoeLayer::backward on DEVICE pointers for the last forward: `grad_output` [T, d] act_dtype in,
- * `grad_input` [T, d] act_dtype out; weight gradients are ACCUMULATED (as Param.grad is) until
+/* MoeLayer::backward on DEVICE pointers for the last forward: `grad_output` [tokens, cols] act_dtype in,
+ * `grad_input` [tokens, cols] act_dtype out; weight gradients are ACCUMULATED (as Param.grad is) until
  * rbmoe_zero_grads.  The gradients of the two auxiliary losses reach the router here, as in the
- * reference (src/moe.rs:343-347).  Enqueued on the context's stream. */
-int rbmoe_backward(rbmoe_layer* layer, const void* grad_output, void* grad_input);
+ * reference (src/moe.rs:343-347).  `tokens` and `cols` are the shape of both buffers and must be the
+ * last forward's (the reference sizes the gradient from the cached input, src/moe.rs:349-350):
+ * anything else is RBMOE_INVALID_INPUT and neither buffer is touched.  Enqueued on the context's stream. */
+int rbmoe_backward(rbmoe_layer* layer, const void* grad_output, int32_t tokens, int32_t cols, void* grad_input);
 /* Same on HOST pointers; synchronises. */
-int rbmoe_backward_host(rbmoe_layer* layer, const void* grad_output, void* grad_input);
+int rbmoe_backward_host(rbmoe_layer* layer, const void* grad_output, int32_t tokens, int32_t cols,
+                        void* grad_input);
 /* Param::zero_grad for every weight of the layer. */
 int rbmoe_zero_grads(rbmoe_layer* layer);
 /* One accumulated weight gradient as f32 [rows, cols] into host memory (same ids and shapes as
@@ -222,10 +225,13 @@ int rbmoe_get_weight_grad(rbmoe_layer* layer, int32_t which, int32_t expert, flo
  *   grad_input     = feed_forward_norm.backward(residual, grad_projected) + grad_output
  * (RmsNorm::backward, src/norm.rs:63-121).  The norm's scale gradient accumulates like the other weight
  * gradients and is read with rbmoe_get_weight_grad(layer, RBMOE_W_NORM, 0, host, 1, d_model).  `grad_input`
- * may be `grad_output` itself.  Needs training mode and a norm (in either order). */
-int rbmoe_backward_block(rbmoe_layer* layer, const void* grad_output, void* grad_input);
+ * may be `grad_output` itself.  Needs training mode and a norm (in either order).  `tokens` and `cols` as
+ * for rbmoe_backward. */
+int rbmoe_backward_block(rbmoe_layer* layer, const void* grad_output, int32_t tokens, int32_t cols,
+                         void* grad_input);
 /* Same on HOST pointers; synchronises. */
-int rbmoe_backward_block_host(rbmoe_layer* layer, const void* grad_output, void* grad_input);
+int rbmoe_backward_block_host(rbmoe_layer* layer, const void* grad_output, int32_t tokens, int32_t cols,
+                              void* grad_input);
 
 /* Per-stage timing of one forward with HIP events on the context's stream.
  * `ms` receives RBMOE_NUM_STAGES durations in milliseconds.  Synchronises.

@@ -244,12 +244,19 @@ impl MoeLayer {
 
     /// `MoeLayer::backward` (src/moe.rs:348-489) for the last `forward_train`: `grad_output` and the
     /// returned gradient of the input are `[rows, d_model]` in the layer's activation type (raw bytes of
-    /// f32 or bf16 values); weight gradients accumulate until `zero_grads`.
-    pub fn backward_raw(&mut self, grad_output: &[u8]) -> Result<Vec<u8>, NetworkError> {
-        let mut grad_input = vec![0u8; grad_output.len()];
+    /// f32 or bf16 values); weight gradients accumulate until `zero_grads`.  `rows` must be the last
+    /// forward's row count: the library refuses anything else before it touches either buffer, and a slice
+    /// whose length is not `rows * d_model` elements is refused here.
+    pub fn backward_raw(&mut self, grad_output: &[u8], rows: usize) -> Result<Vec<u8>, NetworkError> {
+        let elem = 4; // the layer is created with f32 rows on the boundary (see `new`)
+        let expected = rows * self.d_model * elem;
+        if grad_output.len() != expected {
+            return Err(NetworkError::InvalidInput { expected, actual: grad_output.len() });
+        }
+        let mut grad_input = vec![0u8; expected];
         check(unsafe {
-            sys::rbmoe_backward_host(self.layer, grad_output.as_ptr() as *const c_void,
-                                     grad_input.as_mut_ptr() as *mut c_void)
+            sys::rbmoe_backward_host(self.layer, grad_output.as_ptr() as *const c_void, rows as i32,
+                                     self.d_model as i32, grad_input.as_mut_ptr() as *mut c_void)
         }, self.device.raw(), 0, 0)?;
         Ok(grad_input)
     }

@@ -98,10 +98,13 @@ extern "C" {
                                     valid: *const u8, router_bias: *const f32, out: *mut c_void) -> c_int;
     // backward pass (MoeLayer::backward, src/moe.rs:348-489)
     pub fn rbmoe_layer_enable_training(layer: *mut rbmoe_layer) -> c_int;
-    pub fn rbmoe_backward(layer: *mut rbmoe_layer, grad_output: *const c_void, grad_input: *mut c_void) -> c_int;
-    pub fn rbmoe_backward_host(layer: *mut rbmoe_layer, grad_output: *const c_void, grad_input: *mut c_void) -> c_int;
-    pub fn rbmoe_backward_block(layer: *mut rbmoe_layer, grad_output: *const c_void, grad_input: *mut c_void) -> c_int;
-    pub fn rbmoe_backward_block_host(layer: *mut rbmoe_layer, grad_output: *const c_void,
+    pub fn rbmoe_backward(layer: *mut rbmoe_layer, grad_output: *const c_void, tokens: i32, cols: i32,
+                          grad_input: *mut c_void) -> c_int;
+    pub fn rbmoe_backward_host(layer: *mut rbmoe_layer, grad_output: *const c_void, tokens: i32, cols: i32,
+                               grad_input: *mut c_void) -> c_int;
+    pub fn rbmoe_backward_block(layer: *mut rbmoe_layer, grad_output: *const c_void, tokens: i32, cols: i32,
+                                grad_input: *mut c_void) -> c_int;
+    pub fn rbmoe_backward_block_host(layer: *mut rbmoe_layer, grad_output: *const c_void, tokens: i32, cols: i32,
                                      grad_input: *mut c_void) -> c_int;
     pub fn rbmoe_zero_grads(layer: *mut rbmoe_layer) -> c_int;
     pub fn rbmoe_get_weight_grad(layer: *mut rbmoe_layer, which: i32, expert: i32, host: *mut f32, rows: i32,

@@ -72,10 +72,10 @@ SIGNATURES = {
     "rbmoe_forward_block_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p,
                                            C.c_void_p]),
     "rbmoe_layer_enable_training": (C.c_int, [C.c_void_p]),
-    "rbmoe_backward": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
-    "rbmoe_backward_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
-    "rbmoe_backward_block": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
-    "rbmoe_backward_block_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
+    "rbmoe_backward": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
+    "rbmoe_backward_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
+    "rbmoe_backward_block": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
+    "rbmoe_backward_block_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
     "rbmoe_zero_grads": (C.c_int, [C.c_void_p]),
     "rbmoe_get_weight_grad": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_float), C.c_int32, C.c_int32]),
     "rbmoe_version": (C.c_char_p, []),

@@ -491,6 +491,12 @@ hipError_t launch_route_backward(const float* P, const float* lse, const int* ex
     return hipGetLastError();
 }
 
+// Rows up to which the router's weight gradient runs in one launch: at most kRouterGradMaxChunks chunks, a chunk's
+// logit gradients (tokens x kRouterGradExperts floats) held in 48 KiB of LDS.
+int router_grad_max_tokens() {
+    return kRouterGradMaxChunks * (int)((48 * 1024 / sizeof(float) / kRouterGradExperts) / 32 * 32);
+}
+
 // chunks of partial sums a layer of up to `max_tokens` rows needs room for
 int router_grad_chunks(int max_tokens) { return std::min(kRouterGradMaxChunks, (std::max(max_tokens, 1) + 31) / 32); }
 

@@ -6,8 +6,8 @@
 // Data paths (nothing is staged through registers on its way to LDS):
 //   weights      packed at upload into matrix-core operand order (see
 //                pack_weight_bf16 / pack_weight_i8); every wave streams its own
-//                fragments global -> VGPR through an 8-deep register ring, i.e.
-//                the load for reduction step g + 7 is issued while step g runs.
+//                fragments global -> VGPR through a 4-deep register ring, i.e.
+//                the load for reduction step g + 3 is issued while step g runs.
 //                int8 weights are widened to bf16 in registers right before the
 //                multiply; the per-row scale multiplies the accumulator.
 //   activations  128 token rows per workgroup (gathered through an index for
@@ -495,8 +495,8 @@ static hipError_t launch_ring(const GroupedArgs& g, WeightKind wk, hipStream_t s
     return hipErrorInvalidValue;
 }
 
-// variant 0: ring of 4 steps, token fragments read one step ahead
-// variant 1: ring of 8 steps, token fragments read just in time
+// variant 0: ring of 4 steps, token fragments read one step ahead, activation slices by LDS-DMA
+// variant 1: ring of 4 steps, token fragments read just in time, activation slices global -> VGPR -> LDS
 int stream_tile_m() { return BM; }
 
 // K a multiple of 64 (one LDS slice), N a multiple of 32 (row blocks of the packed weights)

@@ -115,6 +115,29 @@ int hip_fail(rbmoe_ctx* ctx, hipError_t e, const char* what) {
 
 }  // namespace
 
+// Where one forward pass keeps its routing tables and expert rows (the layer's workspace).  The getters read
+// the last forward's.
+struct Work {
+    float* P = nullptr;
+    float* lse = nullptr;
+    int* expert_of = nullptr;
+    float* gate_of = nullptr;
+    int* counts = nullptr;
+    int* offsets = nullptr;
+    int* tile_expert = nullptr;
+    int* tile_row0 = nullptr;
+    int* tile_rows = nullptr;
+    int* ntiles = nullptr;
+    float* losses = nullptr;
+    int* perm_slot = nullptr;
+    int* perm_token = nullptr;
+    int* inv_pos = nullptr;
+    void* h = nullptr;
+    void* y = nullptr;
+    void* hs = nullptr;
+    void* ys = nullptr;
+};
+
 struct rbmoe_layer {
     rbmoe_ctx* ctx = nullptr;
     rbmoe_config cfg{};
@@ -131,6 +154,7 @@ struct rbmoe_layer {
     int group_m = 4, variant = 0;
     const char* kernel_name = "none";
     int last_T = -1;
+    Work last;  // tables of the last forward
 
     // weights
     Buf router;            // f32 [E, d]
@@ -667,6 +691,18 @@ int rbmoe_set_weight(rbmoe_layer* L, int32_t which, int32_t expert, const void* 
 
 namespace {
 
+Work work_of_layer(const rbmoe_layer* L) {
+    Work w;
+    w.P = (float*)L->P.p; w.lse = (float*)L->lse.p;
+    w.expert_of = (int*)L->expert_of.p; w.gate_of = (float*)L->gate_of.p;
+    w.counts = (int*)L->counts.p; w.offsets = (int*)L->offsets.p;
+    w.tile_expert = (int*)L->tile_expert.p; w.tile_row0 = (int*)L->tile_row0.p; w.tile_rows = (int*)L->tile_rows.p;
+    w.ntiles = (int*)L->ntiles.p; w.losses = (float*)L->losses.p;
+    w.perm_slot = (int*)L->perm_slot.p; w.perm_token = (int*)L->perm_token.p; w.inv_pos = (int*)L->inv_pos.p;
+    w.h = L->h.p; w.y = L->y.p; w.hs = L->hs.p; w.ys = L->ys.p;
+    return w;
+}
+
 // `norm_src` (block step): the raw rows; `x` is then the layer's buffer of normed rows, filled here - by the
 // small-route kernel itself for a few tokens, by the norm kernel otherwise - before anything reads it.
 int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* valid, const float* router_bias,
@@ -714,6 +750,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
                            (!c.shared_expert || (decode_shape_ok(Fs, d) && decode_shape_ok(d, Fs)));
     const bool norm_in_route = norm_src && decode_ok &&
                                small_route_stages_rows(norm_src, (const float*)L->router.p, T, d, E, abf);
+    Work wk_ = work_of_layer(L);
     if (norm_src && !norm_in_route)
         HIP_TRY(ctx, launch_rmsnorm(norm_src, (const float*)L->norm_w.p, L->norm_eps, T, d, L->xn.p, abf, s));
 
@@ -728,55 +765,55 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
         sr.T = T; sr.d = d; sr.E = E; sr.k = k;
         sr.w_aux = c.aux_loss_weight; sr.w_z = c.router_z_loss_weight;
         sr.tile_m = kDecodeTileM;
-        sr.P = (float*)L->P.p; sr.lse = (float*)L->lse.p;
-        sr.expert_of = (int*)L->expert_of.p; sr.gate_of = (float*)L->gate_of.p;
-        sr.counts = (int*)L->counts.p; sr.offsets = (int*)L->offsets.p;
-        sr.tile_expert = (int*)L->tile_expert.p; sr.tile_row0 = (int*)L->tile_row0.p; sr.tile_rows = (int*)L->tile_rows.p;
-        sr.ntiles = (int*)L->ntiles.p; sr.losses = (float*)L->losses.p;
-        sr.perm_slot = (int*)L->perm_slot.p; sr.perm_token = (int*)L->perm_token.p; sr.inv_pos = (int*)L->inv_pos.p;
+        sr.P = wk_.P; sr.lse = wk_.lse;
+        sr.expert_of = wk_.expert_of; sr.gate_of = wk_.gate_of;
+        sr.counts = wk_.counts; sr.offsets = wk_.offsets;
+        sr.tile_expert = wk_.tile_expert; sr.tile_row0 = wk_.tile_row0; sr.tile_rows = wk_.tile_rows;
+        sr.ntiles = wk_.ntiles; sr.losses = wk_.losses;
+        sr.perm_slot = wk_.perm_slot; sr.perm_token = wk_.perm_token; sr.inv_pos = wk_.inv_pos;
         HIP_TRY(ctx, launch_route_small(sr, abf, s));
         HIP_TRY(ctx, mark(1));
         HIP_TRY(ctx, mark(2));
         HIP_TRY(ctx, mark(3));
 
         DecodeGemmArgs d1{};
-        d1.a = x; d1.row_index = (const int*)L->perm_token.p;
+        d1.a = x; d1.row_index = wk_.perm_token;
         d1.w = L->wgu.p; d1.w_expert_stride = (size_t)2 * F * d;
         d1.scales = wk == WeightKind::I8 ? (const float*)L->sgu.p : nullptr; d1.s_expert_stride = (size_t)2 * F;
         d1.N = F; d1.K = d;
-        d1.tile_expert = (const int*)L->tile_expert.p; d1.tile_row0 = (const int*)L->tile_row0.p;
-        d1.tile_rows = (const int*)L->tile_rows.p; d1.ntiles = (const int*)L->ntiles.p;
+        d1.tile_expert = wk_.tile_expert; d1.tile_row0 = wk_.tile_row0;
+        d1.tile_rows = wk_.tile_rows; d1.ntiles = wk_.ntiles;
         d1.max_tiles = (T * k) / kDecodeTileM + E;
-        d1.out = L->h.p;
+        d1.out = wk_.h;
         d1.swiglu = 1;
         if (c.shared_expert) {
             d1.a_shared = x; d1.w_shared = L->swgu.p;
             d1.scales_shared = wk == WeightKind::I8 ? (const float*)L->ssgu.p : nullptr;
-            d1.N_shared = Fs; d1.K_shared = d; d1.T_shared = T; d1.out_shared = L->hs.p;
+            d1.N_shared = Fs; d1.K_shared = d; d1.T_shared = T; d1.out_shared = wk_.hs;
         }
         HIP_TRY(ctx, launch_decode_gemm(d1, wk, s));
         HIP_TRY(ctx, mark(4));
 
         DecodeGemmArgs d2 = d1;
-        d2.a = L->h.p; d2.row_index = nullptr;
+        d2.a = wk_.h; d2.row_index = nullptr;
         d2.w = L->wd.p; d2.w_expert_stride = (size_t)d * F;
         d2.scales = wk == WeightKind::I8 ? (const float*)L->sd.p : nullptr; d2.s_expert_stride = (size_t)d;
         d2.N = d; d2.K = F;
-        d2.out = L->y.p;
+        d2.out = wk_.y;
         d2.swiglu = 0;
         if (c.shared_expert) {
-            d2.a_shared = L->hs.p; d2.w_shared = L->swd.p;
+            d2.a_shared = wk_.hs; d2.w_shared = L->swd.p;
             d2.scales_shared = wk == WeightKind::I8 ? (const float*)L->ssd.p : nullptr;
-            d2.N_shared = d; d2.K_shared = Fs; d2.out_shared = L->ys.p;
+            d2.N_shared = d; d2.K_shared = Fs; d2.out_shared = wk_.ys;
         }
         HIP_TRY(ctx, launch_decode_gemm(d2, wk, s));
         HIP_TRY(ctx, mark(5));
         HIP_TRY(ctx, mark(6));
-        CombineArgs cd{L->y.p, c.shared_expert ? L->ys.p : nullptr, residual, (const int*)L->inv_pos.p,
-                       (const float*)L->gate_of.p, T, d, k, out};
+        CombineArgs cd{wk_.y, c.shared_expert ? wk_.ys : nullptr, residual, wk_.inv_pos, wk_.gate_of, T, d, k, out};
         HIP_TRY(ctx, launch_combine(cd, abf, s));
         HIP_TRY(ctx, mark(7));
         L->last_T = T;
+        L->last = wk_;
         return RBMOE_OK;
     }
 
@@ -883,13 +920,59 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     HIP_TRY(ctx, launch_combine(ca, abf, s));
     HIP_TRY(ctx, mark(7));
     L->last_T = T;
+    L->last = wk_;
     return RBMOE_OK;
+}
+
+// Allocates and clears the buffers of `p` for a layer that already exists: the budget is checked before
+// anything is allocated, and a failure part-way frees what this call had allocated, so that the layer is left as
+// it was and the call can simply be made again.
+int allocate_plan(rbmoe_layer* L, Plan& p, const char* what) {
+    rbmoe_ctx* ctx = L->ctx;
+    if (ctx->budget_bytes && ctx->allocated + p.total > ctx->budget_bytes) {
+        char buf[200];
+        std::snprintf(buf, sizeof buf, "memory budget exceeded: estimated %zu MiB exceeds budget %zu MiB",
+                      (ctx->allocated + p.total + (1 << 20) - 1) >> 20, ctx->budget_bytes >> 20);
+        return fail(ctx, RBMOE_MEMORY_BUDGET, buf);
+    }
+    size_t done = 0;
+    hipError_t e = hipSetDevice(ctx->device);
+    while (e == hipSuccess && done < p.items.size()) {
+        auto& it = p.items[done];
+        void* q = nullptr;
+        e = hipMalloc(&q, it.second);
+        if (e != hipSuccess) break;
+        it.first->p = q;
+        it.first->bytes = it.second;
+        ctx->allocated += it.second;
+        L->all.push_back(it.first);
+        ++done;
+        e = hipMemsetAsync(q, 0, it.second, ctx->stream);
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e == hipSuccess) return RBMOE_OK;
+    (void)hipGetLastError();
+    (void)hipStreamSynchronize(ctx->stream);
+    for (size_t i = 0; i < done; ++i) {
+        Buf* b = p.items[i].first;
+        (void)hipFree(b->p);
+        if (ctx->allocated >= b->bytes) ctx->allocated -= b->bytes;
+        b->p = nullptr;
+        b->bytes = 0;
+        for (size_t j = L->all.size(); j-- > 0;)
+            if (L->all[j] == b) {
+                L->all.erase(L->all.begin() + (long)j);
+                break;
+            }
+    }
+    if (e == hipErrorOutOfMemory)
+        return fail(ctx, RBMOE_OUT_OF_MEMORY, std::string("out of memory while allocating ") + what);
+    return hip_fail(ctx, e, what);
 }
 
 // Buffers of the backward pass through the norm: allocated by whichever of rbmoe_set_feed_forward_norm and
 // rbmoe_layer_enable_training comes second.
 int ensure_block_training_buffers(rbmoe_layer* L) {
-    rbmoe_ctx* ctx = L->ctx;
     if (!L->training || !L->norm_w.p || L->xraw.p) return RBMOE_OK;
     const rbmoe_config& c = L->cfg;
     const size_t T = L->max_T, d = c.d_model, as = dtype_size(c.act_dtype);
@@ -899,26 +982,7 @@ int ensure_block_training_buffers(rbmoe_layer* L) {
     p.add(&L->inv_rms, T * 4);
     p.add(&L->norm_partial, (size_t)rmsnorm_grad_tiles((int)T) * d * 4);
     p.add(&L->g_norm, d * 4);
-    if (ctx->budget_bytes && ctx->allocated + p.total > ctx->budget_bytes) {
-        char buf[200];
-        std::snprintf(buf, sizeof buf, "memory budget exceeded: estimated %zu MiB exceeds budget %zu MiB",
-                      (ctx->allocated + p.total + (1 << 20) - 1) >> 20, ctx->budget_bytes >> 20);
-        return fail(ctx, RBMOE_MEMORY_BUDGET, buf);
-    }
-    for (auto& it : p.items) {
-        void* q = nullptr;
-        if (hipMalloc(&q, it.second) != hipSuccess) {
-            (void)hipGetLastError();
-            return fail(ctx, RBMOE_OUT_OF_MEMORY, "out of memory while allocating the norm's backward buffers");
-        }
-        it.first->p = q;
-        it.first->bytes = it.second;
-        ctx->allocated += it.second;
-        L->all.push_back(it.first);
-        HIP_TRY(ctx, hipMemsetAsync(q, 0, it.second, ctx->stream));
-    }
-    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
-    return RBMOE_OK;
+    return allocate_plan(L, p, "the norm's backward buffers");
 }
 
 }  // namespace
@@ -995,23 +1059,7 @@ int rbmoe_set_feed_forward_norm(rbmoe_layer* L, const float* weight, int32_t col
         Plan p;
         p.add(&L->xn, (size_t)L->max_T * c.d_model * dtype_size(c.act_dtype));
         p.add(&L->norm_w, (size_t)c.d_model * 4);
-        if (ctx->budget_bytes && ctx->allocated + p.total > ctx->budget_bytes) {
-            char buf[200];
-            std::snprintf(buf, sizeof buf, "memory budget exceeded: estimated %zu MiB exceeds budget %zu MiB",
-                          (ctx->allocated + p.total + (1 << 20) - 1) >> 20, ctx->budget_bytes >> 20);
-            return fail(ctx, RBMOE_MEMORY_BUDGET, buf);
-        }
-        for (auto& it : p.items) {
-            void* q = nullptr;
-            if (hipMalloc(&q, it.second) != hipSuccess) {
-                (void)hipGetLastError();
-                return fail(ctx, RBMOE_OUT_OF_MEMORY, "out of memory while allocating the normed rows");
-            }
-            it.first->p = q;
-            it.first->bytes = it.second;
-            ctx->allocated += it.second;
-            L->all.push_back(it.first);
-        }
+        if (const int rc = allocate_plan(L, p, "the normed rows")) return rc;
     }
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));  // no forward may still read the old weight
     HIP_TRY(ctx, hipMemcpy(L->norm_w.p, weight, (size_t)c.d_model * 4, hipMemcpyHostToDevice));
@@ -1084,6 +1132,12 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
         return fail(ctx, RBMOE_UNSUPPORTED, "the backward pass is not defined for int8 weights");
     if (L->weights_set)
         return fail(ctx, RBMOE_INVALID_CONFIG, "enable training before the weights are set");
+    if (L->max_T > router_grad_max_tokens()) {  // found here, not in the middle of a backward pass
+        char buf[160];
+        std::snprintf(buf, sizeof buf, "the backward pass takes at most %d tokens a call, the layer was created for %d",
+                      router_grad_max_tokens(), L->max_T);
+        return fail(ctx, RBMOE_UNSUPPORTED, buf);
+    }
     const size_t E = c.num_experts, d = c.d_model, F = c.d_ff, Fs = L->Fs, T = L->max_T, S = L->max_S;
     if (bf16_layer) {
         if (!stream_shape_ok((int)d, (int)(2 * F)) || (c.shared_expert && !stream_shape_ok((int)d, (int)(2 * Fs))))
@@ -1126,26 +1180,7 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
         p.add(&L->swdT, Fs * d * ws);
         p.add(&L->swguT, d * 2 * Fs * ws);
     }
-    if (ctx->budget_bytes && ctx->allocated + p.total > ctx->budget_bytes) {
-        char buf[200];
-        std::snprintf(buf, sizeof buf, "memory budget exceeded: estimated %zu MiB exceeds budget %zu MiB",
-                      (ctx->allocated + p.total + (1 << 20) - 1) >> 20, ctx->budget_bytes >> 20);
-        return fail(ctx, RBMOE_MEMORY_BUDGET, buf);
-    }
-    HIP_TRY(ctx, hipSetDevice(ctx->device));
-    for (auto& it : p.items) {
-        void* q = nullptr;
-        hipError_t e = hipMalloc(&q, it.second);
-        if (e != hipSuccess) {
-            (void)hipGetLastError();
-            return fail(ctx, RBMOE_OUT_OF_MEMORY, "out of memory while allocating the training buffers");
-        }
-        it.first->p = q;
-        it.first->bytes = it.second;
-        ctx->allocated += it.second;
-        L->all.push_back(it.first);
-        HIP_TRY(ctx, hipMemsetAsync(q, 0, it.second, ctx->stream));
-    }
+    if (const int rc = allocate_plan(L, p, "the training buffers")) return rc;
     HIP_TRY(ctx, launch_fill_f32((float*)L->ones.p, 1.0f, (long long)S, ctx->stream));
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
     L->wgrad_generic = env_int("RBMOE_WGRAD_GENERIC", 0) == 1;
@@ -1176,11 +1211,30 @@ int rbmoe_zero_grads(rbmoe_layer* L) {
     return RBMOE_OK;
 }
 
-int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
+// The backward entry points differentiate the LAST forward, whose shape the reference takes from the cached input
+// (src/moe.rs:349-350).  Here the cache is the layer's own state, so the caller states the shape of its buffers
+// and a mismatch is refused before any of their bytes is read or written.
+static int backward_shape_problem(rbmoe_layer* L, int32_t tokens, int32_t cols) {
+    rbmoe_ctx* ctx = L->ctx;
+    char buf[160];
+    if (cols != L->cfg.d_model) {
+        std::snprintf(buf, sizeof buf, "gradient length %d does not match expected length %d", cols, L->cfg.d_model);
+        return fail(ctx, RBMOE_INVALID_INPUT, buf);
+    }
+    if (tokens != L->last_T) {
+        std::snprintf(buf, sizeof buf, "gradient rows %d do not match the %d rows of the last forward pass", tokens,
+                      L->last_T);
+        return fail(ctx, RBMOE_INVALID_INPUT, buf);
+    }
+    return RBMOE_OK;
+}
+
+int rbmoe_backward(rbmoe_layer* L, const void* grad_output, int32_t tokens, int32_t cols, void* grad_input) {
     if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
     rbmoe_ctx* ctx = L->ctx;
     if (!L->training) return fail(ctx, RBMOE_INVALID_CONFIG, "training is not enabled on this layer");
     if (L->last_T < 0) return fail(ctx, RBMOE_INVALID_INPUT, "no forward pass has run yet");
+    if (const int rc = backward_shape_problem(L, tokens, cols)) return rc;
     const rbmoe_config& c = L->cfg;
     const int E = c.num_experts, d = c.d_model, F = c.d_ff, k = c.experts_per_token, Fs = L->Fs, T = L->last_T;
     if (T == 0) return RBMOE_OK;
@@ -1207,6 +1261,9 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
         HIP_TRY(ctx, hipEventRecord(ctx->ev_fork, s));
         HIP_TRY(ctx, hipStreamWaitEvent(rs, ctx->ev_fork, 0));
     }
+    // From here to the join the side stream hangs off the main one: an error in between must not leave it forked
+    // (a stream capture in progress could then never end), so the rest runs as one unit that is always joined.
+    auto forked = [&]() -> int {
     HIP_TRY(ctx, launch_route_backward((const float*)L->P.p, (const float*)L->lse.p, (const int*)L->expert_of.p,
                                        (const float*)L->grad_gates.p, counts, offsets, T, E, k, c.aux_loss_weight,
                                        c.router_z_loss_weight, (float*)L->dlogits.p, rs));
@@ -1276,6 +1333,16 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
     }
     // grad_input = sum over a token's slots of its expert rows + shared + router
     if (side) HIP_TRY(ctx, hipStreamWaitEvent(s, ctx->ev_join, 0));
+    return RBMOE_OK;
+    };
+    const int rc = forked();
+    if (rc != RBMOE_OK) {
+        if (side) {  // rejoin whatever the side stream got to
+            (void)hipEventRecord(ctx->ev_join, rs);
+            (void)hipStreamWaitEvent(s, ctx->ev_join, 0);
+        }
+        return rc;
+    }
     CombineArgs ca{L->dxg.p, c.shared_expert ? L->dxs.p : nullptr, L->dxr.p, (const int*)L->inv_pos.p,
                    (const float*)L->ones.p, T, d, k, grad_input};
     HIP_TRY(ctx, launch_combine(ca, abf, s));
@@ -1283,36 +1350,38 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, void* grad_input) {
     return RBMOE_OK;
 }
 
-int rbmoe_backward_host(rbmoe_layer* L, const void* grad_output, void* grad_input) {
+int rbmoe_backward_host(rbmoe_layer* L, const void* grad_output, int32_t tokens, int32_t cols, void* grad_input) {
     if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
     rbmoe_ctx* ctx = L->ctx;
     if (!L->training) return fail(ctx, RBMOE_INVALID_CONFIG, "training is not enabled on this layer");
     if (L->last_T < 0) return fail(ctx, RBMOE_INVALID_INPUT, "no forward pass has run yet");
+    if (const int rc = backward_shape_problem(L, tokens, cols)) return rc;  // before any byte of the buffers is touched
     const int T = L->last_T;
     if (T == 0) return RBMOE_OK;
     if (!grad_output || !grad_input) return fail(ctx, RBMOE_NULL_POINTER, "grad_output or grad_input is NULL");
     const size_t nbytes = (size_t)T * L->cfg.d_model * dtype_size(L->cfg.act_dtype);
     HIP_TRY(ctx, hipSetDevice(ctx->device));
     HIP_TRY(ctx, hipMemcpyAsync(L->st_gout.p, grad_output, nbytes, hipMemcpyHostToDevice, ctx->stream));
-    int rc = rbmoe_backward(L, L->st_gout.p, L->st_gin.p);
+    int rc = rbmoe_backward(L, L->st_gout.p, tokens, cols, L->st_gin.p);
     if (rc != RBMOE_OK) return rc;
     HIP_TRY(ctx, hipMemcpyAsync(grad_input, L->st_gin.p, nbytes, hipMemcpyDeviceToHost, ctx->stream));
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
     return RBMOE_OK;
 }
 
-int rbmoe_backward_block(rbmoe_layer* L, const void* grad_output, void* grad_input) {
+int rbmoe_backward_block(rbmoe_layer* L, const void* grad_output, int32_t tokens, int32_t cols, void* grad_input) {
     if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
     rbmoe_ctx* ctx = L->ctx;
     if (!L->training) return fail(ctx, RBMOE_INVALID_CONFIG, "training is not enabled on this layer");
     if (!L->norm_set) return fail(ctx, RBMOE_INVALID_CONFIG, "the feed-forward norm has not been set");
     if (L->last_T < 0 || !L->last_was_block)
         return fail(ctx, RBMOE_INVALID_INPUT, "the last forward pass was not rbmoe_forward_block");
+    if (const int rc = backward_shape_problem(L, tokens, cols)) return rc;
     const int T = L->last_T, d = L->cfg.d_model;
     if (T == 0) return RBMOE_OK;
     if (!grad_output || !grad_input) return fail(ctx, RBMOE_NULL_POINTER, "grad_output or grad_input is NULL");
     // grad_projected = feed_forward.backward(cache, grad_output)  (src/transformer_block.rs:257)
-    const int rc = rbmoe_backward(L, grad_output, L->dxn.p);
+    const int rc = rbmoe_backward(L, grad_output, tokens, cols, L->dxn.p);
     if (rc != RBMOE_OK) return rc;
     // grad_residual = feed_forward_norm.backward(residual, grad_projected) + grad_output  (:258-263)
     HIP_TRY(ctx, launch_rmsnorm_backward(L->xraw.p, L->dxn.p, (const float*)L->norm_w.p, L->norm_eps, grad_output, T, d,
@@ -1321,20 +1390,22 @@ int rbmoe_backward_block(rbmoe_layer* L, const void* grad_output, void* grad_inp
     return RBMOE_OK;
 }
 
-int rbmoe_backward_block_host(rbmoe_layer* L, const void* grad_output, void* grad_input) {
+int rbmoe_backward_block_host(rbmoe_layer* L, const void* grad_output, int32_t tokens, int32_t cols,
+                              void* grad_input) {
     if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
     rbmoe_ctx* ctx = L->ctx;
     if (!L->training) return fail(ctx, RBMOE_INVALID_CONFIG, "training is not enabled on this layer");
     if (!L->norm_set) return fail(ctx, RBMOE_INVALID_CONFIG, "the feed-forward norm has not been set");
     if (L->last_T < 0 || !L->last_was_block)
         return fail(ctx, RBMOE_INVALID_INPUT, "the last forward pass was not rbmoe_forward_block");
+    if (const int rc = backward_shape_problem(L, tokens, cols)) return rc;  // before any byte of the buffers is touched
     const int T = L->last_T;
     if (T == 0) return RBMOE_OK;
     if (!grad_output || !grad_input) return fail(ctx, RBMOE_NULL_POINTER, "grad_output or grad_input is NULL");
     const size_t nbytes = (size_t)T * L->cfg.d_model * dtype_size(L->cfg.act_dtype);
     HIP_TRY(ctx, hipSetDevice(ctx->device));
     HIP_TRY(ctx, hipMemcpyAsync(L->st_gout.p, grad_output, nbytes, hipMemcpyHostToDevice, ctx->stream));
-    const int rc = rbmoe_backward_block(L, L->st_gout.p, L->st_gin.p);
+    const int rc = rbmoe_backward_block(L, L->st_gout.p, tokens, cols, L->st_gin.p);
     if (rc != RBMOE_OK) return rc;
     HIP_TRY(ctx, hipMemcpyAsync(grad_input, L->st_gin.p, nbytes, hipMemcpyDeviceToHost, ctx->stream));
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
@@ -1400,7 +1471,7 @@ int rbmoe_get_losses(rbmoe_layer* L, float* aux_loss, float* z_loss) {
     if (L->last_T < 0) return fail(ctx, RBMOE_INVALID_INPUT, "no forward pass has run yet");
     float v[2] = {0.f, 0.f};
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
-    HIP_TRY(ctx, hipMemcpy(v, L->losses.p, 8, hipMemcpyDeviceToHost));
+    HIP_TRY(ctx, hipMemcpy(v, L->last.losses, 8, hipMemcpyDeviceToHost));
     if (aux_loss) *aux_loss = v[0];
     if (z_loss) *z_loss = v[1];
     return RBMOE_OK;
@@ -1413,16 +1484,17 @@ int rbmoe_get_routing(rbmoe_layer* L, rbmoe_routing* r) {
     const int T = L->last_T, E = L->cfg.num_experts, k = L->cfg.experts_per_token;
     const size_t S = (size_t)T * k;
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
-    if (r->counts) HIP_TRY(ctx, hipMemcpy(r->counts, L->counts.p, (size_t)E * 4, hipMemcpyDeviceToHost));
-    if (r->offsets) HIP_TRY(ctx, hipMemcpy(r->offsets, L->offsets.p, (size_t)(E + 1) * 4, hipMemcpyDeviceToHost));
+    const Work& w = L->last;
+    if (r->counts) HIP_TRY(ctx, hipMemcpy(r->counts, w.counts, (size_t)E * 4, hipMemcpyDeviceToHost));
+    if (r->offsets) HIP_TRY(ctx, hipMemcpy(r->offsets, w.offsets, (size_t)(E + 1) * 4, hipMemcpyDeviceToHost));
     if (S == 0) return RBMOE_OK;
-    if (r->expert_of) HIP_TRY(ctx, hipMemcpy(r->expert_of, L->expert_of.p, S * 4, hipMemcpyDeviceToHost));
-    if (r->gate_of) HIP_TRY(ctx, hipMemcpy(r->gate_of, L->gate_of.p, S * 4, hipMemcpyDeviceToHost));
-    if (r->perm_slot) HIP_TRY(ctx, hipMemcpy(r->perm_slot, L->perm_slot.p, S * 4, hipMemcpyDeviceToHost));
-    if (r->perm_token) HIP_TRY(ctx, hipMemcpy(r->perm_token, L->perm_token.p, S * 4, hipMemcpyDeviceToHost));
+    if (r->expert_of) HIP_TRY(ctx, hipMemcpy(r->expert_of, w.expert_of, S * 4, hipMemcpyDeviceToHost));
+    if (r->gate_of) HIP_TRY(ctx, hipMemcpy(r->gate_of, w.gate_of, S * 4, hipMemcpyDeviceToHost));
+    if (r->perm_slot) HIP_TRY(ctx, hipMemcpy(r->perm_slot, w.perm_slot, S * 4, hipMemcpyDeviceToHost));
+    if (r->perm_token) HIP_TRY(ctx, hipMemcpy(r->perm_token, w.perm_token, S * 4, hipMemcpyDeviceToHost));
     if (r->probabilities)
-        HIP_TRY(ctx, hipMemcpy(r->probabilities, L->P.p, (size_t)T * E * 4, hipMemcpyDeviceToHost));
-    if (r->log_sum_exp) HIP_TRY(ctx, hipMemcpy(r->log_sum_exp, L->lse.p, (size_t)T * 4, hipMemcpyDeviceToHost));
+        HIP_TRY(ctx, hipMemcpy(r->probabilities, w.P, (size_t)T * E * 4, hipMemcpyDeviceToHost));
+    if (r->log_sum_exp) HIP_TRY(ctx, hipMemcpy(r->log_sum_exp, w.lse, (size_t)T * 4, hipMemcpyDeviceToHost));
     return RBMOE_OK;
 }
 
@@ -1433,22 +1505,22 @@ int rbmoe_get_expert_rows(rbmoe_layer* L, float* hidden, float* expert_out) {
     const int E = L->cfg.num_experts, d = L->cfg.d_model, F = L->cfg.d_ff;
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
     int R = 0;
-    HIP_TRY(ctx, hipMemcpy(&R, static_cast<int*>(L->offsets.p) + E, 4, hipMemcpyDeviceToHost));
+    HIP_TRY(ctx, hipMemcpy(&R, L->last.offsets + E, 4, hipMemcpyDeviceToHost));
     const bool abf = L->cfg.act_dtype == RBMOE_BF16;
-    auto fetch = [&](float* dst, const Buf& src, size_t n) -> int {
+    auto fetch = [&](float* dst, const void* src, size_t n) -> int {
         if (!dst || n == 0) return RBMOE_OK;
         if (!abf) {
-            HIP_TRY(ctx, hipMemcpy(dst, src.p, n * 4, hipMemcpyDeviceToHost));
+            HIP_TRY(ctx, hipMemcpy(dst, src, n * 4, hipMemcpyDeviceToHost));
             return RBMOE_OK;
         }
         std::vector<uint16_t> tmp(n);
-        HIP_TRY(ctx, hipMemcpy(tmp.data(), src.p, n * 2, hipMemcpyDeviceToHost));
+        HIP_TRY(ctx, hipMemcpy(tmp.data(), src, n * 2, hipMemcpyDeviceToHost));
         for (size_t i = 0; i < n; ++i) dst[i] = host_bf16_to_f32(tmp[i]);
         return RBMOE_OK;
     };
-    int rc = fetch(hidden, L->h, (size_t)R * F);
+    int rc = fetch(hidden, L->last.h, (size_t)R * F);
     if (rc != RBMOE_OK) return rc;
-    return fetch(expert_out, L->y, (size_t)R * d);
+    return fetch(expert_out, L->last.y, (size_t)R * d);
 }
 
 const char* rbmoe_expert_kernel_name(const rbmoe_layer* L) { return L ? L->kernel_name : "none"; }

@@ -159,6 +159,7 @@ hipError_t launch_route_backward(const float* P, const float* lse, const int* ex
 // grad_router += dlogits^T . x (through `partial`, router_grad_chunks(max_tokens) * E * d floats) and
 // dxr = dlogits . wr
 int router_grad_chunks(int max_tokens);
+int router_grad_max_tokens();  // launch_router_grad refuses more rows than this
 hipError_t launch_router_grad(const float* dlogits, const void* x, const float* wr, int T, int d, int E,
                               float* partial, float* grad_router, void* dxr, bool bf16, hipStream_t s);
 // RmsNorm::backward (src/norm.rs:63-121): grad_input = d(norm)/dx applied to `up` (+ residual_grad when given),

@@ -12,11 +12,26 @@
 //
 // Nothing here uses floating-point atomics: every sum has a fixed order, so two
 // runs give the same bits.
+#include <atomic>
 #include <cstdlib>
 
 #include "rbmoe_kernels.h"
 
 namespace rbmoe {
+
+// A kernel attribute is set once per device.  `done` has one bit per device; setting an attribute twice is
+// harmless, so two threads that race here only repeat the call.  Devices past the 64th set it on every launch.
+template <typename F>
+static hipError_t once_per_device(std::atomic<unsigned long long>& done, F&& set) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const unsigned long long bit = dev < 64 ? 1ull << dev : 0ull;
+    if (bit && (done.load(std::memory_order_acquire) & bit)) return hipSuccess;
+    e = set();
+    if (e == hipSuccess && bit) done.fetch_or(bit, std::memory_order_release);
+    return e;
+}
 
 // Dynamic LDS layout of router_kernel (floats / ints, in this order):
 //   prob   [TB][ES]   logits, then exp, then probabilities   (ES = E | 1)
@@ -522,7 +537,9 @@ __global__ __launch_bounds__(256) void dispatch_fused_kernel(
         base[tid] = cb;
         mass[tid] = m;
     }
-    if (blk == 0 && tid == E) {
+    // the sum of lse^2 over the parts: by the last thread of the workgroup, which exists for every expert count
+    // (a thread numbered E does not when E is the workgroup size) and owns no expert column unless E is 256
+    if (blk == 0 && tid == 255) {
         float zs = 0.0f;
         for (int q = 0; q < parts; ++q) zs += part_mass[q * (E + 1) + E];
         mass[E] = zs;
@@ -992,15 +1009,17 @@ __global__ __launch_bounds__(256) void combine_any_kernel(
 template <typename XT>
 static hipError_t launch_router_t(const RouterArgs& a, hipStream_t s) {
     const int nb = (a.T + kRouterTokens - 1) / kRouterTokens;
-    static bool attr_set = false;
-    if (!attr_set) {  // allow more than the default 64 KiB of dynamic LDS (gfx950 has 160 KiB per CU)
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(router_kernel<XT, 1>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, kMaxRouterLds);
-        if (e == hipSuccess)
-            e = hipFuncSetAttribute(reinterpret_cast<const void*>(router_kernel<XT, kMaxExperts / 64>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, kMaxRouterLds);
+    static std::atomic<unsigned long long> attr_set{0};
+    {  // allow more than the default 64 KiB of dynamic LDS (gfx950 has 160 KiB per CU)
+        const hipError_t e = once_per_device(attr_set, [] {
+            hipError_t r = hipFuncSetAttribute(reinterpret_cast<const void*>(router_kernel<XT, 1>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kMaxRouterLds);
+            if (r == hipSuccess)
+                r = hipFuncSetAttribute(reinterpret_cast<const void*>(router_kernel<XT, kMaxExperts / 64>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, kMaxRouterLds);
+            return r;
+        });
         if (e != hipSuccess) return e;
-        attr_set = true;
     }
     // eight experts (waves) per workgroup share one staged slice of 64 token rows
     constexpr int NE = 8;
@@ -1041,12 +1060,13 @@ static hipError_t launch_dispatch_t(const DispatchArgs& a, hipStream_t s) {
                            a.perm_slot, a.perm_token, a.inv_pos, static_cast<XT*>(a.xg));
         return hipGetLastError();
     }
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(layout_scan_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+    static std::atomic<unsigned long long> attr_set{0};
+    {
+        const hipError_t e = once_per_device(attr_set, [] {
+            return hipFuncSetAttribute(reinterpret_cast<const void*>(layout_scan_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+        });
         if (e != hipSuccess) return e;
-        attr_set = true;
     }
     // runs for T == 0 too: it then writes zero counts, an empty tile table and zero losses
     hipLaunchKernelGGL(layout_scan_kernel, dim3(1), dim3(kScanThreads), scan_lds_bytes(a.E), s, a.blockcnt, a.partial,

@@ -263,11 +263,14 @@ class MoeLayer {
                                d_model_, grad_output.cols);
         Matrix grad_input(grad_output.rows, d_model_);
         if (act_ == RBMOE_F32) {
-            check(rbmoe_backward_host(layer_, grad_output.data.data(), grad_input.data.data()), device_->raw());
+            check(rbmoe_backward_host(layer_, grad_output.data.data(), (int32_t)grad_output.rows, (int32_t)grad_output.cols,
+                                      grad_input.data.data()),
+                  device_->raw());
         } else {
             std::vector<uint16_t> gin(grad_output.data.size()), gout(grad_output.data.size());
             for (size_t i = 0; i < gin.size(); ++i) gin[i] = to_bf16(grad_output.data[i]);
-            check(rbmoe_backward_host(layer_, gin.data(), gout.data()), device_->raw());
+            check(rbmoe_backward_host(layer_, gin.data(), (int32_t)grad_output.rows, (int32_t)grad_output.cols, gout.data()),
+                  device_->raw());
             for (size_t i = 0; i < gout.size(); ++i) grad_input.data[i] = from_bf16(gout[i]);
         }
         return grad_input;
@@ -304,11 +307,15 @@ class MoeLayer {
     Matrix backward_block(const Matrix& grad_output) {
         Matrix grad_input(grad_output.rows, d_model_);
         if (act_ == RBMOE_F32) {
-            check(rbmoe_backward_block_host(layer_, grad_output.data.data(), grad_input.data.data()), device_->raw());
+            check(rbmoe_backward_block_host(layer_, grad_output.data.data(), (int32_t)grad_output.rows,
+                                            (int32_t)grad_output.cols, grad_input.data.data()),
+                  device_->raw());
         } else {
             std::vector<uint16_t> gin(grad_output.data.size()), gout(grad_output.data.size());
             for (size_t i = 0; i < gin.size(); ++i) gin[i] = to_bf16(grad_output.data[i]);
-            check(rbmoe_backward_block_host(layer_, gin.data(), gout.data()), device_->raw());
+            check(rbmoe_backward_block_host(layer_, gin.data(), (int32_t)grad_output.rows, (int32_t)grad_output.cols,
+                                            gout.data()),
+                  device_->raw());
             for (size_t i = 0; i < gout.size(); ++i) grad_input.data[i] = from_bf16(gout[i]);
         }
         return grad_input;

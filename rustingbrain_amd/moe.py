@@ -452,7 +452,7 @@ class MoeLayer:
                                actual=grad_output.shape[-1] if grad_output.ndim else 0)
         g = self._to_act(grad_output)
         out = np.empty_like(g)
-        _check(self._lib.rbmoe_backward_host(self.handle, g.ctypes.data_as(C.c_void_p),
+        _check(self._lib.rbmoe_backward_host(self.handle, g.ctypes.data_as(C.c_void_p), g.shape[0], g.shape[1],
                                              out.ctypes.data_as(C.c_void_p)), self.device.handle)
         if self.act_dtype == "bf16":
             out = bf16_bits_to_f32(out).reshape(g.shape)
@@ -467,21 +467,23 @@ class MoeLayer:
                                actual=grad_output.shape[-1] if grad_output.ndim else 0)
         g = self._to_act(grad_output)
         out = np.empty_like(g)
-        _check(self._lib.rbmoe_backward_block_host(self.handle, g.ctypes.data_as(C.c_void_p),
+        _check(self._lib.rbmoe_backward_block_host(self.handle, g.ctypes.data_as(C.c_void_p), g.shape[0], g.shape[1],
                                                    out.ctypes.data_as(C.c_void_p)), self.device.handle)
         if self.act_dtype == "bf16":
             out = bf16_bits_to_f32(out).reshape(g.shape)
         return out
 
-    def backward_block_device(self, grad_output_ptr: int, grad_input_ptr: int) -> None:
-        """Enqueue the block step's backward pass on device pointers (no synchronisation)."""
-        _check(self._lib.rbmoe_backward_block(self.handle, C.c_void_p(grad_output_ptr), C.c_void_p(grad_input_ptr)),
-               self.device.handle)
+    def backward_block_device(self, grad_output_ptr: int, tokens: int, grad_input_ptr: int) -> None:
+        """Enqueue the block step's backward pass on device pointers (no synchronisation); both buffers are
+        ``[tokens, d_model]`` and ``tokens`` must be the last forward's."""
+        _check(self._lib.rbmoe_backward_block(self.handle, C.c_void_p(grad_output_ptr), tokens, self._d_model,
+                                              C.c_void_p(grad_input_ptr)), self.device.handle)
 
-    def backward_device(self, grad_output_ptr: int, grad_input_ptr: int) -> None:
-        """Enqueue the backward pass on device pointers (no synchronisation)."""
-        _check(self._lib.rbmoe_backward(self.handle, C.c_void_p(grad_output_ptr), C.c_void_p(grad_input_ptr)),
-               self.device.handle)
+    def backward_device(self, grad_output_ptr: int, tokens: int, grad_input_ptr: int) -> None:
+        """Enqueue the backward pass on device pointers (no synchronisation); both buffers are
+        ``[tokens, d_model]`` and ``tokens`` must be the last forward's."""
+        _check(self._lib.rbmoe_backward(self.handle, C.c_void_p(grad_output_ptr), tokens, self._d_model,
+                                        C.c_void_p(grad_input_ptr)), self.device.handle)
 
     def zero_grads(self) -> None:
         _check(self._lib.rbmoe_zero_grads(self.handle), self.device.handle)

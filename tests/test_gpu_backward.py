@@ -277,6 +277,24 @@ def test_training_mode_errors(device):
     fresh.forward_train(t.x)
     with pytest.raises(rb.InvalidInput):
         fresh.backward(np.zeros((8, 32), np.float32))
+    # buffers that do not have the last forward's rows are refused before a byte of them is touched, on host and
+    # on device pointers, with and without the norm in front
+    for rows in (7, 9, 0):
+        with pytest.raises(rb.InvalidInput, match="rows of the last forward"):
+            fresh.backward(np.zeros((rows, 64), np.float32))
+    lib = L.load()
+    import ctypes as C
+    small = np.zeros((1, 64), np.uint16)
+    for fn in (lib.rbmoe_backward, lib.rbmoe_backward_host):
+        assert fn(fresh.handle, small.ctypes.data_as(C.c_void_p), 9, 64, small.ctypes.data_as(C.c_void_p)) == L.INVALID_INPUT
+        assert fn(fresh.handle, small.ctypes.data_as(C.c_void_p), 8, 63, small.ctypes.data_as(C.c_void_p)) == L.INVALID_INPUT
+    fresh.set_feed_forward_norm(np.ones(64, np.float32))
+    fresh.forward_block(t.x)
+    with pytest.raises(rb.InvalidInput, match="rows of the last forward"):
+        fresh.backward_block(np.zeros((5, 64), np.float32))
+    for fn in (lib.rbmoe_backward_block, lib.rbmoe_backward_block_host):
+        assert fn(fresh.handle, small.ctypes.data_as(C.c_void_p), 1, 64, small.ctypes.data_as(C.c_void_p)) == L.INVALID_INPUT
+    assert fresh.backward_block(np.zeros((8, 64), np.float32)).shape == (8, 64)
     assert fresh.kernel_name().startswith("mfma_bf16")
     fresh.close()
 

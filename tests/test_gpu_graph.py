@@ -105,7 +105,7 @@ def test_training_step_replays_identically(device, hip, monkeypatch):
     def step():
         layer.zero_grads()
         layer.forward_device(x.ptr, T, out.ptr)
-        layer.backward_device(g.ptr, gin.ptr)
+        layer.backward_device(g.ptr, T, gin.ptr)
 
     step()
     device.synchronize()
@@ -114,7 +114,7 @@ def test_training_step_replays_identically(device, hip, monkeypatch):
                                                                       layer.weight_grad(L.W_SHARED_UP)]
     cap = Capture(hip, device, step)
     for _ in range(3):
-        layer.backward_device(g.ptr, gin.ptr)        # eager work in between: gradients now hold twice the values
+        layer.backward_device(g.ptr, T, gin.ptr)        # eager work in between: gradients now hold twice the values
         device.synchronize()
         cap.replay()
         assert np.array_equal(gin.download(np.empty_like(xh)), want_gin)

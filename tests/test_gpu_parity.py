@@ -295,3 +295,24 @@ def test_many_router_blocks_take_the_separate_layout_scan(device):
     valid = (np.arange(2100) % 13 != 5).astype(np.uint8)
     out, cache, ref = check_parity(device, t, valid=valid)
     assert int(cache.offsets[-1]) == int(valid.sum()) * 3
+
+
+@pytest.mark.parametrize("T", [8, 200, 512, 600])
+@pytest.mark.parametrize("act", ["f32", "bf16"])
+def test_the_largest_expert_count_keeps_both_losses(device, T, act):
+    # 256 experts is the routing kernels' limit and the workgroup size of the fused dispatch launch, where no
+    # thread is numbered E: the z-loss (the sum of lse^2 folded by one thread) must still come out.  With bf16
+    # rows T = 8 takes the single-workgroup routing; 200 and 512 take the fused dispatch launch, 600 the
+    # separate layout scan.
+    t = synth.make(small_workload(d=64, E=256, k=3, F=64, T=T, seed=23, act=act, wt=act))
+    ref = oracle_layer(t, z_w=0.7).forward(t.x, threads=8)
+    layer = gpu_layer(device, t, z_w=0.7)
+    out, cache = layer.forward_train(t.x)
+    assert_routing_identical(cache, ref)
+    assert ref.z_loss > 1e-3
+    assert abs(cache.z_loss() - ref.z_loss) <= 1e-5 * abs(ref.z_loss)
+    assert abs(cache.aux_loss() - ref.aux_loss) <= 1e-5 * max(abs(ref.aux_loss), 1e-6)
+    assert rel_l2(out, ref.out) <= tolerance(t.workload)
+    if act == "bf16":
+        assert layer.kernel_name() == ("mfma_bf16_decode" if T <= 32 else "mfma_bf16_stream")
+    layer.close()

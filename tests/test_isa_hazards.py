@@ -40,3 +40,4 @@ def test_streaming_kernel_has_no_use_of_outstanding_loads():
     assert len(res) >= 4, "expected every instantiation of the kernel in the assembly"
     bad = {k: v[:5] for k, v in res.items() if v}
     assert not bad, bad
+
