@@ -156,6 +156,24 @@ int rbmoe_set_weight(rbmoe_layer* layer, int32_t which, int32_t expert, const vo
 int rbmoe_forward(rbmoe_layer* layer, const void* x, int32_t T, int32_t cols, const uint8_t* valid,
                   const float* router_bias, const void* residual, void* out);
 
+/* rbmoe_forward for callers that cannot allocate device memory and want no allocation made on their behalf
+ * either: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference.  Same arguments and same results as rbmoe_forward (bit for bit: the same
+ * kernels run), but every intermediate buffer of the call (probabilities, routing tables, tile table, losses,
+ * hidden and expert output rows) lies in a static device array of RBMOE_STATIC_SCRATCH_BYTES that is part of
+ * the library's code object, instead of in the workspace that rbmoe_layer_create allocated.  The call makes
+ * no hipMalloc, hipFree or other allocating call.
+ * Limits: decode-shaped calls only, i.e. 1 to 32 tokens with tokens * num_experts <= 2048 on a bf16 layer with
+ * bf16 or int8 weights whose widths are multiples of 64, not in training mode; and the buffers of the call
+ * (about tokens * experts_per_token * (d_ff + d_model) * 2 bytes, plus the shared expert's rows and the tables)
+ * must fit the array.  Anything else is RBMOE_UNSUPPORTED with a message that says which limit was hit.
+ * Every call on one GPU, from any layer or context, uses that GPU's one array: calls that overlap in time on
+ * one GPU race, and rbmoe_get_losses / rbmoe_get_routing / rbmoe_get_expert_rows after this call read the array,
+ * so they describe this call only until the next static call on the same GPU. */
+#define RBMOE_STATIC_SCRATCH_BYTES (8u << 20)
+int rbmoe_forward_static(rbmoe_layer* layer, const void* x, int32_t T, int32_t cols, const uint8_t* valid,
+                         const float* router_bias, const void* residual, void* out);
+
 /* Same on HOST pointers: copies in, runs, synchronises, copies out. */
 int rbmoe_forward_host(rbmoe_layer* layer, const void* x, int32_t T, int32_t cols,
                        const uint8_t* valid, const float* router_bias, const void* residual,

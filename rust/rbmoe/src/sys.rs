@@ -82,6 +82,9 @@ extern "C" {
                             scales: *const f32, rows: i32, cols: i32) -> c_int;
     pub fn rbmoe_forward(layer: *mut rbmoe_layer, x: *const c_void, tokens: i32, cols: i32, valid: *const u8,
                          router_bias: *const f32, residual: *const c_void, out: *mut c_void) -> c_int;
+    // rbmoe_forward with every intermediate buffer in the library's static device array (no allocation)
+    pub fn rbmoe_forward_static(layer: *mut rbmoe_layer, x: *const c_void, tokens: i32, cols: i32, valid: *const u8,
+                                router_bias: *const f32, residual: *const c_void, out: *mut c_void) -> c_int;
     pub fn rbmoe_forward_host(layer: *mut rbmoe_layer, x: *const c_void, tokens: i32, cols: i32, valid: *const u8,
                               router_bias: *const f32, residual: *const c_void, out: *mut c_void) -> c_int;
     pub fn rbmoe_forward_timed(layer: *mut rbmoe_layer, x: *const c_void, tokens: i32, cols: i32, valid: *const u8,

@@ -20,6 +20,7 @@ DTYPES = {"f32": F32, "bf16": BF16, "int8": I8}
 # rbmoe_weight
 W_ROUTER, W_GATE, W_UP, W_DOWN, W_SHARED_GATE, W_SHARED_UP, W_SHARED_DOWN, W_NORM = range(8)
 NUM_STAGES = 8
+STATIC_SCRATCH_BYTES = 8 << 20
 STAGE_NAMES = ("router", "empty", "dispatch", "gate_up", "down", "shared", "combine", "total")
 
 
@@ -54,6 +55,8 @@ SIGNATURES = {
                                    C.POINTER(C.c_float), C.c_int32, C.c_int32]),
     "rbmoe_forward": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p,
                                 C.c_void_p, C.c_void_p]),
+    "rbmoe_forward_static": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p,
+                                       C.c_void_p, C.c_void_p]),
     "rbmoe_forward_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p,
                                      C.c_void_p, C.c_void_p]),
     "rbmoe_forward_timed": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p,

@@ -12,6 +12,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -19,7 +20,35 @@
 
 using namespace rbmoe;
 
+// Scratch of rbmoe_forward_static: device memory that exists without any allocation call.  Every GPU the library
+// runs on holds its own copy of the array, at its own address, until the process ends.  In host code the
+// array's name is only a handle for hipGetSymbolAddress: rbmoe_ctx_create resolves it once per device and host
+// code uses the resolved pointer from then on.
+// (No `used` attribute: the compiler makes a static device variable visible to the runtime's lookup by name
+// because host code takes its address below, and only then; marked `used` it stays a local symbol, which
+// hipGetSymbolAddress cannot find.)
+static __device__ __align__(256) unsigned char rbmoe_static_scratch[RBMOE_STATIC_SCRATCH_BYTES];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};  // per device: the address of rbmoe_static_scratch there
+
+// With `device` current.  Resolved once per device and kept.
+hipError_t static_scratch_of(int device, void** out) {
+    *out = nullptr;
+    if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[device]) {
+        void* p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(rbmoe_static_scratch));
+        if (e != hipSuccess) return e;
+        g_scratch_ptr[device] = p;
+    }
+    *out = g_scratch_ptr[device];
+    return hipSuccess;
+}
 
 thread_local std::string g_global_error;
 
@@ -84,6 +113,7 @@ struct rbmoe_ctx {
     hipEvent_t ev_fork = nullptr, ev_fork2 = nullptr, ev_join = nullptr;
     size_t budget_bytes = 0;
     size_t allocated = 0;
+    void* static_scratch = nullptr;  // this device's copy of rbmoe_static_scratch (RBMOE_STATIC_SCRATCH_BYTES)
     std::string last_error;
     int refs = 1;  // the caller's handle + one per live layer; torn down when the last one goes
 };
@@ -115,8 +145,8 @@ int hip_fail(rbmoe_ctx* ctx, hipError_t e, const char* what) {
 
 }  // namespace
 
-// Where one forward pass keeps its routing tables and expert rows (the layer's workspace).  The getters read
-// the last forward's.
+// Where one forward pass keeps its routing tables and expert rows: the layer's own workspace, or a carving of
+// the static scratch array (rbmoe_forward_static).  The getters read the last forward's.
 struct Work {
     float* P = nullptr;
     float* lse = nullptr;
@@ -349,8 +379,11 @@ int rbmoe_ctx_create(int32_t device, size_t budget_mib, rbmoe_ctx** out) {
     if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(nullptr, RBMOE_UNSUPPORTED, std::string("kernels are built for gfx950, device is ") + prop.gcnArchName);
     HIP_TRY(nullptr, hipSetDevice(device));
+    void* scratch = nullptr;
+    HIP_TRY(nullptr, static_scratch_of(device, &scratch));
     rbmoe_ctx* ctx = new rbmoe_ctx();
     ctx->device = device;
+    ctx->static_scratch = scratch;
     ctx->budget_bytes = budget_mib << 20;
     hipError_t se = hipStreamCreateWithFlags(&ctx->own_stream, hipStreamNonBlocking);
     if (se != hipSuccess) {
@@ -703,10 +736,42 @@ Work work_of_layer(const rbmoe_layer* L) {
     return w;
 }
 
+// The buffers of a decode-shaped forward of T tokens carved out of `base` (pieces of 256 bytes); returns the
+// bytes used.  With base == nullptr only the size is computed.
+size_t carve_decode_work(const rbmoe_layer* L, int T, unsigned char* base, Work* w) {
+    const rbmoe_config& c = L->cfg;
+    const size_t E = c.num_experts, d = c.d_model, F = c.d_ff, k = c.experts_per_token, Fs = L->Fs;
+    const size_t S = (size_t)T * k, as = dtype_size(c.act_dtype);
+    const size_t tiles = S / kDecodeTileM + E + 1;
+    size_t used = 0;
+    auto take = [&](size_t bytes) -> void* {
+        void* p = base ? base + used : nullptr;
+        used += (std::max<size_t>(bytes, 1) + 255) & ~(size_t)255;
+        return p;
+    };
+    Work v;
+    v.P = (float*)take((size_t)T * E * 4); v.lse = (float*)take((size_t)T * 4);
+    v.expert_of = (int*)take(S * 4); v.gate_of = (float*)take(S * 4);
+    v.counts = (int*)take(E * 4); v.offsets = (int*)take((E + 1) * 4);
+    v.tile_expert = (int*)take(tiles * 4); v.tile_row0 = (int*)take(tiles * 4); v.tile_rows = (int*)take(tiles * 4);
+    v.ntiles = (int*)take(8); v.losses = (float*)take(8);
+    v.perm_slot = (int*)take(S * 4); v.perm_token = (int*)take(S * 4); v.inv_pos = (int*)take(S * 4);
+    v.h = take(S * F * as); v.y = take(S * d * as);
+    if (c.shared_expert) {
+        v.hs = take((size_t)T * Fs * as);
+        v.ys = take((size_t)T * d * as);
+    }
+    if (w) *w = v;
+    return used;
+}
+
 // `norm_src` (block step): the raw rows; `x` is then the layer's buffer of normed rows, filled here - by the
 // small-route kernel itself for a few tokens, by the norm kernel otherwise - before anything reads it.
+// `static_scratch` (rbmoe_forward_static): this device's copy of the static scratch array; the call must then be
+// decode-shaped, keeps every intermediate result there and touches none of the layer's workspace.
 int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* valid, const float* router_bias,
-                 const void* residual, void* out, bool timed, const void* norm_src = nullptr) {
+                 const void* residual, void* out, bool timed, const void* norm_src = nullptr,
+                 void* static_scratch = nullptr) {
     if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
     rbmoe_ctx* ctx = L->ctx;
     const rbmoe_config& c = L->cfg;
@@ -751,6 +816,27 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     const bool norm_in_route = norm_src && decode_ok &&
                                small_route_stages_rows(norm_src, (const float*)L->router.p, T, d, E, abf);
     Work wk_ = work_of_layer(L);
+    if (static_scratch) {
+        if (!decode_ok) {
+            char buf[200];
+            std::snprintf(buf, sizeof buf,
+                          "rbmoe_forward_static takes decode-shaped calls only: 1 to %d tokens of a bf16 layer with "
+                          "bf16 or int8 weights on the matrix-core path, not in training mode (got %d tokens)",
+                          kSmallRouteMaxTokens, T);
+            return fail(ctx, RBMOE_UNSUPPORTED, buf);
+        }
+        const size_t need = carve_decode_work(L, T, nullptr, nullptr);
+        if (need > (size_t)RBMOE_STATIC_SCRATCH_BYTES) {
+            char buf[200];
+            std::snprintf(buf, sizeof buf, "this call needs %zu bytes of scratch, the static buffer holds %zu", need,
+                          (size_t)RBMOE_STATIC_SCRATCH_BYTES);
+            return fail(ctx, RBMOE_UNSUPPORTED, buf);
+        }
+        // Nothing of it is cleared: every word a kernel of this call reads was written by an earlier kernel of
+        // the same call (the tile-table entries past *ntiles, which the product kernels fetch and drop, may be
+        // a previous call's).
+        carve_decode_work(L, T, static_cast<unsigned char*>(static_scratch), &wk_);
+    }
     if (norm_src && !norm_in_route)
         HIP_TRY(ctx, launch_rmsnorm(norm_src, (const float*)L->norm_w.p, L->norm_eps, T, d, L->xn.p, abf, s));
 
@@ -992,6 +1078,13 @@ extern "C" {
 int rbmoe_forward(rbmoe_layer* L, const void* x, int32_t T, int32_t cols, const uint8_t* valid,
                   const float* router_bias, const void* residual, void* out) {
     return forward_impl(L, x, T, cols, valid, router_bias, residual, out, false);
+}
+
+int rbmoe_forward_static(rbmoe_layer* L, const void* x, int32_t T, int32_t cols, const uint8_t* valid,
+                         const float* router_bias, const void* residual, void* out) {
+    if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
+    if (!L->ctx->static_scratch) return fail(L->ctx, RBMOE_DEVICE_ERROR, "the static scratch buffer was not resolved");
+    return forward_impl(L, x, T, cols, valid, router_bias, residual, out, false, nullptr, L->ctx->static_scratch);
 }
 
 int rbmoe_forward_timed(rbmoe_layer* L, const void* x, int32_t T, int32_t cols, const uint8_t* valid,

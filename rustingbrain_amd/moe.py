@@ -347,6 +347,15 @@ class MoeLayer:
                                        C.c_void_p(valid_ptr or None), C.c_void_p(bias_ptr or None),
                                        C.c_void_p(residual_ptr or None), C.c_void_p(out_ptr)), self.device.handle)
 
+    def forward_static_device(self, x_ptr: int, tokens: int, out_ptr: int, valid_ptr: int = 0, bias_ptr: int = 0,
+                              residual_ptr: int = 0) -> None:
+        """``forward_device`` with every intermediate buffer in the library's static device array: the call
+        allocates nothing.  Decode-shaped calls only (``Unsupported`` otherwise)."""
+        _check(self._lib.rbmoe_forward_static(self.handle, C.c_void_p(x_ptr), tokens, self._d_model,
+                                              C.c_void_p(valid_ptr or None), C.c_void_p(bias_ptr or None),
+                                              C.c_void_p(residual_ptr or None), C.c_void_p(out_ptr)),
+               self.device.handle)
+
     def forward_timed(self, x_ptr: int, tokens: int, out_ptr: int, valid_ptr: int = 0, bias_ptr: int = 0,
                       residual_ptr: int = 0) -> dict:
         ms = (C.c_float * L.NUM_STAGES)()

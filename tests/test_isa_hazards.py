@@ -41,3 +41,20 @@ def test_streaming_kernel_has_no_use_of_outstanding_loads():
     bad = {k: v[:5] for k, v in res.items() if v}
     assert not bad, bad
 
+
+@pytest.mark.skipif(shutil.which("hipcc") is None and not os.path.exists("/opt/rocm/bin/hipcc"), reason="needs hipcc")
+def test_static_scratch_array_is_a_symbol_the_runtime_can_look_up():
+    # rbmoe_forward_static's scratch is a static device array whose address the host asks the runtime for by name
+    # (hipGetSymbolAddress).  The runtime searches the code object's global symbols, and a missing one ends the
+    # process rather than returning an error - so the array must come out of the device compilation as a global
+    # object of the declared size, not as a local one.
+    src = os.path.join(HERE, "..", "rustingbrain_amd", "csrc", "rbmoe_api.hip")
+    with tempfile.TemporaryDirectory() as tmp:
+        out = os.path.join(tmp, "rbmoe_api.s")
+        cmd = [rb_build.HIPCC] + [f for f in rb_build.FLAGS if f != "-fPIC"] + ["-S", "--cuda-device-only", "-o", out, src]
+        subprocess.run(cmd, check=True, capture_output=True)
+        lines = [ln.strip() for ln in open(out) if "rbmoe_static_scratch" in ln]
+    name = next(ln.split()[1].split(",")[0] for ln in lines if ln.startswith(".type"))
+    assert f".globl {name}" in [" ".join(ln.split()) for ln in lines], lines
+    assert not any(ln.startswith(".local") for ln in lines), lines
+    assert any(ln.startswith(".size") and ln.endswith(str(8 << 20)) for ln in lines), lines
