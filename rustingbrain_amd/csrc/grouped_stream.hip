@@ -15,11 +15,15 @@
 //                (global_load_lds_dwordx4): lane l of a wave deposits its 16
 //                bytes at LDS base + 16 l, so the XOR swizzle that keeps the
 //                fragment reads free of bank conflicts is applied by choosing
-//                which global piece each lane fetches.  Two LDS stages; the DMA
-//                for slice k + 1 is issued when slice k starts and is awaited
-//                (vmcnt) just before the barrier that ends slice k.
+//                which global piece each lane fetches.  Three LDS stages: the
+//                DMA for slice k + 2 is issued in the last step of slice k, after
+//                the barrier (behind step KS - 2) that proves its stage free, and
+//                is awaited (vmcnt) just before the barrier of slice k + 1.
 //   fragments    token fragments are read from LDS one step ahead of the
-//                multiplies that use them.
+//                multiplies that use them, across slice boundaries too.
+//   issue order  a wave that is alone on its SIMD must keep the matrix core fed
+//                by itself: every memory instruction of the main loop sits
+//                behind a multiply of its own (see pipe_loop).
 // A workgroup is 4 waves side by side along the output features; a wave owns
 // 128 tokens x 64 weight rows (32 gate + the matching 32 up rows, or 64 down
 // rows).  The weight fragment is the matrix-core A operand and the token
@@ -27,9 +31,17 @@
 // one token and writes them with one 8-byte store.  Token blocks of 32 rows
 // that lie beyond the end of a group are skipped, so a ragged group costs at
 // most 31 rows of padding.
+#include <algorithm>
 #include <type_traits>
 
 #include "rbmoe_kernels.h"
+
+// Hook for timeline studies of the kernels: a harness that includes this file may define it to record a time
+// stamp per tile (`slot` = the tile's number in launch order) at point i (0 tile taken up, 1 main loop entered,
+// 2 main loop left, 3 tile written).  Expands to nothing in the library.
+#ifndef RBMOE_TRACE_AT
+#define RBMOE_TRACE_AT(slot, i)
+#endif
 
 namespace rbmoe {
 
@@ -87,6 +99,14 @@ __device__ __forceinline__ void static_for(F&& f) {
     }
 }
 
+// f(0), f(1), ... while f returns true: slice I + 1 of a loop's remainder is reached only through slice I
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_while(F&& f) {
+    if constexpr (I < N) {
+        if (f(std::integral_constant<int, I>{})) static_while<I + 1, N>(f);
+    }
+}
+
 // One ring slot: the wave's two weight fragments of one reduction step.
 // bf16: 16 bytes per lane per fragment, step g at byte 1024 g + 16 lane of a row block.
 // int8: 8 bytes per lane per fragment; the packed layout is [K/32][64 lanes][16 bytes] with
@@ -101,6 +121,9 @@ struct Slot<false> {
         issue_load(f0, off, p0);
         issue_load(f1, off, p1);
     }
+    static __device__ __forceinline__ uint32_t offset(int g, uint32_t lane16) { return lane16 + (uint32_t)g * 1024u; }
+    __device__ __forceinline__ void load0(const char* p0, uint32_t off) { issue_load(f0, off, p0); }
+    __device__ __forceinline__ void load1(const char* p1, uint32_t off) { issue_load(f1, off, p1); }
     __device__ __forceinline__ bf16x8 a0() const { return __builtin_bit_cast(bf16x8, f0); }
     __device__ __forceinline__ bf16x8 a1() const { return __builtin_bit_cast(bf16x8, f1); }
 };
@@ -112,265 +135,59 @@ struct Slot<true> {
         issue_load(f0, off, p0);
         issue_load(f1, off, p1);
     }
+    static __device__ __forceinline__ uint32_t offset(int g, uint32_t lane16) {
+        return lane16 + (uint32_t)(g >> 1) * 1024u + (uint32_t)(g & 1) * 8u;
+    }
+    __device__ __forceinline__ void load0(const char* p0, uint32_t off) { issue_load(f0, off, p0); }
+    __device__ __forceinline__ void load1(const char* p1, uint32_t off) { issue_load(f1, off, p1); }
     __device__ __forceinline__ bf16x8 a0() const { return widen_i8(make_uint2(f0.x, f0.y)); }
     __device__ __forceinline__ bf16x8 a1() const { return widen_i8(make_uint2(f1.x, f1.y)); }
 };
 
-// RING = weight-fragment steps in flight per wave (register ring depth);
-// TFBUF = 2: token fragments are read from LDS one step ahead, 1: just in time.
-template <bool SWIGLU, bool I8, int RING, int TFBUF, bool AREG>
-__global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
-    const bf16_t* __restrict__ a, const int* __restrict__ row_index, const void* __restrict__ wpacked,
-    size_t w_expert_stride_bytes, const float* __restrict__ scales, size_t s_expert_stride, int N, int K,
-    const int* __restrict__ tile_expert, const int* __restrict__ tile_row0, const int* __restrict__ tile_rows,
-    const int* __restrict__ ntiles, int dense_rows, bf16_t* __restrict__ out, bf16_t* __restrict__ gu_out,
-    const bf16_t* __restrict__ bw_gu,
-    int group_m) {
-    constexpr int BN = SWIGLU ? NW * 32 : NW * 64;  // output features per workgroup
-    // Two LDS stages of one activation slice each; the epilogue reuses both as one
-    // 128 x 128 staging tile for the output.
-    __shared__ uint4 As[2 * BM * CPR];
-    uint4* const As0 = As;
-    uint4* const As1 = As + BM * CPR;
+// ---- epilogue: the accumulators of one tile to memory -------------------------------------------------
+struct TileOut {
+    int rows, row0, tn_idx, N;
+    bool act0, act1;      // whether the wave's two row blocks lie inside N
+    int r0, r1;           // their first weight rows
+    const float* sc;      // int8: the expert's scales, one per weight row
+    bf16_t* out;
+    bf16_t* gu_out;
+    const bf16_t* bw_gu;
+};
 
-    // ---- which tile (each XCD walks a contiguous range, M fastest inside a group)
-    const int tiles_n = (N + BN - 1) / BN;
-    const int tiles_m = dense_rows >= 0 ? (dense_rows + BM - 1) / BM : *ntiles;
-    const int total = tiles_m * tiles_n;
-    const int per_xcd = (total + 7) / 8;
-    const int local = blockIdx.x >> 3;
-    if (local >= per_xcd) return;
-    const int pid = (blockIdx.x & 7) * per_xcd + local;
-    if (pid >= total) return;
-    const int per_group = group_m * tiles_n;
-    const int grp = pid / per_group;
-    const int first_m = grp * group_m;
-    const int gsize = min(group_m, tiles_m - first_m);
-    const int in_g = pid - grp * per_group;
-    const int tm_idx = first_m + in_g % gsize;
-    const int tn_idx = in_g / gsize;
-
-    int expert, row0, rows;
-    if (dense_rows >= 0) {
-        expert = 0;
-        row0 = tm_idx * BM;
-        rows = min(BM, dense_rows - row0);
-    } else {
-        expert = tile_expert[tm_idx];
-        row0 = tile_row0[tm_idx];
-        rows = tile_rows[tm_idx];
-    }
-    const int nblk = (rows + 31) >> 5;  // token blocks that hold at least one row
-
-    const int tid = threadIdx.x;
+// `stage`: 32 KiB of LDS that no wave of the workgroup reads or writes any more (the caller has made sure of
+// that with a barrier).  `before_stores()` is called once, when the first pass has been converted and staged and
+// before its first store to memory is issued.
+template <bool SWIGLU, bool I8, typename F>
+__device__ __forceinline__ void write_tile(const TileOut& o, floatx16 (&acc)[2][TT], char* const stage,
+                                           F&& before_stores) {
+    constexpr int BN = SWIGLU ? NW * 32 : NW * 64;
+    // The thread index is made opaque here: everything derived from it below (LDS and row offsets, two dozen
+    // values per lane) is then worked out where it is used.  Otherwise a caller that writes tile after tile has
+    // them computed once, in front of its tile loop, and carried through the main loop in registers that the
+    // loop does not have.
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-
-    // ---- this wave's two blocks of 32 weight rows ---------------------------
-    // A wave whose rows lie past N (ragged last feature tile) runs the same loop on row
-    // block 0, so that every wave issues the same loads and meets the same barriers; it
-    // stores nothing.
-    // gate/up: gate rows nw .. nw + 31 and the matching up rows; down: rows nw .. nw + 31 and
-    // the rows 128 further on, so that each block index covers 128 consecutive features of
-    // the workgroup's tile.
-    const int nw = tn_idx * BN + wave * 32;
-    const int r0 = nw, r1 = SWIGLU ? N + nw : nw + NW * 32;
-    const bool act0 = nw < N;
-    const bool act1 = SWIGLU ? act0 : (nw + NW * 32 < N);
-    const size_t block_bytes = (size_t)K * 32 * (I8 ? 1 : 2);  // one block of 32 weight rows over all of K
-    const char* wexp = static_cast<const char*>(wpacked) + (size_t)expert * w_expert_stride_bytes;
-    const char* wp0 = wexp + (size_t)(act0 ? r0 / 32 : 0) * block_bytes;
-    const char* wp1 = wexp + (size_t)(act1 ? r1 / 32 : 0) * block_bytes;
-    const uint32_t lane16 = (uint32_t)lane * 16u;
-
-    // ---- LDS-DMA of the activation slice --------------------------------------
-    // Wave w fills LDS rows [32 w, 32 w + 32): instruction j covers rows 32 w + 8 j .. + 7,
-    // lane l lands in row 8 j + l / 8 (of the wave's 32), position l % 8, and therefore
-    // fetches logical piece (l % 8) ^ ((row / 2) % 8): a 16-lane group of a fragment read
-    // (16 consecutive rows, one logical piece) then touches 8 distinct pieces in the even rows
-    // and 8 in the odd rows, i.e. all 64 banks once.  Rows past the end of the group are
-    // clamped to the tile's first row: their products are never stored.
-    // Byte offsets from `a` fit 32 bits (the launcher checks rows * K * 2 < 4 GiB).
-    const char* const a_base = reinterpret_cast<const char*>(a);
-    uint32_t a_src[DMA_PER_WAVE];
-#pragma unroll
-    for (int j = 0; j < DMA_PER_WAVE; ++j) {
-        const int r = wave * 32 + j * 8 + (lane >> 3);
-        const int rr = r < rows ? r : 0;
-        const int grow = row_index ? row_index[row0 + rr] : row0 + rr;
-        a_src[j] = ((uint32_t)grow * (uint32_t)K + 8u * ((lane & 7) ^ ((r >> 1) & 7))) * 2u;
-    }
-    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)As0 + wave * 32 * CPR * 16;
-    const uint32_t lds1 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)As1 + wave * 32 * CPR * 16;
-    auto dma_a = [&](int kt, auto buf_tag) {
-        constexpr int BUF = decltype(buf_tag)::value;
-#pragma unroll
-        for (int j = 0; j < DMA_PER_WAVE; ++j)
-            issue_dma((BUF ? lds1 : lds0) + j * 8 * CPR * 16, a_src[j] + (uint32_t)kt * (BK * 2), a_base);
-    };
-
-    floatx16 acc[2][TT];
-#pragma unroll
-    for (int b = 0; b < 2; ++b)
-#pragma unroll
-        for (int t = 0; t < TT; ++t)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[b][t][v] = 0.0f;
-
     const int lrow = lane & 31;
     const int lhalf = lane >> 5;
-    const int lxor = (lrow >> 1) & 7;
-
-    const int KT = K / BK;
-    const int GS = KT * KS;  // reduction steps in all
-    constexpr int D = RING - 1;  // the load for step g + D is issued while step g runs
-
-    // ---- prologue: first activation slice, first D weight steps -----------------
-    // AREG: the activation slice travels global -> VGPR -> LDS instead of by LDS-DMA, one
-    // 1 KB piece per wave per step: piece j of slice k + 2 is fetched in step j of slice k and
-    // written to LDS in step j of slice k + 1 (into the stage slice k read).  Slices 0 and 1
-    // are placed by the prologue, so that no load is in flight where the loop is entered
-    // (the compiler may copy registers there); the first slice's writes go to a spare row.
-    u32x4 areg[DMA_PER_WAVE];
-    uint4* const a_dst0 = As0 + (wave * 32) * CPR + lane;
-    uint4* const a_dst1 = As1 + (wave * 32) * CPR + lane;
-    __shared__ uint4 spare[AREG ? NT : 1];
-    Slot<I8> ring[RING];
-    if constexpr (AREG) {
-        u32x4 first[DMA_PER_WAVE];
-#pragma unroll
-        for (int j = 0; j < DMA_PER_WAVE; ++j) issue_load(first[j], a_src[j], a_base);
-#pragma unroll
-        for (int j = 0; j < DMA_PER_WAVE; ++j)
-            issue_load(areg[j], a_src[j] + (uint32_t)min(1, KT - 1) * (BK * 2), a_base);
-#pragma unroll
-        for (int g = 0; g < D; ++g) ring[g].load(wp0, wp1, min(g, GS - 1), lane16);
-        wait_outstanding<0>();
-#pragma unroll
-        for (int j = 0; j < DMA_PER_WAVE; ++j) {
-            asm volatile("" : "+v"(first[j]), "+v"(areg[j]));
-            a_dst0[j * 8 * CPR] = make_uint4(first[j].x, first[j].y, first[j].z, first[j].w);
-            a_dst1[j * 8 * CPR] = make_uint4(areg[j].x, areg[j].y, areg[j].z, areg[j].w);
-        }
-        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
-    } else {
-        dma_a(0, std::integral_constant<int, 0>{});
-#pragma unroll
-        for (int g = 0; g < D; ++g) ring[g].load(wp0, wp1, min(g, GS - 1), lane16);
-        wait_outstanding<0>();
-    }
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_sched_barrier(0);
-
-    // One slice = KS steps.  BUF is the LDS stage the slice reads (its parity); the ring
-    // position of the slice's first step is 0, or BUF * KS when the ring holds two slices.
-    // NB = token blocks of this tile that hold rows, a compile-time constant inside the
-    // loop: a run-time branch per block between the multiplies costs far more than the
-    // skipped multiplies save, so the whole loop is specialised instead.
-    // The loop is straight-line and every wave issues, per slice, exactly: 4 DMA
-    // instructions, then 2 weight loads in each of the KS steps.  Past the end the last
-    // slice / step is fetched again, so that the counts below hold everywhere.
-    auto slice = [&](int kt, auto buf_tag, auto nb_tag) {
-        constexpr int BUF = decltype(buf_tag)::value;
-        constexpr int G0 = RING == 2 * KS ? BUF * KS : 0;
-        constexpr int NB = decltype(nb_tag)::value;
-        if constexpr (!AREG) dma_a(min(kt + 1, KT - 1), std::integral_constant<int, BUF ^ 1>{});
-        const uint4* Ab = BUF ? As1 : As0;
-        bf16x8 tf[TFBUF][TT];
-#pragma unroll
-        for (int t = 0; t < NB; ++t) tf[0][t] = lds_frag(Ab, (t * 32 + lrow) * CPR + (lhalf ^ lxor));
-        static_for<0, KS>([&](auto s_tag) {
-            constexpr int s = decltype(s_tag)::value;
-            const int g = kt * KS + s;
-            Slot<I8>& cur = ring[(G0 + s) % RING];
-            // weight fragments for step g + D go into the slot step g - 1 released
-            ring[(G0 + s + D) % RING].load(wp0, wp1, min(g + D, GS - 1), lane16);
-            if constexpr (TFBUF == 2) {
-                if (s + 1 < KS) {
-                    const int piece = (2 * (s + 1) + lhalf) ^ lxor;
-#pragma unroll
-                    for (int t = 0; t < NB; ++t) tf[(s + 1) & 1][t] = lds_frag(Ab, (t * 32 + lrow) * CPR + piece);
-                }
-            } else if (s > 0) {
-                const int piece = (2 * s + lhalf) ^ lxor;
-#pragma unroll
-                for (int t = 0; t < NB; ++t) tf[0][t] = lds_frag(Ab, (t * 32 + lrow) * CPR + piece);
-            }
-            if constexpr (AREG) {
-                // Per step: 2 weight loads, then 1 activation load.  Younger than the weight loads
-                // of step g: 3 per step for D steps.  The activation piece this step writes to LDS
-                // was fetched a whole slice ago, i.e. is older still.
-                static_assert(KS == DMA_PER_WAVE && D <= KS, "one activation piece per step, fetched KS steps before use");
-                wait_for<3 * D>(cur.f0, cur.f1);
-                asm volatile("" : "+v"(areg[s]));
-                uint4* const dst = kt > 0 ? (BUF ? a_dst0 : a_dst1) + s * 8 * CPR : spare + tid;
-                *dst = make_uint4(areg[s].x, areg[s].y, areg[s].z, areg[s].w);
-                issue_load(areg[s], a_src[s] + (uint32_t)min(kt + 2, KT - 1) * (BK * 2), a_base);
-            } else {
-                // Younger than the loads of step g: the weight loads of steps g+1 .. g+D (2 each)
-                // and the DMA (4) of every slice that started after they were issued.
-                wait_for<2 * D + DMA_PER_WAVE * ((D - s + KS - 1) / KS)>(cur.f0, cur.f1);
-            }
-            const bf16x8 w0 = cur.a0();
-            const bf16x8 w1 = cur.a1();
-#pragma unroll
-            for (int t = 0; t < NB; ++t) {
-                acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w0, tf[s % TFBUF][t], acc[0][t], 0, 0, 0);
-                acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w1, tf[s % TFBUF][t], acc[1][t], 0, 0, 0);
-            }
-        });
-        // Every LDS read of this slice has been consumed by a multiply issued above this
-        // point.  The DMA of the next slice is older than this slice's 2 * KS weight loads.
-        __builtin_amdgcn_sched_barrier(0);
-        if constexpr (AREG)
-            asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");  // this wave's pieces of the next slice are in LDS
-        else
-            wait_outstanding<2 * KS>();
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-    };
-
-    static_assert(RING == KS || RING == 2 * KS, "ring depth is one or two slices");
-    static_assert(DMA_PER_WAVE == 4, "the wait counts assume 4 DMA instructions per wave per slice");
-    auto run = [&](auto nb_tag) {
-        int kt = 0;
-        for (; kt + 1 < KT; kt += 2) {
-            slice(kt, std::integral_constant<int, 0>{}, nb_tag);
-            slice(kt + 1, std::integral_constant<int, 1>{}, nb_tag);
-        }
-        if (kt < KT) slice(kt, std::integral_constant<int, 0>{}, nb_tag);
-        // The loads fetched again past the end still target ring registers and LDS.  Naming
-        // the registers after the wait keeps them allocated until their data has arrived: a
-        // loaded value the compiler sees no use for would otherwise hand its register to
-        // something live while the load is still in flight.  (Done here, inside each
-        // specialisation, so that no path leaves it with loads outstanding.)
-        wait_outstanding<0>();
-        auto& ring_ref = ring;
-        auto& areg_ref = areg;
-#pragma unroll
-        for (int i = 0; i < RING; ++i) asm volatile("" : : "v"(ring_ref[i].f0), "v"(ring_ref[i].f1));
-#pragma unroll
-        for (int j = 0; j < DMA_PER_WAVE; ++j) asm volatile("" : : "v"(areg_ref[j]));
-    };
-    static_assert(TT == 4, "one specialisation per possible block count");
-    if (nblk == 4) run(std::integral_constant<int, 4>{});
-    else if (nblk == 3) run(std::integral_constant<int, 3>{});
-    else if (nblk == 2) run(std::integral_constant<int, 2>{});
-    else run(std::integral_constant<int, 1>{});
-    // ---- epilogue -------------------------------------------------------------
+    const int rows = o.rows, row0 = o.row0, tn_idx = o.tn_idx, N = o.N, r0 = o.r0, r1 = o.r1;
+    const bool act0 = o.act0, act1 = o.act1;
+    const float* const sc = o.sc;
+    bf16_t* const out = o.out;
+    bf16_t* const gu_out = o.gu_out;
+    const bf16_t* const bw_gu = o.bw_gu;
     // Accumulator element v of block (b, t): feature 8*(v/4) + 4*(lane/32) + v%4 of the
     // wave's row block b, token t*32 + lane%32 - a lane holds 4 consecutive features of a
     // token, so a direct store would scatter 8-byte pieces over 32 rows per instruction.
     // Instead each block index goes through LDS as a 128-token x 128-feature tile (16-byte
     // pieces, piece p of row r kept at position p ^ (r % 16)), and is written out with
     // 16-byte stores, 16 consecutive lanes covering the 256 contiguous bytes of a row.
-    const float* sc = I8 ? scales + (size_t)expert * s_expert_stride : nullptr;
-    char* const stage = reinterpret_cast<char*>(As);
     // Passes through the staging tile: down product: the two blocks of 128 features; gate/up: the
     // hidden rows, then (only when the caller keeps them for a backward pass) the gate and the
     // up pre-activations, which go to `gu_out` [rows, 2N] with the gate half in columns [0, N).
     constexpr int PASSES = SWIGLU ? 3 : 2;
-    __syncthreads();  // every wave's last DMA has landed and its last fragment reads are done
 #pragma unroll
     for (int b = 0; b < PASSES; ++b) {
         if constexpr (SWIGLU) {
@@ -408,6 +225,7 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
             }
         }
         __syncthreads();
+        if (b == 0) before_stores();
         // where this pass goes: hidden rows and down rows into `out` (row stride N), the
         // pre-activations into `gu_out` (row stride 2 N)
         const int col0 = tn_idx * BN + (SWIGLU ? 0 : b * (NW * 32));
@@ -468,7 +286,349 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
     }
 }
 
-template <bool SWIGLU, bool I8, int RING, int TFBUF, bool AREG>
+// ---- the pipelined main loop: one memory instruction behind each multiply -------------------------
+// A wave issues in order, and while it issues a vector-memory or LDS instruction it issues no multiply: with
+// the loads of a step in one cluster in front of its eight multiplies the matrix core runs dry for the
+// length of the cluster unless another wave of the SIMD fills in - a wave that is alone on its SIMD (the
+// last round of a launch, the partner in its prologue or epilogue) reaches 64 % of the multiply rate that
+// way.  Here every multiply is followed by at most one or two of them, in an order pinned by scheduling
+// barriers, and the slice boundary has no cluster either: three LDS stages, and the workgroup barrier sits
+// behind step KS - 2 of a slice, so that the last step of a slice can already read the first fragments of
+// the next slice and issue the DMA of the slice after that into the stage the barrier has just proven free.
+//   steps 0 .. KS-2 of slice k:  ring loads of step g + D, fragments of step g + 1 (stage k % 3)
+//   then: wait for this wave's DMA of slice k + 1 (issued a slice ago), barrier
+//   step KS-1:                   ring loads, DMA of slice k + 2 (into stage (k + 2) % 3, last read in
+//                                slice k - 1), fragments of step 0 of slice k + 1 (stage (k + 1) % 3)
+// Vector-memory issue order inside a step: ring f0, ring f1, then the DMA instructions.  Younger than the
+// ring loads of step g when step g waits for them (they were issued in step g - D, D = 3): the DMA of that
+// step if it was a last step, then two ring loads per step in between and four DMA if one of them was a last
+// step - 8 in all for the steps 0 .. KS-2 of a slice, 4 for the last one.
+struct PipeCtx {
+    const uint4* As;      // three LDS stages of one activation slice each
+    uint32_t lds0;        // LDS byte address of this wave's rows in stage 0
+    const char* a_base;   // activation rows (DMA source), byte offsets in a_src
+    const char* wp0;      // this wave's two blocks of packed weight rows
+    const char* wp1;
+    uint32_t lane16;
+    int lrow, lhalf, lxor;
+    int KT;               // slices of the reduction
+};
+
+// Before the call: the DMA of slices 0 and 1 (stages 0 and 1) and the ring loads of steps 0 .. D-1 have been issued
+// and have landed, and the workgroup has met at a barrier.  After it: nothing is outstanding; every wave may
+// still be reading the stages until the next barrier.
+template <bool I8, int NB>
+__device__ __forceinline__ void pipe_loop(const PipeCtx& c, floatx16 (&acc)[2][TT], Slot<I8> (&ring)[KS],
+                                          const uint32_t (&a_src)[DMA_PER_WAVE]) {
+    constexpr int RING = KS, D = RING - 1;
+    static_assert(KS == 4 && DMA_PER_WAVE == 4 && D == 3, "the wait counts below are derived for this configuration");
+    const uint4* const As = c.As;
+    const uint32_t lds0 = c.lds0, lane16 = c.lane16;
+    const char* const a_base = c.a_base;
+    const char* const wp0 = c.wp0;
+    const char* const wp1 = c.wp1;
+    const int lrow = c.lrow, lhalf = c.lhalf, lxor = c.lxor, KT = c.KT;
+    const int GS = KT * KS;
+    // The fragment of token block t for the step at position p of a slice sits at piece (2 p + lhalf) ^ lxor of
+    // row t * 32 + lrow, i.e. at index t * 32 * CPR + (frag0 ^ 2 p): one register and an exclusive-or per step.
+    // (Re-read through an empty statement per slice: four precomputed addresses would cost three registers.)
+    static_assert(CPR == 8, "piece index = low three bits of the fragment index");
+    int frag0 = lrow * CPR + (lhalf ^ lxor);
+    bf16x8 tf[2][TT];
+#pragma unroll
+    for (int t = 0; t < NB; ++t) tf[0][t] = lds_frag(As, t * 32 * CPR + frag0);
+    auto pslice = [&](int kt, auto idx_tag) {
+        constexpr int IDX = decltype(idx_tag)::value;
+        constexpr int BUF = IDX % 3, NEXT = (IDX + 1) % 3, FREE = (IDX + 2) % 3;
+        const uint4* const Ab = As + BUF * (BM * CPR);
+        const uint4* const An = As + NEXT * (BM * CPR);
+        asm volatile("" : "+v"(frag0));
+        static_for<0, KS>([&](auto s_tag) {
+            constexpr int s = decltype(s_tag)::value;
+            constexpr bool LAST = s == KS - 1;
+            const int g = kt * KS + s;
+            Slot<I8>& cur = ring[s % RING];
+            Slot<I8>& nxt = ring[(s + D) % RING];
+            wait_for<LAST ? 2 * (D - 1) : 2 * (D - 1) + DMA_PER_WAVE>(cur.f0, cur.f1);
+            const bf16x8 w0 = cur.a0();
+            const bf16x8 w1 = cur.a1();
+            const uint32_t woff = Slot<I8>::offset(min(g + D, GS - 1), lane16);
+            const uint32_t aoff = (uint32_t)min(kt + 2, KT - 1) * (BK * 2);
+            const int frag = frag0 ^ (2 * ((s + 1) % KS));
+            // memory instruction number i of the step
+            constexpr int NOPS = 2 + ((LAST && DMA_PER_WAVE > NB) ? DMA_PER_WAVE : NB);
+            auto op = [&](auto i_tag) {
+                constexpr int i = decltype(i_tag)::value;
+                if constexpr (i == 0) {
+                    nxt.load0(wp0, woff);
+                } else if constexpr (i == 1) {
+                    nxt.load1(wp1, woff);
+                } else {
+                    constexpr int j = i - 2;
+                    if constexpr (LAST && j < DMA_PER_WAVE)
+                        issue_dma(lds0 + FREE * (BM * CPR * 16) + j * 8 * CPR * 16, a_src[j] + aoff, a_base);
+                    if constexpr (j < NB)
+                        tf[(s + 1) & 1][j] = lds_frag(LAST ? An : Ab, j * 32 * CPR + frag);
+                }
+            };
+            static_for<0, 2 * NB>([&](auto m_tag) {
+                constexpr int m = decltype(m_tag)::value;
+                constexpr int b = m & 1, t = m >> 1;
+                acc[b][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b ? w1 : w0, tf[s & 1][t], acc[b][t], 0, 0, 0);
+                if constexpr (m < NOPS) op(m_tag);
+                __builtin_amdgcn_sched_barrier(0);
+            });
+            static_for<2 * NB, NOPS>(op);
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (s == KS - 2) {
+                // this wave's DMA of the next slice (issued in the last step of the slice before this
+                // one) is older than the 2 * (KS - 1) ring loads of this slice so far
+                wait_outstanding<2 * (KS - 1)>();
+                __builtin_amdgcn_s_barrier();
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        });
+    };
+    int kt = 0;
+    for (; kt + 3 <= KT; kt += 3)
+        static_for<0, 3>([&](auto i) { pslice(kt + decltype(i)::value, i); });
+    static_while<0, 2>([&](auto i) {
+        if (kt + decltype(i)::value >= KT) return false;
+        pslice(kt + decltype(i)::value, i);
+        return true;
+    });
+    wait_outstanding<0>();
+    auto& ring_ref = ring;
+#pragma unroll
+    for (int i = 0; i < RING; ++i) asm volatile("" : : "v"(ring_ref[i].f0), "v"(ring_ref[i].f1));
+}
+
+// RING = weight-fragment steps in flight per wave (register ring depth);
+// TFBUF = 2: token fragments are read from LDS one step ahead, 1: just in time;
+// STAGES = LDS stages of one activation slice each: the DMA of slice k + STAGES - 1 is issued when slice k starts;
+// PIPE = the main loop that spreads its memory instructions between the multiplies (see there).
+template <bool SWIGLU, bool I8, int RING, int TFBUF, int STAGES, bool PIPE>
+__global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
+    const bf16_t* __restrict__ a, const int* __restrict__ row_index, const void* __restrict__ wpacked,
+    size_t w_expert_stride_bytes, const float* __restrict__ scales, size_t s_expert_stride, int N, int K,
+    const int* __restrict__ tile_expert, const int* __restrict__ tile_row0, const int* __restrict__ tile_rows,
+    const int* __restrict__ ntiles, int dense_rows, bf16_t* __restrict__ out, bf16_t* __restrict__ gu_out,
+    const bf16_t* __restrict__ bw_gu,
+    int group_m) {
+    constexpr int BN = SWIGLU ? NW * 32 : NW * 64;  // output features per workgroup
+    // LDS stages of one activation slice each; the epilogue reuses the first two as one
+    // 128 x 128 staging tile for the output.
+    static_assert(STAGES == 2 || STAGES == 3, "two or three stages");
+    __shared__ uint4 As[STAGES * BM * CPR];
+
+    // ---- which tile (each XCD walks a contiguous range, M fastest inside a group)
+    const int tiles_n = (N + BN - 1) / BN;
+    const int tiles_m = dense_rows >= 0 ? (dense_rows + BM - 1) / BM : *ntiles;
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) / 8;
+    const int local = blockIdx.x >> 3;
+    if (local >= per_xcd) return;
+    const int pid = (blockIdx.x & 7) * per_xcd + local;
+    if (pid >= total) return;
+    const int per_group = group_m * tiles_n;
+    const int grp = pid / per_group;
+    const int first_m = grp * group_m;
+    const int gsize = min(group_m, tiles_m - first_m);
+    const int in_g = pid - grp * per_group;
+    const int tm_idx = first_m + in_g % gsize;
+    const int tn_idx = in_g / gsize;
+
+    RBMOE_TRACE_AT(blockIdx.x, 0);
+    int expert, row0, rows;
+    if (dense_rows >= 0) {
+        expert = 0;
+        row0 = tm_idx * BM;
+        rows = min(BM, dense_rows - row0);
+    } else {
+        expert = tile_expert[tm_idx];
+        row0 = tile_row0[tm_idx];
+        rows = tile_rows[tm_idx];
+    }
+    const int nblk = (rows + 31) >> 5;  // token blocks that hold at least one row
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    // ---- this wave's two blocks of 32 weight rows ---------------------------
+    // A wave whose rows lie past N (ragged last feature tile) runs the same loop on row
+    // block 0, so that every wave issues the same loads and meets the same barriers; it
+    // stores nothing.
+    // gate/up: gate rows nw .. nw + 31 and the matching up rows; down: rows nw .. nw + 31 and
+    // the rows 128 further on, so that each block index covers 128 consecutive features of
+    // the workgroup's tile.
+    const int nw = tn_idx * BN + wave * 32;
+    const int r0 = nw, r1 = SWIGLU ? N + nw : nw + NW * 32;
+    const bool act0 = nw < N;
+    const bool act1 = SWIGLU ? act0 : (nw + NW * 32 < N);
+    const size_t block_bytes = (size_t)K * 32 * (I8 ? 1 : 2);  // one block of 32 weight rows over all of K
+    const char* wexp = static_cast<const char*>(wpacked) + (size_t)expert * w_expert_stride_bytes;
+    const char* wp0 = wexp + (size_t)(act0 ? r0 / 32 : 0) * block_bytes;
+    const char* wp1 = wexp + (size_t)(act1 ? r1 / 32 : 0) * block_bytes;
+    const uint32_t lane16 = (uint32_t)lane * 16u;
+
+    // ---- LDS-DMA of the activation slice --------------------------------------
+    // Wave w fills LDS rows [32 w, 32 w + 32): instruction j covers rows 32 w + 8 j .. + 7,
+    // lane l lands in row 8 j + l / 8 (of the wave's 32), position l % 8, and therefore
+    // fetches logical piece (l % 8) ^ ((row / 2) % 8): a 16-lane group of a fragment read
+    // (16 consecutive rows, one logical piece) then touches 8 distinct pieces in the even rows
+    // and 8 in the odd rows, i.e. all 64 banks once.  Rows past the end of the group are
+    // clamped to the tile's first row: their products are never stored.
+    // Byte offsets from `a` fit 32 bits (the launcher checks rows * K * 2 < 4 GiB).
+    const char* const a_base = reinterpret_cast<const char*>(a);
+    uint32_t a_src[DMA_PER_WAVE];
+#pragma unroll
+    for (int j = 0; j < DMA_PER_WAVE; ++j) {
+        const int r = wave * 32 + j * 8 + (lane >> 3);
+        const int rr = r < rows ? r : 0;
+        const int grow = row_index ? row_index[row0 + rr] : row0 + rr;
+        a_src[j] = ((uint32_t)grow * (uint32_t)K + 8u * ((lane & 7) ^ ((r >> 1) & 7))) * 2u;
+    }
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)As + wave * 32 * CPR * 16;
+    auto dma_a = [&](int kt, auto buf_tag) {
+        constexpr int BUF = decltype(buf_tag)::value;
+#pragma unroll
+        for (int j = 0; j < DMA_PER_WAVE; ++j)
+            issue_dma(lds0 + BUF * (BM * CPR * 16) + j * 8 * CPR * 16, a_src[j] + (uint32_t)kt * (BK * 2), a_base);
+    };
+
+    floatx16 acc[2][TT];
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int t = 0; t < TT; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[b][t][v] = 0.0f;
+
+    const int lrow = lane & 31;
+    const int lhalf = lane >> 5;
+    const int lxor = (lrow >> 1) & 7;
+
+    const int KT = K / BK;
+    const int GS = KT * KS;  // reduction steps in all
+    constexpr int D = RING - 1;  // the load for step g + D is issued while step g runs
+
+    // ---- prologue: the first STAGES - 1 activation slices, the first D weight steps; nothing is in flight
+    // where the loop is entered (the compiler may copy registers there)
+    Slot<I8> ring[RING];
+    static_for<0, STAGES - 1>([&](auto st) { dma_a(min((int)decltype(st)::value, KT - 1), st); });
+#pragma unroll
+    for (int g = 0; g < D; ++g) ring[g].load(wp0, wp1, min(g, GS - 1), lane16);
+    wait_outstanding<0>();
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    RBMOE_TRACE_AT(blockIdx.x, 1);
+
+    if constexpr (PIPE) {
+        static_assert(STAGES == 3 && RING == KS && TFBUF == 2, "the pipelined loop's configuration");
+        const PipeCtx pc{As, lds0, a_base, wp0, wp1, lane16, lrow, lhalf, lxor, KT};
+        if (nblk == 4) pipe_loop<I8, 4>(pc, acc, ring, a_src);
+        else if (nblk == 3) pipe_loop<I8, 3>(pc, acc, ring, a_src);
+        else if (nblk == 2) pipe_loop<I8, 2>(pc, acc, ring, a_src);
+        else pipe_loop<I8, 1>(pc, acc, ring, a_src);
+    }
+
+    // One slice = KS steps.  BUF is the LDS stage the slice reads (its parity); the ring
+    // position of the slice's first step is 0, or BUF * KS when the ring holds two slices.
+    // NB = token blocks of this tile that hold rows, a compile-time constant inside the
+    // loop: a run-time branch per block between the multiplies costs far more than the
+    // skipped multiplies save, so the whole loop is specialised instead.
+    // The loop is straight-line and every wave issues, per slice, exactly: 4 DMA
+    // instructions, then 2 weight loads in each of the KS steps.  Past the end the last
+    // slice / step is fetched again, so that the counts below hold everywhere.
+    // (IDX = position of the slice inside the unrolled loop body: it fixes the LDS stage and the ring phase)
+    auto slice = [&](int kt, auto idx_tag, auto nb_tag) {
+        constexpr int IDX = decltype(idx_tag)::value;
+        constexpr int BUF = IDX % STAGES;
+        constexpr int G0 = RING == 2 * KS ? (IDX % 2) * KS : 0;
+        constexpr int NB = decltype(nb_tag)::value;
+        dma_a(min(kt + STAGES - 1, KT - 1), std::integral_constant<int, (BUF + STAGES - 1) % STAGES>{});
+        const uint4* Ab = As + BUF * (BM * CPR);
+        bf16x8 tf[TFBUF][TT];
+#pragma unroll
+        for (int t = 0; t < NB; ++t) tf[0][t] = lds_frag(Ab, (t * 32 + lrow) * CPR + (lhalf ^ lxor));
+        static_for<0, KS>([&](auto s_tag) {
+            constexpr int s = decltype(s_tag)::value;
+            const int g = kt * KS + s;
+            Slot<I8>& cur = ring[(G0 + s) % RING];
+            // weight fragments for step g + D go into the slot step g - 1 released
+            ring[(G0 + s + D) % RING].load(wp0, wp1, min(g + D, GS - 1), lane16);
+            if constexpr (TFBUF == 2) {
+                if (s + 1 < KS) {
+                    const int piece = (2 * (s + 1) + lhalf) ^ lxor;
+#pragma unroll
+                    for (int t = 0; t < NB; ++t) tf[(s + 1) & 1][t] = lds_frag(Ab, (t * 32 + lrow) * CPR + piece);
+                }
+            } else if (s > 0) {
+                const int piece = (2 * s + lhalf) ^ lxor;
+#pragma unroll
+                for (int t = 0; t < NB; ++t) tf[0][t] = lds_frag(Ab, (t * 32 + lrow) * CPR + piece);
+            }
+            // Younger than the loads of step g: the weight loads of steps g+1 .. g+D (2 each)
+            // and the DMA (4) of every slice that started after they were issued.
+            wait_for<2 * D + DMA_PER_WAVE * ((D - s + KS - 1) / KS)>(cur.f0, cur.f1);
+            const bf16x8 w0 = cur.a0();
+            const bf16x8 w1 = cur.a1();
+#pragma unroll
+            for (int t = 0; t < NB; ++t) {
+                acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w0, tf[s % TFBUF][t], acc[0][t], 0, 0, 0);
+                acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w1, tf[s % TFBUF][t], acc[1][t], 0, 0, 0);
+            }
+        });
+        // Every LDS read of this slice has been consumed by a multiply issued above this
+        // point.  The DMA of the next slice is older than the 2 * KS weight loads of every slice since it was
+        // issued (STAGES - 1 of them) and than the DMA of the STAGES - 2 slices after it.
+        __builtin_amdgcn_sched_barrier(0);
+        wait_outstanding<2 * KS * (STAGES - 1) + DMA_PER_WAVE * (STAGES - 2)>();
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    static_assert(RING == KS || RING == 2 * KS, "ring depth is one or two slices");
+    static_assert(DMA_PER_WAVE == 4, "the wait counts assume 4 DMA instructions per wave per slice");
+    // the loop body holds as many slices as it takes for the LDS stage and the ring phase to come round again
+    constexpr int UNROLL = (RING == 2 * KS && STAGES % 2) ? 2 * STAGES : (STAGES > 2 ? STAGES : 2);
+    auto run = [&](auto nb_tag) {
+        int kt = 0;
+        for (; kt + UNROLL <= KT; kt += UNROLL)
+            static_for<0, UNROLL>([&](auto i) { slice(kt + decltype(i)::value, i, nb_tag); });
+        static_while<0, UNROLL - 1>([&](auto i) {
+            if (kt + decltype(i)::value >= KT) return false;
+            slice(kt + decltype(i)::value, i, nb_tag);
+            return true;
+        });
+        // The loads fetched again past the end still target ring registers and LDS.  Naming
+        // the registers after the wait keeps them allocated until their data has arrived: a
+        // loaded value the compiler sees no use for would otherwise hand its register to
+        // something live while the load is still in flight.  (Done here, inside each
+        // specialisation, so that no path leaves it with loads outstanding.)
+        wait_outstanding<0>();
+        auto& ring_ref = ring;
+#pragma unroll
+        for (int i = 0; i < RING; ++i) asm volatile("" : : "v"(ring_ref[i].f0), "v"(ring_ref[i].f1));
+    };
+    static_assert(TT == 4, "one specialisation per possible block count");
+    if constexpr (!PIPE) {
+        if (nblk == 4) run(std::integral_constant<int, 4>{});
+        else if (nblk == 3) run(std::integral_constant<int, 3>{});
+        else if (nblk == 2) run(std::integral_constant<int, 2>{});
+        else run(std::integral_constant<int, 1>{});
+    }
+    RBMOE_TRACE_AT(blockIdx.x, 2);
+    // ---- epilogue -------------------------------------------------------------
+    __syncthreads();  // every wave's last DMA has landed and its last fragment reads are done
+    const TileOut to{rows, row0, tn_idx, N, act0, act1, r0, r1, I8 ? scales + (size_t)expert * s_expert_stride : nullptr,
+                     out, gu_out, bw_gu};
+    write_tile<SWIGLU, I8>(to, acc, reinterpret_cast<char*>(As), [] {});
+    RBMOE_TRACE_AT(blockIdx.x, 3);
+}
+
+template <bool SWIGLU, bool I8, int RING, int TFBUF, int STAGES, bool PIPE>
 hipError_t launch_t(const GroupedArgs& g, hipStream_t s) {
     constexpr int BN = SWIGLU ? NW * 32 : NW * 64;
     const int tiles_n = (g.N + BN - 1) / BN;
@@ -476,7 +636,7 @@ hipError_t launch_t(const GroupedArgs& g, hipStream_t s) {
     if (tiles_m <= 0) return hipSuccess;
     const int total = tiles_m * tiles_n;
     const int grid = ((total + 7) / 8) * 8;
-    hipLaunchKernelGGL((grouped_stream_kernel<SWIGLU, I8, RING, TFBUF, AREG>), dim3(grid), dim3(NT), 0, s,
+    hipLaunchKernelGGL((grouped_stream_kernel<SWIGLU, I8, RING, TFBUF, STAGES, PIPE>), dim3(grid), dim3(NT), 0, s,
                        static_cast<const bf16_t*>(g.a), g.row_index, g.w, g.w_expert_stride * (I8 ? 1 : 2), g.scales,
                        g.s_expert_stride, g.N, g.K, g.tile_expert, g.tile_row0, g.tile_rows, g.ntiles, g.dense_rows,
                        static_cast<bf16_t*>(g.out), static_cast<bf16_t*>(g.gu_out), static_cast<const bf16_t*>(g.swiglu_grad_gu),
@@ -484,29 +644,32 @@ hipError_t launch_t(const GroupedArgs& g, hipStream_t s) {
     return hipGetLastError();
 }
 
+
 }  // namespace
 
-template <int RING, int TFBUF, bool AREG>
+template <int RING, int TFBUF, int STAGES, bool PIPE>
 static hipError_t launch_ring(const GroupedArgs& g, WeightKind wk, hipStream_t s) {
     if (wk == WeightKind::BF16)
-        return g.swiglu ? launch_t<true, false, RING, TFBUF, AREG>(g, s) : launch_t<false, false, RING, TFBUF, AREG>(g, s);
+        return g.swiglu ? launch_t<true, false, RING, TFBUF, STAGES, PIPE>(g, s)
+                        : launch_t<false, false, RING, TFBUF, STAGES, PIPE>(g, s);
     if (wk == WeightKind::I8)
-        return g.swiglu ? launch_t<true, true, RING, TFBUF, AREG>(g, s) : launch_t<false, true, RING, TFBUF, AREG>(g, s);
+        return g.swiglu ? launch_t<true, true, RING, TFBUF, STAGES, PIPE>(g, s)
+                        : launch_t<false, true, RING, TFBUF, STAGES, PIPE>(g, s);
     return hipErrorInvalidValue;
 }
 
-// variant 0: ring of 4 steps, token fragments read one step ahead, activation slices by LDS-DMA
-// variant 1: ring of 4 steps, token fragments read just in time, activation slices global -> VGPR -> LDS
 int stream_tile_m() { return BM; }
 
 // K a multiple of 64 (one LDS slice), N a multiple of 32 (row blocks of the packed weights)
 bool stream_shape_ok(int N, int K) { return K % 64 == 0 && K >= 64 && N % 32 == 0 && N >= 32; }
 
+// variant 0: the pipelined main loop (one memory instruction behind each multiply, three LDS stages)
+// variant 1: the loads of a step in one cluster in front of its multiplies, two LDS stages (kept for A/B runs)
 hipError_t launch_grouped_stream(const GroupedArgs& g, WeightKind wk, int variant, hipStream_t s) {
     if (!stream_shape_ok(g.N, g.K)) return hipErrorInvalidValue;
     switch (variant) {
-        case 0: return launch_ring<4, 2, false>(g, wk, s);
-        case 1: return launch_ring<4, 1, true>(g, wk, s);
+        case 0: return launch_ring<4, 2, 3, true>(g, wk, s);
+        case 1: return launch_ring<4, 2, 2, false>(g, wk, s);
     }
     return hipErrorInvalidValue;
 }

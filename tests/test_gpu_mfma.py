@@ -48,7 +48,7 @@ def run(device, t, valid=None, bias=None):
 @pytest.mark.parametrize("shape", [dict(d=128, E=6, k=2, F=192, T=700), dict(d=64, E=3, k=1, F=64, T=130),
                                    dict(d=256, E=16, k=4, F=128, T=333), dict(d=192, E=5, k=2, F=320, T=1000)],
                          ids=lambda s: "d{d}_E{E}_k{k}_F{F}_T{T}".format(**s))
-@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("variant", [0, 1])   # 0: pipelined main loop, 1: clustered loads (two LDS stages)
 def test_matrix_core_kernels(device, kernel_env, shape, wt, variant):
     kernel_env["RBMOE_STREAM_VARIANT"] = str(variant)
     E = shape["E"]
