@@ -195,8 +195,8 @@ impl MoeLayer {
             WeightDtype::Bf16 => sys::RBMOE_BF16,
             WeightDtype::Int8 => sys::RBMOE_I8,
         };
-        // f32 on the boundary; the matrix-core kernels want bf16 activations, which a device-resident
-        // caller passes to `rbmoe_forward` directly.
+        // f32 on the boundary, as the reference's `Matrix`.  With bf16 or int8 weights the library routes on
+        // the f32 rows and runs the expert products on the bf16 matrix cores over a bf16 copy of them.
         c.act_dtype = sys::RBMOE_F32;
         c.max_tokens = max_tokens as i32;
         let mut layer = ptr::null_mut();

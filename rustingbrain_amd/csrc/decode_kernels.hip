@@ -23,7 +23,7 @@ namespace rbmoe {
 // the bucket loop per expert (a stable counting sort), losses per expert in token order.
 // ---------------------------------------------------------------------------
 constexpr int kSmallThreads = 512;
-constexpr int kStageBytes = 44 * 1024;  // LDS for the staged router and token rows
+constexpr int kStageBytes = 96 * 1024;  // LDS for the staged router and token rows (gfx950: 160 KiB per workgroup)
 
 // softmax_rows (src/moe.rs, softmax over one row) and route (src/moe.rs:553-593) of one token, by one
 // thread, the row used where it lies in LDS: the path for more experts than a wave has lanes.
@@ -173,7 +173,8 @@ __global__ __launch_bounds__(kSmallThreads) void route_small_kernel(
     int* __restrict__ counts, int* __restrict__ offsets, int* __restrict__ tile_expert,
     int* __restrict__ tile_row0, int* __restrict__ tile_rows, int* __restrict__ ntiles,
     float* __restrict__ losses, int* __restrict__ perm_slot, int* __restrict__ perm_token,
-    int* __restrict__ inv_pos, const float* __restrict__ norm_w, float norm_eps, XT* __restrict__ xn_out) {
+    int* __restrict__ inv_pos, const float* __restrict__ norm_w, float norm_eps, XT* __restrict__ xn_out,
+    bf16_t* __restrict__ rows16) {
     __shared__ __align__(16) unsigned char stage[kStageBytes];
     __shared__ float prob[kSmallRouteMaxPairs];
     __shared__ float lsev[kSmallRouteMaxTokens];
@@ -254,6 +255,22 @@ __global__ __launch_bounds__(kSmallThreads) void route_small_kernel(
                 Vec16<XT>::store(xn_out + (size_t)t * d + c, o);
             }
             __syncthreads();
+        }
+        if constexpr (sizeof(XT) == 4) {
+            // f32 rows of a layer whose expert products run on the bf16 matrix cores: their bf16 copy (nearest
+            // even), from the staged - and, with a norm, normed - rows
+            if (rows16 != nullptr) {
+                for (int i = tid; i < T * (d / 8); i += kSmallThreads) {
+                    const int t = i / (d / 8), c = (i - t * (d / 8)) * 8;
+                    const float* src = reinterpret_cast<const float*>(xs) + (size_t)t * ds + c;
+                    uint4 o;
+                    o.x = f32_to_bf16_bits(src[0]) | ((uint32_t)f32_to_bf16_bits(src[1]) << 16);
+                    o.y = f32_to_bf16_bits(src[2]) | ((uint32_t)f32_to_bf16_bits(src[3]) << 16);
+                    o.z = f32_to_bf16_bits(src[4]) | ((uint32_t)f32_to_bf16_bits(src[5]) << 16);
+                    o.w = f32_to_bf16_bits(src[6]) | ((uint32_t)f32_to_bf16_bits(src[7]) << 16);
+                    *reinterpret_cast<uint4*>(rows16 + (size_t)t * d + c) = o;
+                }
+            }
         }
         const int tasks = T * E * 8;
         for (int base = 0; base < tasks; base += kSmallThreads) {
@@ -464,18 +481,19 @@ bool small_route_stages_rows(const void* x, const float* wr, int T, int d, int E
 hipError_t launch_route_small(const SmallRouteArgs& a, bool bf16, hipStream_t s) {
     if (!small_route_ok(a.T, a.E, a.k)) return hipErrorInvalidValue;
     if (a.norm_w && (!a.xn_out || !small_route_stages_rows(a.x, a.wr, a.T, a.d, a.E, bf16))) return hipErrorInvalidValue;
+    if (a.rows16 && (bf16 || !small_route_stages_rows(a.x, a.wr, a.T, a.d, a.E, bf16))) return hipErrorInvalidValue;
     if (bf16)
         hipLaunchKernelGGL(route_small_kernel<bf16_t>, dim3(1), dim3(kSmallThreads), 0, s,
                            static_cast<const bf16_t*>(a.x), a.wr, a.bias, a.valid, a.T, a.d, a.E, a.k, a.w_aux, a.w_z,
                            a.tile_m, a.P, a.lse, a.expert_of, a.gate_of, a.counts, a.offsets, a.tile_expert,
                            a.tile_row0, a.tile_rows, a.ntiles, a.losses, a.perm_slot, a.perm_token, a.inv_pos,
-                           a.norm_w, a.norm_eps, static_cast<bf16_t*>(a.xn_out));
+                           a.norm_w, a.norm_eps, static_cast<bf16_t*>(a.xn_out), nullptr);
     else
         hipLaunchKernelGGL(route_small_kernel<float>, dim3(1), dim3(kSmallThreads), 0, s,
                            static_cast<const float*>(a.x), a.wr, a.bias, a.valid, a.T, a.d, a.E, a.k, a.w_aux, a.w_z,
                            a.tile_m, a.P, a.lse, a.expert_of, a.gate_of, a.counts, a.offsets, a.tile_expert,
                            a.tile_row0, a.tile_rows, a.ntiles, a.losses, a.perm_slot, a.perm_token, a.inv_pos,
-                           a.norm_w, a.norm_eps, static_cast<float*>(a.xn_out));
+                           a.norm_w, a.norm_eps, static_cast<float*>(a.xn_out), static_cast<bf16_t*>(a.rows16));
     return hipGetLastError();
 }
 

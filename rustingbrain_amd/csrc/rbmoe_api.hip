@@ -179,6 +179,10 @@ struct rbmoe_layer {
     bool force_generic = false;
     bool explicit_gather = false;  // materialise the gathered rows instead of gathering in the product
     bool use_stream = false;   // bf16 matrix-core kernels (packed weights); otherwise the generic kernels
+    // f32 rows on the boundary of a layer with bf16 / int8 weights: the router reads the f32 rows, the expert
+    // products run on the bf16 matrix cores over a bf16 copy of the rows (nearest even) that the routing kernels
+    // write on the way, hidden and expert rows are bf16, and the combine sums them into f32 again
+    bool cast_rows = false;
     bool use_f32_mc = false;   // all-f32 layer on the f32 matrix cores
     bool decode_path = true;   // few tokens: four launches that stream every touched weight once
     int group_m = 4, variant = 0;
@@ -197,6 +201,7 @@ struct rbmoe_layer {
     Buf counts, offsets, tile_expert, tile_row0, tile_rows, ntiles, losses;
     Buf perm_slot, perm_token, inv_pos;
     Buf xg, h, y, hs, ys;
+    Buf x16;               // [max_T, d] bf16 copy of f32 rows (cast_rows)
     // feed-forward norm in front of the layer (allocated by rbmoe_set_feed_forward_norm)
     Buf xn, norm_w;  // [max_T, d] activation dtype, [d] f32
     float norm_eps = 0.0f;
@@ -286,6 +291,7 @@ Plan make_plan(rbmoe_layer* L) {
     p.add(&L->perm_slot, S * 4);
     p.add(&L->perm_token, S * 4);
     p.add(&L->inv_pos, S * 4);
+    if (L->cast_rows) p.add(&L->x16, T * d * 2);
     p.add(&L->xg, S * d * as);
     p.add(&L->h, S * F * as);
     p.add(&L->y, S * d * as);
@@ -455,10 +461,13 @@ int rbmoe_layer_create(rbmoe_ctx* ctx, const rbmoe_config* cfg, rbmoe_layer** ou
     L->variant = env_int("RBMOE_STREAM_VARIANT", 0) == 1 ? 1 : 0;
     L->decode_path = env_int("RBMOE_NO_DECODE_PATH", 0) != 1;
     // bf16 matrix cores: bf16 activations, bf16 or int8 weights, widths that fit the packed layout
-    const bool mc = !L->force_generic && cfg->act_dtype == RBMOE_BF16 && cfg->weight_dtype != RBMOE_F32;
+    // (f32 rows with bf16 / int8 weights - what a caller with f32 matrices and a quantized or bf16 checkpoint has -
+    // take the same kernels over a bf16 copy of the rows)
+    const bool mc = !L->force_generic && cfg->weight_dtype != RBMOE_F32;
     L->use_stream = mc && stream_shape_ok(cfg->d_ff, cfg->d_model) && stream_shape_ok(cfg->d_model, cfg->d_ff) &&
                     (!cfg->shared_expert ||
                      (stream_shape_ok(L->Fs, cfg->d_model) && stream_shape_ok(cfg->d_model, L->Fs)));
+
     L->use_f32_mc = !L->force_generic && cfg->act_dtype == RBMOE_F32 && cfg->weight_dtype == RBMOE_F32 &&
                     f32_shape_ok(cfg->d_ff, cfg->d_model) && f32_shape_ok(cfg->d_model, cfg->d_ff) &&
                     (!cfg->shared_expert || (f32_shape_ok(L->Fs, cfg->d_model) && f32_shape_ok(cfg->d_model, L->Fs)));
@@ -467,6 +476,11 @@ int rbmoe_layer_create(rbmoe_ctx* ctx, const rbmoe_config* cfg, rbmoe_layer** ou
         const size_t widest = (size_t)std::max(std::max(cfg->d_model, cfg->d_ff), L->Fs);
         const size_t rows = (size_t)cfg->max_tokens * (size_t)std::max(1, cfg->experts_per_token);
         if (rows * widest * 2 >= ((size_t)1 << 32)) L->use_stream = false;
+    }
+    if (cfg->act_dtype == RBMOE_F32 && L->use_stream) {
+        // the bf16 copy is written in 8-element pieces of 16-byte aligned rows
+        if (cfg->d_model % 8 == 0) L->cast_rows = true;
+        else L->use_stream = false;
     }
 
     Plan plan = make_plan(L);
@@ -741,7 +755,7 @@ Work work_of_layer(const rbmoe_layer* L) {
 size_t carve_decode_work(const rbmoe_layer* L, int T, unsigned char* base, Work* w) {
     const rbmoe_config& c = L->cfg;
     const size_t E = c.num_experts, d = c.d_model, F = c.d_ff, k = c.experts_per_token, Fs = L->Fs;
-    const size_t S = (size_t)T * k, as = dtype_size(c.act_dtype);
+    const size_t S = (size_t)T * k, as = L->cast_rows ? 2 : dtype_size(c.act_dtype);
     const size_t tiles = S / kDecodeTileM + E + 1;
     size_t used = 0;
     auto take = [&](size_t bytes) -> void* {
@@ -793,6 +807,9 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     hipStream_t s = ctx->stream;
     L->last_was_block = false;  // rbmoe_forward_block sets it once this call has succeeded
     const bool abf = c.act_dtype == RBMOE_BF16;
+    const bool cast = L->cast_rows;  // f32 rows, bf16 matrix-core products over their bf16 copy
+    // the rows the expert products read
+    const void* const xe = cast ? L->x16.p : x;
     const WeightKind wk = c.weight_dtype == RBMOE_F32 ? WeightKind::F32
                           : c.weight_dtype == RBMOE_BF16 ? WeightKind::BF16 : WeightKind::I8;
     if (timed && !L->have_events) {
@@ -810,11 +827,15 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     // a training layer keeps the gathered rows: the weight gradients of gate and up multiply by them
     const bool gather_in_product = (mfma || f32mc) && !L->explicit_gather && !L->training;
 
+    // whether the single-workgroup routing kernel would stage this call's rows in LDS: only then can it apply the
+    // norm and write the bf16 copy of f32 rows
+    const bool stages_rows = small_route_stages_rows(x, (const float*)L->router.p, T, d, E, abf) &&
+                             (!norm_src || small_route_stages_rows(norm_src, (const float*)L->router.p, T, d, E, abf));
     const bool decode_ok = mfma && L->decode_path && !L->training && small_route_ok(T, E, k) && decode_shape_ok(F, d) &&
                            decode_shape_ok(d, F) &&
-                           (!c.shared_expert || (decode_shape_ok(Fs, d) && decode_shape_ok(d, Fs)));
-    const bool norm_in_route = norm_src && decode_ok &&
-                               small_route_stages_rows(norm_src, (const float*)L->router.p, T, d, E, abf);
+                           (!c.shared_expert || (decode_shape_ok(Fs, d) && decode_shape_ok(d, Fs))) &&
+                           (!cast || stages_rows);
+    const bool norm_in_route = norm_src && decode_ok && stages_rows;
     Work wk_ = work_of_layer(L);
     if (static_scratch) {
         if (!decode_ok) {
@@ -848,6 +869,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
         if (norm_in_route) {
             sr.x = norm_src; sr.norm_w = (const float*)L->norm_w.p; sr.norm_eps = L->norm_eps; sr.xn_out = L->xn.p;
         }
+        if (cast) sr.rows16 = L->x16.p;
         sr.T = T; sr.d = d; sr.E = E; sr.k = k;
         sr.w_aux = c.aux_loss_weight; sr.w_z = c.router_z_loss_weight;
         sr.tile_m = kDecodeTileM;
@@ -863,7 +885,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
         HIP_TRY(ctx, mark(3));
 
         DecodeGemmArgs d1{};
-        d1.a = x; d1.row_index = wk_.perm_token;
+        d1.a = xe; d1.row_index = wk_.perm_token;
         d1.w = L->wgu.p; d1.w_expert_stride = (size_t)2 * F * d;
         d1.scales = wk == WeightKind::I8 ? (const float*)L->sgu.p : nullptr; d1.s_expert_stride = (size_t)2 * F;
         d1.N = F; d1.K = d;
@@ -873,7 +895,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
         d1.out = wk_.h;
         d1.swiglu = 1;
         if (c.shared_expert) {
-            d1.a_shared = x; d1.w_shared = L->swgu.p;
+            d1.a_shared = xe; d1.w_shared = L->swgu.p;
             d1.scales_shared = wk == WeightKind::I8 ? (const float*)L->ssgu.p : nullptr;
             d1.N_shared = Fs; d1.K_shared = d; d1.T_shared = T; d1.out_shared = wk_.hs;
         }
@@ -896,6 +918,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
         HIP_TRY(ctx, mark(5));
         HIP_TRY(ctx, mark(6));
         CombineArgs cd{wk_.y, c.shared_expert ? wk_.ys : nullptr, residual, wk_.inv_pos, wk_.gate_of, T, d, k, out};
+        cd.rows_bf16 = cast;
         HIP_TRY(ctx, launch_combine(cd, abf, s));
         HIP_TRY(ctx, mark(7));
         L->last_T = T;
@@ -909,13 +932,14 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     RouterArgs ra{x, (const float*)L->router.p, router_bias, valid, T, d, E, k,
                   (float*)L->P.p, (float*)L->lse.p, (int*)L->expert_of.p, (float*)L->gate_of.p,
                   (int*)L->rank_in_block.p, (int*)L->blockcnt.p, (float*)L->partial.p};
+    if (cast) ra.rows16 = L->x16.p;
     HIP_TRY(ctx, launch_router(ra, abf, s));
     HIP_TRY(ctx, mark(1));
 
     HIP_TRY(ctx, mark(2));  // an interval with no work in it: the cost of one pair of event records
 
     DispatchArgs da{};
-    da.x = x;
+    da.x = xe;
     da.expert_of = (const int*)L->expert_of.p;
     da.rank_in_block = (const int*)L->rank_in_block.p;
     da.blockcnt = (const int*)L->blockcnt.p;
@@ -929,7 +953,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     da.ntiles = (int*)L->ntiles.p; da.losses = (float*)L->losses.p;
     da.perm_slot = (int*)L->perm_slot.p; da.perm_token = (int*)L->perm_token.p; da.inv_pos = (int*)L->inv_pos.p;
     da.xg = gather_in_product ? nullptr : L->xg.p;
-    HIP_TRY(ctx, launch_dispatch(da, abf, s));
+    HIP_TRY(ctx, launch_dispatch(da, abf || cast, s));
     HIP_TRY(ctx, mark(3));
 
     auto run = [&](const GroupedArgs& g, bool swiglu) -> hipError_t {
@@ -938,7 +962,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
         return launch_grouped_generic(g, abf, wk, kGenericTileM, s);
     };
     GroupedArgs g1{};
-    g1.a = gather_in_product ? x : L->xg.p;
+    g1.a = gather_in_product ? xe : L->xg.p;
     g1.row_index = gather_in_product ? (const int*)L->perm_token.p : nullptr;
     g1.w = L->wgu.p;
     g1.w_expert_stride = (size_t)2 * F * d;
@@ -976,7 +1000,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
 
     if (c.shared_expert && T > 0) {
         GroupedArgs s1 = g1;
-        s1.a = x;
+        s1.a = xe;
         s1.row_index = nullptr;
         s1.w = L->swgu.p;
         s1.w_expert_stride = 0;
@@ -1003,6 +1027,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
 
     CombineArgs ca{L->y.p, c.shared_expert ? L->ys.p : nullptr, residual, (const int*)L->inv_pos.p,
                    (const float*)L->gate_of.p, T, d, k, out};
+    ca.rows_bf16 = cast;
     HIP_TRY(ctx, launch_combine(ca, abf, s));
     HIP_TRY(ctx, mark(7));
     L->last_T = T;
@@ -1220,11 +1245,17 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
     rbmoe_ctx* ctx = L->ctx;
     if (L->training) return RBMOE_OK;
     const rbmoe_config& c = L->cfg;
-    const bool bf16_layer = L->use_stream && c.weight_dtype == RBMOE_BF16;
     if (c.weight_dtype == RBMOE_I8)  // as in the reference: quantized experts are inference-only (src/ffn.rs:87-93)
         return fail(ctx, RBMOE_UNSUPPORTED, "the backward pass is not defined for int8 weights");
     if (L->weights_set)
         return fail(ctx, RBMOE_INVALID_CONFIG, "enable training before the weights are set");
+    if (L->cast_rows) {
+        // f32 rows with bf16 weights differentiate on the plain kernels, in both directions, on the f32 rows
+        // themselves (no weight has been set yet, so none has been packed for the matrix cores)
+        L->cast_rows = false;
+        L->use_stream = false;
+    }
+    const bool bf16_layer = L->use_stream && c.weight_dtype == RBMOE_BF16;
     if (L->max_T > router_grad_max_tokens()) {  // found here, not in the middle of a backward pass
         char buf[160];
         std::snprintf(buf, sizeof buf, "the backward pass takes at most %d tokens a call, the layer was created for %d",
@@ -1599,7 +1630,7 @@ int rbmoe_get_expert_rows(rbmoe_layer* L, float* hidden, float* expert_out) {
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
     int R = 0;
     HIP_TRY(ctx, hipMemcpy(&R, L->last.offsets + E, 4, hipMemcpyDeviceToHost));
-    const bool abf = L->cfg.act_dtype == RBMOE_BF16;
+    const bool abf = L->cfg.act_dtype == RBMOE_BF16 || L->cast_rows;  // the rows of a cast_rows layer are bf16
     auto fetch = [&](float* dst, const void* src, size_t n) -> int {
         if (!dst || n == 0) return RBMOE_OK;
         if (!abf) {

@@ -36,6 +36,7 @@ struct RouterArgs {
     int* rank_in_block;  // [T*k]
     int* blockcnt;       // [nb, E]
     float* partial;      // [nb, E+1]
+    void* rows16 = nullptr;  // f32 rows only: [T, d] bf16 copy of x written on the way (d a multiple of 8), or null
 };
 hipError_t launch_router(const RouterArgs& a, bool bf16, hipStream_t s);
 
@@ -71,6 +72,7 @@ struct CombineArgs {
     const float* gate_of; // [T*k]
     int T, d, k;
     void* out;            // [T, d]
+    bool rows_bf16 = false;  // under f32 activations: y and yshared are bf16 (matrix-core products of a bf16 / int8 layer)
 };
 hipError_t launch_combine(const CombineArgs& a, bool bf16, hipStream_t s);
 
@@ -203,6 +205,9 @@ struct SmallRouteArgs {
     const float* norm_w = nullptr;
     float norm_eps = 0.0f;
     void* xn_out = nullptr;
+    // f32 rows only: a bf16 copy [T, d] of the rows the routing is decided on (after the norm, if any), for the
+    // matrix-core products; only for calls whose rows are staged in LDS (small_route_stages_rows)
+    void* rows16 = nullptr;
 };
 bool small_route_stages_rows(const void* x, const float* wr, int T, int d, int E, bool bf16);
 bool small_route_ok(int T, int E, int k);

@@ -92,11 +92,15 @@ struct XPiece<float> {
 // NE = experts (= waves) per workgroup.
 // (bf16 without AHEAD: 6 waves per SIMD, i.e. three workgroups on a compute unit, is what the launches of many
 // workgroups are tuned for - the bound keeps a later edit from quietly costing one of them)
+// `rows16` (f32 rows only, or null): a bf16 copy of the rows, rounded to nearest even, for the expert products of a
+// layer whose weights are bf16 or int8 - written on the way by the workgroups of the first group of experts, which
+// have every piece of their rows in hand anyway (widths that are multiples of 8).
 template <typename XT, int NE, bool AHEAD>
 __global__ __launch_bounds__(NE * 64, (!AHEAD && sizeof(XT) == 2) ? 6 : 2) void logits_kernel(const XT* __restrict__ x,
                                                                 const float* __restrict__ wr,
                                                                 const float* __restrict__ bias, int T, int d, int E,
-                                                                float* __restrict__ logits) {
+                                                                float* __restrict__ logits,
+                                                                bf16_t* __restrict__ rows16) {
     typedef typename XPiece<XT>::raw_t piece_t;
     constexpr int PIECES = kLogitChunk / 8;  // pieces per row per slice
     constexpr int STRIDE = PIECES + 1;       // one piece of padding per row
@@ -121,12 +125,25 @@ __global__ __launch_bounds__(NE * 64, (!AHEAD && sizeof(XT) == 2) ? 6 : 2) void 
     // pieces in flight occupy would cost one of them.
     constexpr int MAXP = (kLogitTokens * PIECES + kLogitThreads - 1) / kLogitThreads;
     piece_t pre[MAXP];
+    const bool copy16 = sizeof(XT) == 4 && rows16 != nullptr && blockIdx.y == 0;
     auto load_piece = [&](int r, int c) {  // eight elements of row r from column c (zeros past the last row)
         piece_t v = {};
         if (r < nt) {
             const XT* src = x + (size_t)(t0 + r) * d + c;
             if (vec) {
                 v = *reinterpret_cast<const piece_t*>(src);
+                if constexpr (sizeof(XT) == 4) {
+                    if (copy16) {
+                        float f[8];
+                        XPiece<XT>::widen(v, f);
+                        uint4 o;
+                        o.x = f32_to_bf16_bits(f[0]) | ((uint32_t)f32_to_bf16_bits(f[1]) << 16);
+                        o.y = f32_to_bf16_bits(f[2]) | ((uint32_t)f32_to_bf16_bits(f[3]) << 16);
+                        o.z = f32_to_bf16_bits(f[4]) | ((uint32_t)f32_to_bf16_bits(f[5]) << 16);
+                        o.w = f32_to_bf16_bits(f[6]) | ((uint32_t)f32_to_bf16_bits(f[7]) << 16);
+                        *reinterpret_cast<uint4*>(rows16 + (size_t)(t0 + r) * d + c) = o;
+                    }
+                }
             } else {  // rows are not 16-byte aligned: gather the eight elements
                 XT tmp[8];
 #pragma unroll
@@ -894,12 +911,31 @@ __global__ __launch_bounds__(256) void dispatch_kernel(
 // One thread per (token, 16-byte column piece); the token's slots are sorted
 // by position in registers when k <= KMAX, otherwise found by repeated search.
 // ---------------------------------------------------------------------------
-template <typename XT, int KMAX>
+// VN consecutive elements of an expert row, as raw bits and widened: the rows are of the layer's activation type, or
+// bf16 under f32 activations (a layer whose bf16 / int8 expert products run on the matrix cores).
+template <typename YT, typename XT>
+struct RowPiece {  // rows of the activation type itself
+    typedef uint4 raw_t;
+    static __device__ __forceinline__ raw_t load_raw(const YT* p) { return Vec16<YT>::load_raw(p); }
+    static __device__ __forceinline__ void widen(const raw_t& a, float (&v)[Vec16<YT>::N]) { Vec16<YT>::widen(a, v); }
+};
+template <>
+struct RowPiece<bf16_t, float> {  // four bf16 elements beside four f32 ones
+    typedef uint2 raw_t;
+    static __device__ __forceinline__ raw_t load_raw(const bf16_t* p) { return *reinterpret_cast<const uint2*>(p); }
+    static __device__ __forceinline__ void widen(const raw_t& a, float (&v)[4]) {
+        v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xffff0000u);
+        v[2] = __uint_as_float(a.y << 16); v[3] = __uint_as_float(a.y & 0xffff0000u);
+    }
+};
+
+template <typename XT, typename YT, int KMAX>
 __global__ __launch_bounds__(256) void combine_vec_kernel(
-    const XT* __restrict__ y, const XT* __restrict__ yshared, const XT* __restrict__ residual,
+    const YT* __restrict__ y, const YT* __restrict__ yshared, const XT* __restrict__ residual,
     const int* __restrict__ inv_pos, const float* __restrict__ gate_of, int T, int d, int k,
     XT* __restrict__ out) {
     constexpr int VN = Vec16<XT>::N;
+    typedef RowPiece<YT, XT> YP;
     const int pieces = d / VN;
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (long long)T * pieces) return;
@@ -940,24 +976,24 @@ __global__ __launch_bounds__(256) void combine_vec_kernel(
     for (int i = 0; i < VN; ++i) acc[i] = 0.0f;
     // every row piece is fetched before the first add (no branch around a load: an unused slot
     // re-reads row 0), so the k loads of a token are one round trip instead of k
-    uint4 raw[KMAX], raw_s, raw_r;
+    typename YP::raw_t raw[KMAX], raw_s = {};
+    uint4 raw_r = make_uint4(0, 0, 0, 0);
 #pragma unroll
-    for (int r = 0; r < KMAX; ++r) raw[r] = Vec16<XT>::load_raw(y + (size_t)(r < n ? pos[r] : 0) * d + c);
-    raw_s = raw_r = make_uint4(0, 0, 0, 0);
-    if (yshared) raw_s = Vec16<XT>::load_raw(yshared + (size_t)t * d + c);    // uniform over the launch
+    for (int r = 0; r < KMAX; ++r) raw[r] = YP::load_raw(y + (size_t)(r < n ? pos[r] : 0) * d + c);
+    if (yshared) raw_s = YP::load_raw(yshared + (size_t)t * d + c);    // uniform over the launch
     if (residual) raw_r = Vec16<XT>::load_raw(residual + (size_t)t * d + c);
 #pragma unroll
     for (int r = 0; r < KMAX; ++r) {
         if (r < n) {
             float v[VN];
-            Vec16<XT>::widen(raw[r], v);
+            YP::widen(raw[r], v);
 #pragma unroll
             for (int i = 0; i < VN; ++i) acc[i] = __fadd_rn(acc[i], __fmul_rn(gate[r], v[i]));
         }
     }
     if (yshared) {
         float v[VN];
-        Vec16<XT>::widen(raw_s, v);
+        YP::widen(raw_s, v);
 #pragma unroll
         for (int i = 0; i < VN; ++i) acc[i] = __fadd_rn(acc[i], v[i]);
     }
@@ -971,9 +1007,9 @@ __global__ __launch_bounds__(256) void combine_vec_kernel(
 }
 
 // Any k, any d: one wave per token, one column per lane per step.
-template <typename XT>
+template <typename XT, typename YT>
 __global__ __launch_bounds__(256) void combine_any_kernel(
-    const XT* __restrict__ y, const XT* __restrict__ yshared, const XT* __restrict__ residual,
+    const YT* __restrict__ y, const YT* __restrict__ yshared, const XT* __restrict__ residual,
     const int* __restrict__ inv_pos, const float* __restrict__ gate_of, int T, int d, int k,
     XT* __restrict__ out) {
     const int lane = threadIdx.x & 63;
@@ -1027,10 +1063,10 @@ static hipError_t launch_router_t(const RouterArgs& a, hipStream_t s) {
     const dim3 lgrid(tiles_t, (a.E + NE - 1) / NE);
     if ((long long)lgrid.x * lgrid.y <= 512)  // at most two workgroups on a compute unit
         hipLaunchKernelGGL((logits_kernel<XT, NE, true>), lgrid, dim3(NE * 64), 0, s, static_cast<const XT*>(a.x),
-                           a.wr, a.bias, a.T, a.d, a.E, a.P);
+                           a.wr, a.bias, a.T, a.d, a.E, a.P, static_cast<bf16_t*>(a.rows16));
     else
         hipLaunchKernelGGL((logits_kernel<XT, NE, false>), lgrid, dim3(NE * 64), 0, s, static_cast<const XT*>(a.x),
-                           a.wr, a.bias, a.T, a.d, a.E, a.P);
+                           a.wr, a.bias, a.T, a.d, a.E, a.P, static_cast<bf16_t*>(a.rows16));
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     if (a.E <= 64)
@@ -1046,6 +1082,7 @@ static hipError_t launch_router_t(const RouterArgs& a, hipStream_t s) {
 
 hipError_t launch_router(const RouterArgs& a, bool bf16, hipStream_t s) {
     if (a.T <= 0) return hipSuccess;
+    if (a.rows16 && (bf16 || a.d % 8 != 0)) return hipErrorInvalidValue;  // the copy rides on the 8-element pieces
     return bf16 ? launch_router_t<bf16_t>(a, s) : launch_router_t<float>(a, s);
 }
 
@@ -1084,10 +1121,10 @@ hipError_t launch_dispatch(const DispatchArgs& a, bool bf16, hipStream_t s) {
     return bf16 ? launch_dispatch_t<bf16_t>(a, s) : launch_dispatch_t<float>(a, s);
 }
 
-template <typename XT>
+template <typename XT, typename YT>
 static hipError_t launch_combine_t(const CombineArgs& a, hipStream_t s) {
-    const XT* y = static_cast<const XT*>(a.y);
-    const XT* ys = static_cast<const XT*>(a.yshared);
+    const YT* y = static_cast<const YT*>(a.y);
+    const YT* ys = static_cast<const YT*>(a.yshared);
     const XT* res = static_cast<const XT*>(a.residual);
     XT* out = static_cast<XT*>(a.out);
     constexpr int VN = Vec16<XT>::N;
@@ -1095,13 +1132,13 @@ static hipError_t launch_combine_t(const CombineArgs& a, hipStream_t s) {
         const long long total = (long long)a.T * (a.d / VN);
         const dim3 grid((unsigned)((total + 255) / 256)), block(256);
         if (a.k <= 2)
-            hipLaunchKernelGGL((combine_vec_kernel<XT, 2>), grid, block, 0, s, y, ys, res, a.inv_pos, a.gate_of, a.T, a.d, a.k, out);
+            hipLaunchKernelGGL((combine_vec_kernel<XT, YT, 2>), grid, block, 0, s, y, ys, res, a.inv_pos, a.gate_of, a.T, a.d, a.k, out);
         else if (a.k <= 4)
-            hipLaunchKernelGGL((combine_vec_kernel<XT, 4>), grid, block, 0, s, y, ys, res, a.inv_pos, a.gate_of, a.T, a.d, a.k, out);
+            hipLaunchKernelGGL((combine_vec_kernel<XT, YT, 4>), grid, block, 0, s, y, ys, res, a.inv_pos, a.gate_of, a.T, a.d, a.k, out);
         else
-            hipLaunchKernelGGL((combine_vec_kernel<XT, 8>), grid, block, 0, s, y, ys, res, a.inv_pos, a.gate_of, a.T, a.d, a.k, out);
+            hipLaunchKernelGGL((combine_vec_kernel<XT, YT, 8>), grid, block, 0, s, y, ys, res, a.inv_pos, a.gate_of, a.T, a.d, a.k, out);
     } else {
-        hipLaunchKernelGGL((combine_any_kernel<XT>), dim3((a.T + 3) / 4), dim3(256), 0, s, y, ys, res, a.inv_pos,
+        hipLaunchKernelGGL((combine_any_kernel<XT, YT>), dim3((a.T + 3) / 4), dim3(256), 0, s, y, ys, res, a.inv_pos,
                            a.gate_of, a.T, a.d, a.k, out);
     }
     return hipGetLastError();
@@ -1230,7 +1267,8 @@ hipError_t launch_rmsnorm(const void* x, const float* weight, float eps, int T, 
 
 hipError_t launch_combine(const CombineArgs& a, bool bf16, hipStream_t s) {
     if (a.T <= 0) return hipSuccess;
-    return bf16 ? launch_combine_t<bf16_t>(a, s) : launch_combine_t<float>(a, s);
+    if (bf16) return launch_combine_t<bf16_t, bf16_t>(a, s);
+    return a.rows_bf16 ? launch_combine_t<float, bf16_t>(a, s) : launch_combine_t<float, float>(a, s);
 }
 
 }  // namespace rbmoe

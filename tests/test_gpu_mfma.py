@@ -40,8 +40,9 @@ def run(device, t, valid=None, bias=None):
     assert rel_l2(y, ref.expert_out) <= 2e-2, "expert output rows"
     err = rel_l2(out, ref.out)
     assert err <= 2e-2, err
+    name = layer.kernel_name()
     layer.close()
-    return err
+    return name
 
 
 @pytest.mark.parametrize("wt", ["bf16", "int8"])
@@ -98,3 +99,37 @@ def test_matrix_core_and_generic_paths_agree(device, kernel_env):
 def test_small_token_counts(device, T):
     t = synth.make(small_workload(d=64, E=8, k=2, F=64, T=T, seed=37, act="bf16", wt="bf16", shared=True))
     run(device, t)
+
+
+@pytest.mark.parametrize("wt", ["bf16", "int8"])
+@pytest.mark.parametrize("T", [8, 700])
+def test_f32_rows_with_bf16_or_int8_weights_run_on_the_matrix_cores(device, wt, T):
+    # What a caller with f32 matrices and a bf16 or quantized checkpoint has (Matrix is f32, src/matrix.rs:13-18;
+    # after TransformerLm::quantize() the Linear layers take the Quantized branch on f32 inputs,
+    # src/param.rs:778-780, src/quantized.rs:55-99).  The router reads the f32 rows (identical routing), the expert
+    # products read their bf16 copy: the same 2e-2 bar as bf16 rows.  T = 8: the decode-shaped kernels.
+    t = synth.make(small_workload(d=768, E=8, k=2, F=1408, T=T, seed=29, act="f32", wt=wt, shared=True,
+                                  shared_d_ff=704))
+    name = run(device, t)
+    assert name == ("mfma_bf16_decode" if T <= 32 else "mfma_bf16_stream") + ("_int8w" if wt == "int8" else "")
+    valid = (np.arange(T) % 5 != 2).astype(np.uint8)
+    bias = synth.normal((8,), 0.5, 29, 98)
+    run(device, t, valid=valid, bias=bias)
+
+
+def test_f32_rows_block_step_on_the_matrix_cores(device):
+    # norm in front, residual behind, f32 on the boundary, int8 experts on the matrix cores, both kernel sets
+    from helpers import small_workload as sw
+    from oracle import rb_oracle as orc
+    for T in (5, 300):
+        t = synth.make(sw(d=128, E=8, k=2, F=192, T=T, seed=31, act="f32", wt="int8", shared=True, shared_d_ff=64))
+        layer = gpu_layer(device, t)
+        w = (1.0 + 0.1 * synth.normal((128,), 1.0, 31, 97)).astype(np.float32)
+        layer.set_feed_forward_norm(w, 1e-6)
+        out, cache = layer.forward_block(t.x)
+        assert layer.kernel_name().startswith("mfma_bf16")
+        normed = orc.rmsnorm(t.x, w, 1e-6)
+        ref = oracle_layer(t).forward(normed, threads=4)
+        assert_routing_identical(cache, ref)
+        assert rel_l2(out, ref.out + t.x) <= 2e-2
+        layer.close()
