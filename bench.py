@@ -34,12 +34,36 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_F32_TFLOPS = 157.3     # MI355X fp32 matrix
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
-# HBM-side bytes per launch of the gate/up kernel, measured with rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE (each scaled by the reading of a 256 MiB copy; profiles/c3_prefill_hbm_traffic.txt).
-# Valid only for the workload and kernel it was measured on.
-MEASURED_TRAFFIC = {("c3_prefill_d768_e16", "mfma_bf16_stream"): 301.3e6,
-                    # decode gate/up launch (profiles/c2_decode_hbm_traffic.txt): every weight byte once
-                    ("c2_decode_d768_e8", "mfma_bf16_decode"): 39.18e6}
+# HBM-side bytes per launch of the dominant kernel come from rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE), which
+# cannot be taken inside this program: profiles/hbm_traffic.json records them, each with the summary file it was read
+# from and a digest of the kernel sources at the time.  A record whose digest is not that of the sources beside this
+# file describes other kernels and is reported as null.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+KERNEL_SOURCES = ("grouped_stream.hip", "decode_kernels.hip", "grouped_f32.hip")
+
+
+def kernel_digest() -> str:
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "rustingbrain_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload: str, kernel: str):
+    """(bytes per launch or None, where the figure comes from)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            table = json.load(f)
+    except (OSError, ValueError):
+        return None, "no profiles/hbm_traffic.json"
+    rec = table.get(workload)
+    if not rec or rec.get("kernel") != kernel:
+        return None, "no counter run recorded for this workload and kernel"
+    if rec.get("kernel_digest") != kernel_digest():
+        return None, f"{rec.get('source')} was measured on other kernel sources (digest {rec.get('kernel_digest')})"
+    return float(rec["bytes_per_launch"]), rec.get("source")
 
 
 class DeviceBuffer:
@@ -101,7 +125,7 @@ def cpu_baseline(t: synth.Tensors, budget_s: float = 20.0) -> dict:
     on the host cores of this machine.  Only this function touches oracle/."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     from helpers import oracle_layer
-    threads = max(1, min(16, os.cpu_count() or 1))
+    threads = max(1, min(16, os.cpu_count() or 1))   # the GPU box gives one job 16 cores' worth
     layer = oracle_layer(t)
     T = t.x.shape[0]
     layer.forward(t.x, router_bias=t.router_bias, threads=threads)  # warm-up
@@ -112,7 +136,7 @@ def cpu_baseline(t: synth.Tensors, budget_s: float = 20.0) -> dict:
         layer.forward(t.x, router_bias=t.router_bias, threads=threads)
         times.append(time.perf_counter() - t0)
     best = float(np.median(times))
-    return {"value": T / best, "unit": "tokens/s", "cores": threads, "kind": "port",
+    return {"value": T / best, "unit": "tokens/s", "cores": threads, "os_cpu_count": os.cpu_count(), "kind": "port",
             "sample": f"whole workload ({T} tokens), median of {len(times)} forwards after 1 warm-up; "
                       "C++ restatement of the reference's rayon path, not the Rust binary",
             "ms_per_forward": best * 1e3}
@@ -128,7 +152,8 @@ def cpu_baseline_backward(t: synth.Tensors, grad_output: np.ndarray) -> dict:
     t0 = time.perf_counter()
     layer.backward(t.x, grad_output, router_bias=t.router_bias, threads=threads)
     ms = (time.perf_counter() - t0) * 1e3
-    return {"value": t.x.shape[0] / (ms * 1e-3), "unit": "tokens/s", "cores": threads, "kind": "port",
+    return {"value": t.x.shape[0] / (ms * 1e-3), "unit": "tokens/s", "cores": threads, "os_cpu_count": os.cpu_count(),
+            "kind": "port",
             "sample": "whole workload, one forward + backward call of the C++ restatement (experts as parallel "
                       "tasks, like the reference's par_iter over experts)", "ms": ms}
 
@@ -190,32 +215,18 @@ def backward_leg(dev, w, t, x, out, bp, args, alg, with_cpu: bool) -> dict:
     return res
 
 
-def main() -> int:
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c3_prefill_d768_e16", choices=list(synth.WORKLOADS))
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--backward", action="store_true",
-                    help="also time the backward pass (bf16 layers and all-f32 layers)")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run one 256 MiB device-to-device copy (the plain copy that FETCH_SIZE / "
-                         "WRITE_SIZE readings are scaled by when this command runs under rocprofv3 --pmc)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
-        return 2
-
-    w = synth.WORKLOADS[args.workload]
+def measure(dev, name: str, steps: int, warmup: int, repeats: int, act_override: str = None) -> dict:
+    """One workload: `repeats` loops of `steps` forwards (median loop -> ms_per_step), per-stage durations from HIP
+    events on the library's stream, the roofline of the dominant kernel.  Returns the pieces the report is built of."""
+    w = synth.WORKLOADS[name]
     t = synth.make(w)
+    if act_override:
+        w = synth.Workload(**{**w.__dict__, "act_dtype": act_override})
     T = w.tokens
-    dev = rb.Device.open(0)
     cfg = rb.MoeConfig(w.num_experts, w.experts_per_token, w.d_ff, w.shared_expert)
     layer = rb.MoeLayer(w.d_model, cfg, dev, act_dtype=w.act_dtype, weight_dtype=w.weight_dtype, max_tokens=T,
                         shared_d_ff=w.shared_d_ff if w.shared_expert else 0)
     layer.load_tensors(t)
-
     bf16 = w.act_dtype == "bf16"
     xh = synth.f32_to_bf16_bits(t.x) if bf16 else t.x
     x = DeviceBuffer(dev, xh.nbytes).upload(xh)
@@ -223,19 +234,20 @@ def main() -> int:
     bias = DeviceBuffer(dev, 4 * w.num_experts).upload(t.router_bias) if t.router_bias is not None else None
     bp = bias.ptr if bias else 0
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         layer.forward_device(x.ptr, T, out.ptr, bias_ptr=bp)
     dev.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        layer.forward_device(x.ptr, T, out.ptr, bias_ptr=bp)
-    dev.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed * 1e3 / args.steps
+    loops = []
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            layer.forward_device(x.ptr, T, out.ptr, bias_ptr=bp)
+        dev.synchronize()
+        loops.append((time.perf_counter() - t0) * 1e3 / steps)
+    ms_per_step = float(np.median(loops))
 
-    # per-stage durations from HIP events on the library's stream
-    decode = T <= 64
-    nprof = max(10, min(100, args.steps))
+    decode = "decode" in layer.kernel_name()   # the library takes the decode-shaped kernels up to 32 tokens
+    nprof = max(10, min(100, steps))
 
     def timed_stages(flush=None):
         acc = {}
@@ -245,14 +257,14 @@ def main() -> int:
                 assert dev._lib.rbmoe_copy_device(dev.handle, C.c_void_p(flush[1].ptr), C.c_void_p(flush[0].ptr),
                                                   flush[0].nbytes) == L.OK
             st = layer.forward_timed(x.ptr, T, out.ptr, bias_ptr=bp)
-            for name, v in st.items():
-                acc.setdefault(name, []).append(v)
-        raw = {name: float(np.mean(v)) for name, v in acc.items()}
+            for nm, v in st.items():
+                acc.setdefault(nm, []).append(v)
+        raw = {nm: float(np.mean(v)) for nm, v in acc.items()}
         # One interval of forward_timed brackets no work: what a pair of event records adds to every
         # other interval.  Kernel durations are the intervals minus that.
         over = raw["empty"]
-        net = {name: (v if name in ("empty", "total") else max(v - over, 1e-6)) for name, v in raw.items()}
-        mins = {name: float(np.min(v)) for name, v in acc.items()}
+        net = {nm: (v if nm in ("empty", "total") else max(v - over, 1e-6)) for nm, v in raw.items()}
+        mins = {nm: float(np.min(v)) for nm, v in acc.items()}
         return raw, net, mins, over
 
     raw_ms, stage_ms, stage_ms_min, overhead = timed_stages()
@@ -269,7 +281,7 @@ def main() -> int:
     routed = int(cache.offsets[-1])
     touched = int((cache.counts > 0).sum())
     alg = algorithmic(w, T, routed, touched)
-    peak_tf = PEAK_F32_TFLOPS if (w.act_dtype == "f32") else PEAK_BF16_TFLOPS
+    peak_tf = PEAK_F32_TFLOPS if (w.weight_dtype == "f32") else PEAK_BF16_TFLOPS
 
     def tflops(flops, ms):
         return flops / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
@@ -277,23 +289,25 @@ def main() -> int:
     def gbs(nbytes, ms):
         return nbytes / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
 
+    kname = layer.kernel_name()
+    traffic, traffic_source = measured_traffic(w.name, kname)
     gu = tflops(alg["gate_up_flops"], stage_ms["gate_up"])
     if decode:
         # the dominant kernel of the decode-shaped path streams the gate/up weights of the touched experts
         # (and of the shared expert) once: it is bound by HBM
         cold_ms = cold[1]
         gu_gbs = gbs(alg["decode_gate_up_bytes"], cold_ms["gate_up"])
-        roofline = {"bound": "hbm", "kernel": "decode gate/up product + SwiGLU, routed and shared (" +
-                                              layer.kernel_name() + "), caches flushed before every forward",
+        roofline = {"bound": "hbm", "kernel": "decode gate/up product + SwiGLU, routed and shared (" + kname +
+                                              "), caches flushed before every forward",
                     "achieved": gu_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gu_gbs / PEAK_HBM_GBS,
-                    "traffic": MEASURED_TRAFFIC.get((w.name, layer.kernel_name())),
+                    "traffic": traffic, "traffic_source": traffic_source,
                     "bytes_per_launch": alg["decode_gate_up_bytes"],
                     "avg_launch_ms": cold_ms["gate_up"], "touched_experts": touched,
                     "cache_resident_gbs": gbs(alg["decode_gate_up_bytes"], stage_ms["gate_up"])}
     else:
-        roofline = {"bound": "mfma", "kernel": "grouped gate/up product + SwiGLU (" + layer.kernel_name() + ")",
+        roofline = {"bound": "mfma", "kernel": "grouped gate/up product + SwiGLU (" + kname + ")",
                     "achieved": gu, "peak": peak_tf, "unit": "TFLOP/s", "frac": gu / peak_tf,
-                    "traffic": MEASURED_TRAFFIC.get((w.name, layer.kernel_name())),
+                    "traffic": traffic, "traffic_source": traffic_source,
                     "flops_per_launch": alg["gate_up_flops"], "avg_launch_ms": stage_ms["gate_up"]}
     both_ms = stage_ms["gate_up"] + stage_ms["down"] + stage_ms["shared"]
     stages = {
@@ -303,14 +317,12 @@ def main() -> int:
         "down_tflops": tflops(alg["down_flops"], stage_ms["down"]),
         "grouped_gemms_tflops": tflops(alg["gemm_flops"], both_ms),
         "grouped_gemms_frac_of_peak": tflops(alg["gemm_flops"], both_ms) / peak_tf,
-        # The short, HBM-bound stages are priced on their RAW event intervals (kernel plus what the event pair
-        # adds): for a 10 us kernel the subtraction above removes more than the pair really cost, and the
-        # kernel-trace durations under profiles/ lie between the two.  These figures are therefore lower bounds.
-        "router_gbs": gbs(alg["router_bytes"], raw_ms["router"]),
-        "dispatch_gbs": gbs(alg["dispatch_bytes"], raw_ms["dispatch"]),
+        # the HBM-bound stages, on the same net intervals as the products
+        "router_gbs": gbs(alg["router_bytes"], stage_ms["router"]),
+        "dispatch_gbs": gbs(alg["dispatch_bytes"], stage_ms["dispatch"]),
         "dispatch_note": "latency-bound: a few hundred KB of indices per launch, no rows are moved",
-        "combine_gbs": gbs(alg["combine_bytes"], raw_ms["combine"]),
-        "combine_frac_of_hbm": gbs(alg["combine_bytes"], raw_ms["combine"]) / PEAK_HBM_GBS,
+        "combine_gbs": gbs(alg["combine_bytes"], stage_ms["combine"]),
+        "combine_frac_of_hbm": gbs(alg["combine_bytes"], stage_ms["combine"]) / PEAK_HBM_GBS,
     }
     if decode:
         whole = gbs(alg["layer_bytes_decode"], ms_per_step)
@@ -319,24 +331,82 @@ def main() -> int:
         stages.update({"cold_ms_mean": cold_ms,
                        "cold_decode_down_gbs": gbs(alg["decode_down_bytes"], cold_ms["down"]),
                        "cold_decode_down_frac_of_hbm": gbs(alg["decode_down_bytes"], cold_ms["down"]) / PEAK_HBM_GBS,
+                       "cold_whole_layer_ms": cold_kernels,
                        "cold_whole_layer_gbs": gbs(alg["layer_bytes_decode"], cold_kernels),
                        "cold_whole_layer_frac_of_hbm": gbs(alg["layer_bytes_decode"], cold_kernels) / PEAK_HBM_GBS,
                        "cache_resident_whole_layer_gbs": whole,
                        "whole_layer_bytes": alg["layer_bytes_decode"],
                        "note": "value / ms_per_step are back-to-back forwards (weights stay in the 256 MiB "
                                "Infinity Cache); cold_* figures flush L2 and Infinity Cache before every forward"})
+    config = {"workload": w.name, "d_model": w.d_model, "num_experts": w.num_experts,
+              "experts_per_token": w.experts_per_token, "d_ff": w.d_ff, "tokens": T,
+              "shared_expert": w.shared_expert, "weight_dtype": w.weight_dtype, "act_dtype": w.act_dtype,
+              "seed": w.seed, "expert0_share": float(cache.load_fractions()[0]), "routed_slots": routed}
+    return {"w": w, "t": t, "layer": layer, "x": x, "out": out, "bias": bias, "bp": bp, "alg": alg,
+            "ms_per_step": ms_per_step, "loops_ms": loops, "roofline": roofline, "stages": stages, "config": config,
+            "bf16": bf16, "decode": decode}
 
+
+def release(m: dict) -> None:
+    m["layer"].close()
+    for b in (m["x"], m["out"], m["bias"]):
+        if b:
+            b.free()
+
+
+def summary(m: dict) -> dict:
+    """The short form of one workload for the `workloads` object of the report."""
+    r, st = m["roofline"], m["stages"]
+    s = {"tokens_per_s": m["config"]["tokens"] / (m["ms_per_step"] * 1e-3), "ms_per_step": m["ms_per_step"],
+         "kernel": r["kernel"], "bound": r["bound"], "frac": r["frac"], "achieved": r["achieved"], "unit": r["unit"],
+         "peak": r["peak"], "avg_launch_ms": r["avg_launch_ms"], "traffic": r["traffic"],
+         "stage_ms": {k: round(v, 5) for k, v in st["ms_mean"].items()},
+         "grouped_gemms_frac_of_peak": st["grouped_gemms_frac_of_peak"], "config": m["config"]}
+    if m["decode"]:
+        s.update({"cold": {"gate_up_frac_of_hbm": r["frac"], "gate_up_ms": r["avg_launch_ms"],
+                           "down_frac_of_hbm": st["cold_decode_down_frac_of_hbm"],
+                           "whole_layer_ms": st["cold_whole_layer_ms"],
+                           "whole_layer_frac_of_hbm": st["cold_whole_layer_frac_of_hbm"]},
+                  "warm": {"gate_up_gbs": r["cache_resident_gbs"], "whole_layer_ms": m["ms_per_step"],
+                           "whole_layer_gbs": st["cache_resident_whole_layer_gbs"]}})
+    return s
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--repeats", type=int, default=5, help="loops of --steps forwards; ms_per_step is their median")
+    ap.add_argument("--workload", default="c3_prefill_d768_e16", choices=list(synth.WORKLOADS),
+                    help="the workload of the top-level figures (the metric is quoted on the default)")
+    ap.add_argument("--only", action="store_true", help="skip the `workloads` object (the other four workloads)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--backward", action="store_true",
+                    help="also time the backward pass (bf16 layers and all-f32 layers)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 256 MiB device-to-device copy (the plain copy that FETCH_SIZE / "
+                         "WRITE_SIZE readings are scaled by when this command runs under rocprofv3 --pmc)")
+    ap.add_argument("--calibrate-mfma", action="store_true",
+                    help="also run the multiply-only kernel: the rate the matrix cores sustain (`calibration.mfma`)")
+    ap.add_argument("--calibrate-read", action="store_true",
+                    help="also run a plain 39 MiB read with cold and warm caches (`calibration.read`): what a launch "
+                         "the size of the decode gate/up product can get out of HBM")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        return 2
+
+    dev = rb.Device.open(0)
+    m = measure(dev, args.workload, args.steps, args.warmup, args.repeats)
+    w, T = m["w"], m["w"].tokens
     result = {
         "metric": "MoE-layer fwd tokens/sec at d768 E16 k2; grouped-GEMM % of bf16 MFMA peak",
-        "value": T / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16" if bf16 else "f32", "data": "synthetic",
-        "config": {"workload": w.name, "d_model": w.d_model, "num_experts": w.num_experts,
-                   "experts_per_token": w.experts_per_token, "d_ff": w.d_ff, "tokens": T,
-                   "shared_expert": w.shared_expert, "weight_dtype": w.weight_dtype, "seed": w.seed,
-                   "expert0_share": float(cache.load_fractions()[0]), "routed_slots": routed},
-        "roofline": roofline,
-        "stages": stages,
+        "value": T / (m["ms_per_step"] * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "repeats": args.repeats, "ms_per_step": m["ms_per_step"],
+        "ms_per_step_loops": m["loops_ms"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16" if w.weight_dtype != "f32" else "f32", "data": "synthetic",
+        "config": m["config"], "roofline": m["roofline"], "stages": m["stages"],
     }
     if args.calibrate_copy:
         n = 256 << 20
@@ -344,12 +414,49 @@ def main() -> int:
         assert dev._lib.rbmoe_copy_device(dev.handle, C.c_void_p(b.ptr), C.c_void_p(a.ptr), n) == L.OK
         a.free()
         b.free()
+    calibration = {}
+    if args.calibrate_mfma:
+        tf, ms = C.c_double(), C.c_double()
+        assert dev._lib.rbmoe_calibrate_mfma(dev.handle, 10, C.byref(tf), C.byref(ms)) == L.OK
+        calibration["mfma"] = {"tflops": tf.value, "avg_launch_ms": ms.value, "frac_of_published_peak":
+                               tf.value / PEAK_BF16_TFLOPS, "kernel": "mfma_only_kernel: 32x32x16 bf16 multiplies only, "
+                               "two waves per SIMD"}
+    if args.calibrate_read:
+        n = 39 * (1 << 20)
+        rd = {}
+        for label, flush in (("cold", 1), ("warm", 0)):
+            g, ms = C.c_double(), C.c_double()
+            assert dev._lib.rbmoe_calibrate_read(dev.handle, n, 20, flush, C.byref(g), C.byref(ms)) == L.OK
+            rd[label] = {"gbs": g.value, "avg_launch_ms": ms.value, "frac_of_hbm_peak": g.value / PEAK_HBM_GBS}
+        rd["bytes"] = n
+        rd["note"] = ("event interval around each launch of read_only_kernel minus the interval of an empty event "
+                      "pair; cold: a 512 MiB copy runs before every launch")
+        calibration["read"] = rd
+    if calibration:
+        result["calibration"] = calibration
     if args.backward:
-        result["backward"] = backward_leg(dev, w, t, x, out, bp, args, alg, with_cpu=not args.no_cpu)
+        result["backward"] = backward_leg(dev, w, m["t"], m["x"], m["out"], m["bp"], args, m["alg"],
+                                          with_cpu=not args.no_cpu)
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(t)
+        result["cpu_baseline"] = cpu_baseline(m["t"])
+    release(m)
+    if not args.only:
+        # the other workloads, shorter loops: parity-test cases as far as the metric goes, reported for their
+        # kernels' rooflines (C2: the decode-shaped target, cold and warm)
+        others = {}
+        for name in synth.WORKLOADS:
+            if name == args.workload:
+                continue
+            o = measure(dev, name, max(20, args.steps // 4), max(5, args.warmup // 2), max(3, min(args.repeats, 5)))
+            others[name] = summary(o)
+            release(o)
+        # the int8 workload with f32 rows on the boundary: what a caller with f32 matrices and a quantized
+        # checkpoint runs (the router reads the f32 rows, the products their bf16 copy)
+        o = measure(dev, "c5_int8_d768_e8", max(20, args.steps // 4), max(5, args.warmup // 2), 3, act_override="f32")
+        others["c5_int8_d768_e8_f32_rows"] = summary(o)
+        release(o)
+        result["workloads"] = others
     print(json.dumps(result))
-    layer.close()
     return 0
 
 

@@ -283,6 +283,18 @@ int rbmoe_copy_to_host(rbmoe_ctx* ctx, void* dst, const void* src, size_t bytes)
  * plain copy of known size that hardware-counter readings are calibrated against). */
 int rbmoe_copy_device(rbmoe_ctx* ctx, void* dst, const void* src, size_t bytes);
 
+/* ---- calibration: what the device sustains, for roofline figures to be read against.  No counterpart in the
+ * reference; neither touches a layer.  Both allocate their own buffers, time `launches` launches with HIP events on
+ * the context's stream and synchronise.  rbmoe_calibrate_read times every launch by itself and takes off what a pair
+ * of event records with nothing between them reads in the same call (a few microseconds, as much as the launch).
+ * rbmoe_calibrate_mfma: a kernel of nothing but 32x32x16 bf16 matrix-core multiplies, two waves on every SIMD, about
+ * 0.25 ms a launch -> the multiply rate the matrix cores sustain at the clock they settle at.
+ * rbmoe_calibrate_read: a plain read of `bytes` (16-byte loads, 1024 workgroups); with `flush_caches` != 0 a 512 MiB
+ * copy runs before every launch so that the read comes from HBM, as a decode step's weights do. */
+int rbmoe_calibrate_mfma(rbmoe_ctx* ctx, int32_t launches, double* tflops, double* avg_launch_ms);
+int rbmoe_calibrate_read(rbmoe_ctx* ctx, size_t bytes, int32_t launches, int32_t flush_caches, double* gbs,
+                         double* avg_launch_ms);
+
 const char* rbmoe_version(void);
 
 #ifdef __cplusplus

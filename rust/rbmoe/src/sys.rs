@@ -118,5 +118,9 @@ extern "C" {
     pub fn rbmoe_copy_to_device(ctx: *mut rbmoe_ctx, dst: *mut c_void, src: *const c_void, bytes: usize) -> c_int;
     pub fn rbmoe_copy_to_host(ctx: *mut rbmoe_ctx, dst: *mut c_void, src: *const c_void, bytes: usize) -> c_int;
     pub fn rbmoe_copy_device(ctx: *mut rbmoe_ctx, dst: *mut c_void, src: *const c_void, bytes: usize) -> c_int;
+    // calibration: a multiply-only kernel and a plain read, for roofline figures to be read against
+    pub fn rbmoe_calibrate_mfma(ctx: *mut rbmoe_ctx, launches: i32, tflops: *mut f64, avg_launch_ms: *mut f64) -> c_int;
+    pub fn rbmoe_calibrate_read(ctx: *mut rbmoe_ctx, bytes: usize, launches: i32, flush_caches: i32, gbs: *mut f64,
+                                avg_launch_ms: *mut f64) -> c_int;
     pub fn rbmoe_version() -> *const c_char;
 }

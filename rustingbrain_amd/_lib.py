@@ -81,6 +81,9 @@ SIGNATURES = {
     "rbmoe_backward_block_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
     "rbmoe_zero_grads": (C.c_int, [C.c_void_p]),
     "rbmoe_get_weight_grad": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_float), C.c_int32, C.c_int32]),
+    "rbmoe_calibrate_mfma": (C.c_int, [C.c_void_p, C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+    "rbmoe_calibrate_read": (C.c_int, [C.c_void_p, C.c_size_t, C.c_int32, C.c_int32, C.POINTER(C.c_double),
+                                       C.POINTER(C.c_double)]),
     "rbmoe_version": (C.c_char_p, []),
 }
 

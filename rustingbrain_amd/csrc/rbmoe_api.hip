@@ -1680,6 +1680,91 @@ int rbmoe_copy_to_host(rbmoe_ctx* ctx, void* dst, const void* src, size_t bytes)
     return RBMOE_OK;
 }
 
+int rbmoe_calibrate_mfma(rbmoe_ctx* ctx, int32_t launches, double* tflops, double* avg_launch_ms) {
+    if (!ctx || !tflops) return fail(ctx, RBMOE_NULL_POINTER, "ctx or tflops is NULL");
+    if (launches <= 0) return fail(ctx, RBMOE_INVALID_INPUT, "launches must be positive");
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    int cus = 0;
+    HIP_TRY(ctx, hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, ctx->device));
+    const int workgroups = 2 * cus, steps = 2048;  // two waves on every SIMD
+    float* out = nullptr;
+    HIP_TRY(ctx, hipMalloc(&out, (size_t)workgroups * 256 * sizeof(float)));
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipError_t e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    hipStream_t s = ctx->stream;
+    if (e == hipSuccess) e = launch_mfma_only(out, workgroups, steps, s);  // warm-up
+    if (e == hipSuccess) e = hipEventRecord(e0, s);
+    for (int i = 0; i < launches && e == hipSuccess; ++i) e = launch_mfma_only(out, workgroups, steps, s);
+    if (e == hipSuccess) e = hipEventRecord(e1, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    float ms = 0.0f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    (void)hipFree(out);
+    if (e != hipSuccess) return hip_fail(ctx, e, "rbmoe_calibrate_mfma");
+    const double flops = (double)workgroups * 4 * steps * 8 * 32768.0;  // 2 * 32 * 32 * 16 per multiply
+    const double avg = (double)ms / launches;
+    *tflops = flops / (avg * 1e-3) / 1e12;
+    if (avg_launch_ms) *avg_launch_ms = avg;
+    return RBMOE_OK;
+}
+
+int rbmoe_calibrate_read(rbmoe_ctx* ctx, size_t bytes, int32_t launches, int32_t flush_caches, double* gbs,
+                         double* avg_launch_ms) {
+    if (!ctx || !gbs) return fail(ctx, RBMOE_NULL_POINTER, "ctx or gbs is NULL");
+    if (launches <= 0 || bytes < 16 || bytes % 16 != 0)
+        return fail(ctx, RBMOE_INVALID_INPUT, "launches must be positive and bytes a positive multiple of 16");
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    hipStream_t s = ctx->stream;
+    const size_t flush_bytes = (size_t)512 << 20;  // twice the 256 MiB Infinity Cache through L2
+    void *buf = nullptr, *fa = nullptr, *fb = nullptr;
+    uint32_t* sink = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipError_t e = hipMalloc(&buf, bytes);
+    if (e == hipSuccess) e = hipMalloc(&sink, 256);
+    if (e == hipSuccess) e = hipMemsetAsync(buf, 1, bytes, s);
+    if (e == hipSuccess && flush_caches) e = hipMalloc(&fa, flush_bytes);
+    if (e == hipSuccess && flush_caches) e = hipMalloc(&fb, flush_bytes);
+    if (e == hipSuccess) e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    const int workgroups = 1024;
+    if (e == hipSuccess) e = launch_read_only(buf, bytes, workgroups, sink, s);  // warm-up
+    // what a pair of event records adds to the interval between them: taken off every launch's interval below
+    double empty = 0.0;
+    for (int i = 0; i < 8 && e == hipSuccess; ++i) {
+        e = hipEventRecord(e0, s);
+        if (e == hipSuccess) e = hipEventRecord(e1, s);
+        if (e == hipSuccess) e = hipStreamSynchronize(s);
+        float ms = 0.0f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+        empty += ms / 8.0;
+    }
+    double total = 0.0;
+    for (int i = 0; i < launches && e == hipSuccess; ++i) {
+        if (flush_caches) e = hipMemcpyAsync(fb, fa, flush_bytes, hipMemcpyDeviceToDevice, s);
+        if (e == hipSuccess) e = hipEventRecord(e0, s);
+        if (e == hipSuccess) e = launch_read_only(buf, bytes, workgroups, sink, s);
+        if (e == hipSuccess) e = hipEventRecord(e1, s);
+        if (e == hipSuccess) e = hipStreamSynchronize(s);
+        float ms = 0.0f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+        total += std::max((double)ms - empty, 1e-6);
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    (void)hipFree(buf);
+    (void)hipFree(sink);
+    if (fa) (void)hipFree(fa);
+    if (fb) (void)hipFree(fb);
+    if (e != hipSuccess) return hip_fail(ctx, e, "rbmoe_calibrate_read");
+    const double avg = total / launches;
+    *gbs = (double)bytes / (avg * 1e-3) / 1e9;
+    if (avg_launch_ms) *avg_launch_ms = avg;
+    return RBMOE_OK;
+}
+
 int rbmoe_copy_device(rbmoe_ctx* ctx, void* dst, const void* src, size_t bytes) {
     if (!ctx) return fail(nullptr, RBMOE_NULL_POINTER, "ctx is NULL");
     if (bytes == 0) return RBMOE_OK;

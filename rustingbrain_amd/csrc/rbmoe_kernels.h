@@ -239,4 +239,10 @@ struct DecodeGemmArgs {
 bool decode_shape_ok(int N, int K);
 hipError_t launch_decode_gemm(const DecodeGemmArgs& g, WeightKind wk, hipStream_t s);
 
+// ---- calibration (calibrate.hip): what the device sustains, for the roofline figures to be read against ----
+// 4 waves per workgroup, each issuing steps * 8 independent 32x32x16 bf16 multiplies; out: workgroups * 256 floats
+hipError_t launch_mfma_only(float* out, int workgroups, int steps, hipStream_t s);
+// a plain read of `bytes` (a multiple of 16) split over the workgroups
+hipError_t launch_read_only(const void* src, size_t bytes, int workgroups, uint32_t* out, hipStream_t s);
+
 }  // namespace rbmoe

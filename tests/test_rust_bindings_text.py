@@ -21,14 +21,14 @@ def c_kind(decl):
     if "*" in decl:
         return "ptr"
     base = decl.rsplit(" ", 1)[0] if " " in decl else decl
-    return {"int32_t": "i32", "int": "i32", "size_t": "usize", "float": "f32", "uint64_t": "u64"}[base.replace("const ", "").strip()]
+    return {"int32_t": "i32", "int": "i32", "size_t": "usize", "float": "f32", "double": "f64", "uint64_t": "u64"}[base.replace("const ", "").strip()]
 
 
 def rust_kind(ty):
     ty = ty.strip()
     if ty.startswith("*"):
         return "ptr"
-    return {"i32": "i32", "c_int": "i32", "usize": "usize", "f32": "f32", "u64": "u64"}[ty]
+    return {"i32": "i32", "c_int": "i32", "usize": "usize", "f32": "f32", "f64": "f64", "u64": "u64"}[ty]
 
 
 def c_functions():
