@@ -24,6 +24,13 @@ namespace rbmoe {
 // ---------------------------------------------------------------------------
 constexpr int kSmallThreads = 512;
 constexpr int kStageBytes = 96 * 1024;  // LDS for the staged router and token rows (gfx950: 160 KiB per workgroup)
+// LDS of the routing code behind the staging area: prob, lsev, sexp, cnt, off, aux_term (see route_small_body)
+constexpr int kRouteFixedBytes = (kSmallRouteMaxPairs + kSmallRouteMaxTokens + kSmallRouteMaxTokens * kMaxTopK +
+                                  2 * (kMaxExperts + 1) + kMaxExperts) * 4 + 64;
+// The launch that runs the routing beside the gate/up products (decode_front_kernel) keeps two workgroups on a
+// compute unit: 80 KiB each, of which the routing workgroup stages rows in this much.
+constexpr int kFrontLdsBytes = 80 * 1024;
+constexpr int kFrontStageBytes = (kFrontLdsBytes - kRouteFixedBytes) / 16 * 16;
 
 // softmax_rows (src/moe.rs, softmax over one row) and route (src/moe.rs:553-593) of one token, by one
 // thread, the row used where it lies in LDS: the path for more experts than a wave has lanes.
@@ -165,8 +172,10 @@ __device__ __forceinline__ void token_phase_lanes(float* row_lds, int t, int j, 
     }
 }
 
-template <typename XT>
-__global__ __launch_bounds__(kSmallThreads) void route_small_kernel(
+// STAGE = bytes of `smem` for the staged router and token rows; the routing arrays follow them.
+template <typename XT, int STAGE>
+__device__ __forceinline__ void route_small_body(
+    unsigned char* __restrict__ smem,
     const XT* __restrict__ x, const float* __restrict__ wr, const float* __restrict__ bias,
     const uint8_t* __restrict__ valid, int T, int d, int E, int k, float w_aux, float w_z, int tile_m,
     float* __restrict__ P, float* __restrict__ lse, int* __restrict__ expert_of, float* __restrict__ gate_of,
@@ -175,13 +184,14 @@ __global__ __launch_bounds__(kSmallThreads) void route_small_kernel(
     float* __restrict__ losses, int* __restrict__ perm_slot, int* __restrict__ perm_token,
     int* __restrict__ inv_pos, const float* __restrict__ norm_w, float norm_eps, XT* __restrict__ xn_out,
     bf16_t* __restrict__ rows16) {
-    __shared__ __align__(16) unsigned char stage[kStageBytes];
-    __shared__ float prob[kSmallRouteMaxPairs];
-    __shared__ float lsev[kSmallRouteMaxTokens];
-    __shared__ int sexp[kSmallRouteMaxTokens * kMaxTopK];
-    __shared__ int cnt[kMaxExperts + 1];
-    __shared__ int off[kMaxExperts + 1];
-    __shared__ float aux_term[kMaxExperts];
+    static_assert(STAGE % 16 == 0, "the arrays behind the staging area stay aligned");
+    unsigned char* const stage = smem;
+    float* const prob = reinterpret_cast<float*>(smem + STAGE);                 // [kSmallRouteMaxPairs]
+    float* const lsev = prob + kSmallRouteMaxPairs;                             // [kSmallRouteMaxTokens]
+    int* const sexp = reinterpret_cast<int*>(lsev + kSmallRouteMaxTokens);      // [kSmallRouteMaxTokens * kMaxTopK]
+    int* const cnt = sexp + kSmallRouteMaxTokens * kMaxTopK;                    // [kMaxExperts + 1]
+    int* const off = cnt + (kMaxExperts + 1);                                   // [kMaxExperts + 1]
+    float* const aux_term = reinterpret_cast<float*>(off + (kMaxExperts + 1));  // [kMaxExperts]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -192,7 +202,7 @@ __global__ __launch_bounds__(kSmallThreads) void route_small_kernel(
     // coalesced loads (one round trip to memory instead of one per batch of columns); rows are
     // padded by 8 elements so that the eight pairs a wave works on fall into different banks.
     const int ds = d + 8;
-    const bool staged = (d % 8 == 0) && ((size_t)E * ds * 4 + (size_t)T * ds * sizeof(XT) <= (size_t)kStageBytes) &&
+    const bool staged = (d % 8 == 0) && ((size_t)E * ds * 4 + (size_t)T * ds * sizeof(XT) <= (size_t)STAGE) &&
                         (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(wr) % 16 == 0);
     if (staged) {
         float* ws = reinterpret_cast<float*>(stage);
@@ -465,6 +475,22 @@ __global__ __launch_bounds__(kSmallThreads) void route_small_kernel(
     }
 }
 
+template <typename XT>
+__global__ __launch_bounds__(kSmallThreads) void route_small_kernel(
+    const XT* __restrict__ x, const float* __restrict__ wr, const float* __restrict__ bias,
+    const uint8_t* __restrict__ valid, int T, int d, int E, int k, float w_aux, float w_z, int tile_m,
+    float* __restrict__ P, float* __restrict__ lse, int* __restrict__ expert_of, float* __restrict__ gate_of,
+    int* __restrict__ counts, int* __restrict__ offsets, int* __restrict__ tile_expert,
+    int* __restrict__ tile_row0, int* __restrict__ tile_rows, int* __restrict__ ntiles,
+    float* __restrict__ losses, int* __restrict__ perm_slot, int* __restrict__ perm_token,
+    int* __restrict__ inv_pos, const float* __restrict__ norm_w, float norm_eps, XT* __restrict__ xn_out,
+    bf16_t* __restrict__ rows16) {
+    __shared__ __align__(16) unsigned char smem[kStageBytes + kRouteFixedBytes];
+    route_small_body<XT, kStageBytes>(smem, x, wr, bias, valid, T, d, E, k, w_aux, w_z, tile_m, P, lse, expert_of, gate_of,
+                                      counts, offsets, tile_expert, tile_row0, tile_rows, ntiles, losses, perm_slot,
+                                      perm_token, inv_pos, norm_w, norm_eps, xn_out, rows16);
+}
+
 bool small_route_ok(int T, int E, int k) {
     return T >= 1 && T <= kSmallRouteMaxTokens && E <= kMaxExperts && k <= kMaxTopK &&
            T * E <= kSmallRouteMaxPairs;
@@ -517,17 +543,24 @@ struct DecodeSide {
     const float* scales;
     bf16_t* out;
     int N, K, row0, rows;
+    int a_row0;    // added to a row's number in `a` (rows of one expert inside a per-expert array)
+    int out_row0;  // first output row is out_row0 + row0
 };
 
 // NW = waves of a workgroup, each with 1 / NW of the reduction steps: 4 for the gate/up product, 8 for the
 // down product (a third of the workgroups and twice the reduction length: with 8 waves every weight byte of
 // the launch is requested before the first multiply there as well).
+template <bool SWIGLU, bool I8, int NW, int BATCH>
+__device__ __forceinline__ void decode_gemm_body(const DecodeSide& sd, int fb, float* red_raw);
+
 template <bool SWIGLU, bool I8, int NW>
 __global__ __launch_bounds__(NW * 64) void decode_gemm_kernel(DecodeGemmArgs g) {
-    __shared__ float red[NW][SWIGLU ? 2 : 1][16][64];
+    __shared__ float red[NW * (SWIGLU ? 2 : 1) * 16 * 64];
     const int fb = blockIdx.x;
     const int ty = blockIdx.y;
     DecodeSide sd;
+    sd.a_row0 = 0;
+    sd.out_row0 = 0;
     // One round trip for the whole tile table: the four entries are fetched side by side (a stale entry past
     // *ntiles is read and dropped), not one after the other - with cold caches every dependent scalar load in
     // front of the first weight load is a few hundred nanoseconds of a launch that lasts ten microseconds.
@@ -548,6 +581,7 @@ __global__ __launch_bounds__(NW * 64) void decode_gemm_kernel(DecodeGemmArgs g) 
         sd.K = g.K;
         sd.row0 = t_row0;
         sd.rows = t_rows;
+        sd.a_row0 = expert * g.a_expert_rows;
     } else {
         const int st = ty - g.max_tiles;
         sd.a = static_cast<const bf16_t*>(g.a_shared);
@@ -561,7 +595,13 @@ __global__ __launch_bounds__(NW * 64) void decode_gemm_kernel(DecodeGemmArgs g) 
         sd.rows = min(32, g.T_shared - sd.row0);
     }
     if (fb * 32 >= sd.N) return;
+    decode_gemm_body<SWIGLU, I8, NW, kBatch>(sd, fb, red);
+}
 
+// red_raw: NW * (SWIGLU ? 2 : 1) * 1024 floats of LDS; BATCH: reduction steps whose loads a wave issues together
+template <bool SWIGLU, bool I8, int NW, int BATCH>
+__device__ __forceinline__ void decode_gemm_body(const DecodeSide& sd, int fb, float* red_raw) {
+    float (*red)[SWIGLU ? 2 : 1][16][64] = reinterpret_cast<float (*)[SWIGLU ? 2 : 1][16][64]>(red_raw);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -586,18 +626,18 @@ __global__ __launch_bounds__(NW * 64) void decode_gemm_kernel(DecodeGemmArgs g) 
     };
     // token fragment: lane -> token lane % 32, columns 16 s + 8 (lane / 32) .. + 7
     const int trow = (lane & 31) < sd.rows ? (lane & 31) : 0;
-    int grow = sd.row_index ? sd.row_index[sd.row0 + trow] : sd.row0 + trow;  // awaited after the weight loads
+    int grow = (sd.row_index ? sd.row_index[sd.row0 + trow] : sd.row0 + trow) + sd.a_row0;  // awaited after the weight loads
 
     floatx16 acc0, acc1;
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc0[v] = acc1[v] = 0.0f;
 
-    for (int s0 = g0; s0 < g1; s0 += kBatch) {
-        bf16x8 wa[kBatch], wb[kBatch], tf[kBatch];
+    for (int s0 = g0; s0 < g1; s0 += BATCH) {
+        bf16x8 wa[BATCH], wb[BATCH], tf[BATCH];
         // the weights first: the address of a token row depends on a load of its own (the row index), and
         // loads are issued in order - nothing of the stream may queue up behind that wait
 #pragma unroll
-        for (int u = 0; u < kBatch; ++u) {
+        for (int u = 0; u < BATCH; ++u) {
             const int s = min(s0 + u, g1 - 1);
             wa[u] = wfrag(w0, s);
             if constexpr (SWIGLU) wb[u] = wfrag(w1, s);
@@ -608,13 +648,13 @@ __global__ __launch_bounds__(NW * 64) void decode_gemm_kernel(DecodeGemmArgs g) 
         asm volatile("" : "+v"(grow));
         const bf16_t* arow = sd.a + (size_t)grow * K + 8 * (lane >> 5);
 #pragma unroll
-        for (int u = 0; u < kBatch; ++u) {
+        for (int u = 0; u < BATCH; ++u) {
             const int s = min(s0 + u, g1 - 1);
             tf[u] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(arow + 16 * s));
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int u = 0; u < kBatch; ++u) {
+        for (int u = 0; u < BATCH; ++u) {
             if (s0 + u < g1) {
                 acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wa[u], tf[u], acc0, 0, 0, 0);
                 if constexpr (SWIGLU) acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[u], tf[u], acc1, 0, 0, 0);
@@ -646,8 +686,87 @@ __global__ __launch_bounds__(NW * 64) void decode_gemm_kernel(DecodeGemmArgs g) 
             if constexpr (I8) u *= sd.scales[sd.N + fb * 32 + f];
             y = silu_bf16_grade(y) * u;
         }
-        if (token < sd.rows) sd.out[(size_t)(sd.row0 + token) * sd.N + fb * 32 + f] = from_f32<bf16_t>(y);
+        if (token < sd.rows) sd.out[(size_t)(sd.out_row0 + sd.row0 + token) * sd.N + fb * 32 + f] = from_f32<bf16_t>(y);
     }
+}
+
+// ---------------------------------------------------------------------------
+// decode_front_kernel: the routing and the gate/up products in ONE launch, side by side.
+// The routing is one workgroup walking a dependent chain for about ten microseconds; the gate/up
+// product of a routed expert needs nothing of it but WHICH rows the expert takes.  With at most 32
+// tokens an expert's rows are one tile whatever the routing says, so every expert's gate/up product
+// is taken over ALL the call's rows - hidden rows [E][T, F] - without waiting for the routing: an
+// expert that turns out unrouted costs its weights' bytes (the caller takes this launch only when
+// most experts will be touched), the rows nobody routed to an expert cost nothing (the tile is 32
+// rows either way).  Workgroup 0 routes; workgroup 1 + side * (N / 32) + fb takes feature block fb
+// of side `side`: experts 0 .. E-1, then the shared expert's 32-row blocks.  The down product then
+// picks the routed rows out of the per-expert hidden rows (DecodeGemmArgs::a_expert_rows).
+// ---------------------------------------------------------------------------
+template <bool I8>
+__global__ __launch_bounds__(kSmallThreads, 2) void decode_front_kernel(SmallRouteArgs r, DecodeGemmArgs g, int E, int T) {
+    __shared__ __align__(16) unsigned char smem[kFrontLdsBytes];
+    if (blockIdx.x == 0) {
+        route_small_body<bf16_t, kFrontStageBytes>(
+            smem, static_cast<const bf16_t*>(r.x), r.wr, r.bias, r.valid, r.T, r.d, r.E, r.k, r.w_aux, r.w_z, r.tile_m, r.P,
+            r.lse, r.expert_of, r.gate_of, r.counts, r.offsets, r.tile_expert, r.tile_row0, r.tile_rows, r.ntiles, r.losses,
+            r.perm_slot, r.perm_token, r.inv_pos, nullptr, 0.0f, nullptr, nullptr);
+        return;
+    }
+    const int widest = g.a_shared ? max(g.N, g.N_shared) : g.N;
+    const int nfb = widest / 32;
+    const int idx = blockIdx.x - 1;
+    const int fb = idx % nfb, side = idx / nfb;
+    DecodeSide sd;
+    sd.row_index = nullptr;
+    sd.row0 = 0;
+    sd.a_row0 = 0;
+    if (side < E) {
+        sd.a = static_cast<const bf16_t*>(g.a);
+        sd.w = static_cast<const char*>(g.w) + (size_t)side * g.w_expert_stride * (I8 ? 1 : 2);
+        sd.scales = I8 ? g.scales + (size_t)side * g.s_expert_stride : nullptr;
+        sd.out = static_cast<bf16_t*>(g.out);
+        sd.N = g.N;
+        sd.K = g.K;
+        sd.rows = T;
+        sd.out_row0 = side * T;
+    } else {
+        const int st = side - E;
+        sd.a = static_cast<const bf16_t*>(g.a_shared);
+        sd.w = static_cast<const char*>(g.w_shared);
+        sd.scales = I8 ? g.scales_shared : nullptr;
+        sd.out = static_cast<bf16_t*>(g.out_shared);
+        sd.N = g.N_shared;
+        sd.K = g.K_shared;
+        sd.row0 = st * 32;
+        sd.rows = min(32, g.T_shared - sd.row0);
+        sd.out_row0 = 0;
+    }
+    if (fb * 32 >= sd.N) return;
+    decode_gemm_body<true, I8, kSmallThreads / 64, kBatch / 2>(sd, fb, reinterpret_cast<float*>(smem));
+}
+
+bool decode_front_ok(const void* x, const float* wr, int T, int d, int E, int k) {
+    // the routing workgroup of the fused launch has a smaller staging area; rows that do not fit it are read from
+    // memory piecemeal, which takes longer than the products beside it: not worth it
+    const size_t ds = (size_t)d + 8;
+    const bool staged = d % 8 == 0 && (size_t)E * ds * 4 + (size_t)T * ds * 2 <= (size_t)kFrontStageBytes &&
+                        reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(wr) % 16 == 0;
+    // most experts must be about to be touched: an unrouted expert's gate/up weights are fetched for nothing
+    return staged && T <= 32 && (long long)T * k >= 2LL * E;
+}
+
+hipError_t launch_decode_front(const SmallRouteArgs& r, const DecodeGemmArgs& g, WeightKind wk, hipStream_t s) {
+    if (!small_route_ok(r.T, r.E, r.k) || r.norm_w || r.rows16 || !g.swiglu) return hipErrorInvalidValue;
+    const int shared_tiles = g.a_shared ? (g.T_shared + 31) / 32 : 0;
+    const int widest = g.a_shared ? (g.N > g.N_shared ? g.N : g.N_shared) : g.N;
+    const int grid = 1 + (r.E + shared_tiles) * (widest / 32);
+    if (wk == WeightKind::BF16)
+        hipLaunchKernelGGL(decode_front_kernel<false>, dim3(grid), dim3(kSmallThreads), 0, s, r, g, r.E, r.T);
+    else if (wk == WeightKind::I8)
+        hipLaunchKernelGGL(decode_front_kernel<true>, dim3(grid), dim3(kSmallThreads), 0, s, r, g, r.E, r.T);
+    else
+        return hipErrorInvalidValue;
+    return hipGetLastError();
 }
 
 bool decode_shape_ok(int N, int K) { return K % 32 == 0 && K >= 32 && N % 32 == 0 && N >= 32; }

@@ -166,6 +166,7 @@ struct Work {
     void* y = nullptr;
     void* hs = nullptr;
     void* ys = nullptr;
+    void* hall = nullptr;  // hidden rows of every expert over every row, [E][T, F] (decode_front launches), or null
 };
 
 struct rbmoe_layer {
@@ -185,6 +186,8 @@ struct rbmoe_layer {
     bool cast_rows = false;
     bool use_f32_mc = false;   // all-f32 layer on the f32 matrix cores
     bool decode_path = true;   // few tokens: four launches that stream every touched weight once
+    bool decode_front = true;  // ... three, with the routing beside the gate/up products, when most experts are touched
+    bool last_front = false;   // the last forward's hidden rows are per expert over all rows (Work::hall)
     int group_m = 4, variant = 0;
     const char* kernel_name = "none";
     int last_T = -1;
@@ -202,6 +205,7 @@ struct rbmoe_layer {
     Buf perm_slot, perm_token, inv_pos;
     Buf xg, h, y, hs, ys;
     Buf x16;               // [max_T, d] bf16 copy of f32 rows (cast_rows)
+    Buf hall;              // [E][min(max_T, 32), F] hidden rows of decode_front launches
     // feed-forward norm in front of the layer (allocated by rbmoe_set_feed_forward_norm)
     Buf xn, norm_w;  // [max_T, d] activation dtype, [d] f32
     float norm_eps = 0.0f;
@@ -292,6 +296,8 @@ Plan make_plan(rbmoe_layer* L) {
     p.add(&L->perm_token, S * 4);
     p.add(&L->inv_pos, S * 4);
     if (L->cast_rows) p.add(&L->x16, T * d * 2);
+    // decode_front launches need most experts touched (tokens * k >= 2 E, at most 32 tokens): none when E > 16 k
+    if (L->use_stream && E <= 16 * k) p.add(&L->hall, E * std::min<size_t>(T, kSmallRouteMaxTokens) * F * 2);
     p.add(&L->xg, S * d * as);
     p.add(&L->h, S * F * as);
     p.add(&L->y, S * d * as);
@@ -460,6 +466,7 @@ int rbmoe_layer_create(rbmoe_ctx* ctx, const rbmoe_config* cfg, rbmoe_layer** ou
     L->group_m = std::max(1, env_int("RBMOE_GROUP_M", 4));
     L->variant = env_int("RBMOE_STREAM_VARIANT", 0) == 1 ? 1 : 0;
     L->decode_path = env_int("RBMOE_NO_DECODE_PATH", 0) != 1;
+    L->decode_front = env_int("RBMOE_NO_DECODE_FRONT", 0) != 1;
     // bf16 matrix cores: bf16 activations, bf16 or int8 weights, widths that fit the packed layout
     // (f32 rows with bf16 / int8 weights - what a caller with f32 matrices and a quantized or bf16 checkpoint has -
     // take the same kernels over a bf16 copy of the rows)
@@ -747,6 +754,7 @@ Work work_of_layer(const rbmoe_layer* L) {
     w.ntiles = (int*)L->ntiles.p; w.losses = (float*)L->losses.p;
     w.perm_slot = (int*)L->perm_slot.p; w.perm_token = (int*)L->perm_token.p; w.inv_pos = (int*)L->inv_pos.p;
     w.h = L->h.p; w.y = L->y.p; w.hs = L->hs.p; w.ys = L->ys.p;
+    w.hall = L->hall.p;
     return w;
 }
 
@@ -771,6 +779,7 @@ size_t carve_decode_work(const rbmoe_layer* L, int T, unsigned char* base, Work*
     v.ntiles = (int*)take(8); v.losses = (float*)take(8);
     v.perm_slot = (int*)take(S * 4); v.perm_token = (int*)take(S * 4); v.inv_pos = (int*)take(S * 4);
     v.h = take(S * F * as); v.y = take(S * d * as);
+    if ((size_t)T * k >= 2 * E) v.hall = take(E * (size_t)T * F * 2);  // (the condition of decode_front_ok)
     if (c.shared_expert) {
         v.hs = take((size_t)T * Fs * as);
         v.ys = take((size_t)T * d * as);
@@ -870,6 +879,9 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
             sr.x = norm_src; sr.norm_w = (const float*)L->norm_w.p; sr.norm_eps = L->norm_eps; sr.xn_out = L->xn.p;
         }
         if (cast) sr.rows16 = L->x16.p;
+        // the routing beside the gate/up products, in one launch: bf16 rows as they are (no norm to apply first)
+        const bool front = L->decode_front && !norm_src && !cast && wk_.hall != nullptr &&
+                           decode_front_ok(x, (const float*)L->router.p, T, d, E, k);
         sr.T = T; sr.d = d; sr.E = E; sr.k = k;
         sr.w_aux = c.aux_loss_weight; sr.w_z = c.router_z_loss_weight;
         sr.tile_m = kDecodeTileM;
@@ -879,7 +891,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
         sr.tile_expert = wk_.tile_expert; sr.tile_row0 = wk_.tile_row0; sr.tile_rows = wk_.tile_rows;
         sr.ntiles = wk_.ntiles; sr.losses = wk_.losses;
         sr.perm_slot = wk_.perm_slot; sr.perm_token = wk_.perm_token; sr.inv_pos = wk_.inv_pos;
-        HIP_TRY(ctx, launch_route_small(sr, abf, s));
+        if (!front) HIP_TRY(ctx, launch_route_small(sr, abf, s));
         HIP_TRY(ctx, mark(1));
         HIP_TRY(ctx, mark(2));
         HIP_TRY(ctx, mark(3));
@@ -899,11 +911,20 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
             d1.scales_shared = wk == WeightKind::I8 ? (const float*)L->ssgu.p : nullptr;
             d1.N_shared = Fs; d1.K_shared = d; d1.T_shared = T; d1.out_shared = wk_.hs;
         }
-        HIP_TRY(ctx, launch_decode_gemm(d1, wk, s));
+        if (front) {
+            d1.row_index = nullptr;
+            d1.out = wk_.hall;
+            HIP_TRY(ctx, launch_decode_front(sr, d1, wk, s));
+        } else {
+            HIP_TRY(ctx, launch_decode_gemm(d1, wk, s));
+        }
         HIP_TRY(ctx, mark(4));
 
         DecodeGemmArgs d2 = d1;
         d2.a = wk_.h; d2.row_index = nullptr;
+        if (front) {  // the routed rows are picked out of the per-expert hidden rows: row token of expert e
+            d2.a = wk_.hall; d2.row_index = wk_.perm_token; d2.a_expert_rows = T;
+        }
         d2.w = L->wd.p; d2.w_expert_stride = (size_t)d * F;
         d2.scales = wk == WeightKind::I8 ? (const float*)L->sd.p : nullptr; d2.s_expert_stride = (size_t)d;
         d2.N = d; d2.K = F;
@@ -923,6 +944,9 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
         HIP_TRY(ctx, mark(7));
         L->last_T = T;
         L->last = wk_;
+        L->last_front = front;
+        L->kernel_name = front ? (wk == WeightKind::I8 ? "mfma_bf16_decode_front_int8w" : "mfma_bf16_decode_front")
+                               : L->kernel_name;
         return RBMOE_OK;
     }
 
@@ -1032,6 +1056,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     HIP_TRY(ctx, mark(7));
     L->last_T = T;
     L->last = wk_;
+    L->last_front = false;
     return RBMOE_OK;
 }
 
@@ -1642,7 +1667,22 @@ int rbmoe_get_expert_rows(rbmoe_layer* L, float* hidden, float* expert_out) {
         for (size_t i = 0; i < n; ++i) dst[i] = host_bf16_to_f32(tmp[i]);
         return RBMOE_OK;
     };
-    int rc = fetch(hidden, L->last.h, (size_t)R * F);
+    int rc = RBMOE_OK;
+    if (L->last_front && hidden && R > 0) {
+        // the hidden rows lie per expert over all the call's rows: pick the routed ones, in permuted order
+        const int T = L->last_T;
+        std::vector<float> all((size_t)E * T * F);
+        std::vector<int> offs(E + 1), ptok(R);
+        rc = fetch(all.data(), L->last.hall, all.size());
+        if (rc != RBMOE_OK) return rc;
+        HIP_TRY(ctx, hipMemcpy(offs.data(), L->last.offsets, (size_t)(E + 1) * 4, hipMemcpyDeviceToHost));
+        HIP_TRY(ctx, hipMemcpy(ptok.data(), L->last.perm_token, (size_t)R * 4, hipMemcpyDeviceToHost));
+        for (int e = 0; e < E; ++e)
+            for (int pos = offs[e]; pos < offs[e + 1]; ++pos)
+                std::memcpy(hidden + (size_t)pos * F, all.data() + ((size_t)e * T + ptok[pos]) * F, (size_t)F * 4);
+    } else {
+        rc = fetch(hidden, L->last.h, (size_t)R * F);
+    }
     if (rc != RBMOE_OK) return rc;
     return fetch(expert_out, L->last.y, (size_t)R * d);
 }

@@ -229,6 +229,7 @@ struct DecodeGemmArgs {
     const int* ntiles;
     int max_tiles;
     void* out;
+    int a_expert_rows = 0;  // rows of `a` per expert: a routed row r of expert e is a[e * a_expert_rows + row]
     const void* a_shared;
     const void* w_shared;
     const float* scales_shared;
@@ -238,6 +239,10 @@ struct DecodeGemmArgs {
 };
 bool decode_shape_ok(int N, int K);
 hipError_t launch_decode_gemm(const DecodeGemmArgs& g, WeightKind wk, hipStream_t s);
+// Routing and gate/up products in one launch (bf16 rows, no norm): every expert's gate/up product over all T rows,
+// hidden rows to g.out as [E][T, N]; the shared expert as in launch_decode_gemm.  g.a / g.a_shared: the T rows.
+bool decode_front_ok(const void* x, const float* wr, int T, int d, int E, int k);
+hipError_t launch_decode_front(const SmallRouteArgs& r, const DecodeGemmArgs& g, WeightKind wk, hipStream_t s);
 
 // ---- calibration (calibrate.hip): what the device sustains, for the roofline figures to be read against ----
 // 4 waves per workgroup, each issuing steps * 8 independent 32x32x16 bf16 multiplies; out: workgroups * 256 floats

@@ -15,12 +15,14 @@ pytestmark = pytest.mark.gpu
 
 @pytest.fixture
 def env():
-    saved = os.environ.get("RBMOE_NO_DECODE_PATH")
+    keys = ("RBMOE_NO_DECODE_PATH", "RBMOE_NO_DECODE_FRONT")
+    saved = {k: os.environ.get(k) for k in keys}
     yield os.environ
-    if saved is None:
-        os.environ.pop("RBMOE_NO_DECODE_PATH", None)
-    else:
-        os.environ["RBMOE_NO_DECODE_PATH"] = saved
+    for k, v in saved.items():
+        if v is None:
+            os.environ.pop(k, None)
+        else:
+            os.environ[k] = v
 
 
 def run(device, t, valid=None, bias=None, residual=None):
@@ -109,7 +111,7 @@ def test_decode_and_large_batch_paths_agree(device, env):
     env.pop("RBMOE_NO_DECODE_PATH", None)
     small = gpu_layer(device, t)
     out_s, cache_s = small.forward_train(t.x)
-    assert small.kernel_name() == "mfma_bf16_decode"
+    assert small.kernel_name() == "mfma_bf16_decode_front"   # 48 slots on 8 experts: routing beside the gate/up products
     env["RBMOE_NO_DECODE_PATH"] = "1"
     large = gpu_layer(device, t)
     out_l, cache_l = large.forward_train(t.x)
@@ -121,3 +123,33 @@ def test_decode_and_large_batch_paths_agree(device, env):
     assert rel_l2(out_s, out_l) <= 5e-3
     small.close()
     large.close()
+
+
+@pytest.mark.parametrize("wt", ["bf16", "int8"])
+def test_routing_beside_the_products_changes_nothing_but_the_launch_count(device, env, wt):
+    # When most experts are about to be touched (tokens * k >= 2 E) the routing workgroup runs in the same launch as
+    # the gate/up products, which are then taken for every expert over every row; the routing tables are the same
+    # bits, the routed hidden rows and outputs the same within the reduction order of the products (8 waves
+    # split the reduction there, 4 in the product launch of its own).
+    shape = dict(d=256, E=8, k=2, F=192, T=11)
+    t = synth.make(small_workload(seed=41, act="bf16", wt=wt, shared=True, shared_d_ff=128, **shape))
+    valid = (np.arange(11) % 5 != 3).astype(np.uint8)
+    bias = synth.normal((8,), 0.5, 41, 98)
+    env.pop("RBMOE_NO_DECODE_PATH", None)
+    env.pop("RBMOE_NO_DECODE_FRONT", None)
+    name_f, out_f, cache_f = run(device, t, valid=valid, bias=bias)
+    assert name_f.startswith("mfma_bf16_decode_front")
+    env["RBMOE_NO_DECODE_FRONT"] = "1"
+    name_p, out_p, cache_p = run(device, t, valid=valid, bias=bias)
+    assert name_p.startswith("mfma_bf16_decode") and "front" not in name_p
+    for f in ("expert_of", "counts", "offsets", "perm_slot", "perm_token"):
+        assert np.array_equal(getattr(cache_f, f), getattr(cache_p, f)), f
+    assert np.array_equal(cache_f.probabilities.view(np.uint32), cache_p.probabilities.view(np.uint32))
+    assert np.array_equal(cache_f.gate_of.view(np.uint32), cache_p.gate_of.view(np.uint32))
+    assert cache_f.aux_loss() == cache_p.aux_loss() and cache_f.z_loss() == cache_p.z_loss()
+    assert rel_l2(out_f, out_p) <= 5e-3
+    # few slots on many experts: the launches stay apart (an unrouted expert's weights would be fetched for nothing)
+    t = synth.make(small_workload(seed=41, act="bf16", wt=wt, d=64, E=16, k=2, F=64, T=4))
+    env.pop("RBMOE_NO_DECODE_FRONT", None)
+    name, _, _ = run(device, t)
+    assert name.startswith("mfma_bf16_decode") and "front" not in name
