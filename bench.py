@@ -215,6 +215,41 @@ def backward_leg(dev, w, t, x, out, bp, args, alg, with_cpu: bool) -> dict:
     return res
 
 
+class ForwardGraph:
+    """One forward captured into a HIP graph on a stream of its own (the entry points that take device pointers only
+    enqueue kernels, so they can be captured); a replay is one step without the host's launch calls."""
+
+    def __init__(self, dev, enqueue):
+        self.hip = C.CDLL("libamdhip64.so")
+        self.dev = dev
+        self.stream, self.graph, self.exe = C.c_void_p(), C.c_void_p(), C.c_void_p()
+        self._ck(self.hip.hipStreamCreateWithFlags(C.byref(self.stream), 1), "hipStreamCreateWithFlags")
+        dev.synchronize()
+        dev.set_stream(self.stream.value)
+        self._ck(self.hip.hipStreamBeginCapture(self.stream, 0), "hipStreamBeginCapture")
+        enqueue()
+        self._ck(self.hip.hipStreamEndCapture(self.stream, C.byref(self.graph)), "hipStreamEndCapture")
+        self._ck(self.hip.hipGraphInstantiate(C.byref(self.exe), self.graph, None, None, 0), "hipGraphInstantiate")
+
+    @staticmethod
+    def _ck(rc, what):
+        if rc != 0:
+            raise RuntimeError(f"{what} failed with hipError {rc}")
+
+    def replay(self):
+        self._ck(self.hip.hipGraphLaunch(self.exe, self.stream), "hipGraphLaunch")
+
+    def synchronize(self):
+        self._ck(self.hip.hipStreamSynchronize(self.stream), "hipStreamSynchronize")
+
+    def close(self):
+        self.synchronize()
+        self.dev.set_stream(None)
+        self.hip.hipGraphExecDestroy(self.exe)
+        self.hip.hipGraphDestroy(self.graph)
+        self.hip.hipStreamDestroy(self.stream)
+
+
 def measure(dev, name: str, steps: int, warmup: int, repeats: int, act_override: str = None) -> dict:
     """One workload: `repeats` loops of `steps` forwards (median loop -> ms_per_step), per-stage durations from HIP
     events on the library's stream, the roofline of the dominant kernel.  Returns the pieces the report is built of."""
@@ -247,6 +282,23 @@ def measure(dev, name: str, steps: int, warmup: int, repeats: int, act_override:
     ms_per_step = float(np.median(loops))
 
     decode = "decode" in layer.kernel_name()   # the library takes the decode-shaped kernels up to 32 tokens
+    graph_ms = None
+    if decode:
+        # A decode step is three short launches: issued one by one from this interpreter, the host's launch calls
+        # are part of the step.  The same forward replayed from a HIP graph, timed the same way:
+        g = ForwardGraph(dev, lambda: layer.forward_device(x.ptr, T, out.ptr, bias_ptr=bp))
+        for _ in range(warmup):
+            g.replay()
+        g.synchronize()
+        gl = []
+        for _ in range(repeats):
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                g.replay()
+            g.synchronize()
+            gl.append((time.perf_counter() - t0) * 1e3 / steps)
+        g.close()
+        graph_ms = float(np.median(gl))
     nprof = max(10, min(100, steps))
 
     def timed_stages(flush=None):
@@ -344,7 +396,7 @@ def measure(dev, name: str, steps: int, warmup: int, repeats: int, act_override:
               "seed": w.seed, "expert0_share": float(cache.load_fractions()[0]), "routed_slots": routed}
     return {"w": w, "t": t, "layer": layer, "x": x, "out": out, "bias": bias, "bp": bp, "alg": alg,
             "ms_per_step": ms_per_step, "loops_ms": loops, "roofline": roofline, "stages": stages, "config": config,
-            "bf16": bf16, "decode": decode}
+            "bf16": bf16, "decode": decode, "graph_ms": graph_ms}
 
 
 def release(m: dict) -> None:
@@ -368,7 +420,8 @@ def summary(m: dict) -> dict:
                            "whole_layer_ms": st["cold_whole_layer_ms"],
                            "whole_layer_frac_of_hbm": st["cold_whole_layer_frac_of_hbm"]},
                   "warm": {"gate_up_gbs": r["cache_resident_gbs"], "whole_layer_ms": m["ms_per_step"],
-                           "whole_layer_gbs": st["cache_resident_whole_layer_gbs"]}})
+                           "whole_layer_gbs": st["cache_resident_whole_layer_gbs"],
+                           "whole_layer_ms_graph_replay": m["graph_ms"]}})
     return s
 
 
@@ -408,6 +461,8 @@ def main() -> int:
         "vs_baseline": None, "dtype": "bf16" if w.weight_dtype != "f32" else "f32", "data": "synthetic",
         "config": m["config"], "roofline": m["roofline"], "stages": m["stages"],
     }
+    if m["graph_ms"] is not None:
+        result["ms_per_step_graph_replay"] = m["graph_ms"]
     if args.calibrate_copy:
         n = 256 << 20
         a, b = DeviceBuffer(dev, n), DeviceBuffer(dev, n)
