@@ -223,7 +223,9 @@ struct rbmoe_layer {
     Buf grad_gates, ones, dlogits, dxr, rpartial;
     Buf g_router, g_gu, g_down, g_sgu, g_sdown;   // f32 weight gradients, accumulated
     Buf wg_chunks;                        // chunk table of the weight-gradient products
-    bool wgrad_generic = false, wgrad_split = true, side_branch = true;
+    Buf wg_partial;                       // partial matrices of cut experts (ordered accumulation)
+    bool wgrad_generic = false, side_branch = true;
+    WgradSplit wgrad_split = WgradSplit::Ordered;
     // The expert gradients count as zero without having been cleared (set by rbmoe_zero_grads): the next
     // backward pass overwrites them.
     bool grads_clear = false;
@@ -1317,7 +1319,21 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
     p.add(&L->g_down, E * d * F * 4);
     p.add(&L->wdT, E * F * d * ws);
     p.add(&L->wguT, E * d * 2 * F * ws);
-    p.add(&L->wg_chunks, (size_t)(4 * std::max(weight_grad_max_chunks((int)E, (int)S), weight_grad_max_chunks(1, (int)T)) + 1) * 4);
+    p.add(&L->wg_chunks, (size_t)std::max(weight_grad_table_ints((int)E, (int)S), weight_grad_table_ints(1, (int)T)) * 4);
+    // How the weight gradients treat an expert far above the average share (and the shared expert, whose one
+    // group of rows is always cut): in a fixed order by default, RBMOE_ATOMIC_WGRAD=1 for f32 atomics,
+    // RBMOE_DETERMINISTIC=1 for no cut at all.
+    L->wgrad_split = env_int("RBMOE_DETERMINISTIC", 0) == 1 ? WgradSplit::None
+                     : env_int("RBMOE_ATOMIC_WGRAD", 0) == 1 ? WgradSplit::Atomic : WgradSplit::Ordered;
+    if (L->wgrad_split == WgradSplit::Ordered) {
+        const bool wbf = c.act_dtype == RBMOE_BF16;
+        size_t need = std::max(weight_grad_partial_bytes((int)d, (int)F, (int)E, -1, (int)S, wbf),
+                               weight_grad_partial_bytes((int)(2 * F), (int)d, (int)E, -1, (int)S, wbf));
+        if (c.shared_expert)
+            need = std::max(need, std::max(weight_grad_partial_bytes((int)d, (int)Fs, 1, (int)T, (int)T, wbf),
+                                           weight_grad_partial_bytes((int)(2 * Fs), (int)d, 1, (int)T, (int)T, wbf)));
+        p.add(&L->wg_partial, need);
+    }
     p.add(&L->st_gout, T * d * as);
     p.add(&L->st_gin, T * d * as);
     if (c.shared_expert) {
@@ -1333,7 +1349,6 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
     HIP_TRY(ctx, launch_fill_f32((float*)L->ones.p, 1.0f, (long long)S, ctx->stream));
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
     L->wgrad_generic = env_int("RBMOE_WGRAD_GENERIC", 0) == 1;
-    L->wgrad_split = env_int("RBMOE_DETERMINISTIC", 0) != 1;
     L->side_branch = env_int("RBMOE_NO_SIDE_STREAM", 0) != 1;
     if (L->side_branch && !ctx->side_stream) {
         HIP_TRY(ctx, hipStreamCreateWithFlags(&ctx->side_stream, hipStreamNonBlocking));
@@ -1457,7 +1472,8 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, int32_t tokens, int3
                      int total_rows, float* out, size_t stride) -> hipError_t {
         if (!L->wgrad_generic && !b_rows && weight_grad_shape_ok(M, N, abf))
             return launch_weight_grad(a, M, b, N, counts, offsets, groups, dense_rows, total_rows,
-                                      L->wgrad_split, L->grads_clear, (int*)L->wg_chunks.p, out, stride, abf, s);
+                                      L->wgrad_split, L->grads_clear, (int*)L->wg_chunks.p, (float*)L->wg_partial.p,
+                                      L->wg_partial.bytes, out, stride, abf, s);
         if (L->grads_clear) {
             const hipError_t e = launch_fill_f32(out, 0.0f, (long long)((size_t)groups * (stride ? stride : (size_t)M * N)), s);
             if (e != hipSuccess) return e;

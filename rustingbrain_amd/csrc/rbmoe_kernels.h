@@ -145,14 +145,22 @@ hipError_t launch_grouped_tn(const void* a, int M, const void* b, const int* b_r
                              bool bf16, hipStream_t s);
 
 // Weight gradients on the matrix cores (bf16 or f32 operands): out[e] += A_e^T . B_e with the rows of a group cut into
-// chunks (`allow_split`: an expert far above the average share is cut into several chunks, which
-// then add with f32 atomics; `overwrite`: out is known to hold zeros, whatever its bytes are, and is
-// written instead of added to).  `chunks` is scratch of 4 * weight_grad_max_chunks(...) + 1 ints.
+// chunks.  How an expert far above the average share is handled:
+//   None     one chunk per expert (a skewed load then serialises the launch)
+//   Ordered  cut into several chunks; the first adds in place, the others store partial matrices (`partial`) that
+//            a second kernel adds in chunk order: identical bits run to run
+//   Atomic   cut into several chunks that all add with f32 atomics, in whatever order they arrive
+// `overwrite`: out is known to hold zeros, whatever its bytes are, and is written instead of added to.
+// `chunks` is scratch of weight_grad_table_ints(...) ints, `partial` of weight_grad_partial_bytes(...) bytes.
+enum class WgradSplit : int { None = 0, Ordered = 1, Atomic = 2 };
 bool weight_grad_shape_ok(int M, int N, bool bf16);
 int weight_grad_max_chunks(int groups, int total_rows);
+int weight_grad_table_ints(int groups, int total_rows);
+size_t weight_grad_partial_bytes(int M, int N, int groups, int dense_rows, int total_rows, bool bf16);
 hipError_t launch_weight_grad(const void* a, int M, const void* b, int N, const int* counts, const int* offsets,
-                              int groups, int dense_rows, int total_rows, bool allow_split, bool overwrite, int* chunks,
-                              float* out, size_t out_expert_stride, bool bf16, hipStream_t s);
+                              int groups, int dense_rows, int total_rows, WgradSplit split_mode, bool overwrite,
+                              int* chunks, float* partial, size_t partial_bytes, float* out, size_t out_expert_stride,
+                              bool bf16, hipStream_t s);
 
 // gates -> probabilities -> logits, with the gradients of the two auxiliary losses
 hipError_t launch_route_backward(const float* P, const float* lse, const int* expert_of, const float* grad_gates,

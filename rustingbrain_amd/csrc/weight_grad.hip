@@ -16,11 +16,14 @@
 // a wave owns 64 x 128 (2 x 4 accumulator blocks of 32 x 32).  Rows go through LDS 32 at a
 // time, double buffered; the global loads run three stages ahead in three register sets, so a
 // load has two full stages of products to arrive in.  An expert with many more rows than the
-// others is cut into several chunks so that the launch stays balanced; chunks of one expert add
-// into the same matrix with hardware f32 atomics (their order is not fixed; an expert with a
-// single chunk adds in place, in one fixed order).  When the caller knows that the gradient is
-// zero (first backward pass after it was cleared), a single chunk stores instead of adding, and
-// only the experts that have no chunk or several are cleared beforehand.
+// others is cut into several chunks so that the launch stays balanced.  The sums of a cut expert's
+// chunks meet in a fixed order (the reference's convention for reductions, src/norm.rs:8-14): the first
+// chunk adds in place like an expert's only chunk, every further chunk stores its tile sums into a
+// partial matrix of its own, and a second kernel adds the partial matrices to the gradient in chunk
+// order - two runs give identical bits.  (Opt-in alternative: the chunks add into the gradient with
+// hardware f32 atomics, in whatever order they arrive.)  When the caller knows that the gradient is
+// zero (first backward pass after it was cleared), a first chunk stores instead of adding, and only
+// the experts without rows are cleared beforehand.
 #include "rbmoe_kernels.h"
 
 namespace rbmoe {
@@ -54,9 +57,13 @@ __device__ __forceinline__ bf16x8 tr_fragment(const char* p, int pitch) {
 // elements: it reads the 16 values of a block, adds, and stores (M is a multiple of 4, so a group of 4
 // rows is inside or outside as a whole) - or just stores when the gradient is known to be zero.  The chunks
 // of a cut expert meet on the same elements and add with no-return f32 atomics.
+// mode: 0 = add in place (or store when `overwrite`), 1 = atomic add, 2 = plain store (`o` is then the chunk's
+// partial matrix).
 template <int NI, int NJ>
 __device__ __forceinline__ void add_tiles(const floatx16 (&acc)[NI][NJ], float* __restrict__ o, int M, int N, int mw,
-                                          int nw, int lane, bool split, bool overwrite) {
+                                          int nw, int lane, int mode, bool overwrite) {
+    const bool split = mode == 1;
+    overwrite = overwrite || mode == 2;
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
         const int mb = mw + i * 32 + 4 * (lane >> 5);
@@ -92,16 +99,21 @@ __device__ __forceinline__ void add_tiles(const floatx16 (&acc)[NI][NJ], float* 
 }
 
 // chunk table: expert e with c rows gets ceil(c / limit) chunks of equal size (a multiple of 32)
+// chunk_split[c]: 0 = the expert's only or first chunk (adds in place), 1 = adds with atomics (`ordered` off),
+// 2 + s = stores into partial matrix s; slot_first[e] / slot_count[e]: the partial matrices of expert e, in chunk order
 __global__ __launch_bounds__(256) void chunk_table_kernel(const int* __restrict__ counts,
                                                           const int* __restrict__ offsets, int groups,
-                                                          int dense_rows, int limit, int max_chunks,
+                                                          int dense_rows, int limit, int max_chunks, int ordered,
+                                                          int max_slots,
                                                           int* __restrict__ chunk_expert, int* __restrict__ chunk_row0,
                                                           int* __restrict__ chunk_rows, int* __restrict__ chunk_split,
-                                                          int* __restrict__ nchunks) {
+                                                          int* __restrict__ nchunks, int* __restrict__ slot_first,
+                                                          int* __restrict__ slot_count) {
     __shared__ int scan[256];
-    __shared__ int base;
+    __shared__ int scan_x[256];
+    __shared__ int base, base_x;
     const int tid = threadIdx.x;
-    if (tid == 0) base = 0;
+    if (tid == 0) base = base_x = 0;
     __syncthreads();
     for (int e0 = 0; e0 < groups; e0 += 256) {
         const int e = e0 + tid;
@@ -111,15 +123,26 @@ __global__ __launch_bounds__(256) void chunk_table_kernel(const int* __restrict_
             row0 = dense_rows >= 0 ? 0 : offsets[e];
         }
         const int n = rows > 0 ? (rows + limit - 1) / limit : 0;
+        const int nx = n > 1 ? n - 1 : 0;  // chunks beyond the first
         scan[tid] = n;
+        scan_x[tid] = nx;
         __syncthreads();
         for (int o = 1; o < 256; o <<= 1) {
             const int v = tid >= o ? scan[tid - o] : 0;
+            const int vx = tid >= o ? scan_x[tid - o] : 0;
             __syncthreads();
             scan[tid] += v;
+            scan_x[tid] += vx;
             __syncthreads();
         }
         const int first = base + scan[tid] - n;
+        const int first_x = base_x + scan_x[tid] - nx;
+        if (e < groups) {
+            // (more partial matrices than there is room for cannot happen: the launcher sizes the limit for it;
+            // should it, the surplus chunks are dropped from the count here and their rows are not added)
+            slot_first[e] = first_x;
+            slot_count[e] = ordered ? max(0, min(nx, max_slots - first_x)) : 0;
+        }
         if (n > 0) {
             const int per = (((rows + n - 1) / n) + 31) & ~31;
             for (int c = 0; c < n; ++c) {
@@ -128,8 +151,9 @@ __global__ __launch_bounds__(256) void chunk_table_kernel(const int* __restrict_
                 if (first + c < max_chunks && r > 0) {
                     chunk_expert[first + c] = e;
                     chunk_row0[first + c] = row0 + r0;
-                    chunk_rows[first + c] = r;
-                    chunk_split[first + c] = n > 1;
+                    const bool room = !ordered || c == 0 || first_x + c - 1 < max_slots;
+                    chunk_rows[first + c] = room ? r : 0;
+                    chunk_split[first + c] = !ordered ? (n > 1) : (c == 0 ? 0 : 2 + first_x + c - 1);
                 } else if (first + c < max_chunks) {
                     chunk_expert[first + c] = e;
                     chunk_row0[first + c] = row0;
@@ -139,17 +163,39 @@ __global__ __launch_bounds__(256) void chunk_table_kernel(const int* __restrict_
             }
         }
         __syncthreads();
-        if (tid == 255) base += scan[255];
+        if (tid == 255) {
+            base += scan[255];
+            base_x += scan_x[255];
+        }
         __syncthreads();
     }
     if (tid == 0) *nchunks = min(base, max_chunks);
+}
+
+// out[e] += partial[slot_first[e]] + partial[slot_first[e] + 1] + ... in that order, element by element
+__global__ __launch_bounds__(256) void add_partials_kernel(const int* __restrict__ slot_first,
+                                                           const int* __restrict__ slot_count,
+                                                           const float* __restrict__ partial, size_t elems,
+                                                           float* __restrict__ out, size_t out_expert_stride) {
+    const int e = blockIdx.y;
+    const int ns = slot_count[e];
+    if (ns <= 0) return;
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    const f32x4* const p = reinterpret_cast<const f32x4*>(partial + (size_t)slot_first[e] * elems);
+    f32x4* const o = reinterpret_cast<f32x4*>(out + (size_t)e * out_expert_stride);
+    const size_t n4 = elems / 4;  // M and N are multiples of 4
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (size_t)gridDim.x * 256) {
+        f32x4 v = o[i];
+        for (int s = 0; s < ns; ++s) v += __builtin_nontemporal_load(p + (size_t)s * n4 + i);  // read once
+        o[i] = v;
+    }
 }
 
 __global__ __launch_bounds__(GT) void weight_grad_kernel(
     const bf16_t* __restrict__ a, int M, const bf16_t* __restrict__ b, int N, int tiles_m, int tiles_n,
     const int* __restrict__ chunk_expert, const int* __restrict__ chunk_row0, const int* __restrict__ chunk_rows,
     const int* __restrict__ chunk_split, const int* __restrict__ nchunks, float* __restrict__ out,
-    size_t out_expert_stride, int overwrite) {
+    size_t out_expert_stride, int overwrite, float* __restrict__ partial) {
     extern __shared__ __attribute__((aligned(16))) char lds[];  // 2 * GSTAGE
 
     // Workgroup i runs on XCD i % 8.  A unit is one chunk's row of tiles (same m, every n): its
@@ -164,8 +210,9 @@ __global__ __launch_bounds__(GT) void weight_grad_kernel(
     const int rows = chunk_rows[ch];
     if (rows <= 0) return;
     const int row0 = chunk_row0[ch];
-    const bool split = chunk_split[ch] != 0;
-    float* const o = out + (size_t)chunk_expert[ch] * out_expert_stride;
+    const int cs = chunk_split[ch];
+    const int mode = cs >= 2 ? 2 : cs;
+    float* const o = cs >= 2 ? partial + (size_t)(cs - 2) * M * N : out + (size_t)chunk_expert[ch] * out_expert_stride;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
@@ -262,7 +309,7 @@ __global__ __launch_bounds__(GT) void weight_grad_kernel(
         step(I2{}, s + 2);
     }
 
-    add_tiles<2, 4>(acc, o, M, N, m0 + wm * 64, n0 + wn * 128, lane, split, overwrite != 0);
+    add_tiles<2, 4>(acc, o, M, N, m0 + wm * 64, n0 + wn * 128, lane, mode, overwrite != 0);
 }
 
 // ---------------------------------------------------------------------------
@@ -280,7 +327,7 @@ __global__ __launch_bounds__(FT, 2) void weight_grad_f32_kernel(
     const float* __restrict__ a, int M, const float* __restrict__ b, int N, int tiles_m, int tiles_n,
     const int* __restrict__ chunk_expert, const int* __restrict__ chunk_row0, const int* __restrict__ chunk_rows,
     const int* __restrict__ chunk_split, const int* __restrict__ nchunks, float* __restrict__ out,
-    size_t out_expert_stride, int overwrite) {
+    size_t out_expert_stride, int overwrite, float* __restrict__ partial) {
     __shared__ __attribute__((aligned(16))) float lds[2 * FSTAGE];  // 40 KB
 
     const int idx = (int)(blockIdx.x >> 3);
@@ -291,8 +338,9 @@ __global__ __launch_bounds__(FT, 2) void weight_grad_f32_kernel(
     const int rows = chunk_rows[ch];
     if (rows <= 0) return;
     const int row0 = chunk_row0[ch];
-    const bool split = chunk_split[ch] != 0;
-    float* const o = out + (size_t)chunk_expert[ch] * out_expert_stride;
+    const int cs = chunk_split[ch];
+    const int mode = cs >= 2 ? 2 : cs;
+    float* const o = cs >= 2 ? partial + (size_t)(cs - 2) * M * N : out + (size_t)chunk_expert[ch] * out_expert_stride;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
@@ -373,17 +421,17 @@ __global__ __launch_bounds__(FT, 2) void weight_grad_f32_kernel(
         step(I1{}, s + 1);
         step(I2{}, s + 2);
     }
-    add_tiles<2, 2>(acc, o, M, N, m0 + wm * 64, n0 + wn * 64, lane, split, overwrite != 0);
+    add_tiles<2, 2>(acc, o, M, N, m0 + wm * 64, n0 + wn * 64, lane, mode, overwrite != 0);
 }
 
 // Overwrite mode: an expert with exactly one chunk is written in full by that chunk's tiles; every
 // other expert (no rows, or cut into chunks that add atomically) is cleared here first.
 __global__ __launch_bounds__(256) void clear_other_experts_kernel(const int* __restrict__ counts, int dense_rows,
-                                                                  int limit, float* __restrict__ out,
+                                                                  int limit, int ordered, float* __restrict__ out,
                                                                   size_t out_expert_stride, size_t elems) {
     const int e = blockIdx.y;
     const int rows = dense_rows >= 0 ? dense_rows : counts[e];
-    if (rows > 0 && rows <= limit) return;  // exactly one chunk
+    if (rows > 0 && (rows <= limit || ordered)) return;  // a chunk that stores: the only one, or the first of an ordered cut
     float4* const o = reinterpret_cast<float4*>(out + (size_t)e * out_expert_stride);
     const size_t n4 = elems / 4;  // M and N are multiples of 4
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (size_t)gridDim.x * 256)
@@ -397,12 +445,34 @@ bool weight_grad_shape_ok(int M, int N, bool bf16) {
     return M % q == 0 && N % q == 0 && M >= q && N >= q;
 }
 
-// Upper bound of the number of chunks of one launch; `chunks` needs 4 * bound + 1 ints.
+// Upper bound of the number of chunks of one launch; `chunks` needs weight_grad_table_ints(...) ints.
 int weight_grad_max_chunks(int groups, int total_rows) { return groups + total_rows / 256 + 1; }
+int weight_grad_table_ints(int groups, int total_rows) { return 4 * weight_grad_max_chunks(groups, total_rows) + 1 + 2 * groups; }
+
+namespace {
+// rows above which an expert is cut: enough (chunk, tile) pairs to fill the chip twice, and no chunk longer than
+// twice the average expert's share (a cut costs a partial matrix per further chunk)
+int cut_limit(int M, int N, int groups, int dense_rows, int total_rows, bool bf16) {
+    const int tile_m = bf16 ? GM : FM, tile_n = bf16 ? GN : FN;
+    const int tiles = ((M + tile_m - 1) / tile_m) * ((N + tile_n - 1) / tile_n);
+    const int want = std::max(groups, (512 + tiles - 1) / tiles);
+    const int share = (total_rows + want - 1) / want;
+    return std::max(256, ((dense_rows >= 0 ? share : 2 * share) + 31) & ~31);
+}
+}  // namespace
+
+// Partial matrices an ordered launch may need: every further chunk of a cut expert has one; there are at most
+// total_rows / limit of them.
+size_t weight_grad_partial_bytes(int M, int N, int groups, int dense_rows, int total_rows, bool bf16) {
+    if (groups <= 0 || total_rows <= 0) return 0;
+    const int limit = cut_limit(M, N, groups, dense_rows, total_rows, bf16);
+    return (size_t)(total_rows / limit + 1) * M * N * sizeof(float);
+}
 
 hipError_t launch_weight_grad(const void* a, int M, const void* b, int N, const int* counts, const int* offsets,
-                              int groups, int dense_rows, int total_rows, bool allow_split, bool overwrite, int* chunks,
-                              float* out, size_t out_expert_stride, bool bf16, hipStream_t s) {
+                              int groups, int dense_rows, int total_rows, WgradSplit split_mode, bool overwrite,
+                              int* chunks, float* partial, size_t partial_bytes, float* out, size_t out_expert_stride,
+                              bool bf16, hipStream_t s) {
     if (groups <= 0 || total_rows <= 0) return hipSuccess;
     if (!weight_grad_shape_ok(M, N, bf16)) return hipErrorInvalidValue;
     if (bf16) {
@@ -412,15 +482,16 @@ hipError_t launch_weight_grad(const void* a, int M, const void* b, int N, const 
     }
     const int tile_m = bf16 ? GM : FM, tile_n = bf16 ? GN : FN;
     const int tiles_m = (M + tile_m - 1) / tile_m, tiles_n = (N + tile_n - 1) / tile_n;
-    const int tiles = tiles_m * tiles_n;
-    // Enough (chunk, tile) pairs to fill the chip twice, and no chunk longer than twice the average
-    // expert's share: an expert above that is cut into equal pieces (the cut costs atomics, which
-    // are several times slower than the read-add-store of an expert's only chunk).
-    int limit = 1 << 30;
-    if (allow_split) {
-        const int want = std::max(groups, (512 + tiles - 1) / tiles);
-        const int share = (total_rows + want - 1) / want;
-        limit = std::max(256, ((dense_rows >= 0 ? share : 2 * share) + 31) & ~31);
+    int limit = 1 << 30;  // WgradSplit::None: an expert is one chunk, whatever its share
+    int max_slots = 0;
+    bool ordered = false;
+    if (split_mode != WgradSplit::None) {
+        limit = cut_limit(M, N, groups, dense_rows, total_rows, bf16);
+        if (split_mode == WgradSplit::Ordered) {
+            ordered = true;
+            max_slots = (int)(partial_bytes / ((size_t)M * N * sizeof(float)));
+            if (partial == nullptr || max_slots < total_rows / limit + 1) return hipErrorInvalidValue;
+        }
     }
     const int max_chunks = weight_grad_max_chunks(groups, total_rows);
     int* const chunk_expert = chunks;
@@ -428,20 +499,26 @@ hipError_t launch_weight_grad(const void* a, int M, const void* b, int N, const 
     int* const chunk_rows = chunks + 2 * max_chunks;
     int* const chunk_split = chunks + 3 * max_chunks;
     int* const nchunks = chunks + 4 * max_chunks;
+    int* const slot_first = nchunks + 1;
+    int* const slot_count = slot_first + groups;
     hipLaunchKernelGGL(chunk_table_kernel, dim3(1), dim3(256), 0, s, counts, offsets, groups, dense_rows, limit,
-                       max_chunks, chunk_expert, chunk_row0, chunk_rows, chunk_split, nchunks);
+                       max_chunks, ordered ? 1 : 0, max_slots, chunk_expert, chunk_row0, chunk_rows, chunk_split, nchunks,
+                       slot_first, slot_count);
     if (overwrite)
-        hipLaunchKernelGGL(clear_other_experts_kernel, dim3(64, groups), dim3(256), 0, s, counts, dense_rows, limit, out,
-                           out_expert_stride, (size_t)M * N);
+        hipLaunchKernelGGL(clear_other_experts_kernel, dim3(64, groups), dim3(256), 0, s, counts, dense_rows, limit,
+                           ordered ? 1 : 0, out, out_expert_stride, (size_t)M * N);
     const int grid = ((max_chunks * tiles_m + 7) / 8) * 8 * tiles_n;
     if (bf16)
         hipLaunchKernelGGL(weight_grad_kernel, dim3(grid), dim3(GT), 2 * GSTAGE, s, static_cast<const bf16_t*>(a), M,
                            static_cast<const bf16_t*>(b), N, tiles_m, tiles_n, chunk_expert, chunk_row0, chunk_rows,
-                           chunk_split, nchunks, out, out_expert_stride, overwrite ? 1 : 0);
+                           chunk_split, nchunks, out, out_expert_stride, overwrite ? 1 : 0, partial);
     else
         hipLaunchKernelGGL(weight_grad_f32_kernel, dim3(grid), dim3(FT), 0, s, static_cast<const float*>(a), M,
                            static_cast<const float*>(b), N, tiles_m, tiles_n, chunk_expert, chunk_row0, chunk_rows,
-                           chunk_split, nchunks, out, out_expert_stride, overwrite ? 1 : 0);
+                           chunk_split, nchunks, out, out_expert_stride, overwrite ? 1 : 0, partial);
+    if (ordered)
+        hipLaunchKernelGGL(add_partials_kernel, dim3(128, groups), dim3(256), 0, s, slot_first, slot_count, partial,
+                           (size_t)M * N, out, out_expert_stride);
     return hipGetLastError();
 }
 

@@ -187,19 +187,33 @@ def test_cleared_gradients_are_overwritten_not_added_to(device):
     layer.close()
 
 
-def test_deterministic_mode_gives_identical_bits(device, monkeypatch):
-    # RBMOE_DETERMINISTIC=1: no expert is cut into chunks, so no sum depends on the order of atomics
-    monkeypatch.setenv("RBMOE_DETERMINISTIC", "1")
-    t = synth.make(small_workload(d=64, E=4, k=2, F=128, T=900, seed=29, act="bf16", wt="bf16"))
+@pytest.mark.parametrize("mode", ["default", "uncut", "atomic"])
+@pytest.mark.parametrize("act", ["bf16", "f32"])
+def test_weight_gradients_of_a_cut_expert(device, monkeypatch, mode, act):
+    # One expert far above its share is cut into chunks of rows (a shared expert always is).  By default the
+    # chunks meet in a fixed order (the first adds in place, the others store partial matrices that are added in
+    # chunk order), so two runs give identical bits - with gradients accumulated over two passes and after
+    # zero_grads alike; RBMOE_DETERMINISTIC=1 cuts nothing; RBMOE_ATOMIC_WGRAD=1 adds with f32 atomics (right
+    # within the tolerance, in no fixed order).
+    if mode == "uncut":
+        monkeypatch.setenv("RBMOE_DETERMINISTIC", "1")
+    if mode == "atomic":
+        monkeypatch.setenv("RBMOE_ATOMIC_WGRAD", "1")
+    t = synth.make(small_workload(d=64, E=4, k=2, F=128, T=2600, seed=29, act=act, wt=act, shared=True))
     bias = np.array([2.5, 0.0, 0.0, 0.0], np.float32)          # one expert far above its share
     runs = []
     for _ in range(2):
         layer, ref, gout = check_backward(device, t, bias=bias)
-        runs.append([layer.weight_grad(w, e) for w in (L.W_GATE, L.W_UP, L.W_DOWN) for e in range(4)] +
-                    [layer.weight_grad(L.W_ROUTER)])
+        first = [layer.weight_grad(w, e) for w in (L.W_GATE, L.W_UP, L.W_DOWN) for e in range(4)] + \
+                [layer.weight_grad(L.W_ROUTER), layer.weight_grad(L.W_SHARED_DOWN), layer.weight_grad(L.W_SHARED_UP)]
+        layer.backward(gout)                                    # a second pass adds to the gradients
+        twice = [layer.weight_grad(L.W_DOWN, 0), layer.weight_grad(L.W_SHARED_DOWN)]
+        assert rel_l2(twice[0], 2.0 * ref.grad_down[0]) <= (2e-2 if act == "bf16" else 1e-5)
+        runs.append(first + twice)
         layer.close()
-    for a, b in zip(*runs):
-        assert np.array_equal(a, b)
+    if mode != "atomic":
+        for a, b in zip(*runs):
+            assert np.array_equal(a, b)
 
 
 def test_plain_f32_weight_gradient_kernel_agrees(device, monkeypatch):
