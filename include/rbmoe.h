@@ -289,8 +289,9 @@ int rbmoe_copy_device(rbmoe_ctx* ctx, void* dst, const void* src, size_t bytes);
  * of event records with nothing between them reads in the same call (a few microseconds, as much as the launch).
  * rbmoe_calibrate_mfma: a kernel of nothing but 32x32x16 bf16 matrix-core multiplies, two waves on every SIMD, about
  * 0.25 ms a launch -> the multiply rate the matrix cores sustain at the clock they settle at.
- * rbmoe_calibrate_read: a plain read of `bytes` (16-byte loads, 1024 workgroups); with `flush_caches` != 0 a 512 MiB
- * copy runs before every launch so that the read comes from HBM, as a decode step's weights do. */
+ * rbmoe_calibrate_read: a plain read of `bytes` (16-byte loads; split over 512, 1024 and 2048 workgroups, the fastest
+ * split is reported); with `flush_caches` != 0 a 512 MiB copy runs before every launch, which is then timed by
+ * itself, so that the read comes from HBM as a decode step's weights do; otherwise the launches run back to back. */
 int rbmoe_calibrate_mfma(rbmoe_ctx* ctx, int32_t launches, double* tflops, double* avg_launch_ms);
 int rbmoe_calibrate_read(rbmoe_ctx* ctx, size_t bytes, int32_t launches, int32_t flush_caches, double* gbs,
                          double* avg_launch_ms);

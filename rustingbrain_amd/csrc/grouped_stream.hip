@@ -640,7 +640,7 @@ hipError_t launch_t(const GroupedArgs& g, hipStream_t s) {
                        static_cast<const bf16_t*>(g.a), g.row_index, g.w, g.w_expert_stride * (I8 ? 1 : 2), g.scales,
                        g.s_expert_stride, g.N, g.K, g.tile_expert, g.tile_row0, g.tile_rows, g.ntiles, g.dense_rows,
                        static_cast<bf16_t*>(g.out), static_cast<bf16_t*>(g.gu_out), static_cast<const bf16_t*>(g.swiglu_grad_gu),
-                       g.group_m > 0 ? g.group_m : 4);
+                       g.group_m > 0 ? g.group_m : 8);
     return hipGetLastError();
 }
 
