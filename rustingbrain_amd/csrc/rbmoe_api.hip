@@ -187,6 +187,7 @@ struct rbmoe_layer {
     bool use_f32_mc = false;   // all-f32 layer on the f32 matrix cores
     bool decode_path = true;   // few tokens: four launches that stream every touched weight once
     bool decode_front = true;  // ... three, with the routing beside the gate/up products, when most experts are touched
+    bool shared_beside = true; // large batches: the shared expert's products on the side stream, beside the routing
     bool last_front = false;   // the last forward's hidden rows are per expert over all rows (Work::hall)
     int group_m = 0, variant = 0;
     const char* kernel_name = "none";
@@ -469,6 +470,7 @@ int rbmoe_layer_create(rbmoe_ctx* ctx, const rbmoe_config* cfg, rbmoe_layer** ou
     L->variant = env_int("RBMOE_STREAM_VARIANT", 0) == 1 ? 1 : 0;
     L->decode_path = env_int("RBMOE_NO_DECODE_PATH", 0) != 1;
     L->decode_front = env_int("RBMOE_NO_DECODE_FRONT", 0) != 1;
+    L->shared_beside = env_int("RBMOE_NO_SIDE_STREAM", 0) != 1;
     // bf16 matrix cores: bf16 activations, bf16 or int8 weights, widths that fit the packed layout
     // (f32 rows with bf16 / int8 weights - what a caller with f32 matrices and a quantized or bf16 checkpoint has -
     // take the same kernels over a bf16 copy of the rows)
@@ -747,6 +749,18 @@ int rbmoe_set_weight(rbmoe_layer* L, int32_t which, int32_t expert, const void* 
 
 namespace {
 
+// The second stream of a context (default priority, like the first) and the events that fork it from and join it
+// to the main one: the backward pass runs the router's branch there, the forward pass the shared expert.
+int ensure_side_stream(rbmoe_ctx* ctx) {
+    if (ctx->side_stream) return RBMOE_OK;
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    HIP_TRY(ctx, hipStreamCreateWithFlags(&ctx->side_stream, hipStreamNonBlocking));
+    HIP_TRY(ctx, hipEventCreateWithFlags(&ctx->ev_fork, hipEventDisableTiming));
+    HIP_TRY(ctx, hipEventCreateWithFlags(&ctx->ev_fork2, hipEventDisableTiming));
+    HIP_TRY(ctx, hipEventCreateWithFlags(&ctx->ev_join, hipEventDisableTiming));
+    return RBMOE_OK;
+}
+
 Work work_of_layer(const rbmoe_layer* L) {
     Work w;
     w.P = (float*)L->P.p; w.lse = (float*)L->lse.p;
@@ -955,6 +969,62 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     if (L->training && T > 0)  // MoeCache keeps the input (src/moe.rs:133-135)
         HIP_TRY(ctx, hipMemcpyAsync(L->xc.p, x, (size_t)T * d * dtype_size(c.act_dtype), hipMemcpyDeviceToDevice, s));
 
+    auto run_on = [&](const GroupedArgs& g, hipStream_t st) -> hipError_t {
+        if (mfma) return launch_grouped_stream(g, wk, L->variant, st);
+        if (f32mc) return launch_grouped_f32(g, st);
+        return launch_grouped_generic(g, abf, wk, kGenericTileM, st);
+    };
+    auto run = [&](const GroupedArgs& g, bool) -> hipError_t { return run_on(g, s); };
+    // The shared expert (src/moe.rs:313-319) takes every row and needs nothing of the routing: with a second stream
+    // its two products run beside the routing kernels, which are bound by the vector units and by latency and
+    // leave the matrix cores idle.  (Not when the stages are timed one by one, and not over f32 rows, whose bf16
+    // copy the logits kernel has yet to write.)
+    auto shared_expert = [&](hipStream_t st) -> hipError_t {
+        GroupedArgs s1{};
+        s1.a = xe;
+        s1.w = L->swgu.p;
+        s1.scales = wk == WeightKind::I8 ? (const float*)L->ssgu.p : nullptr;
+        s1.N = Fs;
+        s1.K = d;
+        s1.dense_rows = T;
+        s1.out = L->hs.p;
+        s1.swiglu = true;
+        s1.group_m = L->group_m;
+        if (L->training) s1.gu_out = L->gus.p;
+        hipError_t e = run_on(s1, st);
+        if (e != hipSuccess) return e;
+        GroupedArgs s2 = s1;
+        s2.a = L->hs.p;
+        s2.w = L->swd.p;
+        s2.scales = wk == WeightKind::I8 ? (const float*)L->ssd.p : nullptr;
+        s2.gu_out = nullptr;
+        s2.N = d;
+        s2.K = Fs;
+        s2.out = L->ys.p;
+        s2.swiglu = false;
+        if (L->group_m == 0) s2.group_m = 4;
+        return run_on(s2, st);
+    };
+    struct JoinGuard {  // an error between fork and join must not leave the side stream forked (a capture could not end)
+        rbmoe_ctx* ctx;
+        hipStream_t main;
+        bool armed = false;
+        ~JoinGuard() {
+            if (armed) (void)hipStreamWaitEvent(main, ctx->ev_join, 0);
+        }
+    } join_guard{ctx, s};
+    bool shared_forked = false;
+    if (c.shared_expert && T >= 1024 && !timed && !cast && L->shared_beside && (mfma || f32mc) &&
+        ensure_side_stream(ctx) == RBMOE_OK) {
+        HIP_TRY(ctx, hipEventRecord(ctx->ev_fork, s));
+        HIP_TRY(ctx, hipStreamWaitEvent(ctx->side_stream, ctx->ev_fork, 0));
+        const hipError_t e = shared_expert(ctx->side_stream);
+        (void)hipEventRecord(ctx->ev_join, ctx->side_stream);  // recorded whatever happened: the join below always works
+        join_guard.armed = true;
+        shared_forked = true;
+        if (e != hipSuccess) return hip_fail(ctx, e, "shared expert on the side stream");
+    }
+
     RouterArgs ra{x, (const float*)L->router.p, router_bias, valid, T, d, E, k,
                   (float*)L->P.p, (float*)L->lse.p, (int*)L->expert_of.p, (float*)L->gate_of.p,
                   (int*)L->rank_in_block.p, (int*)L->blockcnt.p, (float*)L->partial.p};
@@ -982,11 +1052,6 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     HIP_TRY(ctx, launch_dispatch(da, abf || cast, s));
     HIP_TRY(ctx, mark(3));
 
-    auto run = [&](const GroupedArgs& g, bool swiglu) -> hipError_t {
-        if (mfma) return launch_grouped_stream(g, wk, L->variant, s);
-        if (f32mc) return launch_grouped_f32(g, s);
-        return launch_grouped_generic(g, abf, wk, kGenericTileM, s);
-    };
     GroupedArgs g1{};
     g1.a = gather_in_product ? xe : L->xg.p;
     g1.row_index = gather_in_product ? (const int*)L->perm_token.p : nullptr;
@@ -1029,31 +1094,10 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     HIP_TRY(ctx, run(g2, false));
     HIP_TRY(ctx, mark(5));
 
-    if (c.shared_expert && T > 0) {
-        GroupedArgs s1 = g1;
-        s1.a = xe;
-        s1.row_index = nullptr;
-        s1.w = L->swgu.p;
-        s1.w_expert_stride = 0;
-        s1.scales = wk == WeightKind::I8 ? (const float*)L->ssgu.p : nullptr;
-        s1.s_expert_stride = 0;
-        s1.N = Fs;
-        s1.K = d;
-        s1.dense_rows = T;
-        s1.out = L->hs.p;
-        if (L->training) s1.gu_out = L->gus.p;
-        HIP_TRY(ctx, run(s1, true));
-        GroupedArgs s2 = s1;
-        s2.a = L->hs.p;
-        s2.w = L->swd.p;
-        s2.scales = wk == WeightKind::I8 ? (const float*)L->ssd.p : nullptr;
-        s2.gu_out = nullptr;
-        s2.N = d;
-        s2.K = Fs;
-        s2.out = L->ys.p;
-        s2.swiglu = false;
-        if (L->group_m == 0) s2.group_m = 4;
-        HIP_TRY(ctx, run(s2, false));
+    if (c.shared_expert && T > 0 && !shared_forked) HIP_TRY(ctx, shared_expert(s));
+    if (shared_forked) {
+        HIP_TRY(ctx, hipStreamWaitEvent(s, ctx->ev_join, 0));
+        join_guard.armed = false;
     }
     HIP_TRY(ctx, mark(6));
 
@@ -1356,12 +1400,8 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
     L->wgrad_generic = env_int("RBMOE_WGRAD_GENERIC", 0) == 1;
     L->side_branch = env_int("RBMOE_NO_SIDE_STREAM", 0) != 1;
-    if (L->side_branch && !ctx->side_stream) {
-        HIP_TRY(ctx, hipStreamCreateWithFlags(&ctx->side_stream, hipStreamNonBlocking));
-        HIP_TRY(ctx, hipEventCreateWithFlags(&ctx->ev_fork, hipEventDisableTiming));
-        HIP_TRY(ctx, hipEventCreateWithFlags(&ctx->ev_fork2, hipEventDisableTiming));
-        HIP_TRY(ctx, hipEventCreateWithFlags(&ctx->ev_join, hipEventDisableTiming));
-    }
+    if (L->side_branch)
+        if (const int rc = ensure_side_stream(ctx)) return rc;
     L->training = true;
     L->grads_clear = true;
     return ensure_block_training_buffers(L);
