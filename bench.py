@@ -373,8 +373,12 @@ def measure(dev, name: str, steps: int, warmup: int, repeats: int, act_override:
         "router_gbs": gbs(alg["router_bytes"], stage_ms["router"]),
         "dispatch_gbs": gbs(alg["dispatch_bytes"], stage_ms["dispatch"]),
         "dispatch_note": "latency-bound: a few hundred KB of indices per launch, no rows are moved",
+        # A launch of a few microseconds sits between its raw event interval (launch plus what an event pair adds)
+        # and the net one (which takes off more than the pair really cost): both are given, the kernel-trace
+        # duration under profiles/ lies between them.
         "combine_gbs": gbs(alg["combine_bytes"], stage_ms["combine"]),
         "combine_frac_of_hbm": gbs(alg["combine_bytes"], stage_ms["combine"]) / PEAK_HBM_GBS,
+        "combine_frac_of_hbm_raw_interval": gbs(alg["combine_bytes"], raw_ms["combine"]) / PEAK_HBM_GBS,
     }
     if decode:
         whole = gbs(alg["layer_bytes_decode"], ms_per_step)
