@@ -403,6 +403,51 @@ def measure(dev, name: str, steps: int, warmup: int, repeats: int, act_override:
             "bf16": bf16, "decode": decode, "graph_ms": graph_ms}
 
 
+def two_in_flight(w, t, steps: int, warmup: int, repeats: int) -> dict:
+    """Throughput with two independent batches in flight: two contexts (a stream each), a layer with the same weights
+    on each, forwards issued alternately.  The routing kernels of one forward (vector units, latency) then run beside
+    the expert products of the other (matrix cores).  Not the headline figure: inside one model consecutive layers
+    depend on each other; this is what independent micro-batches get."""
+    T = w.tokens
+    devs = [rb.Device.open(0) for _ in range(2)]
+    layers, bufs = [], []
+    xh = synth.f32_to_bf16_bits(t.x) if w.act_dtype == "bf16" else t.x
+    for dev in devs:
+        cfg = rb.MoeConfig(w.num_experts, w.experts_per_token, w.d_ff, w.shared_expert)
+        layer = rb.MoeLayer(w.d_model, cfg, dev, act_dtype=w.act_dtype, weight_dtype=w.weight_dtype, max_tokens=T,
+                            shared_d_ff=w.shared_d_ff if w.shared_expert else 0)
+        layer.load_tensors(t)
+        x, out = DeviceBuffer(dev, xh.nbytes).upload(xh), DeviceBuffer(dev, xh.nbytes)
+        bias = DeviceBuffer(dev, 4 * w.num_experts).upload(t.router_bias) if t.router_bias is not None else None
+        layers.append(layer)
+        bufs.append((x, out, bias))
+
+    def run(n):
+        for i in range(n):
+            x, out, bias = bufs[i % 2]
+            layers[i % 2].forward_device(x.ptr, T, out.ptr, bias_ptr=bias.ptr if bias else 0)
+        for dev in devs:
+            dev.synchronize()
+
+    run(2 * warmup)
+    loops = []
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        run(steps)
+        loops.append((time.perf_counter() - t0) * 1e3 / steps)
+    ms = float(np.median(loops))
+    for layer in layers:
+        layer.close()
+    for x, out, bias in bufs:
+        for b in (x, out, bias):
+            if b:
+                b.free()
+    for dev in devs:
+        dev.close()
+    return {"ms_per_forward": ms, "tokens_per_s": T / (ms * 1e-3), "steps": steps, "repeats": repeats,
+            "note": "two contexts and two layers with the same weights, forwards issued alternately; not the headline value"}
+
+
 def release(m: dict) -> None:
     m["layer"].close()
     for b in (m["x"], m["out"], m["bias"]):
@@ -498,6 +543,8 @@ def main() -> int:
                                           with_cpu=not args.no_cpu)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(m["t"])
+    if not m["decode"]:
+        result["two_batches_in_flight"] = two_in_flight(w, m["t"], args.steps, args.warmup, max(3, min(args.repeats, 5)))
     release(m)
     if not args.only:
         # the other workloads, shorter loops: parity-test cases as far as the metric goes, reported for their
