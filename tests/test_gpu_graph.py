@@ -61,6 +61,8 @@ def bits(t, a):
     (dict(d=768, E=8, k=2, F=128, T=8, shared=True), True),      # ... with the norm inside the routing kernel
     (dict(d=128, E=8, k=2, F=64, T=600, shared=True), False),    # large-batch kernels
     (dict(d=128, E=8, k=2, F=64, T=600), True),                  # ... behind the norm kernel, residual added
+    (dict(d=128, E=8, k=2, F=64, T=1100, shared=True), False),   # the shared expert forked onto the side stream and
+    (dict(d=128, E=8, k=2, F=64, T=1100, shared=True), True),    # joined again inside the capture
 ])
 def test_forward_replays_identically(device, hip, shape, block):
     t = synth.make(small_workload(seed=61, act="bf16", wt="bf16", **shape))
