@@ -754,10 +754,21 @@ namespace {
 int ensure_side_stream(rbmoe_ctx* ctx) {
     if (ctx->side_stream) return RBMOE_OK;
     HIP_TRY(ctx, hipSetDevice(ctx->device));
-    HIP_TRY(ctx, hipStreamCreateWithFlags(&ctx->side_stream, hipStreamNonBlocking));
-    HIP_TRY(ctx, hipEventCreateWithFlags(&ctx->ev_fork, hipEventDisableTiming));
-    HIP_TRY(ctx, hipEventCreateWithFlags(&ctx->ev_fork2, hipEventDisableTiming));
-    HIP_TRY(ctx, hipEventCreateWithFlags(&ctx->ev_join, hipEventDisableTiming));
+    // all four or none: a stream without its events would be used as if it were complete
+    hipStream_t st = nullptr;
+    hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
+    hipError_t e = hipStreamCreateWithFlags(&st, hipStreamNonBlocking);
+    for (int i = 0; i < 3 && e == hipSuccess; ++i) e = hipEventCreateWithFlags(&ev[i], hipEventDisableTiming);
+    if (e != hipSuccess) {
+        for (hipEvent_t x : ev)
+            if (x) (void)hipEventDestroy(x);
+        if (st) (void)hipStreamDestroy(st);
+        return hip_fail(ctx, e, "creating the context's second stream");
+    }
+    ctx->side_stream = st;
+    ctx->ev_fork = ev[0];
+    ctx->ev_fork2 = ev[1];
+    ctx->ev_join = ev[2];
     return RBMOE_OK;
 }
 
