@@ -517,7 +517,9 @@ hipError_t launch_weight_grad(const void* a, int M, const void* b, int N, const 
                            static_cast<const float*>(b), N, tiles_m, tiles_n, chunk_expert, chunk_row0, chunk_rows,
                            chunk_split, nchunks, out, out_expert_stride, overwrite ? 1 : 0, partial);
     if (ordered)
-        hipLaunchKernelGGL(add_partials_kernel, dim3(128, groups), dim3(256), 0, s, slot_first, slot_count, partial,
+        // (most experts have nothing to add and leave at once: enough workgroups per expert for one cut expert to
+        // fill the chip by itself)
+        hipLaunchKernelGGL(add_partials_kernel, dim3(1024, groups), dim3(256), 0, s, slot_first, slot_count, partial,
                            (size_t)M * N, out, out_expert_stride);
     return hipGetLastError();
 }
