@@ -479,7 +479,10 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--repeats", type=int, default=5, help="loops of --steps forwards; ms_per_step is their median")
+    ap.add_argument("--repeats", type=int, default=0,
+                    help="loops of --steps forwards; ms_per_step is their median (default: 5, more for short loops, so "
+                         "that about 300 forwards are timed in all - a loop of 20 forwards lasts 3 ms, less than "
+                         "the device takes to settle at its clocks)")
     ap.add_argument("--workload", default="c3_prefill_d768_e16", choices=list(synth.WORKLOADS),
                     help="the workload of the top-level figures (the metric is quoted on the default)")
     ap.add_argument("--only", action="store_true", help="skip the `workloads` object (the other four workloads)")
@@ -495,6 +498,8 @@ def main() -> int:
                     help="also run a plain 39 MiB read with cold and warm caches (`calibration.read`): what a launch "
                          "the size of the decode gate/up product can get out of HBM")
     args = ap.parse_args()
+    if args.repeats <= 0:
+        args.repeats = max(5, min(25, 300 // max(args.steps, 1)))
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         return 2
