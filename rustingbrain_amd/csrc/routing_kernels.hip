@@ -14,6 +14,7 @@
 // runs give the same bits.
 #include <atomic>
 #include <cstdlib>
+#include <type_traits>
 
 #include "rbmoe_kernels.h"
 
@@ -221,14 +222,15 @@ __global__ __launch_bounds__(NE * 64, (!AHEAD && sizeof(XT) == 2) ? 6 : 2) void 
     }
 }
 
+// router_tail: everything behind the logits for the 32 tokens of router block `blk` - softmax, log-sum-exp, top-k,
+// gates, ranks, block histogram, partial sums of the losses.  LOADED = false: the logits are read from P;
+// true: the caller has put them into the `prob` array of `lds_raw` (row pitch E | 1) and met at a barrier.
 // MAXJ = experts a lane may own: 1 when E <= 64 (a lane owns one expert), kMaxExperts / 64 otherwise.
-template <typename XT, int MAXJ>
-__global__ __launch_bounds__(kRouterThreads) void router_kernel(
-    const XT* __restrict__ x, const float* __restrict__ wr, const float* __restrict__ bias,
-    const uint8_t* __restrict__ valid, int T, int d, int E, int k, float* __restrict__ P,
-    float* __restrict__ lse, int* __restrict__ expert_of, float* __restrict__ gate_of,
+template <int MAXJ, bool LOADED>
+__device__ __forceinline__ void router_tail(
+    unsigned char* __restrict__ lds_raw, int blk, const uint8_t* __restrict__ valid, int T, int E, int k,
+    float* __restrict__ P, float* __restrict__ lse, int* __restrict__ expert_of, float* __restrict__ gate_of,
     int* __restrict__ rank_in_block, int* __restrict__ blockcnt, float* __restrict__ partial) {
-    extern __shared__ __align__(16) unsigned char lds_raw[];
     constexpr int TB = kRouterTokens;
     const int ES = E | 1;
     float* prob = reinterpret_cast<float*>(lds_raw);
@@ -239,14 +241,15 @@ __global__ __launch_bounds__(kRouterThreads) void router_kernel(
     int* running = wcount + kRouterWaves * E;
 
     const int tid = threadIdx.x;
-    const int blk = blockIdx.x;
     const int t0 = blk * TB;
     const int nt = min(TB, T - t0);
 
     // ---- logits were written to P by logits_kernel ------------------------------
-    for (int idx = tid; idx < nt * E; idx += kRouterThreads) {
-        const int i = idx / E;
-        prob[i * ES + (idx - i * E)] = P[(size_t)t0 * E + idx];
+    if constexpr (!LOADED) {
+        for (int idx = tid; idx < nt * E; idx += kRouterThreads) {
+            const int i = idx / E;
+            prob[i * ES + (idx - i * E)] = P[(size_t)t0 * E + idx];
+        }
     }
     for (int idx = tid; idx < E; idx += kRouterThreads) running[idx] = 0;
     __syncthreads();
@@ -440,6 +443,166 @@ __global__ __launch_bounds__(kRouterThreads) void router_kernel(
         __syncthreads();
     }
     for (int idx = tid; idx < E; idx += kRouterThreads) blockcnt[(size_t)blk * E + idx] = running[idx];
+}
+
+// ---------------------------------------------------------------------------
+// route_fused_kernel: the logits AND everything behind them for the 32 tokens of a router block, in one workgroup
+// - one launch and one trip of the logits through memory less than logits_kernel + router_kernel.  A workgroup
+// must then hold every expert of its tokens, and with 32 tokens a wave's 64 lanes are two experts side by side:
+// lane = (token, half), wave w takes the experts 2 w + half (+ 16, + 32, ... for more than 16 experts).  The router
+// rows are no longer uniform over a wave, so they are staged in LDS beside the token rows, a slice of columns at a
+// time, and read from there (one address per half-wave: a broadcast).  The arithmetic is logits_kernel's, element by
+// element: lanes[c % 8] += x[c] * w[c] in increasing c, a rounded multiply and a rounded add, the lanes folded left
+// to right (widths that are multiples of 8: no tail).
+// Dynamic LDS: the arrays of router_tail, then 32 token rows and E router rows of one slice.
+// NI = experts per lane = ceil(E / 16).
+// ---------------------------------------------------------------------------
+__host__ __device__ static size_t fused_lds_bytes(int E, int k, int cols, size_t xsize) {
+    return router_fixed_bytes(E, k) + (size_t)kRouterTokens * (cols * xsize + 16) + (size_t)E * (cols * 4 + 16);
+}
+
+template <typename XT, int NI>
+__global__ __launch_bounds__(kRouterThreads) void route_fused_kernel(
+    const XT* __restrict__ x, const float* __restrict__ wr, const float* __restrict__ bias,
+    const uint8_t* __restrict__ valid, int T, int d, int E, int k, int cols, float* __restrict__ P,
+    float* __restrict__ lse, int* __restrict__ expert_of, float* __restrict__ gate_of,
+    int* __restrict__ rank_in_block, int* __restrict__ blockcnt, float* __restrict__ partial,
+    bf16_t* __restrict__ rows16) {
+    typedef typename XPiece<XT>::raw_t piece_t;
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    constexpr int TB = kRouterTokens;
+    const int ES = E | 1;
+    float* const prob = reinterpret_cast<float*>(lds_raw);
+    const int xpitch = cols * (int)sizeof(XT) + 16, wpitch = cols * 4 + 16;  // bytes; + 16: rows start in different banks
+    unsigned char* const xs = lds_raw + router_fixed_bytes(E, k);
+    unsigned char* const ws = xs + (size_t)TB * xpitch;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int t = lane & 31, half = lane >> 5;
+    const int blk = blockIdx.x;
+    const int t0 = blk * TB;
+    const int nt = min(TB, T - t0);
+
+    float la[NI][8];
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+        for (int l = 0; l < 8; ++l) la[i][l] = 0.0f;
+
+    // A slice travels global -> registers -> LDS; the loads of the next slice are issued before the products of the
+    // current one, so that their latency is covered by arithmetic.  A thread moves up to MAXX pieces of token rows
+    // (32 rows x 32 pieces at most) and MAXW 16-byte pieces of router rows (E rows x 64 at most) per slice.
+    constexpr int MAXX = (kRouterTokens * 32 + kRouterThreads - 1) / kRouterThreads;
+    constexpr int MAXW = (NI * 16 * 64 + kRouterThreads - 1) / kRouterThreads;
+    piece_t pre_x[MAXX];
+    float4 pre_w[MAXW];
+    auto fetch = [&](int c0) {
+        const int nc = min(cols, d - c0);
+        const int np = nc / 8, nq = nc / 4;
+#pragma unroll
+        for (int u = 0; u < MAXX; ++u) {
+            const int idx = tid + u * kRouterThreads;
+            const int r = idx / np, q = idx - r * np;
+            pre_x[u] = (idx < TB * np && r < nt) ? *reinterpret_cast<const piece_t*>(x + (size_t)(t0 + r) * d + c0 + 8 * q)
+                                                 : piece_t{};
+        }
+#pragma unroll
+        for (int u = 0; u < MAXW; ++u) {
+            const int idx = tid + u * kRouterThreads;
+            const int e = idx / nq, j = idx - e * nq;
+            pre_w[u] = idx < E * nq ? *reinterpret_cast<const float4*>(wr + (size_t)e * d + c0 + 4 * j)
+                                    : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+    };
+    auto stage = [&](int c0) {
+        const int nc = min(cols, d - c0);
+        const int np = nc / 8, nq = nc / 4;
+#pragma unroll
+        for (int u = 0; u < MAXX; ++u) {
+            const int idx = tid + u * kRouterThreads;
+            if (idx < TB * np) {
+                const int r = idx / np, q = idx - r * np;
+                *reinterpret_cast<piece_t*>(xs + (size_t)r * xpitch + (size_t)q * sizeof(piece_t)) = pre_x[u];
+                if constexpr (sizeof(XT) == 4) {
+                    if (rows16 != nullptr && r < nt) {  // the bf16 copy of f32 rows for the expert products (see logits_kernel)
+                        float f[8];
+                        XPiece<XT>::widen(pre_x[u], f);
+                        uint4 o;
+                        o.x = f32_to_bf16_bits(f[0]) | ((uint32_t)f32_to_bf16_bits(f[1]) << 16);
+                        o.y = f32_to_bf16_bits(f[2]) | ((uint32_t)f32_to_bf16_bits(f[3]) << 16);
+                        o.z = f32_to_bf16_bits(f[4]) | ((uint32_t)f32_to_bf16_bits(f[5]) << 16);
+                        o.w = f32_to_bf16_bits(f[6]) | ((uint32_t)f32_to_bf16_bits(f[7]) << 16);
+                        *reinterpret_cast<uint4*>(rows16 + (size_t)(t0 + r) * d + c0 + 8 * q) = o;
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < MAXW; ++u) {
+            const int idx = tid + u * kRouterThreads;
+            if (idx < E * nq) {
+                const int e = idx / nq, j = idx - e * nq;
+                *reinterpret_cast<float4*>(ws + (size_t)e * wpitch + 16 * j) = pre_w[u];
+            }
+        }
+    };
+    fetch(0);
+    for (int c0 = 0; c0 < d; c0 += cols) {
+        const int nc = min(cols, d - c0);
+        const int np = nc / 8;  // pieces of 8 columns in this slice
+        __syncthreads();        // the slice before has been consumed
+        stage(c0);
+        __syncthreads();
+        if (c0 + cols < d) fetch(c0 + cols);
+        const unsigned char* const xrow = xs + (size_t)t * xpitch;
+        for (int q = 0; q < np; ++q) {
+            float xv[8];
+            XPiece<XT>::widen(*reinterpret_cast<const piece_t*>(xrow + (size_t)q * sizeof(piece_t)), xv);
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                const int e = 2 * wave + half + 16 * i;
+                if (e < E) {
+                    const float4 wa = *reinterpret_cast<const float4*>(ws + (size_t)e * wpitch + 32 * q);
+                    const float4 wb = *reinterpret_cast<const float4*>(ws + (size_t)e * wpitch + 32 * q + 16);
+                    la[i][0] = __fadd_rn(la[i][0], __fmul_rn(xv[0], wa.x));
+                    la[i][1] = __fadd_rn(la[i][1], __fmul_rn(xv[1], wa.y));
+                    la[i][2] = __fadd_rn(la[i][2], __fmul_rn(xv[2], wa.z));
+                    la[i][3] = __fadd_rn(la[i][3], __fmul_rn(xv[3], wa.w));
+                    la[i][4] = __fadd_rn(la[i][4], __fmul_rn(xv[4], wb.x));
+                    la[i][5] = __fadd_rn(la[i][5], __fmul_rn(xv[5], wb.y));
+                    la[i][6] = __fadd_rn(la[i][6], __fmul_rn(xv[6], wb.z));
+                    la[i][7] = __fadd_rn(la[i][7], __fmul_rn(xv[7], wb.w));
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        const int e = 2 * wave + half + 16 * i;
+        if (e < E && t < nt) {
+            float sum = 0.0f;
+#pragma unroll
+            for (int l = 0; l < 8; ++l) sum = __fadd_rn(sum, la[i][l]);
+            float v = __fadd_rn(sum, 0.0f);  // the reference adds its (empty) scalar rest: sum + 0
+            if (bias) v = __fadd_rn(v, bias[e]);
+            prob[t * ES + e] = v;
+        }
+    }
+    __syncthreads();
+    router_tail<1, true>(lds_raw, blk, valid, T, E, k, P, lse, expert_of, gate_of, rank_in_block, blockcnt, partial);
+}
+
+template <typename XT, int MAXJ>
+__global__ __launch_bounds__(kRouterThreads) void router_kernel(
+    const XT* __restrict__ x, const float* __restrict__ wr, const float* __restrict__ bias,
+    const uint8_t* __restrict__ valid, int T, int d, int E, int k, float* __restrict__ P,
+    float* __restrict__ lse, int* __restrict__ expert_of, float* __restrict__ gate_of,
+    int* __restrict__ rank_in_block, int* __restrict__ blockcnt, float* __restrict__ partial) {
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    router_tail<MAXJ, false>(lds_raw, blockIdx.x, valid, T, E, k, P, lse, expert_of, gate_of, rank_in_block, blockcnt,
+                             partial);
 }
 
 // ---------------------------------------------------------------------------
@@ -1042,9 +1205,33 @@ __global__ __launch_bounds__(256) void combine_any_kernel(
 // ---------------------------------------------------------------------------
 // launchers
 // ---------------------------------------------------------------------------
+// Whether route_fused_kernel takes the call: every expert of a token in one workgroup (at most 64, four per lane),
+// rows of whole 8-element pieces on 16-byte boundaries, and a slice of columns that fits LDS.
+static int fused_cols(const RouterArgs& a, size_t xsize) {
+    static const bool off = [] { const char* v = std::getenv("RBMOE_NO_FUSED_ROUTER"); return v && v[0] == '1'; }();
+    if (off || a.E > 64 || a.d % 8 != 0 || a.d < 8) return 0;
+    if ((reinterpret_cast<uintptr_t>(a.x) & 15) || (reinterpret_cast<uintptr_t>(a.wr) & 15)) return 0;
+    if (((size_t)a.d * xsize) % 16 != 0) return 0;
+    const int cols = a.E <= 32 ? 256 : 128;
+    return fused_lds_bytes(a.E, a.k, cols, xsize) <= 64 * 1024 ? cols : 0;
+}
+
 template <typename XT>
 static hipError_t launch_router_t(const RouterArgs& a, hipStream_t s) {
     const int nb = (a.T + kRouterTokens - 1) / kRouterTokens;
+    if (const int cols = fused_cols(a, sizeof(XT))) {
+        const size_t lds = fused_lds_bytes(a.E, a.k, cols, sizeof(XT));
+        auto go = [&](auto ni) {
+            hipLaunchKernelGGL((route_fused_kernel<XT, decltype(ni)::value>), dim3(nb), dim3(kRouterThreads), lds, s,
+                               static_cast<const XT*>(a.x), a.wr, a.bias, a.valid, a.T, a.d, a.E, a.k, cols, a.P, a.lse,
+                               a.expert_of, a.gate_of, a.rank_in_block, a.blockcnt, a.partial,
+                               static_cast<bf16_t*>(a.rows16));
+        };
+        if (a.E <= 16) go(std::integral_constant<int, 1>{});
+        else if (a.E <= 32) go(std::integral_constant<int, 2>{});
+        else go(std::integral_constant<int, 4>{});
+        return hipGetLastError();
+    }
     static std::atomic<unsigned long long> attr_set{0};
     {  // allow more than the default 64 KiB of dynamic LDS (gfx950 has 160 KiB per CU)
         const hipError_t e = once_per_device(attr_set, [] {
