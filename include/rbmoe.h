@@ -163,10 +163,10 @@ int rbmoe_forward(rbmoe_layer* layer, const void* x, int32_t T, int32_t cols, co
  * hidden and expert output rows) lies in a static device array of RBMOE_STATIC_SCRATCH_BYTES that is part of
  * the library's code object, instead of in the workspace that rbmoe_layer_create allocated.  The call makes
  * no hipMalloc, hipFree or other allocating call.
- * Limits: decode-shaped calls only, i.e. 1 to 32 tokens with tokens * num_experts <= 2048 on a bf16 layer with
- * bf16 or int8 weights whose widths are multiples of 64, not in training mode; and the buffers of the call
- * (about tokens * experts_per_token * (d_ff + d_model) * 2 bytes, plus the shared expert's rows and the tables)
- * must fit the array.  Anything else is RBMOE_UNSUPPORTED with a message that says which limit was hit.
+ * Limits: decode-shaped calls only, i.e. 1 to 32 tokens with tokens * num_experts <= 2048 on a layer with bf16
+ * or int8 weights whose widths are multiples of 64 (bf16 rows, or f32 rows whose bf16 copy then lies in the
+ * array as well), not in training mode; and the buffers of the call (about tokens * experts_per_token *
+ * (d_ff + d_model) * 2 bytes, plus the shared expert's rows and the tables) must fit the array.  Anything else is RBMOE_UNSUPPORTED with a message that says which limit was hit.
  * Every call on one GPU, from any layer or context, uses that GPU's one array: calls that overlap in time on
  * one GPU race, and rbmoe_get_losses / rbmoe_get_routing / rbmoe_get_expert_rows after this call read the array,
  * so they describe this call only until the next static call on the same GPU. */

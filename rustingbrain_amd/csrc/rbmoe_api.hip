@@ -167,6 +167,7 @@ struct Work {
     void* hs = nullptr;
     void* ys = nullptr;
     void* hall = nullptr;  // hidden rows of every expert over every row, [E][T, F] (decode_front launches), or null
+    void* x16 = nullptr;   // bf16 copy of f32 rows [T, d] (layers with cast_rows), or null
 };
 
 struct rbmoe_layer {
@@ -782,6 +783,7 @@ Work work_of_layer(const rbmoe_layer* L) {
     w.perm_slot = (int*)L->perm_slot.p; w.perm_token = (int*)L->perm_token.p; w.inv_pos = (int*)L->inv_pos.p;
     w.h = L->h.p; w.y = L->y.p; w.hs = L->hs.p; w.ys = L->ys.p;
     w.hall = L->hall.p;
+    w.x16 = L->x16.p;
     return w;
 }
 
@@ -811,6 +813,7 @@ size_t carve_decode_work(const rbmoe_layer* L, int T, unsigned char* base, Work*
         v.hs = take((size_t)T * Fs * as);
         v.ys = take((size_t)T * d * as);
     }
+    if (L->cast_rows) v.x16 = take((size_t)T * d * 2);
     if (w) *w = v;
     return used;
 }
@@ -844,8 +847,6 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     L->last_was_block = false;  // rbmoe_forward_block sets it once this call has succeeded
     const bool abf = c.act_dtype == RBMOE_BF16;
     const bool cast = L->cast_rows;  // f32 rows, bf16 matrix-core products over their bf16 copy
-    // the rows the expert products read
-    const void* const xe = cast ? L->x16.p : x;
     const WeightKind wk = c.weight_dtype == RBMOE_F32 ? WeightKind::F32
                           : c.weight_dtype == RBMOE_BF16 ? WeightKind::BF16 : WeightKind::I8;
     if (timed && !L->have_events) {
@@ -877,8 +878,8 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
         if (!decode_ok) {
             char buf[200];
             std::snprintf(buf, sizeof buf,
-                          "rbmoe_forward_static takes decode-shaped calls only: 1 to %d tokens of a bf16 layer with "
-                          "bf16 or int8 weights on the matrix-core path, not in training mode (got %d tokens)",
+                          "rbmoe_forward_static takes decode-shaped calls only: 1 to %d tokens of a layer with bf16 or "
+                          "int8 weights on the matrix-core path, not in training mode (got %d tokens)",
                           kSmallRouteMaxTokens, T);
             return fail(ctx, RBMOE_UNSUPPORTED, buf);
         }
@@ -894,6 +895,8 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
         // a previous call's).
         carve_decode_work(L, T, static_cast<unsigned char*>(static_scratch), &wk_);
     }
+    // the rows the expert products read
+    const void* const xe = cast ? wk_.x16 : x;
     if (norm_src && !norm_in_route)
         HIP_TRY(ctx, launch_rmsnorm(norm_src, (const float*)L->norm_w.p, L->norm_eps, T, d, L->xn.p, abf, s));
 
@@ -905,7 +908,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
         if (norm_in_route) {
             sr.x = norm_src; sr.norm_w = (const float*)L->norm_w.p; sr.norm_eps = L->norm_eps; sr.xn_out = L->xn.p;
         }
-        if (cast) sr.rows16 = L->x16.p;
+        if (cast) sr.rows16 = wk_.x16;
         // the routing beside the gate/up products, in one launch: bf16 rows as they are (no norm to apply first)
         const bool front = L->decode_front && !norm_src && !cast && wk_.hall != nullptr &&
                            decode_front_ok(x, (const float*)L->router.p, T, d, E, k);
@@ -1388,11 +1391,14 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
                      : env_int("RBMOE_ATOMIC_WGRAD", 0) == 1 ? WgradSplit::Atomic : WgradSplit::Ordered;
     if (L->wgrad_split == WgradSplit::Ordered) {
         const bool wbf = c.act_dtype == RBMOE_BF16;
-        size_t need = std::max(weight_grad_partial_bytes((int)d, (int)F, (int)E, -1, (int)S, wbf),
-                               weight_grad_partial_bytes((int)(2 * F), (int)d, (int)E, -1, (int)S, wbf));
+        // sized for every token count up to max_tokens: a smaller batch can need more partial matrices than the
+        // largest one, because the cut limit follows the row count with a floor and a rounding
+        const int k = c.experts_per_token;
+        size_t need = std::max(weight_grad_partial_bytes_upto((int)d, (int)F, (int)E, false, (int)T, k, wbf),
+                               weight_grad_partial_bytes_upto((int)(2 * F), (int)d, (int)E, false, (int)T, k, wbf));
         if (c.shared_expert)
-            need = std::max(need, std::max(weight_grad_partial_bytes((int)d, (int)Fs, 1, (int)T, (int)T, wbf),
-                                           weight_grad_partial_bytes((int)(2 * Fs), (int)d, 1, (int)T, (int)T, wbf)));
+            need = std::max(need, std::max(weight_grad_partial_bytes_upto((int)d, (int)Fs, 1, true, (int)T, 1, wbf),
+                                           weight_grad_partial_bytes_upto((int)(2 * Fs), (int)d, 1, true, (int)T, 1, wbf)));
         p.add(&L->wg_partial, need);
     }
     p.add(&L->st_gout, T * d * as);
@@ -1892,6 +1898,19 @@ int rbmoe_calibrate_read(rbmoe_ctx* ctx, size_t bytes, int32_t launches, int32_t
     const double avg = total / launches;
     *gbs = (double)bytes / (avg * 1e-3) / 1e9;
     if (avg_launch_ms) *avg_launch_ms = avg;
+    return RBMOE_OK;
+}
+
+// Test hook (not part of rbmoe.h): the partial matrices an ordered weight-gradient launch over `tokens` tokens cuts
+// out, and how many a buffer sized for `max_tokens` holds.
+int rbmoe_internal_weight_grad_slots(int32_t M, int32_t N, int32_t groups, int32_t dense, int32_t tokens,
+                                     int32_t rows_per_token, int32_t bf16, int32_t max_tokens, int64_t* needed,
+                                     int64_t* held) {
+    if (!needed || !held) return RBMOE_NULL_POINTER;
+    const size_t one = (size_t)M * N * sizeof(float);
+    const int rows = dense ? tokens : tokens * rows_per_token;
+    *needed = (int64_t)(weight_grad_partial_bytes(M, N, groups, dense ? rows : -1, rows, bf16 != 0) / one);
+    *held = (int64_t)(weight_grad_partial_bytes_upto(M, N, groups, dense != 0, max_tokens, rows_per_token, bf16 != 0) / one);
     return RBMOE_OK;
 }
 

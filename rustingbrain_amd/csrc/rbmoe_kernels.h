@@ -151,12 +151,16 @@ hipError_t launch_grouped_tn(const void* a, int M, const void* b, const int* b_r
 //            a second kernel adds in chunk order: identical bits run to run
 //   Atomic   cut into several chunks that all add with f32 atomics, in whatever order they arrive
 // `overwrite`: out is known to hold zeros, whatever its bytes are, and is written instead of added to.
-// `chunks` is scratch of weight_grad_table_ints(...) ints, `partial` of weight_grad_partial_bytes(...) bytes.
+// `chunks` is scratch of weight_grad_table_ints(...) ints, `partial` of weight_grad_partial_bytes(...) bytes
+// (a smaller buffer is legal: the launch then cuts less).
 enum class WgradSplit : int { None = 0, Ordered = 1, Atomic = 2 };
 bool weight_grad_shape_ok(int M, int N, bool bf16);
 int weight_grad_max_chunks(int groups, int total_rows);
 int weight_grad_table_ints(int groups, int total_rows);
 size_t weight_grad_partial_bytes(int M, int N, int groups, int dense_rows, int total_rows, bool bf16);
+// ... for a buffer that serves every launch of 1 .. max_tokens tokens (rows_per_token rows each; dense: rows = tokens)
+size_t weight_grad_partial_bytes_upto(int M, int N, int groups, bool dense, int max_tokens, int rows_per_token,
+                                      bool bf16);
 hipError_t launch_weight_grad(const void* a, int M, const void* b, int N, const int* counts, const int* offsets,
                               int groups, int dense_rows, int total_rows, WgradSplit split_mode, bool overwrite,
                               int* chunks, float* partial, size_t partial_bytes, float* out, size_t out_expert_stride,

@@ -137,29 +137,24 @@ __global__ __launch_bounds__(256) void chunk_table_kernel(const int* __restrict_
         }
         const int first = base + scan[tid] - n;
         const int first_x = base_x + scan_x[tid] - nx;
+        // An ordered cut needs a partial matrix per further chunk.  The launcher sizes the limit so that there is
+        // always room; should there not be, the expert is not cut at all (one chunk over all its rows: slower,
+        // never wrong), and its unused table entries are empty chunks.
+        const bool cut = n > 1 && (!ordered || first_x + nx <= max_slots);
         if (e < groups) {
-            // (more partial matrices than there is room for cannot happen: the launcher sizes the limit for it;
-            // should it, the surplus chunks are dropped from the count here and their rows are not added)
             slot_first[e] = first_x;
-            slot_count[e] = ordered ? max(0, min(nx, max_slots - first_x)) : 0;
+            slot_count[e] = (ordered && cut) ? nx : 0;
         }
         if (n > 0) {
-            const int per = (((rows + n - 1) / n) + 31) & ~31;
+            const int per = cut ? (((rows + n - 1) / n) + 31) & ~31 : rows;
             for (int c = 0; c < n; ++c) {
+                if (first + c >= max_chunks) break;
                 const int r0 = c * per;
-                const int r = min(per, rows - r0);
-                if (first + c < max_chunks && r > 0) {
-                    chunk_expert[first + c] = e;
-                    chunk_row0[first + c] = row0 + r0;
-                    const bool room = !ordered || c == 0 || first_x + c - 1 < max_slots;
-                    chunk_rows[first + c] = room ? r : 0;
-                    chunk_split[first + c] = !ordered ? (n > 1) : (c == 0 ? 0 : 2 + first_x + c - 1);
-                } else if (first + c < max_chunks) {
-                    chunk_expert[first + c] = e;
-                    chunk_row0[first + c] = row0;
-                    chunk_rows[first + c] = 0;
-                    chunk_split[first + c] = 1;
-                }
+                const int r = max(0, min(per, rows - r0));
+                chunk_expert[first + c] = e;
+                chunk_row0[first + c] = r > 0 ? row0 + r0 : row0;
+                chunk_rows[first + c] = r;
+                chunk_split[first + c] = !cut ? 0 : (!ordered ? 1 : (c == 0 ? 0 : 2 + first_x + c - 1));
             }
         }
         __syncthreads();
@@ -461,12 +456,25 @@ int cut_limit(int M, int N, int groups, int dense_rows, int total_rows, bool bf1
 }
 }  // namespace
 
-// Partial matrices an ordered launch may need: every further chunk of a cut expert has one; there are at most
-// total_rows / limit of them.
+// Partial matrices an ordered launch of `total_rows` rows needs: every further chunk of a cut expert has one, and
+// there are at most total_rows / limit of them.
 size_t weight_grad_partial_bytes(int M, int N, int groups, int dense_rows, int total_rows, bool bf16) {
     if (groups <= 0 || total_rows <= 0) return 0;
     const int limit = cut_limit(M, N, groups, dense_rows, total_rows, bf16);
     return (size_t)(total_rows / limit + 1) * M * N * sizeof(float);
+}
+
+// The same for a buffer that has to serve every launch of 1 .. max_tokens tokens (rows_per_token rows each; for
+// a dense launch the rows are the tokens).  The cut limit follows the row count with a floor and a rounding, so
+// the number of partial matrices is not monotone in the row count: a smaller batch can need more of them.
+size_t weight_grad_partial_bytes_upto(int M, int N, int groups, bool dense, int max_tokens, int rows_per_token,
+                                      bool bf16) {
+    size_t need = 0;
+    for (int t = 1; t <= max_tokens; ++t) {
+        const int rows = dense ? t : t * rows_per_token;
+        need = std::max(need, weight_grad_partial_bytes(M, N, groups, dense ? rows : -1, rows, bf16));
+    }
+    return need;
 }
 
 hipError_t launch_weight_grad(const void* a, int M, const void* b, int N, const int* counts, const int* offsets,
@@ -489,8 +497,11 @@ hipError_t launch_weight_grad(const void* a, int M, const void* b, int N, const 
         limit = cut_limit(M, N, groups, dense_rows, total_rows, bf16);
         if (split_mode == WgradSplit::Ordered) {
             ordered = true;
-            max_slots = (int)(partial_bytes / ((size_t)M * N * sizeof(float)));
-            if (partial == nullptr || max_slots < total_rows / limit + 1) return hipErrorInvalidValue;
+            max_slots = partial ? (int)std::min<size_t>(partial_bytes / ((size_t)M * N * sizeof(float)), 1 << 20) : 0;
+            // A buffer with fewer partial matrices than this row count would cut out (total_rows / limit at most)
+            // gets longer chunks, down to no cut at all, instead of a refusal.
+            if (max_slots == 0) limit = 1 << 30;
+            else if (total_rows / limit > max_slots) limit = ((total_rows / max_slots + 1) + 31) & ~31;
         }
     }
     const int max_chunks = weight_grad_max_chunks(groups, total_rows);

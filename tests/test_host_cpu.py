@@ -165,3 +165,25 @@ def test_skewed_workload_puts_about_thirty_percent_on_expert_zero():
     logits = t.x.astype(np.float64) @ t.router.astype(np.float64).T + t.router_bias
     top = np.argsort(-logits, axis=1, kind="stable")[:, :2]
     assert 0.28 <= float(np.mean(top == 0)) <= 0.32
+
+
+def test_weight_gradient_workspace_holds_every_batch_up_to_max_tokens():
+    """The ordered weight gradients keep one partial matrix per further chunk of a cut expert.  How many a launch
+    cuts out depends on its own row count (not monotonically), the buffer is sized once for max_tokens: it must
+    hold what every token count up to max_tokens asks for."""
+    import ctypes as C
+    lib = L.load()
+    fn = lib.rbmoe_internal_weight_grad_slots
+    fn.restype = C.c_int
+    fn.argtypes = [C.c_int32] * 8 + [C.POINTER(C.c_int64)] * 2
+    cases = [(768, 2048, 16, 0, 2, 1, 1200), (4096, 768, 16, 0, 2, 1, 2000), (768, 2048, 16, 0, 2, 1, 3072),
+             (768, 1408, 16, 0, 2, 1, 1536), (1024, 704, 64, 0, 6, 1, 900), (512, 1408, 8, 0, 2, 0, 1024),
+             (768, 1408, 1, 1, 1, 1, 1300), (2816, 768, 1, 1, 1, 1, 700)]
+    for M, N, groups, dense, k, bf16, max_tokens in cases:
+        need, held = C.c_int64(), C.c_int64()
+        worst = 0
+        for tokens in range(1, max_tokens + 1):
+            assert fn(M, N, groups, dense, tokens, k, bf16, max_tokens, C.byref(need), C.byref(held)) == L.OK
+            worst = max(worst, need.value)
+            assert need.value <= held.value, (M, N, groups, tokens, need.value, held.value)
+        assert worst == held.value   # and no more than the worst case asks for

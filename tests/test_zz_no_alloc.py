@@ -75,6 +75,35 @@ def test_static_forward_matches_the_allocating_one_twice_in_a_row(device, wt):
     layer.close()
 
 
+def test_static_forward_over_f32_rows_keeps_their_bf16_copy_in_the_static_array_too(device):
+    """f32 rows over bf16 weights: the bf16 copy of the rows that the products read is one more buffer of the
+    call and lies in the static array like the others; same bits as the allocating entry point, twice in a row."""
+    t = synth.make(small_workload(d=128, E=8, k=2, F=192, T=24, seed=73, act="f32", wt="bf16", shared=True,
+                                  shared_d_ff=64))
+    layer = gpu_layer(device, t)
+    ref_layer = oracle_layer(t)
+    for rows in (24, 7):
+        x = np.ascontiguousarray(t.x[:rows], dtype=np.float32)
+        xb, ob = DeviceBuffer(device, x.nbytes).upload(x), DeviceBuffer(device, x.nbytes)
+        got = []
+        for fn in (layer.forward_device, layer.forward_static_device):
+            ob.upload(np.zeros_like(x))
+            fn(xb.ptr, rows, ob.ptr)
+            device.synchronize()
+            got.append((ob.download(np.empty_like(x)).copy(), layer.cache(rows)))
+        assert layer.kernel_name().startswith("mfma_bf16_decode")
+        (out_a, cache_a), (out_s, cache_s) = got
+        assert same(out_s, out_a), f"{rows} rows: outputs differ between the two entry points"
+        for name in ("expert_of", "gate_of", "counts", "offsets", "perm_slot", "perm_token", "probabilities"):
+            assert same(getattr(cache_s, name), getattr(cache_a, name)), f"{rows} rows: {name}"
+        ref = ref_layer.forward(t.x[:rows], threads=4)
+        assert_routing_identical(cache_s, ref)
+        assert rel_l2(out_s.reshape(rows, 128), ref.out) <= 2e-2
+        xb.free()
+        ob.free()
+    layer.close()
+
+
 def test_static_forward_refuses_what_it_cannot_take(device):
     t = synth.make(small_workload(d=64, E=4, k=2, F=64, T=40, seed=72, act="bf16", wt="bf16"))
     layer = gpu_layer(device, t)
