@@ -134,6 +134,23 @@ const char* rbmoe_last_global_error(void);
 int rbmoe_layer_create(rbmoe_ctx* ctx, const rbmoe_config* cfg, rbmoe_layer** out);
 void rbmoe_layer_destroy(rbmoe_layer* layer);
 
+/* Behaviour switches of a layer, the counterpart of the reference's test hooks and environment switches
+ * (CHUNK_ROWS_OVERRIDE src/gpu_model.rs:2948, cuda_flash::DISABLED src/cuda_flash.rs:898-907): every default is
+ * the fast path, the other settings exist for A/B measurements and for tests that hold one kernel set against
+ * another.  The library itself reads no environment variable. */
+typedef enum rbmoe_option {
+    RBMOE_OPT_FORCE_GENERIC = 0,   /* 1: the any-shape kernels for every product; only before the first weight is set */
+    RBMOE_OPT_EXPLICIT_GATHER = 1, /* 1: gathered rows are written out instead of gathered inside the gate/up product */
+    RBMOE_OPT_GROUP_M = 2,         /* row tiles that walk the column tiles together on one XCD; 0: each product's default */
+    RBMOE_OPT_DECODE_PATH = 3,     /* 0: a few tokens take the large-batch kernels too */
+    RBMOE_OPT_DECODE_FRONT = 4,    /* 0: decode-shaped calls route in a launch of their own */
+    RBMOE_OPT_FUSED_ROUTER = 5,    /* 0: router logits and the routing behind them in separate launches */
+    RBMOE_OPT_SIDE_STREAM = 6,     /* 0: everything on the context's one stream */
+    RBMOE_OPT_WGRAD_MODE = 7,      /* cut experts' weight gradients: 0 fixed order (default), 1 f32 atomics, 2 never cut */
+    RBMOE_OPT_WGRAD_GENERIC = 8    /* 1: the plain kernel for the weight gradients */
+} rbmoe_option;
+int rbmoe_layer_set_option(rbmoe_layer* layer, int32_t option, int32_t value);
+
 /* DeviceParam::new (src/gpu_transformer.rs:471-490): copies one weight matrix
  * from HOST memory to the device (the caller keeps its buffer).  `dtype` is the
  * dtype of `data`; f32 data is converted to the layer's weight dtype (bf16 by

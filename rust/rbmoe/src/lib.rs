@@ -238,6 +238,11 @@ impl MoeLayer {
     /// Makes the forward pass keep what `backward` needs and allocates the f32 gradient accumulators (the
     /// role of `Param.grad`).  Call before the weights are set.  Every f32 and bf16 layer has a backward pass
     /// (matrix-core kernels where the widths fit them, plain ones otherwise); int8 layers report `UnsupportedCuda`.
+    /// A behaviour switch of the layer (`sys::RBMOE_OPT_*`); every default is the fast path.
+    pub fn set_option(&mut self, option: i32, value: i32) -> Result<(), NetworkError> {
+        check(unsafe { sys::rbmoe_layer_set_option(self.layer, option, value) }, self.device.raw(), 0, 0)
+    }
+
     pub fn enable_training(&mut self) -> Result<(), NetworkError> {
         check(unsafe { sys::rbmoe_layer_enable_training(self.layer) }, self.device.raw(), 0, 0)
     }

@@ -26,6 +26,16 @@ pub const RBMOE_W_SHARED_UP: i32 = 5;
 pub const RBMOE_W_SHARED_DOWN: i32 = 6;
 pub const RBMOE_W_NORM: i32 = 7;
 
+pub const RBMOE_OPT_FORCE_GENERIC: i32 = 0;
+pub const RBMOE_OPT_EXPLICIT_GATHER: i32 = 1;
+pub const RBMOE_OPT_GROUP_M: i32 = 2;
+pub const RBMOE_OPT_DECODE_PATH: i32 = 3;
+pub const RBMOE_OPT_DECODE_FRONT: i32 = 4;
+pub const RBMOE_OPT_FUSED_ROUTER: i32 = 5;
+pub const RBMOE_OPT_SIDE_STREAM: i32 = 6;
+pub const RBMOE_OPT_WGRAD_MODE: i32 = 7;
+pub const RBMOE_OPT_WGRAD_GENERIC: i32 = 8;
+
 pub const RBMOE_NUM_STAGES: usize = 8;
 
 #[repr(C)]
@@ -78,6 +88,7 @@ extern "C" {
     pub fn rbmoe_last_global_error() -> *const c_char;
     pub fn rbmoe_layer_create(ctx: *mut rbmoe_ctx, cfg: *const rbmoe_config, out: *mut *mut rbmoe_layer) -> c_int;
     pub fn rbmoe_layer_destroy(layer: *mut rbmoe_layer);
+    pub fn rbmoe_layer_set_option(layer: *mut rbmoe_layer, option: i32, value: i32) -> c_int;
     pub fn rbmoe_set_weight(layer: *mut rbmoe_layer, which: i32, expert: i32, data: *const c_void, dtype: i32,
                             scales: *const f32, rows: i32, cols: i32) -> c_int;
     pub fn rbmoe_forward(layer: *mut rbmoe_layer, x: *const c_void, tokens: i32, cols: i32, valid: *const u8,

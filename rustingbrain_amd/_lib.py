@@ -19,6 +19,9 @@ F32, BF16, I8 = 0, 1, 2
 DTYPES = {"f32": F32, "bf16": BF16, "int8": I8}
 # rbmoe_weight
 W_ROUTER, W_GATE, W_UP, W_DOWN, W_SHARED_GATE, W_SHARED_UP, W_SHARED_DOWN, W_NORM = range(8)
+# rbmoe_option
+(OPT_FORCE_GENERIC, OPT_EXPLICIT_GATHER, OPT_GROUP_M, OPT_DECODE_PATH, OPT_DECODE_FRONT, OPT_FUSED_ROUTER,
+ OPT_SIDE_STREAM, OPT_WGRAD_MODE, OPT_WGRAD_GENERIC) = range(9)
 NUM_STAGES = 8
 STATIC_SCRATCH_BYTES = 8 << 20
 STAGE_NAMES = ("router", "empty", "dispatch", "gate_up", "down", "shared", "combine", "total")
@@ -51,6 +54,7 @@ SIGNATURES = {
     "rbmoe_last_global_error": (C.c_char_p, []),
     "rbmoe_layer_create": (C.c_int, [C.c_void_p, C.POINTER(Config), C.POINTER(C.c_void_p)]),
     "rbmoe_layer_destroy": (None, [C.c_void_p]),
+    "rbmoe_layer_set_option": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32]),
     "rbmoe_set_weight": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_int32,
                                    C.POINTER(C.c_float), C.c_int32, C.c_int32]),
     "rbmoe_forward": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p,

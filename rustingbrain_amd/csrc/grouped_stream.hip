@@ -47,14 +47,22 @@ namespace rbmoe {
 
 namespace {
 
-constexpr int BM = 128;   // token rows per workgroup
+#ifndef RBMOE_STREAM_BM
+#define RBMOE_STREAM_BM 128
+#endif
+#ifndef RBMOE_STREAM_OCC
+#define RBMOE_STREAM_OCC 2
+#endif
+constexpr int BM = RBMOE_STREAM_BM;   // token rows per workgroup
 constexpr int BK = 64;    // reduction slice held in one LDS stage
 constexpr int NW = 4;     // waves per workgroup
 constexpr int NT = NW * 64;
 constexpr int CPR = BK / 8;            // 16-byte pieces per LDS row
 constexpr int TT = BM / 32;            // token blocks per wave
 constexpr int KS = BK / 16;            // matrix-core steps per slice
-constexpr int DMA_PER_WAVE = BM * CPR / 64 / NW;  // LDS-DMA instructions per wave per slice (4)
+constexpr int DMA_PER_WAVE = BM * CPR / 64 / NW;  // LDS-DMA instructions per wave per slice
+constexpr int RING = KS;    // weight-fragment steps in flight per wave (register ring depth)
+constexpr int STAGES = 3;   // LDS stages of one activation slice each
 
 // Token fragment read from LDS.
 __device__ __forceinline__ bf16x8 lds_frag(const uint4* __restrict__ base, int idx) {
@@ -320,8 +328,8 @@ struct PipeCtx {
 template <bool I8, int NB>
 __device__ __forceinline__ void pipe_loop(const PipeCtx& c, floatx16 (&acc)[2][TT], Slot<I8> (&ring)[KS],
                                           const uint32_t (&a_src)[DMA_PER_WAVE]) {
-    constexpr int RING = KS, D = RING - 1;
-    static_assert(KS == 4 && DMA_PER_WAVE == 4 && D == 3, "the wait counts below are derived for this configuration");
+    constexpr int D = RING - 1;
+    static_assert(KS == 4 && D == 3, "the wait counts below are derived for this configuration");
     const uint4* const As = c.As;
     const uint32_t lds0 = c.lds0, lane16 = c.lane16;
     const char* const a_base = c.a_base;
@@ -403,12 +411,8 @@ __device__ __forceinline__ void pipe_loop(const PipeCtx& c, floatx16 (&acc)[2][T
     for (int i = 0; i < RING; ++i) asm volatile("" : : "v"(ring_ref[i].f0), "v"(ring_ref[i].f1));
 }
 
-// RING = weight-fragment steps in flight per wave (register ring depth);
-// TFBUF = 2: token fragments are read from LDS one step ahead, 1: just in time;
-// STAGES = LDS stages of one activation slice each: the DMA of slice k + STAGES - 1 is issued when slice k starts;
-// PIPE = the main loop that spreads its memory instructions between the multiplies (see there).
-template <bool SWIGLU, bool I8, int RING, int TFBUF, int STAGES, bool PIPE>
-__global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
+template <bool SWIGLU, bool I8>
+__global__ __launch_bounds__(NT, RBMOE_STREAM_OCC) void grouped_stream_kernel(
     const bf16_t* __restrict__ a, const int* __restrict__ row_index, const void* __restrict__ wpacked,
     size_t w_expert_stride_bytes, const float* __restrict__ scales, size_t s_expert_stride, int N, int K,
     const int* __restrict__ tile_expert, const int* __restrict__ tile_row0, const int* __restrict__ tile_rows,
@@ -418,7 +422,6 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
     constexpr int BN = SWIGLU ? NW * 32 : NW * 64;  // output features per workgroup
     // LDS stages of one activation slice each; the epilogue reuses the first two as one
     // 128 x 128 staging tile for the output.
-    static_assert(STAGES == 2 || STAGES == 3, "two or three stages");
     __shared__ uint4 As[STAGES * BM * CPR];
 
     // ---- which tile (each XCD walks a contiguous range, M fastest inside a group)
@@ -484,12 +487,12 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
     uint32_t a_src[DMA_PER_WAVE];
 #pragma unroll
     for (int j = 0; j < DMA_PER_WAVE; ++j) {
-        const int r = wave * 32 + j * 8 + (lane >> 3);
+        const int r = wave * (BM / NW) + j * 8 + (lane >> 3);
         const int rr = r < rows ? r : 0;
         const int grow = row_index ? row_index[row0 + rr] : row0 + rr;
         a_src[j] = ((uint32_t)grow * (uint32_t)K + 8u * ((lane & 7) ^ ((r >> 1) & 7))) * 2u;
     }
-    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)As + wave * 32 * CPR * 16;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)As + wave * (BM / NW) * CPR * 16;
     auto dma_a = [&](int kt, auto buf_tag) {
         constexpr int BUF = decltype(buf_tag)::value;
 #pragma unroll
@@ -524,100 +527,15 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
     __builtin_amdgcn_sched_barrier(0);
     RBMOE_TRACE_AT(blockIdx.x, 1);
 
-    if constexpr (PIPE) {
-        static_assert(STAGES == 3 && RING == KS && TFBUF == 2, "the pipelined loop's configuration");
+    // The loop is specialised at compile time for the number of token blocks that hold rows: a run-time branch per
+    // block between the multiplies costs far more than the skipped multiplies save.
+    {
         const PipeCtx pc{As, lds0, a_base, wp0, wp1, lane16, lrow, lhalf, lxor, KT};
-        if (nblk == 4) pipe_loop<I8, 4>(pc, acc, ring, a_src);
-        else if (nblk == 3) pipe_loop<I8, 3>(pc, acc, ring, a_src);
+        static_assert(TT >= 2 && TT <= 4, "one specialisation per possible block count");
+        if (TT >= 4 && nblk >= 4) pipe_loop<I8, (TT >= 4 ? 4 : TT)>(pc, acc, ring, a_src);
+        else if (TT >= 3 && nblk == 3) pipe_loop<I8, (TT >= 3 ? 3 : TT)>(pc, acc, ring, a_src);
         else if (nblk == 2) pipe_loop<I8, 2>(pc, acc, ring, a_src);
         else pipe_loop<I8, 1>(pc, acc, ring, a_src);
-    }
-
-    // One slice = KS steps.  BUF is the LDS stage the slice reads (its parity); the ring
-    // position of the slice's first step is 0, or BUF * KS when the ring holds two slices.
-    // NB = token blocks of this tile that hold rows, a compile-time constant inside the
-    // loop: a run-time branch per block between the multiplies costs far more than the
-    // skipped multiplies save, so the whole loop is specialised instead.
-    // The loop is straight-line and every wave issues, per slice, exactly: 4 DMA
-    // instructions, then 2 weight loads in each of the KS steps.  Past the end the last
-    // slice / step is fetched again, so that the counts below hold everywhere.
-    // (IDX = position of the slice inside the unrolled loop body: it fixes the LDS stage and the ring phase)
-    auto slice = [&](int kt, auto idx_tag, auto nb_tag) {
-        constexpr int IDX = decltype(idx_tag)::value;
-        constexpr int BUF = IDX % STAGES;
-        constexpr int G0 = RING == 2 * KS ? (IDX % 2) * KS : 0;
-        constexpr int NB = decltype(nb_tag)::value;
-        dma_a(min(kt + STAGES - 1, KT - 1), std::integral_constant<int, (BUF + STAGES - 1) % STAGES>{});
-        const uint4* Ab = As + BUF * (BM * CPR);
-        bf16x8 tf[TFBUF][TT];
-#pragma unroll
-        for (int t = 0; t < NB; ++t) tf[0][t] = lds_frag(Ab, (t * 32 + lrow) * CPR + (lhalf ^ lxor));
-        static_for<0, KS>([&](auto s_tag) {
-            constexpr int s = decltype(s_tag)::value;
-            const int g = kt * KS + s;
-            Slot<I8>& cur = ring[(G0 + s) % RING];
-            // weight fragments for step g + D go into the slot step g - 1 released
-            ring[(G0 + s + D) % RING].load(wp0, wp1, min(g + D, GS - 1), lane16);
-            if constexpr (TFBUF == 2) {
-                if (s + 1 < KS) {
-                    const int piece = (2 * (s + 1) + lhalf) ^ lxor;
-#pragma unroll
-                    for (int t = 0; t < NB; ++t) tf[(s + 1) & 1][t] = lds_frag(Ab, (t * 32 + lrow) * CPR + piece);
-                }
-            } else if (s > 0) {
-                const int piece = (2 * s + lhalf) ^ lxor;
-#pragma unroll
-                for (int t = 0; t < NB; ++t) tf[0][t] = lds_frag(Ab, (t * 32 + lrow) * CPR + piece);
-            }
-            // Younger than the loads of step g: the weight loads of steps g+1 .. g+D (2 each)
-            // and the DMA (4) of every slice that started after they were issued.
-            wait_for<2 * D + DMA_PER_WAVE * ((D - s + KS - 1) / KS)>(cur.f0, cur.f1);
-            const bf16x8 w0 = cur.a0();
-            const bf16x8 w1 = cur.a1();
-#pragma unroll
-            for (int t = 0; t < NB; ++t) {
-                acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w0, tf[s % TFBUF][t], acc[0][t], 0, 0, 0);
-                acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w1, tf[s % TFBUF][t], acc[1][t], 0, 0, 0);
-            }
-        });
-        // Every LDS read of this slice has been consumed by a multiply issued above this
-        // point.  The DMA of the next slice is older than the 2 * KS weight loads of every slice since it was
-        // issued (STAGES - 1 of them) and than the DMA of the STAGES - 2 slices after it.
-        __builtin_amdgcn_sched_barrier(0);
-        wait_outstanding<2 * KS * (STAGES - 1) + DMA_PER_WAVE * (STAGES - 2)>();
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-    };
-
-    static_assert(RING == KS || RING == 2 * KS, "ring depth is one or two slices");
-    static_assert(DMA_PER_WAVE == 4, "the wait counts assume 4 DMA instructions per wave per slice");
-    // the loop body holds as many slices as it takes for the LDS stage and the ring phase to come round again
-    constexpr int UNROLL = (RING == 2 * KS && STAGES % 2) ? 2 * STAGES : (STAGES > 2 ? STAGES : 2);
-    auto run = [&](auto nb_tag) {
-        int kt = 0;
-        for (; kt + UNROLL <= KT; kt += UNROLL)
-            static_for<0, UNROLL>([&](auto i) { slice(kt + decltype(i)::value, i, nb_tag); });
-        static_while<0, UNROLL - 1>([&](auto i) {
-            if (kt + decltype(i)::value >= KT) return false;
-            slice(kt + decltype(i)::value, i, nb_tag);
-            return true;
-        });
-        // The loads fetched again past the end still target ring registers and LDS.  Naming
-        // the registers after the wait keeps them allocated until their data has arrived: a
-        // loaded value the compiler sees no use for would otherwise hand its register to
-        // something live while the load is still in flight.  (Done here, inside each
-        // specialisation, so that no path leaves it with loads outstanding.)
-        wait_outstanding<0>();
-        auto& ring_ref = ring;
-#pragma unroll
-        for (int i = 0; i < RING; ++i) asm volatile("" : : "v"(ring_ref[i].f0), "v"(ring_ref[i].f1));
-    };
-    static_assert(TT == 4, "one specialisation per possible block count");
-    if constexpr (!PIPE) {
-        if (nblk == 4) run(std::integral_constant<int, 4>{});
-        else if (nblk == 3) run(std::integral_constant<int, 3>{});
-        else if (nblk == 2) run(std::integral_constant<int, 2>{});
-        else run(std::integral_constant<int, 1>{});
     }
     RBMOE_TRACE_AT(blockIdx.x, 2);
     // ---- epilogue -------------------------------------------------------------
@@ -628,7 +546,7 @@ __global__ __launch_bounds__(NT, 2) void grouped_stream_kernel(
     RBMOE_TRACE_AT(blockIdx.x, 3);
 }
 
-template <bool SWIGLU, bool I8, int RING, int TFBUF, int STAGES, bool PIPE>
+template <bool SWIGLU, bool I8>
 hipError_t launch_t(const GroupedArgs& g, hipStream_t s) {
     constexpr int BN = SWIGLU ? NW * 32 : NW * 64;
     const int tiles_n = (g.N + BN - 1) / BN;
@@ -636,7 +554,7 @@ hipError_t launch_t(const GroupedArgs& g, hipStream_t s) {
     if (tiles_m <= 0) return hipSuccess;
     const int total = tiles_m * tiles_n;
     const int grid = ((total + 7) / 8) * 8;
-    hipLaunchKernelGGL((grouped_stream_kernel<SWIGLU, I8, RING, TFBUF, STAGES, PIPE>), dim3(grid), dim3(NT), 0, s,
+    hipLaunchKernelGGL((grouped_stream_kernel<SWIGLU, I8>), dim3(grid), dim3(NT), 0, s,
                        static_cast<const bf16_t*>(g.a), g.row_index, g.w, g.w_expert_stride * (I8 ? 1 : 2), g.scales,
                        g.s_expert_stride, g.N, g.K, g.tile_expert, g.tile_row0, g.tile_rows, g.ntiles, g.dense_rows,
                        static_cast<bf16_t*>(g.out), static_cast<bf16_t*>(g.gu_out), static_cast<const bf16_t*>(g.swiglu_grad_gu),
@@ -647,30 +565,15 @@ hipError_t launch_t(const GroupedArgs& g, hipStream_t s) {
 
 }  // namespace
 
-template <int RING, int TFBUF, int STAGES, bool PIPE>
-static hipError_t launch_ring(const GroupedArgs& g, WeightKind wk, hipStream_t s) {
-    if (wk == WeightKind::BF16)
-        return g.swiglu ? launch_t<true, false, RING, TFBUF, STAGES, PIPE>(g, s)
-                        : launch_t<false, false, RING, TFBUF, STAGES, PIPE>(g, s);
-    if (wk == WeightKind::I8)
-        return g.swiglu ? launch_t<true, true, RING, TFBUF, STAGES, PIPE>(g, s)
-                        : launch_t<false, true, RING, TFBUF, STAGES, PIPE>(g, s);
-    return hipErrorInvalidValue;
-}
-
 int stream_tile_m() { return BM; }
 
 // K a multiple of 64 (one LDS slice), N a multiple of 32 (row blocks of the packed weights)
 bool stream_shape_ok(int N, int K) { return K % 64 == 0 && K >= 64 && N % 32 == 0 && N >= 32; }
 
-// variant 0: the pipelined main loop (one memory instruction behind each multiply, three LDS stages)
-// variant 1: the loads of a step in one cluster in front of its multiplies, two LDS stages (kept for A/B runs)
-hipError_t launch_grouped_stream(const GroupedArgs& g, WeightKind wk, int variant, hipStream_t s) {
+hipError_t launch_grouped_stream(const GroupedArgs& g, WeightKind wk, hipStream_t s) {
     if (!stream_shape_ok(g.N, g.K)) return hipErrorInvalidValue;
-    switch (variant) {
-        case 0: return launch_ring<4, 2, 3, true>(g, wk, s);
-        case 1: return launch_ring<4, 2, 2, false>(g, wk, s);
-    }
+    if (wk == WeightKind::BF16) return g.swiglu ? launch_t<true, false>(g, s) : launch_t<false, false>(g, s);
+    if (wk == WeightKind::I8) return g.swiglu ? launch_t<true, true>(g, s) : launch_t<false, true>(g, s);
     return hipErrorInvalidValue;
 }
 

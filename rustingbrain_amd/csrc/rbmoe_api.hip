@@ -189,8 +189,9 @@ struct rbmoe_layer {
     bool decode_path = true;   // few tokens: four launches that stream every touched weight once
     bool decode_front = true;  // ... three, with the routing beside the gate/up products, when most experts are touched
     bool shared_beside = true; // large batches: the shared expert's products on the side stream, beside the routing
+    bool fused_router = true;  // logits and everything behind them in one launch where the shapes allow
     bool last_front = false;   // the last forward's hidden rows are per expert over all rows (Work::hall)
-    int group_m = 0, variant = 0;
+    int group_m = 0;
     const char* kernel_name = "none";
     int last_T = -1;
     Work last;  // tables of the last forward
@@ -242,11 +243,6 @@ struct rbmoe_layer {
 
 namespace {
 
-int env_int(const char* name, int fallback) {
-    const char* v = std::getenv(name);
-    return v && v[0] ? std::atoi(v) : fallback;
-}
-
 struct Plan {
     std::vector<std::pair<Buf*, size_t>> items;
     size_t total = 0;
@@ -257,6 +253,34 @@ struct Plan {
         total += bytes;
     }
 };
+
+// Which kernel sets the layer's shapes and dtypes allow (and `force_generic` does not rule out).
+void choose_kernel_sets(rbmoe_layer* L) {
+    const rbmoe_config* cfg = &L->cfg;
+    L->use_stream = L->use_f32_mc = L->cast_rows = false;
+    // bf16 matrix cores: bf16 activations, bf16 or int8 weights, widths that fit the packed layout
+    // (f32 rows with bf16 / int8 weights - what a caller with f32 matrices and a quantized or bf16 checkpoint has -
+    // take the same kernels over a bf16 copy of the rows)
+    const bool mc = !L->force_generic && cfg->weight_dtype != RBMOE_F32;
+    L->use_stream = mc && stream_shape_ok(cfg->d_ff, cfg->d_model) && stream_shape_ok(cfg->d_model, cfg->d_ff) &&
+                    (!cfg->shared_expert ||
+                     (stream_shape_ok(L->Fs, cfg->d_model) && stream_shape_ok(cfg->d_model, L->Fs)));
+
+    L->use_f32_mc = !L->force_generic && cfg->act_dtype == RBMOE_F32 && cfg->weight_dtype == RBMOE_F32 &&
+                    f32_shape_ok(cfg->d_ff, cfg->d_model) && f32_shape_ok(cfg->d_model, cfg->d_ff) &&
+                    (!cfg->shared_expert || (f32_shape_ok(L->Fs, cfg->d_model) && f32_shape_ok(cfg->d_model, L->Fs)));
+    {
+        // the streaming kernel addresses activation rows with 32-bit byte offsets
+        const size_t widest = (size_t)std::max(std::max(cfg->d_model, cfg->d_ff), L->Fs);
+        const size_t rows = (size_t)cfg->max_tokens * (size_t)std::max(1, cfg->experts_per_token);
+        if (rows * widest * 2 >= ((size_t)1 << 32)) L->use_stream = false;
+    }
+    if (cfg->act_dtype == RBMOE_F32 && L->use_stream) {
+        // the bf16 copy is written in 8-element pieces of 16-byte aligned rows
+        if (cfg->d_model % 8 == 0) L->cast_rows = true;
+        else L->use_stream = false;
+    }
+}
 
 Plan make_plan(rbmoe_layer* L) {
     const rbmoe_config& c = L->cfg;
@@ -465,35 +489,11 @@ int rbmoe_layer_create(rbmoe_ctx* ctx, const rbmoe_config* cfg, rbmoe_layer** ou
     L->max_S = cfg->max_tokens * cfg->experts_per_token;
     L->max_nb = (cfg->max_tokens + kRouterTokens - 1) / kRouterTokens;
     L->max_tiles = L->max_S / kGenericTileM + cfg->num_experts + 1;
-    L->force_generic = env_int("RBMOE_FORCE_GENERIC", 0) == 1;
-    L->explicit_gather = env_int("RBMOE_EXPLICIT_GATHER", 0) == 1;
-    L->group_m = std::max(0, env_int("RBMOE_GROUP_M", 0));  // 0: each product's own default
-    L->variant = env_int("RBMOE_STREAM_VARIANT", 0) == 1 ? 1 : 0;
-    L->decode_path = env_int("RBMOE_NO_DECODE_PATH", 0) != 1;
-    L->decode_front = env_int("RBMOE_NO_DECODE_FRONT", 0) != 1;
-    L->shared_beside = env_int("RBMOE_NO_SIDE_STREAM", 0) != 1;
+    // (behaviour switches keep their defaults here: rbmoe_layer_set_option changes them)
     // bf16 matrix cores: bf16 activations, bf16 or int8 weights, widths that fit the packed layout
     // (f32 rows with bf16 / int8 weights - what a caller with f32 matrices and a quantized or bf16 checkpoint has -
     // take the same kernels over a bf16 copy of the rows)
-    const bool mc = !L->force_generic && cfg->weight_dtype != RBMOE_F32;
-    L->use_stream = mc && stream_shape_ok(cfg->d_ff, cfg->d_model) && stream_shape_ok(cfg->d_model, cfg->d_ff) &&
-                    (!cfg->shared_expert ||
-                     (stream_shape_ok(L->Fs, cfg->d_model) && stream_shape_ok(cfg->d_model, L->Fs)));
-
-    L->use_f32_mc = !L->force_generic && cfg->act_dtype == RBMOE_F32 && cfg->weight_dtype == RBMOE_F32 &&
-                    f32_shape_ok(cfg->d_ff, cfg->d_model) && f32_shape_ok(cfg->d_model, cfg->d_ff) &&
-                    (!cfg->shared_expert || (f32_shape_ok(L->Fs, cfg->d_model) && f32_shape_ok(cfg->d_model, L->Fs)));
-    {
-        // the streaming kernel addresses activation rows with 32-bit byte offsets
-        const size_t widest = (size_t)std::max(std::max(cfg->d_model, cfg->d_ff), L->Fs);
-        const size_t rows = (size_t)cfg->max_tokens * (size_t)std::max(1, cfg->experts_per_token);
-        if (rows * widest * 2 >= ((size_t)1 << 32)) L->use_stream = false;
-    }
-    if (cfg->act_dtype == RBMOE_F32 && L->use_stream) {
-        // the bf16 copy is written in 8-element pieces of 16-byte aligned rows
-        if (cfg->d_model % 8 == 0) L->cast_rows = true;
-        else L->use_stream = false;
-    }
+    choose_kernel_sets(L);
 
     Plan plan = make_plan(L);
     // Refuse before allocating anything, as the reference's budget check does
@@ -984,7 +984,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
         HIP_TRY(ctx, hipMemcpyAsync(L->xc.p, x, (size_t)T * d * dtype_size(c.act_dtype), hipMemcpyDeviceToDevice, s));
 
     auto run_on = [&](const GroupedArgs& g, hipStream_t st) -> hipError_t {
-        if (mfma) return launch_grouped_stream(g, wk, L->variant, st);
+        if (mfma) return launch_grouped_stream(g, wk, st);
         if (f32mc) return launch_grouped_f32(g, st);
         return launch_grouped_generic(g, abf, wk, kGenericTileM, st);
     };
@@ -1043,6 +1043,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
                   (float*)L->P.p, (float*)L->lse.p, (int*)L->expert_of.p, (float*)L->gate_of.p,
                   (int*)L->rank_in_block.p, (int*)L->blockcnt.p, (float*)L->partial.p};
     if (cast) ra.rows16 = L->x16.p;
+    ra.allow_fused = L->fused_router;
     HIP_TRY(ctx, launch_router(ra, abf, s));
     HIP_TRY(ctx, mark(1));
 
@@ -1385,10 +1386,7 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
     p.add(&L->wguT, E * d * 2 * F * ws);
     p.add(&L->wg_chunks, (size_t)std::max(weight_grad_table_ints((int)E, (int)S), weight_grad_table_ints(1, (int)T)) * 4);
     // How the weight gradients treat an expert far above the average share (and the shared expert, whose one
-    // group of rows is always cut): in a fixed order by default, RBMOE_ATOMIC_WGRAD=1 for f32 atomics,
-    // RBMOE_DETERMINISTIC=1 for no cut at all.
-    L->wgrad_split = env_int("RBMOE_DETERMINISTIC", 0) == 1 ? WgradSplit::None
-                     : env_int("RBMOE_ATOMIC_WGRAD", 0) == 1 ? WgradSplit::Atomic : WgradSplit::Ordered;
+    // group of rows is always cut): in a fixed order by default (RBMOE_OPT_WGRAD_MODE for f32 atomics or no cut).
     if (L->wgrad_split == WgradSplit::Ordered) {
         const bool wbf = c.act_dtype == RBMOE_BF16;
         // sized for every token count up to max_tokens: a smaller batch can need more partial matrices than the
@@ -1415,13 +1413,46 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
     if (const int rc = allocate_plan(L, p, "the training buffers")) return rc;
     HIP_TRY(ctx, launch_fill_f32((float*)L->ones.p, 1.0f, (long long)S, ctx->stream));
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
-    L->wgrad_generic = env_int("RBMOE_WGRAD_GENERIC", 0) == 1;
-    L->side_branch = env_int("RBMOE_NO_SIDE_STREAM", 0) != 1;
+    L->side_branch = L->shared_beside;
     if (L->side_branch)
         if (const int rc = ensure_side_stream(ctx)) return rc;
     L->training = true;
     L->grads_clear = true;
     return ensure_block_training_buffers(L);
+}
+
+int rbmoe_layer_set_option(rbmoe_layer* L, int32_t option, int32_t value) {
+    if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
+    rbmoe_ctx* ctx = L->ctx;
+    switch (option) {
+        case RBMOE_OPT_FORCE_GENERIC:
+            // the kernel set decides how the weights are laid out on the device
+            if (L->weights_set || L->training)
+                return fail(ctx, RBMOE_INVALID_CONFIG, "choose the kernel set before weights are set or training is enabled");
+            L->force_generic = value != 0;
+            choose_kernel_sets(L);
+            return RBMOE_OK;
+        case RBMOE_OPT_EXPLICIT_GATHER: L->explicit_gather = value != 0; return RBMOE_OK;
+        case RBMOE_OPT_GROUP_M:
+            if (value < 0) return fail(ctx, RBMOE_INVALID_CONFIG, "the group size must not be negative");
+            L->group_m = value;
+            return RBMOE_OK;
+        case RBMOE_OPT_DECODE_PATH: L->decode_path = value != 0; return RBMOE_OK;
+        case RBMOE_OPT_DECODE_FRONT: L->decode_front = value != 0; return RBMOE_OK;
+        case RBMOE_OPT_FUSED_ROUTER: L->fused_router = value != 0; return RBMOE_OK;
+        case RBMOE_OPT_SIDE_STREAM:
+            if (value != 0 && L->training)
+                if (const int rc = ensure_side_stream(ctx)) return rc;
+            L->shared_beside = value != 0;
+            L->side_branch = value != 0;
+            return RBMOE_OK;
+        case RBMOE_OPT_WGRAD_MODE:
+            if (value < 0 || value > 2) return fail(ctx, RBMOE_INVALID_CONFIG, "weight-gradient mode must be 0, 1 or 2");
+            L->wgrad_split = value == 0 ? WgradSplit::Ordered : value == 1 ? WgradSplit::Atomic : WgradSplit::None;
+            return RBMOE_OK;
+        case RBMOE_OPT_WGRAD_GENERIC: L->wgrad_generic = value != 0; return RBMOE_OK;
+    }
+    return fail(ctx, RBMOE_INVALID_CONFIG, "unknown option");
 }
 
 int rbmoe_zero_grads(rbmoe_layer* L) {
@@ -1512,7 +1543,7 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, int32_t tokens, int3
     gh.swiglu_grad_gu = L->gu.p; gh.gu_out = L->dgu.p;  // the hidden gradient goes straight through SwiGLU's backward
     const WeightKind wk = c.weight_dtype == RBMOE_F32 ? WeightKind::F32 : WeightKind::BF16;
     auto prod_on = [&](const GroupedArgs& a, hipStream_t st) -> hipError_t {
-        if (L->use_stream) return launch_grouped_stream(a, WeightKind::BF16, L->variant, st);
+        if (L->use_stream) return launch_grouped_stream(a, WeightKind::BF16, st);
         if (L->use_f32_mc) return launch_grouped_f32(a, st);
         return launch_grouped_generic(a, abf, wk, kGenericTileM, st);
     };

@@ -37,6 +37,7 @@ struct RouterArgs {
     int* blockcnt;       // [nb, E]
     float* partial;      // [nb, E+1]
     void* rows16 = nullptr;  // f32 rows only: [T, d] bf16 copy of x written on the way (d a multiple of 8), or null
+    bool allow_fused = true; // logits and everything behind them in one launch where the shapes allow
 };
 hipError_t launch_router(const RouterArgs& a, bool bf16, hipStream_t s);
 
@@ -125,7 +126,7 @@ constexpr int kGenericTileM = 16;
 // global -> LDS by DMA.  `w` must have been packed matrix by matrix.
 int stream_tile_m();
 bool stream_shape_ok(int N, int K);
-hipError_t launch_grouped_stream(const GroupedArgs& a, WeightKind wk, int variant, hipStream_t s);  // variant 0..1
+hipError_t launch_grouped_stream(const GroupedArgs& a, WeightKind wk, hipStream_t s);
 void pack_weight_bf16(const uint16_t* src, int rows, int cols, uint16_t* dst);
 void pack_weight_i8(const int8_t* src, int rows, int cols, int8_t* dst);
 

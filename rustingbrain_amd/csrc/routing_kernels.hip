@@ -1208,8 +1208,7 @@ __global__ __launch_bounds__(256) void combine_any_kernel(
 // Whether route_fused_kernel takes the call: every expert of a token in one workgroup (at most 64, four per lane),
 // rows of whole 8-element pieces on 16-byte boundaries, and a slice of columns that fits LDS.
 static int fused_cols(const RouterArgs& a, size_t xsize) {
-    static const bool off = [] { const char* v = std::getenv("RBMOE_NO_FUSED_ROUTER"); return v && v[0] == '1'; }();
-    if (off || a.E > 64 || a.d % 8 != 0 || a.d < 8) return 0;
+    if (!a.allow_fused || a.E > 64 || a.d % 8 != 0 || a.d < 8) return 0;
     if ((reinterpret_cast<uintptr_t>(a.x) & 15) || (reinterpret_cast<uintptr_t>(a.wr) & 15)) return 0;
     if (((size_t)a.d * xsize) % 16 != 0) return 0;
     const int cols = a.E <= 32 ? 256 : 128;

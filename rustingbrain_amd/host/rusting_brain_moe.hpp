@@ -256,6 +256,9 @@ class MoeLayer {
     // as an argument; the device layer keeps that state itself, so backward differentiates the last forward.
     void enable_training() { check(rbmoe_layer_enable_training(layer_), device_->raw()); }
 
+    // a behaviour switch of the layer (RBMOE_OPT_*); every default is the fast path
+    void set_option(int option, int value) { check(rbmoe_layer_set_option(layer_, option, value), device_->raw()); }
+
     Matrix backward(const Matrix& grad_output) {
         if (grad_output.cols != d_model_)
             throw InvalidInput("grad_output length " + std::to_string(grad_output.cols) +

@@ -76,6 +76,29 @@ def _check(rc: int, ctx=None) -> None:
     raise _ERRORS.get(rc, NetworkError)((msg or b"").decode() or f"rbmoe status {rc}")
 
 
+# --------------------------------------------------------------------------- switches
+# The library reads no environment variable; this host layer does, for A/B runs of the benchmark and the tests:
+# variable -> (option, value it sets when the variable is "1"), RBMOE_GROUP_M carries its value.
+_ENV_SWITCHES = {
+    "RBMOE_FORCE_GENERIC": (L.OPT_FORCE_GENERIC, 1), "RBMOE_EXPLICIT_GATHER": (L.OPT_EXPLICIT_GATHER, 1),
+    "RBMOE_NO_DECODE_PATH": (L.OPT_DECODE_PATH, 0), "RBMOE_NO_DECODE_FRONT": (L.OPT_DECODE_FRONT, 0),
+    "RBMOE_NO_FUSED_ROUTER": (L.OPT_FUSED_ROUTER, 0), "RBMOE_NO_SIDE_STREAM": (L.OPT_SIDE_STREAM, 0),
+    "RBMOE_ATOMIC_WGRAD": (L.OPT_WGRAD_MODE, 1), "RBMOE_DETERMINISTIC": (L.OPT_WGRAD_MODE, 2),
+    "RBMOE_WGRAD_GENERIC": (L.OPT_WGRAD_GENERIC, 1),
+}
+
+
+def options_from_environment() -> dict:
+    import os
+    out = {}
+    for name, (option, value) in _ENV_SWITCHES.items():
+        if os.environ.get(name, "") == "1":
+            out[option] = value
+    if os.environ.get("RBMOE_GROUP_M", ""):
+        out[L.OPT_GROUP_M] = max(0, int(os.environ["RBMOE_GROUP_M"]))
+    return out
+
+
 # --------------------------------------------------------------------------- config
 @dataclass(frozen=True)
 class MoeConfig:
@@ -232,6 +255,12 @@ class MoeLayer:
         h = C.c_void_p()
         _check(self._lib.rbmoe_layer_create(device.handle, C.byref(cfg), C.byref(h)), device.handle)
         self.handle = h
+        for option, value in options_from_environment().items():
+            self.set_option(option, value)
+
+    def set_option(self, option: int, value: int) -> None:
+        """A behaviour switch of the layer (``_lib.OPT_*``); every default is the fast path."""
+        _check(self._lib.rbmoe_layer_set_option(self.handle, option, value), self.device.handle)
 
     @staticmethod
     def new(d_model: int, config: MoeConfig, device: Device, **kw) -> "MoeLayer":

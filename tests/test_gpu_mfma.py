@@ -17,7 +17,7 @@ pytestmark = pytest.mark.gpu
 
 @pytest.fixture
 def kernel_env():
-    keys = ("RBMOE_GROUP_M", "RBMOE_EXPLICIT_GATHER", "RBMOE_FORCE_GENERIC", "RBMOE_STREAM_VARIANT")
+    keys = ("RBMOE_GROUP_M", "RBMOE_EXPLICIT_GATHER", "RBMOE_FORCE_GENERIC")
     saved = {k: os.environ.get(k) for k in keys}
     yield os.environ
     for k, v in saved.items():
@@ -49,9 +49,7 @@ def run(device, t, valid=None, bias=None):
 @pytest.mark.parametrize("shape", [dict(d=128, E=6, k=2, F=192, T=700), dict(d=64, E=3, k=1, F=64, T=130),
                                    dict(d=256, E=16, k=4, F=128, T=333), dict(d=192, E=5, k=2, F=320, T=1000)],
                          ids=lambda s: "d{d}_E{E}_k{k}_F{F}_T{T}".format(**s))
-@pytest.mark.parametrize("variant", [0, 1])   # 0: pipelined main loop, 1: clustered loads (two LDS stages)
-def test_matrix_core_kernels(device, kernel_env, shape, wt, variant):
-    kernel_env["RBMOE_STREAM_VARIANT"] = str(variant)
+def test_matrix_core_kernels(device, kernel_env, shape, wt):
     E = shape["E"]
     t = synth.make(small_workload(seed=19, act="bf16", wt=wt, shared=True, shared_d_ff=shape["F"] + 64, **shape))
     bias = np.zeros(E, np.float32)
