@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the mixture-of-experts layer forward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--backward]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-backward]
 
 A step is one forward pass of the layer (router, dispatch, grouped SwiGLU expert
 products, combine, auxiliary losses) over one batch of seeded synthetic tokens
@@ -9,8 +9,9 @@ already resident in HBM.  Prints ONE JSON line: tokens/s for the whole layer, th
 roofline of the dominant kernel (the grouped gate/up product) measured with HIP
 events on the library's stream, per-stage figures, and the CPU restatement of
 the reference's rayon path timed on this machine's host cores.  With --backward
-a second layer in training mode is also timed: forward with the backward pass's
-state kept, the backward pass, and both (a "backward" object in the same line).
+a second layer in training mode is also timed (unless --no-backward): forward
+with the backward pass's state kept, the backward pass, and both (a "backward"
+object in the same line).
 """
 from __future__ import annotations
 
@@ -215,13 +216,64 @@ def backward_leg(dev, w, t, x, out, bp, args, alg, with_cpu: bool) -> dict:
     return res
 
 
+class Tools:
+    """The benchmark's helpers (librbmoe_bench.so): one stream that the layer's kernels, the cache flush and the
+    event timer share, set on the device context."""
+
+    def __init__(self, dev):
+        self.lib = L.load_bench()
+        self.dev = dev
+        self.stream, self.timer, self._flush = C.c_void_p(), C.c_void_p(), None
+        self._ck(self.lib.rbbench_stream_create(C.byref(self.stream)), "rbbench_stream_create")
+        self._ck(self.lib.rbbench_timer_create(C.byref(self.timer)), "rbbench_timer_create")
+        dev.set_stream(self.stream.value)
+
+    @staticmethod
+    def _ck(rc, what):
+        if rc != 0:
+            raise RuntimeError(f"{what} failed with code {rc}")
+
+    def use_stream(self):
+        self.dev.set_stream(self.stream.value)
+
+    def start(self):
+        self._ck(self.lib.rbbench_timer_start(self.timer, self.stream), "rbbench_timer_start")
+
+    def stop(self) -> float:
+        ms = C.c_float()
+        self._ck(self.lib.rbbench_timer_stop(self.timer, self.stream, C.byref(ms)), "rbbench_timer_stop")
+        return float(ms.value)
+
+    def flush(self):
+        """Evict L2 and the 256 MiB Infinity Cache with a read-only sweep of 512 MiB (no dirty lines are left to
+        drain while the next kernel runs)."""
+        if self._flush is None:
+            self._flush = C.c_void_p()
+            self._ck(self.lib.rbbench_flush_create(512 << 20, C.byref(self._flush)), "rbbench_flush_create")
+        self._ck(self.lib.rbbench_flush(self._flush, self.stream), "rbbench_flush")
+
+    def flush_handle(self):
+        if self._flush is None:
+            self.flush()
+            self.dev.synchronize()
+        return self._flush
+
+    def close(self):
+        self.dev.synchronize()
+        self.dev.set_stream(None)
+        if self._flush is not None:
+            self.lib.rbbench_flush_destroy(self._flush)
+        self.lib.rbbench_timer_destroy(self.timer)
+        self.lib.rbbench_stream_destroy(self.stream)
+
+
 class ForwardGraph:
     """One forward captured into a HIP graph on a stream of its own (the entry points that take device pointers only
     enqueue kernels, so they can be captured); a replay is one step without the host's launch calls."""
 
-    def __init__(self, dev, enqueue):
+    def __init__(self, dev, tools, enqueue):
         self.hip = C.CDLL("libamdhip64.so")
-        self.dev = dev
+        self.dev, self.tools = dev, tools
         self.stream, self.graph, self.exe = C.c_void_p(), C.c_void_p(), C.c_void_p()
         self._ck(self.hip.hipStreamCreateWithFlags(C.byref(self.stream), 1), "hipStreamCreateWithFlags")
         dev.synchronize()
@@ -230,6 +282,10 @@ class ForwardGraph:
         enqueue()
         self._ck(self.hip.hipStreamEndCapture(self.stream, C.byref(self.graph)), "hipStreamEndCapture")
         self._ck(self.hip.hipGraphInstantiate(C.byref(self.exe), self.graph, None, None, 0), "hipGraphInstantiate")
+        n = C.c_size_t()
+        self.nodes = None
+        if self.hip.hipGraphGetNodes(self.graph, None, C.byref(n)) == 0:
+            self.nodes = int(n.value)
 
     @staticmethod
     def _ck(rc, what):
@@ -244,24 +300,46 @@ class ForwardGraph:
 
     def close(self):
         self.synchronize()
-        self.dev.set_stream(None)
+        self.tools.use_stream()
         self.hip.hipGraphExecDestroy(self.exe)
         self.hip.hipGraphDestroy(self.graph)
         self.hip.hipStreamDestroy(self.stream)
 
 
-def measure(dev, name: str, steps: int, warmup: int, repeats: int, act_override: str = None) -> dict:
-    """One workload: `repeats` loops of `steps` forwards (median loop -> ms_per_step), per-stage durations from HIP
-    events on the library's stream, the roofline of the dominant kernel.  Returns the pieces the report is built of."""
+REPLAY_STAGES = ("router", "dispatch", "gate_up", "down", "combine")
+
+
+def weight_bytes(w: synth.Workload) -> int:
+    sw = {"f32": 4, "bf16": 2, "int8": 1}[w.weight_dtype]
+    Fs = w.shared_d_ff if w.shared_expert else 0
+    return w.num_experts * 3 * w.d_model * w.d_ff * sw + 3 * w.d_model * Fs * sw + w.num_experts * w.d_model * 4
+
+
+def measure(dev, tools, name: str, steps: int, warmup: int, repeats: int, act_override: str = None) -> dict:
+    """One workload.
+    * `repeats` loops of `steps` forwards of one layer back to back (median loop -> ms_per_step): weights that fit
+      the 256 MiB Infinity Cache stay there;
+    * the launch time of each stage by itself: the stage's launches of the last forward replayed 20 times between
+      ONE pair of events (rbmoe_replay_stage), median of three such runs -> the roofline of the dominant kernel;
+    * the same two measurements over several layers with their own copies of the weights (more than the Infinity
+      Cache holds in all), forwards and stage launches issued in rotation: every launch finds its weights in HBM;
+    * forwards with L2 and Infinity Cache flushed by a read-only sweep before each one, each forward timed by an
+      event pair of its own (raw interval);
+    * per-stage event intervals inside one forward (rbmoe_forward_timed), kept for comparison."""
     w = synth.WORKLOADS[name]
     t = synth.make(w)
     if act_override:
         w = synth.Workload(**{**w.__dict__, "act_dtype": act_override})
     T = w.tokens
     cfg = rb.MoeConfig(w.num_experts, w.experts_per_token, w.d_ff, w.shared_expert)
-    layer = rb.MoeLayer(w.d_model, cfg, dev, act_dtype=w.act_dtype, weight_dtype=w.weight_dtype, max_tokens=T,
-                        shared_d_ff=w.shared_d_ff if w.shared_expert else 0)
-    layer.load_tensors(t)
+
+    def new_layer():
+        layer = rb.MoeLayer(w.d_model, cfg, dev, act_dtype=w.act_dtype, weight_dtype=w.weight_dtype, max_tokens=T,
+                            shared_d_ff=w.shared_d_ff if w.shared_expert else 0)
+        layer.load_tensors(t)
+        return layer
+
+    layer = new_layer()
     bf16 = w.act_dtype == "bf16"
     xh = synth.f32_to_bf16_bits(t.x) if bf16 else t.x
     x = DeviceBuffer(dev, xh.nbytes).upload(xh)
@@ -269,65 +347,115 @@ def measure(dev, name: str, steps: int, warmup: int, repeats: int, act_override:
     bias = DeviceBuffer(dev, 4 * w.num_experts).upload(t.router_bias) if t.router_bias is not None else None
     bp = bias.ptr if bias else 0
 
+    def fwd(lay=None):
+        (lay or layer).forward_device(x.ptr, T, out.ptr, bias_ptr=bp)
+
+    def wall_loops(fn, n_steps, n_repeats, sync):
+        loops = []
+        for _ in range(n_repeats):
+            t0 = time.perf_counter()
+            for i in range(n_steps):
+                fn(i)
+            sync()
+            loops.append((time.perf_counter() - t0) * 1e3 / n_steps)
+        return loops
+
     for _ in range(warmup):
-        layer.forward_device(x.ptr, T, out.ptr, bias_ptr=bp)
+        fwd()
     dev.synchronize()
-    loops = []
-    for _ in range(repeats):
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            layer.forward_device(x.ptr, T, out.ptr, bias_ptr=bp)
-        dev.synchronize()
-        loops.append((time.perf_counter() - t0) * 1e3 / steps)
+    loops = wall_loops(lambda i: fwd(), steps, repeats, dev.synchronize)
     ms_per_step = float(np.median(loops))
 
     decode = "decode" in layer.kernel_name()   # the library takes the decode-shaped kernels up to 32 tokens
-    graph_ms = None
+    graph = None
     if decode:
         # A decode step is three short launches: issued one by one from this interpreter, the host's launch calls
         # are part of the step.  The same forward replayed from a HIP graph, timed the same way:
-        g = ForwardGraph(dev, lambda: layer.forward_device(x.ptr, T, out.ptr, bias_ptr=bp))
+        g = ForwardGraph(dev, tools, fwd)
         for _ in range(warmup):
             g.replay()
         g.synchronize()
-        gl = []
-        for _ in range(repeats):
-            t0 = time.perf_counter()
-            for _ in range(steps):
-                g.replay()
-            g.synchronize()
-            gl.append((time.perf_counter() - t0) * 1e3 / steps)
+        gl = wall_loops(lambda i: g.replay(), steps, repeats, g.synchronize)
+        graph = {"ms_per_step": float(np.median(gl)), "nodes": g.nodes}
         g.close()
-        graph_ms = float(np.median(gl))
-    nprof = max(10, min(100, steps))
 
-    def timed_stages(flush=None):
+    # ---- each stage by itself, one event pair over 20 launches
+    fwd()
+    dev.synchronize()
+    launch_ms = {}
+    for st in REPLAY_STAGES:
+        v = [layer.replay_stage(st, 20) for _ in range(3)]
+        launch_ms[st] = None if v[0] is None else float(np.median(v))
+
+    # ---- kernel durations inside a forward: every launch carries its own start / stop events, which receive the
+    # dispatch's own begin and end time stamps (what a kernel trace reports for the same launch)
+    nprof = max(10, min(50, steps))
+
+    def kernel_times(flush: bool):
         acc = {}
         for _ in range(nprof):
-            if flush is not None:
-                # evict the weights from L2 and the 256 MiB Infinity Cache: stream 2 x 512 MiB through them
-                assert dev._lib.rbmoe_copy_device(dev.handle, C.c_void_p(flush[1].ptr), C.c_void_p(flush[0].ptr),
-                                                  flush[0].nbytes) == L.OK
-            st = layer.forward_timed(x.ptr, T, out.ptr, bias_ptr=bp)
-            for nm, v in st.items():
+            if flush:
+                tools.flush()
+            for nm, v in layer.forward_kernel_times(x.ptr, T, out.ptr, bias_ptr=bp).items():
                 acc.setdefault(nm, []).append(v)
-        raw = {nm: float(np.mean(v)) for nm, v in acc.items()}
-        # One interval of forward_timed brackets no work: what a pair of event records adds to every
-        # other interval.  Kernel durations are the intervals minus that.
-        over = raw["empty"]
-        net = {nm: (v if nm in ("empty", "total") else max(v - over, 1e-6)) for nm, v in raw.items()}
-        mins = {nm: float(np.min(v)) for nm, v in acc.items()}
-        return raw, net, mins, over
+        return {nm: float(np.mean(v)) for nm, v in acc.items()}, {nm: float(np.min(v)) for nm, v in acc.items()}
 
-    raw_ms, stage_ms, stage_ms_min, overhead = timed_stages()
-    cold = None
-    if decode:
-        # A decode step's 58 MB of weights fit the Infinity Cache, so back-to-back forwards never go to
-        # HBM.  The roofline figure is therefore taken with the caches flushed before every forward.
-        fl = (DeviceBuffer(dev, 512 << 20), DeviceBuffer(dev, 512 << 20))
-        cold = timed_stages(flush=fl)
-        fl[0].free()
-        fl[1].free()
+    kernel_ms, kernel_ms_min = kernel_times(False)
+    # ---- event intervals between the stages of one forward (each carries the cost of an event pair: `empty`)
+    acc = {}
+    for _ in range(nprof):
+        for nm, v in layer.forward_timed(x.ptr, T, out.ptr, bias_ptr=bp).items():
+            acc.setdefault(nm, []).append(v)
+    raw_ms = {nm: float(np.mean(v)) for nm, v in acc.items()}
+    over = raw_ms["empty"]
+
+    # ---- caches flushed (a read-only sweep of 512 MiB) before every forward
+    cold_kernel_ms, _ = kernel_times(True)
+    flushed = []
+    for _ in range(max(10, min(30, steps))):
+        tools.flush()
+        tools.start()
+        fwd()
+        flushed.append(tools.stop())
+    cold_flush = {"kernel_ms": cold_kernel_ms, "ms_per_step_raw_interval": float(np.median(flushed)),
+                  "event_interval_overhead_ms": over,
+                  "note": "a read-only sweep of 512 MiB before every forward.  kernel_ms: the dispatches' own time "
+                          "stamps, per stage; ms_per_step_raw_interval: one event pair around the whole forward, "
+                          "nothing subtracted"}
+
+    # ---- several layers with their own copies of the weights, in rotation
+    wb = weight_bytes(w)
+    nlayers = int(max(4, min(16, -(-(512 << 20) // wb))))
+    layers = [layer] + [new_layer() for _ in range(nlayers - 1)]
+    for lay in layers:
+        fwd(lay)
+    dev.synchronize()
+    rr_steps = max(nlayers * 2, (max(20, steps // 2) // nlayers) * nlayers)
+    rr_loops = wall_loops(lambda i: fwd(layers[i % nlayers]), rr_steps, max(3, min(repeats, 5)), dev.synchronize)
+    rr_ms = float(np.median(rr_loops))
+    rr_launch = {}
+    rounds = max(1, 20 // nlayers)
+    for st in REPLAY_STAGES:
+        if launch_ms[st] is None:
+            rr_launch[st] = None
+            continue
+        v = []
+        for _ in range(3):
+            for lay in layers:      # untimed: the rotation is in steady state when the interval starts
+                lay.enqueue_stage(st)
+            tools.start()
+            for _ in range(rounds):
+                for lay in layers:
+                    lay.enqueue_stage(st)
+            v.append(tools.stop() / (rounds * nlayers))
+        rr_launch[st] = float(np.median(v))
+    for lay in layers[1:]:
+        lay.close()
+    round_robin = {"layers": nlayers, "weight_bytes_per_layer": wb, "weight_bytes_total": wb * nlayers,
+                   "ms_per_step": rr_ms, "tokens_per_s": T / (rr_ms * 1e-3), "stage_launch_ms": rr_launch,
+                   "note": "layers with their own copies of the weights (same values, distinct addresses, more than "
+                           "the 256 MiB Infinity Cache in all), forwards issued in rotation; stage_launch_ms: the "
+                           "stage's launches of all layers in rotation between one pair of events"}
 
     cache = layer.cache(T)
     routed = int(cache.offsets[-1])
@@ -336,71 +464,78 @@ def measure(dev, name: str, steps: int, warmup: int, repeats: int, act_override:
     peak_tf = PEAK_F32_TFLOPS if (w.weight_dtype == "f32") else PEAK_BF16_TFLOPS
 
     def tflops(flops, ms):
-        return flops / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
+        return flops / (ms * 1e-3) / 1e12 if ms and ms > 0 else 0.0
 
     def gbs(nbytes, ms):
-        return nbytes / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
+        return nbytes / (ms * 1e-3) / 1e9 if ms and ms > 0 else 0.0
 
     kname = layer.kernel_name()
     traffic, traffic_source = measured_traffic(w.name, kname)
-    gu = tflops(alg["gate_up_flops"], stage_ms["gate_up"])
+    timing = ("start / stop events carried by the launch itself (the dispatch's own begin and end time stamps, as in a "
+              "kernel trace), mean over %d forwards" % nprof)
     if decode:
-        # the dominant kernel of the decode-shaped path streams the gate/up weights of the touched experts
-        # (and of the shared expert) once: it is bound by HBM
-        cold_ms = cold[1]
-        gu_gbs = gbs(alg["decode_gate_up_bytes"], cold_ms["gate_up"])
+        # the dominant kernel of the decode-shaped path streams the gate/up weights of the touched experts (and of
+        # the shared expert) once: it is bound by HBM, and is measured where its weights come from HBM
+        ms_gu = cold_kernel_ms["gate_up"]
+        gu_gbs = gbs(alg["decode_gate_up_bytes"], ms_gu)
         roofline = {"bound": "hbm", "kernel": "decode gate/up product + SwiGLU, routed and shared (" + kname +
                                               "), caches flushed before every forward",
                     "achieved": gu_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gu_gbs / PEAK_HBM_GBS,
                     "traffic": traffic, "traffic_source": traffic_source,
-                    "bytes_per_launch": alg["decode_gate_up_bytes"],
-                    "avg_launch_ms": cold_ms["gate_up"], "touched_experts": touched,
-                    "cache_resident_gbs": gbs(alg["decode_gate_up_bytes"], stage_ms["gate_up"])}
+                    "bytes_per_launch": alg["decode_gate_up_bytes"], "avg_launch_ms": ms_gu, "timing": timing,
+                    "touched_experts": touched,
+                    "frac_layers_in_rotation": gbs(alg["decode_gate_up_bytes"], rr_launch["gate_up"]) / PEAK_HBM_GBS,
+                    "cache_resident_gbs": gbs(alg["decode_gate_up_bytes"], kernel_ms["gate_up"])}
     else:
+        gu = tflops(alg["gate_up_flops"], kernel_ms["gate_up"])
         roofline = {"bound": "mfma", "kernel": "grouped gate/up product + SwiGLU (" + kname + ")",
                     "achieved": gu, "peak": peak_tf, "unit": "TFLOP/s", "frac": gu / peak_tf,
                     "traffic": traffic, "traffic_source": traffic_source,
-                    "flops_per_launch": alg["gate_up_flops"], "avg_launch_ms": stage_ms["gate_up"]}
-    both_ms = stage_ms["gate_up"] + stage_ms["down"] + stage_ms["shared"]
+                    "flops_per_launch": alg["gate_up_flops"], "avg_launch_ms": kernel_ms["gate_up"],
+                    "min_launch_ms": kernel_ms_min["gate_up"], "timing": timing,
+                    "frac_back_to_back": tflops(alg["gate_up_flops"], launch_ms["gate_up"]) / peak_tf,
+                    "frac_weights_from_hbm": tflops(alg["gate_up_flops"], cold_kernel_ms["gate_up"]) / peak_tf}
+    prod_ms = kernel_ms["gate_up"] + kernel_ms["down"]
     stages = {
-        "ms_mean": stage_ms, "ms_mean_raw_intervals": raw_ms, "ms_min_raw_intervals": stage_ms_min,
-        "event_interval_overhead_ms": overhead,
-        "gate_up_tflops": gu,
-        "down_tflops": tflops(alg["down_flops"], stage_ms["down"]),
-        "grouped_gemms_tflops": tflops(alg["gemm_flops"], both_ms),
-        "grouped_gemms_frac_of_peak": tflops(alg["gemm_flops"], both_ms) / peak_tf,
-        # the HBM-bound stages, on the same net intervals as the products
-        "router_gbs": gbs(alg["router_bytes"], stage_ms["router"]),
-        "dispatch_gbs": gbs(alg["dispatch_bytes"], stage_ms["dispatch"]),
+        "kernel_ms": kernel_ms, "kernel_ms_min": kernel_ms_min, "kernel_ms_timing": timing,
+        "launch_ms_back_to_back": launch_ms,
+        "launch_ms_back_to_back_timing": "20 launches of the stage between one pair of HIP events, median of 3 runs "
+                                         "(sustained: the clocks settle lower than inside a forward)",
+        "ms_mean_raw_intervals": raw_ms, "event_interval_overhead_ms": over,
+        "gate_up_tflops": tflops(alg["gate_up_flops"], kernel_ms["gate_up"]),
+        "down_tflops": tflops(alg["down_flops"], kernel_ms["down"]),
+        "down_frac_of_peak": tflops(alg["down_flops"], kernel_ms["down"]) / peak_tf,
+        # the routed experts' two products
+        "grouped_gemms_tflops": tflops(alg["gate_up_flops"] + alg["down_flops"], prod_ms),
+        "grouped_gemms_frac_of_peak": tflops(alg["gate_up_flops"] + alg["down_flops"], prod_ms) / peak_tf,
+        "router_gbs": gbs(alg["router_bytes"], kernel_ms["router"]),
+        "dispatch_gbs": gbs(alg["dispatch_bytes"], kernel_ms["dispatch"]),
         "dispatch_note": "latency-bound: a few hundred KB of indices per launch, no rows are moved",
-        # A launch of a few microseconds sits between its raw event interval (launch plus what an event pair adds)
-        # and the net one (which takes off more than the pair really cost): both are given, the kernel-trace
-        # duration under profiles/ lies between them.
-        "combine_gbs": gbs(alg["combine_bytes"], stage_ms["combine"]),
-        "combine_frac_of_hbm": gbs(alg["combine_bytes"], stage_ms["combine"]) / PEAK_HBM_GBS,
-        "combine_frac_of_hbm_raw_interval": gbs(alg["combine_bytes"], raw_ms["combine"]) / PEAK_HBM_GBS,
+        "combine_gbs": gbs(alg["combine_bytes"], kernel_ms["combine"]),
+        "combine_frac_of_hbm": gbs(alg["combine_bytes"], kernel_ms["combine"]) / PEAK_HBM_GBS,
+        "launch_gaps_ms": ms_per_step - kernel_ms["total"],
     }
     if decode:
-        whole = gbs(alg["layer_bytes_decode"], ms_per_step)
-        cold_ms = cold[1]
-        cold_kernels = sum(cold_ms[n] for n in ("router", "dispatch", "gate_up", "down", "shared", "combine"))
-        stages.update({"cold_ms_mean": cold_ms,
-                       "cold_decode_down_gbs": gbs(alg["decode_down_bytes"], cold_ms["down"]),
-                       "cold_decode_down_frac_of_hbm": gbs(alg["decode_down_bytes"], cold_ms["down"]) / PEAK_HBM_GBS,
-                       "cold_whole_layer_ms": cold_kernels,
-                       "cold_whole_layer_gbs": gbs(alg["layer_bytes_decode"], cold_kernels),
-                       "cold_whole_layer_frac_of_hbm": gbs(alg["layer_bytes_decode"], cold_kernels) / PEAK_HBM_GBS,
-                       "cache_resident_whole_layer_gbs": whole,
-                       "whole_layer_bytes": alg["layer_bytes_decode"],
-                       "note": "value / ms_per_step are back-to-back forwards (weights stay in the 256 MiB "
-                               "Infinity Cache); cold_* figures flush L2 and Infinity Cache before every forward"})
+        cold_kernels = cold_kernel_ms["total"]
+        stages.update({
+            "whole_layer_bytes": alg["layer_bytes_decode"],
+            "cold_kernel_ms": cold_kernel_ms,
+            "cold_decode_down_frac_of_hbm": gbs(alg["decode_down_bytes"], cold_kernel_ms["down"]) / PEAK_HBM_GBS,
+            "cold_whole_layer_ms": cold_kernels,
+            "cold_whole_layer_frac_of_hbm": gbs(alg["layer_bytes_decode"], cold_kernels) / PEAK_HBM_GBS,
+            "rotation_whole_layer_frac_of_hbm_per_step": gbs(alg["layer_bytes_decode"], rr_ms) / PEAK_HBM_GBS,
+            "cache_resident_whole_layer_gbs": gbs(alg["layer_bytes_decode"], ms_per_step),
+            "note": "value / ms_per_step are back-to-back forwards of one layer (weights stay in the 256 MiB "
+                    "Infinity Cache); cold_* figures flush L2 and Infinity Cache before every forward and sum the "
+                    "kernels' own durations; rotation_*: layers with their own weights in rotation, whole step "
+                    "(launch gaps included)"})
     config = {"workload": w.name, "d_model": w.d_model, "num_experts": w.num_experts,
               "experts_per_token": w.experts_per_token, "d_ff": w.d_ff, "tokens": T,
               "shared_expert": w.shared_expert, "weight_dtype": w.weight_dtype, "act_dtype": w.act_dtype,
               "seed": w.seed, "expert0_share": float(cache.load_fractions()[0]), "routed_slots": routed}
     return {"w": w, "t": t, "layer": layer, "x": x, "out": out, "bias": bias, "bp": bp, "alg": alg,
             "ms_per_step": ms_per_step, "loops_ms": loops, "roofline": roofline, "stages": stages, "config": config,
-            "bf16": bf16, "decode": decode, "graph_ms": graph_ms}
+            "bf16": bf16, "decode": decode, "graph": graph, "cold_flush": cold_flush, "round_robin": round_robin}
 
 
 def two_in_flight(w, t, steps: int, warmup: int, repeats: int) -> dict:
@@ -457,20 +592,29 @@ def release(m: dict) -> None:
 
 def summary(m: dict) -> dict:
     """The short form of one workload for the `workloads` object of the report."""
-    r, st = m["roofline"], m["stages"]
+    r, st, rr = m["roofline"], m["stages"], m["round_robin"]
     s = {"tokens_per_s": m["config"]["tokens"] / (m["ms_per_step"] * 1e-3), "ms_per_step": m["ms_per_step"],
          "kernel": r["kernel"], "bound": r["bound"], "frac": r["frac"], "achieved": r["achieved"], "unit": r["unit"],
          "peak": r["peak"], "avg_launch_ms": r["avg_launch_ms"], "traffic": r["traffic"],
-         "stage_ms": {k: round(v, 5) for k, v in st["ms_mean"].items()},
-         "grouped_gemms_frac_of_peak": st["grouped_gemms_frac_of_peak"], "config": m["config"]}
+         "kernel_ms": {k: round(v, 5) for k, v in st["kernel_ms"].items()},
+         "launch_gaps_ms": st["launch_gaps_ms"],
+         "down_frac_of_peak": st["down_frac_of_peak"],
+         "grouped_gemms_frac_of_peak": st["grouped_gemms_frac_of_peak"],
+         "cold": m["cold_flush"],
+         "layers_round_robin": {"layers": rr["layers"], "ms_per_step": rr["ms_per_step"],
+                                "tokens_per_s": rr["tokens_per_s"],
+                                "stage_launch_ms": {k: (None if v is None else round(v, 5))
+                                                    for k, v in rr["stage_launch_ms"].items()}},
+         "config": m["config"]}
     if m["decode"]:
-        s.update({"cold": {"gate_up_frac_of_hbm": r["frac"], "gate_up_ms": r["avg_launch_ms"],
-                           "down_frac_of_hbm": st["cold_decode_down_frac_of_hbm"],
-                           "whole_layer_ms": st["cold_whole_layer_ms"],
-                           "whole_layer_frac_of_hbm": st["cold_whole_layer_frac_of_hbm"]},
-                  "warm": {"gate_up_gbs": r["cache_resident_gbs"], "whole_layer_ms": m["ms_per_step"],
-                           "whole_layer_gbs": st["cache_resident_whole_layer_gbs"],
-                           "whole_layer_ms_graph_replay": m["graph_ms"]}})
+        s["cold"] = dict(m["cold_flush"], gate_up_frac_of_hbm=r["frac"], gate_up_ms=r["avg_launch_ms"],
+                         down_frac_of_hbm=st["cold_decode_down_frac_of_hbm"], whole_layer_ms=st["cold_whole_layer_ms"],
+                         whole_layer_frac_of_hbm=st["cold_whole_layer_frac_of_hbm"],
+                         rotation_whole_layer_frac_of_hbm_per_step=st["rotation_whole_layer_frac_of_hbm_per_step"])
+        s["warm"] = {"gate_up_gbs": r["cache_resident_gbs"], "whole_layer_ms": m["ms_per_step"],
+                     "whole_layer_gbs": st["cache_resident_whole_layer_gbs"],
+                     "whole_layer_ms_graph_replay": m["graph"]["ms_per_step"] if m["graph"] else None,
+                     "graph_nodes": m["graph"]["nodes"] if m["graph"] else None}
     return s
 
 
@@ -487,8 +631,10 @@ def main() -> int:
                     help="the workload of the top-level figures (the metric is quoted on the default)")
     ap.add_argument("--only", action="store_true", help="skip the `workloads` object (the other four workloads)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--backward", action="store_true",
-                    help="also time the backward pass (bf16 layers and all-f32 layers)")
+    ap.add_argument("--no-backward", action="store_true",
+                    help="skip the training-step figures (the `backward` object: forward in training mode, backward "
+                         "pass, both; bf16 layers and all-f32 layers)")
+    ap.add_argument("--backward", action="store_true", help="(the training-step figures are on by default)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (the plain copy that FETCH_SIZE / "
                          "WRITE_SIZE readings are scaled by when this command runs under rocprofv3 --pmc)")
@@ -505,7 +651,8 @@ def main() -> int:
         return 2
 
     dev = rb.Device.open(0)
-    m = measure(dev, args.workload, args.steps, args.warmup, args.repeats)
+    tools = Tools(dev)
+    m = measure(dev, tools, args.workload, args.steps, args.warmup, args.repeats)
     w, T = m["w"], m["w"].tokens
     result = {
         "metric": "MoE-layer fwd tokens/sec at d768 E16 k2; grouped-GEMM % of bf16 MFMA peak",
@@ -513,10 +660,11 @@ def main() -> int:
         "warmup": args.warmup, "repeats": args.repeats, "ms_per_step": m["ms_per_step"],
         "ms_per_step_loops": m["loops_ms"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16" if w.weight_dtype != "f32" else "f32", "data": "synthetic",
-        "config": m["config"], "roofline": m["roofline"], "stages": m["stages"],
+        "config": m["config"], "roofline": m["roofline"], "stages": m["stages"], "cold": m["cold_flush"],
+        "layers_round_robin": m["round_robin"],
     }
-    if m["graph_ms"] is not None:
-        result["ms_per_step_graph_replay"] = m["graph_ms"]
+    if m["graph"] is not None:
+        result["graph_replay"] = m["graph"]
     if args.calibrate_copy:
         n = 256 << 20
         a, b = DeviceBuffer(dev, n), DeviceBuffer(dev, n)
@@ -526,47 +674,50 @@ def main() -> int:
     calibration = {}
     if args.calibrate_mfma:
         tf, ms = C.c_double(), C.c_double()
-        assert dev._lib.rbmoe_calibrate_mfma(dev.handle, 10, C.byref(tf), C.byref(ms)) == L.OK
+        assert tools.lib.rbbench_mfma_only(tools.stream, 10, C.byref(tf), C.byref(ms)) == 0
         calibration["mfma"] = {"tflops": tf.value, "avg_launch_ms": ms.value, "frac_of_published_peak":
                                tf.value / PEAK_BF16_TFLOPS, "kernel": "mfma_only_kernel: 32x32x16 bf16 multiplies only, "
-                               "two waves per SIMD"}
+                               "two waves per SIMD, 10 launches between one pair of events"}
     if args.calibrate_read:
         n = 39 * (1 << 20)
         rd = {}
-        for label, flush in (("cold", 1), ("warm", 0)):
+        for label, flush in (("cold", tools.flush_handle()), ("warm", None)):
             g, ms = C.c_double(), C.c_double()
-            assert dev._lib.rbmoe_calibrate_read(dev.handle, n, 20, flush, C.byref(g), C.byref(ms)) == L.OK
+            assert tools.lib.rbbench_read(tools.stream, n, 20, flush, C.byref(g), C.byref(ms)) == 0
             rd[label] = {"gbs": g.value, "avg_launch_ms": ms.value, "frac_of_hbm_peak": g.value / PEAK_HBM_GBS}
         rd["bytes"] = n
-        rd["note"] = ("event interval around each launch of read_only_kernel minus the interval of an empty event "
-                      "pair; cold: a 512 MiB copy runs before every launch")
+        rd["note"] = ("warm: 20 launches of read_only_kernel between one pair of events; cold: a read-only sweep of "
+                      "512 MiB before every launch, each launch in an event pair of its own, raw interval")
         calibration["read"] = rd
     if calibration:
         result["calibration"] = calibration
-    if args.backward:
+    if not args.no_backward:
         result["backward"] = backward_leg(dev, w, m["t"], m["x"], m["out"], m["bp"], args, m["alg"],
-                                          with_cpu=not args.no_cpu)
+                                          with_cpu=args.backward and not args.no_cpu)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(m["t"])
-    if not m["decode"]:
-        result["two_batches_in_flight"] = two_in_flight(w, m["t"], args.steps, args.warmup, max(3, min(args.repeats, 5)))
     release(m)
+    if not m["decode"]:
+        tools.close()
+        result["two_batches_in_flight"] = two_in_flight(w, m["t"], args.steps, args.warmup, max(3, min(args.repeats, 5)))
+        tools = Tools(dev)
     if not args.only:
         # the other workloads, shorter loops: parity-test cases as far as the metric goes, reported for their
-        # kernels' rooflines (C2: the decode-shaped target, cold and warm)
+        # kernels' rooflines (C2: the decode-shaped target, with weights from HBM and cache-resident)
         others = {}
         for name in synth.WORKLOADS:
             if name == args.workload:
                 continue
-            o = measure(dev, name, max(20, args.steps // 4), max(5, args.warmup // 2), max(3, min(args.repeats, 5)))
+            o = measure(dev, tools, name, max(20, args.steps // 4), max(5, args.warmup // 2), max(3, min(args.repeats, 5)))
             others[name] = summary(o)
             release(o)
         # the int8 workload with f32 rows on the boundary: what a caller with f32 matrices and a quantized
         # checkpoint runs (the router reads the f32 rows, the products their bf16 copy)
-        o = measure(dev, "c5_int8_d768_e8", max(20, args.steps // 4), max(5, args.warmup // 2), 3, act_override="f32")
+        o = measure(dev, tools, "c5_int8_d768_e8", max(20, args.steps // 4), max(5, args.warmup // 2), 3, act_override="f32")
         others["c5_int8_d768_e8_f32_rows"] = summary(o)
         release(o)
         result["workloads"] = others
+    tools.close()
     print(json.dumps(result))
     return 0
 

@@ -287,6 +287,27 @@ int rbmoe_forward_timed(rbmoe_layer* layer, const void* x, int32_t T, int32_t co
                         const uint8_t* valid, const float* router_bias, const void* residual,
                         void* out, float* ms);
 
+/* Kernel durations of one forward the way a kernel trace reports them: every launch of the forward carries its own
+ * start and stop events, which receive the begin and end time stamps of that dispatch itself (no launch gap, no
+ * event-pair overhead, no events between the stages).  `ms` receives RBMOE_NUM_STAGES values in milliseconds: per
+ * stage the sum over its launches (RBMOE_STAGE_EMPTY: 0), RBMOE_STAGE_TOTAL: their sum - the time the device spent
+ * inside kernels, which is less than the forward took by the gaps between the launches.  Synchronises.  Like
+ * rbmoe_forward_timed, the call runs the shared expert on the main stream. */
+int rbmoe_forward_kernel_times(rbmoe_layer* layer, const void* x, int32_t T, int32_t cols,
+                               const uint8_t* valid, const float* router_bias, const void* residual,
+                               void* out, float* ms);
+
+/* Launch time of one stage by itself: enqueues the launches of stage `stage` (RBMOE_STAGE_ROUTER, _DISPATCH,
+ * _GATE_UP, _DOWN or _COMBINE) of the LAST forward again, on the same buffers, once untimed and then `launches`
+ * times back to back between ONE pair of events, and returns the average in milliseconds.  Synchronises.  The
+ * stages read their inputs and overwrite their outputs with the same values, so the layer's state is unchanged.
+ * A figure taken this way contains no event-pair overhead (one pair over many launches) and cannot fall below
+ * what a kernel trace shows for the launch; the operands a stage shares with its neighbours in a forward may sit
+ * in other cache levels here.  With ms_per_launch == NULL the launches are only enqueued (no warm-up, no events, no
+ * synchronisation): for a caller that times a sequence of its own, e.g. the same stage of several layers in
+ * rotation.  RBMOE_UNSUPPORTED when the last forward had no launch of its own for the stage. */
+int rbmoe_replay_stage(rbmoe_layer* layer, int32_t stage, int32_t launches, float* ms_per_launch);
+
 /* Name of the kernel variant the last forward used for the expert products
  * ("mfma_bf16", "generic", ...), for reports.  Static storage. */
 const char* rbmoe_expert_kernel_name(const rbmoe_layer* layer);
@@ -300,18 +321,6 @@ int rbmoe_copy_to_host(rbmoe_ctx* ctx, void* dst, const void* src, size_t bytes)
  * plain copy of known size that hardware-counter readings are calibrated against). */
 int rbmoe_copy_device(rbmoe_ctx* ctx, void* dst, const void* src, size_t bytes);
 
-/* ---- calibration: what the device sustains, for roofline figures to be read against.  No counterpart in the
- * reference; neither touches a layer.  Both allocate their own buffers, time `launches` launches with HIP events on
- * the context's stream and synchronise.  rbmoe_calibrate_read times every launch by itself and takes off what a pair
- * of event records with nothing between them reads in the same call (a few microseconds, as much as the launch).
- * rbmoe_calibrate_mfma: a kernel of nothing but 32x32x16 bf16 matrix-core multiplies, two waves on every SIMD, about
- * 0.25 ms a launch -> the multiply rate the matrix cores sustain at the clock they settle at.
- * rbmoe_calibrate_read: a plain read of `bytes` (16-byte loads; split over 512, 1024 and 2048 workgroups, the fastest
- * split is reported); with `flush_caches` != 0 a 512 MiB copy runs before every launch, which is then timed by
- * itself, so that the read comes from HBM as a decode step's weights do; otherwise the launches run back to back. */
-int rbmoe_calibrate_mfma(rbmoe_ctx* ctx, int32_t launches, double* tflops, double* avg_launch_ms);
-int rbmoe_calibrate_read(rbmoe_ctx* ctx, size_t bytes, int32_t launches, int32_t flush_caches, double* gbs,
-                         double* avg_launch_ms);
 
 const char* rbmoe_version(void);
 

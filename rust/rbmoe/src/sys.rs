@@ -101,6 +101,9 @@ extern "C" {
     pub fn rbmoe_forward_timed(layer: *mut rbmoe_layer, x: *const c_void, tokens: i32, cols: i32, valid: *const u8,
                                router_bias: *const f32, residual: *const c_void, out: *mut c_void,
                                ms: *mut f32) -> c_int;
+    pub fn rbmoe_forward_kernel_times(layer: *mut rbmoe_layer, x: *const c_void, tokens: i32, cols: i32, valid: *const u8,
+                               router_bias: *const f32, residual: *const c_void, out: *mut c_void,
+                               ms: *mut f32) -> c_int;
     pub fn rbmoe_get_losses(layer: *mut rbmoe_layer, aux_loss: *mut f32, z_loss: *mut f32) -> c_int;
     pub fn rbmoe_get_routing(layer: *mut rbmoe_layer, routing: *mut rbmoe_routing) -> c_int;
     pub fn rbmoe_get_expert_rows(layer: *mut rbmoe_layer, hidden: *mut f32, expert_out: *mut f32) -> c_int;
@@ -130,8 +133,6 @@ extern "C" {
     pub fn rbmoe_copy_to_host(ctx: *mut rbmoe_ctx, dst: *mut c_void, src: *const c_void, bytes: usize) -> c_int;
     pub fn rbmoe_copy_device(ctx: *mut rbmoe_ctx, dst: *mut c_void, src: *const c_void, bytes: usize) -> c_int;
     // calibration: a multiply-only kernel and a plain read, for roofline figures to be read against
-    pub fn rbmoe_calibrate_mfma(ctx: *mut rbmoe_ctx, launches: i32, tflops: *mut f64, avg_launch_ms: *mut f64) -> c_int;
-    pub fn rbmoe_calibrate_read(ctx: *mut rbmoe_ctx, bytes: usize, launches: i32, flush_caches: i32, gbs: *mut f64,
-                                avg_launch_ms: *mut f64) -> c_int;
+    pub fn rbmoe_replay_stage(layer: *mut rbmoe_layer, stage: i32, launches: i32, ms_per_launch: *mut f32) -> c_int;
     pub fn rbmoe_version() -> *const c_char;
 }

@@ -85,9 +85,9 @@ SIGNATURES = {
     "rbmoe_backward_block_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
     "rbmoe_zero_grads": (C.c_int, [C.c_void_p]),
     "rbmoe_get_weight_grad": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_float), C.c_int32, C.c_int32]),
-    "rbmoe_calibrate_mfma": (C.c_int, [C.c_void_p, C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
-    "rbmoe_calibrate_read": (C.c_int, [C.c_void_p, C.c_size_t, C.c_int32, C.c_int32, C.POINTER(C.c_double),
-                                       C.POINTER(C.c_double)]),
+    "rbmoe_forward_kernel_times": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p,
+                                             C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
+    "rbmoe_replay_stage": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_float)]),
     "rbmoe_version": (C.c_char_p, []),
 }
 
@@ -109,4 +109,39 @@ def load() -> C.CDLL:
         fn.restype = restype
         fn.argtypes = argtypes
     _lib = lib
+    return lib
+
+
+# include/rbmoe_bench.h: the benchmark's measurement helpers, a library of their own
+BENCH_LIB_PATH = os.path.join(_HERE, "librbmoe_bench.so")
+BENCH_SIGNATURES = {
+    "rbbench_stream_create": (C.c_int, [C.POINTER(C.c_void_p)]),
+    "rbbench_stream_destroy": (C.c_int, [C.c_void_p]),
+    "rbbench_timer_create": (C.c_int, [C.POINTER(C.c_void_p)]),
+    "rbbench_timer_start": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "rbbench_timer_stop": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
+    "rbbench_timer_destroy": (None, [C.c_void_p]),
+    "rbbench_flush_create": (C.c_int, [C.c_size_t, C.POINTER(C.c_void_p)]),
+    "rbbench_flush": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "rbbench_flush_destroy": (None, [C.c_void_p]),
+    "rbbench_mfma_only": (C.c_int, [C.c_void_p, C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+    "rbbench_read": (C.c_int, [C.c_void_p, C.c_size_t, C.c_int32, C.c_void_p, C.POINTER(C.c_double),
+                               C.POINTER(C.c_double)]),
+}
+_bench_lib = None
+
+
+def load_bench() -> C.CDLL:
+    """Load librbmoe_bench.so (the benchmark's helpers); raises if it has not been built."""
+    global _bench_lib
+    if _bench_lib is not None:
+        return _bench_lib
+    if not os.path.exists(BENCH_LIB_PATH):
+        raise ImportError(f"{BENCH_LIB_PATH} is missing: build it with `python -m rustingbrain_amd.build`")
+    lib = C.CDLL(BENCH_LIB_PATH)
+    for name, (restype, argtypes) in BENCH_SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _bench_lib = lib
     return lib

@@ -50,8 +50,22 @@ def build(jobs: int = 4) -> str:
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError("link failed:\n" + res.stderr)
+    build_bench()
     build_host()
     return LIB
+
+
+BENCH_SRC = os.path.join(CSRC, "bench", "rbmoe_bench.hip")
+BENCH_LIB = os.path.join(HERE, "librbmoe_bench.so")
+
+
+def build_bench() -> str:
+    """The benchmark's measurement helpers (include/rbmoe_bench.h): a library of their own, not part of librbmoe.so."""
+    cmd = [HIPCC, *FLAGS, "-shared", BENCH_SRC, "-o", BENCH_LIB]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("bench helper build failed:\n" + res.stderr)
+    return BENCH_LIB
 
 
 HOST = os.path.join(HERE, "host")

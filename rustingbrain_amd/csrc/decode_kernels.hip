@@ -509,13 +509,13 @@ hipError_t launch_route_small(const SmallRouteArgs& a, bool bf16, hipStream_t s)
     if (a.norm_w && (!a.xn_out || !small_route_stages_rows(a.x, a.wr, a.T, a.d, a.E, bf16))) return hipErrorInvalidValue;
     if (a.rows16 && (bf16 || !small_route_stages_rows(a.x, a.wr, a.T, a.d, a.E, bf16))) return hipErrorInvalidValue;
     if (bf16)
-        hipLaunchKernelGGL(route_small_kernel<bf16_t>, dim3(1), dim3(kSmallThreads), 0, s,
+        RB_LAUNCH(route_small_kernel<bf16_t>, dim3(1), dim3(kSmallThreads), 0, s,
                            static_cast<const bf16_t*>(a.x), a.wr, a.bias, a.valid, a.T, a.d, a.E, a.k, a.w_aux, a.w_z,
                            a.tile_m, a.P, a.lse, a.expert_of, a.gate_of, a.counts, a.offsets, a.tile_expert,
                            a.tile_row0, a.tile_rows, a.ntiles, a.losses, a.perm_slot, a.perm_token, a.inv_pos,
                            a.norm_w, a.norm_eps, static_cast<bf16_t*>(a.xn_out), nullptr);
     else
-        hipLaunchKernelGGL(route_small_kernel<float>, dim3(1), dim3(kSmallThreads), 0, s,
+        RB_LAUNCH(route_small_kernel<float>, dim3(1), dim3(kSmallThreads), 0, s,
                            static_cast<const float*>(a.x), a.wr, a.bias, a.valid, a.T, a.d, a.E, a.k, a.w_aux, a.w_z,
                            a.tile_m, a.P, a.lse, a.expert_of, a.gate_of, a.counts, a.offsets, a.tile_expert,
                            a.tile_row0, a.tile_rows, a.ntiles, a.losses, a.perm_slot, a.perm_token, a.inv_pos,
@@ -761,9 +761,9 @@ hipError_t launch_decode_front(const SmallRouteArgs& r, const DecodeGemmArgs& g,
     const int widest = g.a_shared ? (g.N > g.N_shared ? g.N : g.N_shared) : g.N;
     const int grid = 1 + (r.E + shared_tiles) * (widest / 32);
     if (wk == WeightKind::BF16)
-        hipLaunchKernelGGL(decode_front_kernel<false>, dim3(grid), dim3(kSmallThreads), 0, s, r, g, r.E, r.T);
+        RB_LAUNCH(decode_front_kernel<false>, dim3(grid), dim3(kSmallThreads), 0, s, r, g, r.E, r.T);
     else if (wk == WeightKind::I8)
-        hipLaunchKernelGGL(decode_front_kernel<true>, dim3(grid), dim3(kSmallThreads), 0, s, r, g, r.E, r.T);
+        RB_LAUNCH(decode_front_kernel<true>, dim3(grid), dim3(kSmallThreads), 0, s, r, g, r.E, r.T);
     else
         return hipErrorInvalidValue;
     return hipGetLastError();
@@ -778,11 +778,11 @@ hipError_t launch_decode_gemm(const DecodeGemmArgs& g, WeightKind wk, hipStream_
     const int widest = g.a_shared ? (g.N > g.N_shared ? g.N : g.N_shared) : g.N;
     const dim3 grid(widest / 32, tiles);
     if (wk == WeightKind::BF16) {
-        if (g.swiglu) hipLaunchKernelGGL((decode_gemm_kernel<true, false, 4>), grid, dim3(256), 0, s, g);
-        else hipLaunchKernelGGL((decode_gemm_kernel<false, false, 8>), grid, dim3(512), 0, s, g);
+        if (g.swiglu) RB_LAUNCH((decode_gemm_kernel<true, false, 4>), grid, dim3(256), 0, s, g);
+        else RB_LAUNCH((decode_gemm_kernel<false, false, 8>), grid, dim3(512), 0, s, g);
     } else if (wk == WeightKind::I8) {
-        if (g.swiglu) hipLaunchKernelGGL((decode_gemm_kernel<true, true, 4>), grid, dim3(256), 0, s, g);
-        else hipLaunchKernelGGL((decode_gemm_kernel<false, true, 8>), grid, dim3(512), 0, s, g);
+        if (g.swiglu) RB_LAUNCH((decode_gemm_kernel<true, true, 4>), grid, dim3(256), 0, s, g);
+        else RB_LAUNCH((decode_gemm_kernel<false, true, 8>), grid, dim3(512), 0, s, g);
     } else {
         return hipErrorInvalidValue;
     }

@@ -94,13 +94,13 @@ static hipError_t launch_t(const GroupedArgs& g, hipStream_t s) {
     if (tiles <= 0) return hipSuccess;
     const dim3 grid(tiles, (g.N + 15) / 16), block(256);
     if (g.swiglu)
-        hipLaunchKernelGGL((grouped_generic_kernel<AT, WT, true>), grid, block, 0, s,
+        RB_LAUNCH((grouped_generic_kernel<AT, WT, true>), grid, block, 0, s,
                            static_cast<const AT*>(g.a), g.row_index, static_cast<const WT*>(g.w),
                            g.w_expert_stride, g.scales, g.s_expert_stride, g.N, g.K, g.tile_expert,
                            g.tile_row0, g.tile_rows, g.ntiles, g.dense_rows, static_cast<AT*>(g.out),
                            static_cast<AT*>(g.gu_out), static_cast<const AT*>(g.swiglu_grad_gu));
     else
-        hipLaunchKernelGGL((grouped_generic_kernel<AT, WT, false>), grid, block, 0, s,
+        RB_LAUNCH((grouped_generic_kernel<AT, WT, false>), grid, block, 0, s,
                            static_cast<const AT*>(g.a), g.row_index, static_cast<const WT*>(g.w),
                            g.w_expert_stride, g.scales, g.s_expert_stride, g.N, g.K, g.tile_expert,
                            g.tile_row0, g.tile_rows, g.ntiles, g.dense_rows, static_cast<AT*>(g.out),

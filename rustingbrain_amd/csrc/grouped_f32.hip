@@ -186,12 +186,12 @@ hipError_t launch_grouped_f32(const GroupedArgs& g, hipStream_t s) {
     if (tiles_m <= 0) return hipSuccess;
     const dim3 grid((g.N + FN - 1) / FN, tiles_m), block(256);
     if (g.swiglu)
-        hipLaunchKernelGGL((grouped_f32_kernel<true>), grid, block, 0, s, static_cast<const float*>(g.a), g.row_index,
+        RB_LAUNCH((grouped_f32_kernel<true>), grid, block, 0, s, static_cast<const float*>(g.a), g.row_index,
                            static_cast<const float*>(g.w), g.w_expert_stride, g.N, g.K, g.tile_expert, g.tile_row0,
                            g.tile_rows, g.ntiles, g.dense_rows, static_cast<float*>(g.out), static_cast<float*>(g.gu_out),
                            static_cast<const float*>(g.swiglu_grad_gu));
     else
-        hipLaunchKernelGGL((grouped_f32_kernel<false>), grid, block, 0, s, static_cast<const float*>(g.a), g.row_index,
+        RB_LAUNCH((grouped_f32_kernel<false>), grid, block, 0, s, static_cast<const float*>(g.a), g.row_index,
                            static_cast<const float*>(g.w), g.w_expert_stride, g.N, g.K, g.tile_expert, g.tile_row0,
                            g.tile_rows, g.ntiles, g.dense_rows, static_cast<float*>(g.out), static_cast<float*>(g.gu_out),
                            static_cast<const float*>(g.swiglu_grad_gu));

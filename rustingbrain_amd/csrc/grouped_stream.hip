@@ -554,7 +554,7 @@ hipError_t launch_t(const GroupedArgs& g, hipStream_t s) {
     if (tiles_m <= 0) return hipSuccess;
     const int total = tiles_m * tiles_n;
     const int grid = ((total + 7) / 8) * 8;
-    hipLaunchKernelGGL((grouped_stream_kernel<SWIGLU, I8>), dim3(grid), dim3(NT), 0, s,
+    RB_LAUNCH((grouped_stream_kernel<SWIGLU, I8>), dim3(grid), dim3(NT), 0, s,
                        static_cast<const bf16_t*>(g.a), g.row_index, g.w, g.w_expert_stride * (I8 ? 1 : 2), g.scales,
                        g.s_expert_stride, g.N, g.K, g.tile_expert, g.tile_row0, g.tile_rows, g.ntiles, g.dense_rows,
                        static_cast<bf16_t*>(g.out), static_cast<bf16_t*>(g.gu_out), static_cast<const bf16_t*>(g.swiglu_grad_gu),

@@ -12,6 +12,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <functional>
 #include <mutex>
 #include <string>
 #include <vector>
@@ -19,6 +20,8 @@
 #include "rbmoe_kernels.h"
 
 using namespace rbmoe;
+
+thread_local rbmoe::KernelTimer* rbmoe::g_kernel_timer = nullptr;
 
 // Scratch of rbmoe_forward_static: device memory that exists without any allocation call.  Every GPU the library
 // runs on holds its own copy of the array, at its own address, until the process ends.  In host code the
@@ -239,6 +242,10 @@ struct rbmoe_layer {
     std::vector<Buf*> all;
     hipEvent_t ev[RBMOE_NUM_STAGES + 1] = {};
     bool have_events = false;
+    KernelTimer ktimer[RBMOE_NUM_STAGES];  // rbmoe_forward_kernel_times: events carried by the stages' own dispatches
+    bool have_ktimers = false;
+    // the launches of the last forward, stage by stage, for rbmoe_replay_stage (empty: the stage had no launch)
+    std::function<hipError_t(hipStream_t)> replay[RBMOE_NUM_STAGES];
 };
 
 namespace {
@@ -553,6 +560,10 @@ void rbmoe_layer_destroy(rbmoe_layer* L) {
     if (L->have_events)
         for (auto& ev : L->ev)
             if (ev) (void)hipEventDestroy(ev);
+    if (L->have_ktimers)
+        for (auto& kt : L->ktimer)
+            for (auto& ev : kt.ev)
+                if (ev) (void)hipEventDestroy(ev);
     free_layer_buffers(L);
     delete L;
     ctx_release(owner);
@@ -822,9 +833,12 @@ size_t carve_decode_work(const rbmoe_layer* L, int T, unsigned char* base, Work*
 // small-route kernel itself for a few tokens, by the norm kernel otherwise - before anything reads it.
 // `static_scratch` (rbmoe_forward_static): this device's copy of the static scratch array; the call must then be
 // decode-shaped, keeps every intermediate result there and touches none of the layer's workspace.
+// `timing`: 0 none; 1 an event between the stages (rbmoe_forward_timed); 2 every stage's dispatches carry their own
+// start and stop events (rbmoe_forward_kernel_times).
 int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* valid, const float* router_bias,
-                 const void* residual, void* out, bool timed, const void* norm_src = nullptr,
+                 const void* residual, void* out, int timing, const void* norm_src = nullptr,
                  void* static_scratch = nullptr) {
+    const bool timed = timing != 0;
     if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
     rbmoe_ctx* ctx = L->ctx;
     const rbmoe_config& c = L->cfg;
@@ -849,11 +863,25 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     const bool cast = L->cast_rows;  // f32 rows, bf16 matrix-core products over their bf16 copy
     const WeightKind wk = c.weight_dtype == RBMOE_F32 ? WeightKind::F32
                           : c.weight_dtype == RBMOE_BF16 ? WeightKind::BF16 : WeightKind::I8;
-    if (timed && !L->have_events) {
+    if (timing == 1 && !L->have_events) {
         for (auto& ev : L->ev) HIP_TRY(ctx, hipEventCreate(&ev));
         L->have_events = true;
     }
-    auto mark = [&](int i) -> hipError_t { return timed ? hipEventRecord(L->ev[i], s) : hipSuccess; };
+    if (timing == 2 && !L->have_ktimers) {
+        for (auto& kt : L->ktimer)
+            for (auto& ev : kt.ev) HIP_TRY(ctx, hipEventCreate(&ev));
+        L->have_ktimers = true;
+    }
+    struct TimerScope {  // whatever path leaves this function, the thread's launches are plain again
+        ~TimerScope() { g_kernel_timer = nullptr; }
+    } timer_scope;
+    if (timing == 2)
+        for (auto& kt : L->ktimer) kt.used = 0;
+    // mark(i): stage i - 1 ends here and stage i begins
+    auto mark = [&](int i) -> hipError_t {
+        if (timing == 2) g_kernel_timer = i < RBMOE_NUM_STAGES - 1 ? &L->ktimer[i] : nullptr;
+        return timing == 1 ? hipEventRecord(L->ev[i], s) : hipSuccess;
+    };
     HIP_TRY(ctx, mark(0));
 
     const bool mfma = L->use_stream;
@@ -921,7 +949,11 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
         sr.tile_expert = wk_.tile_expert; sr.tile_row0 = wk_.tile_row0; sr.tile_rows = wk_.tile_rows;
         sr.ntiles = wk_.ntiles; sr.losses = wk_.losses;
         sr.perm_slot = wk_.perm_slot; sr.perm_token = wk_.perm_token; sr.inv_pos = wk_.inv_pos;
-        if (!front) HIP_TRY(ctx, launch_route_small(sr, abf, s));
+        for (auto& r : L->replay) r = nullptr;
+        if (!front) {
+            HIP_TRY(ctx, launch_route_small(sr, abf, s));
+            L->replay[RBMOE_STAGE_ROUTER] = [=](hipStream_t st) { return launch_route_small(sr, abf, st); };
+        }
         HIP_TRY(ctx, mark(1));
         HIP_TRY(ctx, mark(2));
         HIP_TRY(ctx, mark(3));
@@ -945,8 +977,10 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
             d1.row_index = nullptr;
             d1.out = wk_.hall;
             HIP_TRY(ctx, launch_decode_front(sr, d1, wk, s));
+            L->replay[RBMOE_STAGE_GATE_UP] = [=](hipStream_t st) { return launch_decode_front(sr, d1, wk, st); };
         } else {
             HIP_TRY(ctx, launch_decode_gemm(d1, wk, s));
+            L->replay[RBMOE_STAGE_GATE_UP] = [=](hipStream_t st) { return launch_decode_gemm(d1, wk, st); };
         }
         HIP_TRY(ctx, mark(4));
 
@@ -966,11 +1000,13 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
             d2.N_shared = d; d2.K_shared = Fs; d2.out_shared = wk_.ys;
         }
         HIP_TRY(ctx, launch_decode_gemm(d2, wk, s));
+        L->replay[RBMOE_STAGE_DOWN] = [=](hipStream_t st) { return launch_decode_gemm(d2, wk, st); };
         HIP_TRY(ctx, mark(5));
         HIP_TRY(ctx, mark(6));
         CombineArgs cd{wk_.y, c.shared_expert ? wk_.ys : nullptr, residual, wk_.inv_pos, wk_.gate_of, T, d, k, out};
         cd.rows_bf16 = cast;
         HIP_TRY(ctx, launch_combine(cd, abf, s));
+        L->replay[RBMOE_STAGE_COMBINE] = [=](hipStream_t st) { return launch_combine(cd, abf, st); };
         HIP_TRY(ctx, mark(7));
         L->last_T = T;
         L->last = wk_;
@@ -983,7 +1019,8 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     if (L->training && T > 0)  // MoeCache keeps the input (src/moe.rs:133-135)
         HIP_TRY(ctx, hipMemcpyAsync(L->xc.p, x, (size_t)T * d * dtype_size(c.act_dtype), hipMemcpyDeviceToDevice, s));
 
-    auto run_on = [&](const GroupedArgs& g, hipStream_t st) -> hipError_t {
+    for (auto& r : L->replay) r = nullptr;
+    auto run_on = [=](const GroupedArgs& g, hipStream_t st) -> hipError_t {
         if (mfma) return launch_grouped_stream(g, wk, st);
         if (f32mc) return launch_grouped_f32(g, st);
         return launch_grouped_generic(g, abf, wk, kGenericTileM, st);
@@ -1045,6 +1082,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     if (cast) ra.rows16 = L->x16.p;
     ra.allow_fused = L->fused_router;
     HIP_TRY(ctx, launch_router(ra, abf, s));
+    L->replay[RBMOE_STAGE_ROUTER] = [=](hipStream_t st) { return launch_router(ra, abf, st); };
     HIP_TRY(ctx, mark(1));
 
     HIP_TRY(ctx, mark(2));  // an interval with no work in it: the cost of one pair of event records
@@ -1065,6 +1103,10 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     da.perm_slot = (int*)L->perm_slot.p; da.perm_token = (int*)L->perm_token.p; da.inv_pos = (int*)L->inv_pos.p;
     da.xg = gather_in_product ? nullptr : L->xg.p;
     HIP_TRY(ctx, launch_dispatch(da, abf || cast, s));
+    {
+        const bool rows_bf16 = abf || cast;
+        L->replay[RBMOE_STAGE_DISPATCH] = [=](hipStream_t st) { return launch_dispatch(da, rows_bf16, st); };
+    }
     HIP_TRY(ctx, mark(3));
 
     GroupedArgs g1{};
@@ -1087,6 +1129,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     g1.group_m = L->group_m;
     if (L->training) g1.gu_out = L->gu.p;
     HIP_TRY(ctx, run(g1, true));
+    L->replay[RBMOE_STAGE_GATE_UP] = [=](hipStream_t st) { return run_on(g1, st); };
     HIP_TRY(ctx, mark(4));
 
     GroupedArgs g2 = g1;
@@ -1107,6 +1150,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     // against 4 for gate/up, 147 against 166 MB with 4 against 8 for down)
     if (L->group_m == 0) g2.group_m = 4;
     HIP_TRY(ctx, run(g2, false));
+    L->replay[RBMOE_STAGE_DOWN] = [=](hipStream_t st) { return run_on(g2, st); };
     HIP_TRY(ctx, mark(5));
 
     if (c.shared_expert && T > 0 && !shared_forked) HIP_TRY(ctx, shared_expert(s));
@@ -1120,6 +1164,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
                    (const float*)L->gate_of.p, T, d, k, out};
     ca.rows_bf16 = cast;
     HIP_TRY(ctx, launch_combine(ca, abf, s));
+    L->replay[RBMOE_STAGE_COMBINE] = [=](hipStream_t st) { return launch_combine(ca, abf, st); };
     HIP_TRY(ctx, mark(7));
     L->last_T = T;
     L->last = wk_;
@@ -1194,26 +1239,75 @@ extern "C" {
 
 int rbmoe_forward(rbmoe_layer* L, const void* x, int32_t T, int32_t cols, const uint8_t* valid,
                   const float* router_bias, const void* residual, void* out) {
-    return forward_impl(L, x, T, cols, valid, router_bias, residual, out, false);
+    return forward_impl(L, x, T, cols, valid, router_bias, residual, out, 0);
 }
 
 int rbmoe_forward_static(rbmoe_layer* L, const void* x, int32_t T, int32_t cols, const uint8_t* valid,
                          const float* router_bias, const void* residual, void* out) {
     if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
     if (!L->ctx->static_scratch) return fail(L->ctx, RBMOE_DEVICE_ERROR, "the static scratch buffer was not resolved");
-    return forward_impl(L, x, T, cols, valid, router_bias, residual, out, false, nullptr, L->ctx->static_scratch);
+    return forward_impl(L, x, T, cols, valid, router_bias, residual, out, 0, nullptr, L->ctx->static_scratch);
 }
 
 int rbmoe_forward_timed(rbmoe_layer* L, const void* x, int32_t T, int32_t cols, const uint8_t* valid,
                         const float* router_bias, const void* residual, void* out, float* ms) {
     if (!ms) return fail(L ? L->ctx : nullptr, RBMOE_NULL_POINTER, "ms is NULL");
-    int rc = forward_impl(L, x, T, cols, valid, router_bias, residual, out, true);
+    int rc = forward_impl(L, x, T, cols, valid, router_bias, residual, out, 1);
     if (rc != RBMOE_OK) return rc;
     rbmoe_ctx* ctx = L->ctx;
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
     for (int i = 0; i < RBMOE_NUM_STAGES - 1; ++i)
         HIP_TRY(ctx, hipEventElapsedTime(&ms[i], L->ev[i], L->ev[i + 1]));
     HIP_TRY(ctx, hipEventElapsedTime(&ms[RBMOE_STAGE_TOTAL], L->ev[0], L->ev[RBMOE_NUM_STAGES - 1]));
+    return RBMOE_OK;
+}
+
+int rbmoe_forward_kernel_times(rbmoe_layer* L, const void* x, int32_t T, int32_t cols, const uint8_t* valid,
+                               const float* router_bias, const void* residual, void* out, float* ms) {
+    if (!ms) return fail(L ? L->ctx : nullptr, RBMOE_NULL_POINTER, "ms is NULL");
+    int rc = forward_impl(L, x, T, cols, valid, router_bias, residual, out, 2);
+    if (rc != RBMOE_OK) return rc;
+    rbmoe_ctx* ctx = L->ctx;
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    float total = 0.0f;
+    for (int i = 0; i < RBMOE_NUM_STAGES - 1; ++i) {
+        ms[i] = 0.0f;
+        for (int u = 0; u < L->ktimer[i].used; ++u) {
+            float one = 0.0f;
+            HIP_TRY(ctx, hipEventElapsedTime(&one, L->ktimer[i].ev[2 * u], L->ktimer[i].ev[2 * u + 1]));
+            ms[i] += one;
+        }
+        total += ms[i];
+    }
+    ms[RBMOE_STAGE_TOTAL] = total;
+    return RBMOE_OK;
+}
+
+int rbmoe_replay_stage(rbmoe_layer* L, int32_t stage, int32_t launches, float* ms_per_launch) {
+    if (!L) return fail(nullptr, RBMOE_NULL_POINTER, "layer is NULL");
+    rbmoe_ctx* ctx = L->ctx;
+    if (stage < 0 || stage >= RBMOE_NUM_STAGES || launches <= 0)
+        return fail(ctx, RBMOE_INVALID_INPUT, "stage out of range or launches not positive");
+    if (L->last_T < 0) return fail(ctx, RBMOE_INVALID_INPUT, "no forward pass has run yet");
+    if (!L->replay[stage]) return fail(ctx, RBMOE_UNSUPPORTED, "the last forward had no launch of its own for this stage");
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    hipStream_t s = ctx->stream;
+    if (!ms_per_launch) {  // enqueue only: the caller times a sequence of its own
+        for (int i = 0; i < launches; ++i) HIP_TRY(ctx, L->replay[stage](s));
+        return RBMOE_OK;
+    }
+    if (!L->have_events) {
+        for (auto& ev : L->ev) HIP_TRY(ctx, hipEventCreate(&ev));
+        L->have_events = true;
+    }
+    HIP_TRY(ctx, L->replay[stage](s));  // warm-up: the stage's operands are back in the caches it usually finds them in
+    HIP_TRY(ctx, hipEventRecord(L->ev[0], s));
+    for (int i = 0; i < launches; ++i) HIP_TRY(ctx, L->replay[stage](s));
+    HIP_TRY(ctx, hipEventRecord(L->ev[1], s));
+    HIP_TRY(ctx, hipStreamSynchronize(s));
+    float ms = 0.0f;
+    HIP_TRY(ctx, hipEventElapsedTime(&ms, L->ev[0], L->ev[1]));
+    *ms_per_launch = ms / (float)launches;
     return RBMOE_OK;
 }
 
@@ -1242,7 +1336,7 @@ int rbmoe_forward_host(rbmoe_layer* L, const void* x, int32_t T, int32_t cols, c
         HIP_TRY(ctx, hipMemcpyAsync(L->st_bias.p, router_bias, (size_t)c.num_experts * 4, hipMemcpyHostToDevice, s));
     int rc = forward_impl(L, L->st_x.p, T, cols, valid ? (const uint8_t*)L->st_valid.p : nullptr,
                           router_bias ? (const float*)L->st_bias.p : nullptr, residual ? L->st_res.p : nullptr,
-                          L->st_out.p, false);
+                          L->st_out.p, 0);
     if (rc != RBMOE_OK) return rc;
     if (T > 0) HIP_TRY(ctx, hipMemcpyAsync(out, L->st_out.p, nbytes, hipMemcpyDeviceToHost, s));
     HIP_TRY(ctx, hipStreamSynchronize(s));
@@ -1294,7 +1388,7 @@ int rbmoe_forward_block(rbmoe_layer* L, const void* x, int32_t T, int32_t cols, 
     if (L->training && T > 0)  // TransformerBlockCache keeps the residual (src/transformer_block.rs:224-232)
         HIP_TRY(ctx, hipMemcpyAsync(L->xraw.p, x, (size_t)T * cols * dtype_size(L->cfg.act_dtype),
                                     hipMemcpyDeviceToDevice, ctx->stream));
-    const int rc = forward_impl(L, L->xn.p, T, cols, valid, router_bias, x, out, false, x);
+    const int rc = forward_impl(L, L->xn.p, T, cols, valid, router_bias, x, out, 0, x);
     if (rc == RBMOE_OK) L->last_was_block = true;
     return rc;
 }
@@ -1827,108 +1921,6 @@ int rbmoe_copy_to_host(rbmoe_ctx* ctx, void* dst, const void* src, size_t bytes)
     if (!dst || !src) return fail(ctx, RBMOE_NULL_POINTER, "dst or src is NULL");
     HIP_TRY(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
-    return RBMOE_OK;
-}
-
-int rbmoe_calibrate_mfma(rbmoe_ctx* ctx, int32_t launches, double* tflops, double* avg_launch_ms) {
-    if (!ctx || !tflops) return fail(ctx, RBMOE_NULL_POINTER, "ctx or tflops is NULL");
-    if (launches <= 0) return fail(ctx, RBMOE_INVALID_INPUT, "launches must be positive");
-    HIP_TRY(ctx, hipSetDevice(ctx->device));
-    int cus = 0;
-    HIP_TRY(ctx, hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, ctx->device));
-    const int workgroups = 2 * cus, steps = 2048;  // two waves on every SIMD
-    float* out = nullptr;
-    HIP_TRY(ctx, hipMalloc(&out, (size_t)workgroups * 256 * sizeof(float)));
-    hipEvent_t e0 = nullptr, e1 = nullptr;
-    hipError_t e = hipEventCreate(&e0);
-    if (e == hipSuccess) e = hipEventCreate(&e1);
-    hipStream_t s = ctx->stream;
-    if (e == hipSuccess) e = launch_mfma_only(out, workgroups, steps, s);  // warm-up
-    if (e == hipSuccess) e = hipEventRecord(e0, s);
-    for (int i = 0; i < launches && e == hipSuccess; ++i) e = launch_mfma_only(out, workgroups, steps, s);
-    if (e == hipSuccess) e = hipEventRecord(e1, s);
-    if (e == hipSuccess) e = hipStreamSynchronize(s);
-    float ms = 0.0f;
-    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
-    if (e0) (void)hipEventDestroy(e0);
-    if (e1) (void)hipEventDestroy(e1);
-    (void)hipFree(out);
-    if (e != hipSuccess) return hip_fail(ctx, e, "rbmoe_calibrate_mfma");
-    const double flops = (double)workgroups * 4 * steps * 8 * 32768.0;  // 2 * 32 * 32 * 16 per multiply
-    const double avg = (double)ms / launches;
-    *tflops = flops / (avg * 1e-3) / 1e12;
-    if (avg_launch_ms) *avg_launch_ms = avg;
-    return RBMOE_OK;
-}
-
-int rbmoe_calibrate_read(rbmoe_ctx* ctx, size_t bytes, int32_t launches, int32_t flush_caches, double* gbs,
-                         double* avg_launch_ms) {
-    if (!ctx || !gbs) return fail(ctx, RBMOE_NULL_POINTER, "ctx or gbs is NULL");
-    if (launches <= 0 || bytes < 16 || bytes % 16 != 0)
-        return fail(ctx, RBMOE_INVALID_INPUT, "launches must be positive and bytes a positive multiple of 16");
-    HIP_TRY(ctx, hipSetDevice(ctx->device));
-    hipStream_t s = ctx->stream;
-    const size_t flush_bytes = (size_t)512 << 20;  // twice the 256 MiB Infinity Cache through L2
-    void *buf = nullptr, *fa = nullptr, *fb = nullptr;
-    uint32_t* sink = nullptr;
-    hipEvent_t e0 = nullptr, e1 = nullptr;
-    hipError_t e = hipMalloc(&buf, bytes);
-    if (e == hipSuccess) e = hipMalloc(&sink, 256);
-    if (e == hipSuccess) e = hipMemsetAsync(buf, 1, bytes, s);
-    if (e == hipSuccess && flush_caches) e = hipMalloc(&fa, flush_bytes);
-    if (e == hipSuccess && flush_caches) e = hipMalloc(&fb, flush_bytes);
-    if (e == hipSuccess) e = hipEventCreate(&e0);
-    if (e == hipSuccess) e = hipEventCreate(&e1);
-    // what a pair of event records adds to the interval between them: taken off every timed interval below
-    double empty = 0.0;
-    for (int i = 0; i < 8 && e == hipSuccess; ++i) {
-        e = hipEventRecord(e0, s);
-        if (e == hipSuccess) e = hipEventRecord(e1, s);
-        if (e == hipSuccess) e = hipStreamSynchronize(s);
-        float ms = 0.0f;
-        if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
-        empty += ms / 8.0;
-    }
-    // the split over workgroups that reads fastest is the one reported
-    double best = 1e30;
-    const int splits[3] = {512, 1024, 2048};
-    for (int sp = 0; sp < 3 && e == hipSuccess; ++sp) {
-        const int workgroups = splits[sp];
-        e = launch_read_only(buf, bytes, workgroups, sink, s);  // warm-up
-        double total = 0.0;
-        if (flush_caches) {
-            for (int i = 0; i < launches && e == hipSuccess; ++i) {
-                e = hipMemcpyAsync(fb, fa, flush_bytes, hipMemcpyDeviceToDevice, s);
-                if (e == hipSuccess) e = hipEventRecord(e0, s);
-                if (e == hipSuccess) e = launch_read_only(buf, bytes, workgroups, sink, s);
-                if (e == hipSuccess) e = hipEventRecord(e1, s);
-                if (e == hipSuccess) e = hipStreamSynchronize(s);
-                float ms = 0.0f;
-                if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
-                total += std::max((double)ms - empty, 1e-6);
-            }
-        } else {  // back to back between one pair of events
-            if (e == hipSuccess) e = hipEventRecord(e0, s);
-            for (int i = 0; i < launches && e == hipSuccess; ++i) e = launch_read_only(buf, bytes, workgroups, sink, s);
-            if (e == hipSuccess) e = hipEventRecord(e1, s);
-            if (e == hipSuccess) e = hipStreamSynchronize(s);
-            float ms = 0.0f;
-            if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
-            total = std::max((double)ms - empty, 1e-6);
-        }
-        best = std::min(best, total / launches);
-    }
-    const double total = best * launches;
-    if (e0) (void)hipEventDestroy(e0);
-    if (e1) (void)hipEventDestroy(e1);
-    (void)hipFree(buf);
-    (void)hipFree(sink);
-    if (fa) (void)hipFree(fa);
-    if (fb) (void)hipFree(fb);
-    if (e != hipSuccess) return hip_fail(ctx, e, "rbmoe_calibrate_read");
-    const double avg = total / launches;
-    *gbs = (double)bytes / (avg * 1e-3) / 1e9;
-    if (avg_launch_ms) *avg_launch_ms = avg;
     return RBMOE_OK;
 }
 

@@ -2,12 +2,35 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stddef.h>
 #include <stdint.h>
 
 #include "rbmoe_device.h"
 
 namespace rbmoe {
+
+// Kernel durations the way a kernel trace reports them: while a KernelTimer is installed on the calling thread,
+// every forward-path launch below carries its own start and stop events (hipExtLaunchKernelGGL), which receive the
+// begin and end time stamps of that dispatch itself - no launch gap, no event-pair overhead.  Up to kMaxTimedLaunches
+// launches per timer; further ones are plain launches.
+constexpr int kMaxTimedLaunches = 4;
+struct KernelTimer {
+    hipEvent_t ev[2 * kMaxTimedLaunches] = {};
+    int used = 0;
+};
+extern thread_local KernelTimer* g_kernel_timer;  // null (the default): plain launches
+#define RB_LAUNCH(kernel, grid, block, lds, stream, ...)                                                        \
+    do {                                                                                                        \
+        ::rbmoe::KernelTimer* const kt_ = ::rbmoe::g_kernel_timer;                                              \
+        if (kt_ != nullptr && kt_->used < ::rbmoe::kMaxTimedLaunches) {                                         \
+            hipExtLaunchKernelGGL(kernel, grid, block, lds, stream, kt_->ev[2 * kt_->used],                     \
+                                  kt_->ev[2 * kt_->used + 1], 0, __VA_ARGS__);                                  \
+            ++kt_->used;                                                                                        \
+        } else {                                                                                                \
+            hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);                                  \
+        }                                                                                                       \
+    } while (0)
 
 // Tokens owned by one router / dispatch block.  Slots are numbered
 // token * k + rank, so a block owns a contiguous slot range.
@@ -256,11 +279,5 @@ hipError_t launch_decode_gemm(const DecodeGemmArgs& g, WeightKind wk, hipStream_
 // hidden rows to g.out as [E][T, N]; the shared expert as in launch_decode_gemm.  g.a / g.a_shared: the T rows.
 bool decode_front_ok(const void* x, const float* wr, int T, int d, int E, int k);
 hipError_t launch_decode_front(const SmallRouteArgs& r, const DecodeGemmArgs& g, WeightKind wk, hipStream_t s);
-
-// ---- calibration (calibrate.hip): what the device sustains, for the roofline figures to be read against ----
-// 4 waves per workgroup, each issuing steps * 8 independent 32x32x16 bf16 multiplies; out: workgroups * 256 floats
-hipError_t launch_mfma_only(float* out, int workgroups, int steps, hipStream_t s);
-// a plain read of `bytes` (a multiple of 16) split over the workgroups
-hipError_t launch_read_only(const void* src, size_t bytes, int workgroups, uint32_t* out, hipStream_t s);
 
 }  // namespace rbmoe

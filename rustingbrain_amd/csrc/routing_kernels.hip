@@ -1221,7 +1221,7 @@ static hipError_t launch_router_t(const RouterArgs& a, hipStream_t s) {
     if (const int cols = fused_cols(a, sizeof(XT))) {
         const size_t lds = fused_lds_bytes(a.E, a.k, cols, sizeof(XT));
         auto go = [&](auto ni) {
-            hipLaunchKernelGGL((route_fused_kernel<XT, decltype(ni)::value>), dim3(nb), dim3(kRouterThreads), lds, s,
+            RB_LAUNCH((route_fused_kernel<XT, decltype(ni)::value>), dim3(nb), dim3(kRouterThreads), lds, s,
                                static_cast<const XT*>(a.x), a.wr, a.bias, a.valid, a.T, a.d, a.E, a.k, cols, a.P, a.lse,
                                a.expert_of, a.gate_of, a.rank_in_block, a.blockcnt, a.partial,
                                static_cast<bf16_t*>(a.rows16));
@@ -1248,19 +1248,19 @@ static hipError_t launch_router_t(const RouterArgs& a, hipStream_t s) {
     const int tiles_t = (a.T + kLogitTokens - 1) / kLogitTokens;
     const dim3 lgrid(tiles_t, (a.E + NE - 1) / NE);
     if ((long long)lgrid.x * lgrid.y <= 512)  // at most two workgroups on a compute unit
-        hipLaunchKernelGGL((logits_kernel<XT, NE, true>), lgrid, dim3(NE * 64), 0, s, static_cast<const XT*>(a.x),
+        RB_LAUNCH((logits_kernel<XT, NE, true>), lgrid, dim3(NE * 64), 0, s, static_cast<const XT*>(a.x),
                            a.wr, a.bias, a.T, a.d, a.E, a.P, static_cast<bf16_t*>(a.rows16));
     else
-        hipLaunchKernelGGL((logits_kernel<XT, NE, false>), lgrid, dim3(NE * 64), 0, s, static_cast<const XT*>(a.x),
+        RB_LAUNCH((logits_kernel<XT, NE, false>), lgrid, dim3(NE * 64), 0, s, static_cast<const XT*>(a.x),
                            a.wr, a.bias, a.T, a.d, a.E, a.P, static_cast<bf16_t*>(a.rows16));
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     if (a.E <= 64)
-        hipLaunchKernelGGL((router_kernel<XT, 1>), dim3(nb), dim3(kRouterThreads), router_lds_bytes(a.E, a.k), s,
+        RB_LAUNCH((router_kernel<XT, 1>), dim3(nb), dim3(kRouterThreads), router_lds_bytes(a.E, a.k), s,
                            static_cast<const XT*>(a.x), a.wr, a.bias, a.valid, a.T, a.d, a.E, a.k, a.P, a.lse,
                            a.expert_of, a.gate_of, a.rank_in_block, a.blockcnt, a.partial);
     else
-        hipLaunchKernelGGL((router_kernel<XT, kMaxExperts / 64>), dim3(nb), dim3(kRouterThreads),
+        RB_LAUNCH((router_kernel<XT, kMaxExperts / 64>), dim3(nb), dim3(kRouterThreads),
                            router_lds_bytes(a.E, a.k), s, static_cast<const XT*>(a.x), a.wr, a.bias, a.valid, a.T, a.d,
                            a.E, a.k, a.P, a.lse, a.expert_of, a.gate_of, a.rank_in_block, a.blockcnt, a.partial);
     return hipGetLastError();
@@ -1276,7 +1276,7 @@ template <typename XT>
 static hipError_t launch_dispatch_t(const DispatchArgs& a, hipStream_t s) {
     const int nb = (a.T + kRouterTokens - 1) / kRouterTokens;
     if ((long long)nb * a.E <= kFusedScanLimit) {
-        hipLaunchKernelGGL(dispatch_fused_kernel<XT>, dim3(nb > 0 ? nb : 1), dim3(256),
+        RB_LAUNCH(dispatch_fused_kernel<XT>, dim3(nb > 0 ? nb : 1), dim3(256),
                            dispatch_fused_lds_bytes(a.E, a.k), s, static_cast<const XT*>(a.x), a.expert_of,
                            a.rank_in_block, a.blockcnt, a.partial, a.T, a.d, a.E, a.k, a.w_aux, a.w_z, a.tile_m,
                            a.counts, a.offsets, a.tile_expert, a.tile_row0, a.tile_rows, a.ntiles, a.losses,
@@ -1292,12 +1292,12 @@ static hipError_t launch_dispatch_t(const DispatchArgs& a, hipStream_t s) {
         if (e != hipSuccess) return e;
     }
     // runs for T == 0 too: it then writes zero counts, an empty tile table and zero losses
-    hipLaunchKernelGGL(layout_scan_kernel, dim3(1), dim3(kScanThreads), scan_lds_bytes(a.E), s, a.blockcnt, a.partial,
+    RB_LAUNCH(layout_scan_kernel, dim3(1), dim3(kScanThreads), scan_lds_bytes(a.E), s, a.blockcnt, a.partial,
                        nb, a.E, a.k, a.w_aux, a.w_z, a.tile_m, a.blockbase, a.counts, a.offsets, a.tile_expert,
                        a.tile_row0, a.tile_rows, a.ntiles, a.losses);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || nb == 0) return e;
-    hipLaunchKernelGGL(dispatch_kernel<XT>, dim3(nb), dim3(256), dispatch_lds_bytes(a.E, a.k), s,
+    RB_LAUNCH(dispatch_kernel<XT>, dim3(nb), dim3(256), dispatch_lds_bytes(a.E, a.k), s,
                        static_cast<const XT*>(a.x), a.expert_of, a.rank_in_block, a.blockbase, a.offsets, a.T, a.d,
                        a.E, a.k, a.perm_slot, a.perm_token, a.inv_pos, static_cast<XT*>(a.xg));
     return hipGetLastError();
@@ -1318,13 +1318,13 @@ static hipError_t launch_combine_t(const CombineArgs& a, hipStream_t s) {
         const long long total = (long long)a.T * (a.d / VN);
         const dim3 grid((unsigned)((total + 255) / 256)), block(256);
         if (a.k <= 2)
-            hipLaunchKernelGGL((combine_vec_kernel<XT, YT, 2>), grid, block, 0, s, y, ys, res, a.inv_pos, a.gate_of, a.T, a.d, a.k, out);
+            RB_LAUNCH((combine_vec_kernel<XT, YT, 2>), grid, block, 0, s, y, ys, res, a.inv_pos, a.gate_of, a.T, a.d, a.k, out);
         else if (a.k <= 4)
-            hipLaunchKernelGGL((combine_vec_kernel<XT, YT, 4>), grid, block, 0, s, y, ys, res, a.inv_pos, a.gate_of, a.T, a.d, a.k, out);
+            RB_LAUNCH((combine_vec_kernel<XT, YT, 4>), grid, block, 0, s, y, ys, res, a.inv_pos, a.gate_of, a.T, a.d, a.k, out);
         else
-            hipLaunchKernelGGL((combine_vec_kernel<XT, YT, 8>), grid, block, 0, s, y, ys, res, a.inv_pos, a.gate_of, a.T, a.d, a.k, out);
+            RB_LAUNCH((combine_vec_kernel<XT, YT, 8>), grid, block, 0, s, y, ys, res, a.inv_pos, a.gate_of, a.T, a.d, a.k, out);
     } else {
-        hipLaunchKernelGGL((combine_any_kernel<XT, YT>), dim3((a.T + 3) / 4), dim3(256), 0, s, y, ys, res, a.inv_pos,
+        RB_LAUNCH((combine_any_kernel<XT, YT>), dim3((a.T + 3) / 4), dim3(256), 0, s, y, ys, res, a.inv_pos,
                            a.gate_of, a.T, a.d, a.k, out);
     }
     return hipGetLastError();
@@ -1435,10 +1435,10 @@ hipError_t launch_rmsnorm_t(const XT* x, const float* weight, float eps, int T, 
     if (pieces_ok && pitch + 4 <= 40 * 1024) {
         const int R = std::max(1, std::min(64, (32 * 1024) / pitch));
         const size_t lds = (size_t)R * pitch + (size_t)R * 4;
-        hipLaunchKernelGGL(rmsnorm_rows_kernel<XT>, dim3((T + R - 1) / R), dim3(256), lds, s, x, weight, eps, T, d, R,
+        RB_LAUNCH(rmsnorm_rows_kernel<XT>, dim3((T + R - 1) / R), dim3(256), lds, s, x, weight, eps, T, d, R,
                            pitch, out);
     } else {
-        hipLaunchKernelGGL(rmsnorm_rows_direct_kernel<XT>, dim3((T + 63) / 64), dim3(64), 0, s, x, weight, eps, T, d,
+        RB_LAUNCH(rmsnorm_rows_direct_kernel<XT>, dim3((T + 63) / 64), dim3(64), 0, s, x, weight, eps, T, d,
                            out);
     }
     return hipGetLastError();

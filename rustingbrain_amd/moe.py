@@ -394,6 +394,35 @@ class MoeLayer:
                self.device.handle)
         return {name: float(ms[i]) for i, name in enumerate(L.STAGE_NAMES)}
 
+    def forward_kernel_times(self, x_ptr: int, tokens: int, out_ptr: int, valid_ptr: int = 0, bias_ptr: int = 0,
+                             residual_ptr: int = 0) -> dict:
+        """One forward whose launches carry their own start/stop events: kernel durations per stage in milliseconds,
+        as a kernel trace would report them."""
+        ms = (C.c_float * L.NUM_STAGES)()
+        _check(self._lib.rbmoe_forward_kernel_times(self.handle, C.c_void_p(x_ptr), tokens, self._d_model,
+                                                    C.c_void_p(valid_ptr or None), C.c_void_p(bias_ptr or None),
+                                                    C.c_void_p(residual_ptr or None), C.c_void_p(out_ptr), ms),
+               self.device.handle)
+        return {name: float(ms[i]) for i, name in enumerate(L.STAGE_NAMES)}
+
+    def replay_stage(self, stage: str, launches: int = 20) -> Optional[float]:
+        """Average launch time in milliseconds of one stage of the last forward (``_lib.STAGE_NAMES``), replayed
+        ``launches`` times between one pair of events; None when the last forward had no launch for the stage."""
+        ms = C.c_float()
+        rc = self._lib.rbmoe_replay_stage(self.handle, L.STAGE_NAMES.index(stage), launches, C.byref(ms))
+        if rc == L.UNSUPPORTED:
+            return None
+        _check(rc, self.device.handle)
+        return float(ms.value)
+
+    def enqueue_stage(self, stage: str, launches: int = 1) -> bool:
+        """The launches of one stage of the last forward again, enqueued only (the caller times the sequence)."""
+        rc = self._lib.rbmoe_replay_stage(self.handle, L.STAGE_NAMES.index(stage), launches, None)
+        if rc == L.UNSUPPORTED:
+            return False
+        _check(rc, self.device.handle)
+        return True
+
     def losses(self) -> Tuple[float, float]:
         aux, z = C.c_float(), C.c_float()
         _check(self._lib.rbmoe_get_losses(self.handle, C.byref(aux), C.byref(z)), self.device.handle)

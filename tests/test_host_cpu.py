@@ -187,3 +187,16 @@ def test_weight_gradient_workspace_holds_every_batch_up_to_max_tokens():
             worst = max(worst, need.value)
             assert need.value <= held.value, (M, N, groups, tokens, need.value, held.value)
         assert worst == held.value   # and no more than the worst case asks for
+
+
+def test_bench_helper_library_exports_what_its_header_declares():
+    header = open(os.path.join(ROOT, "include", "rbmoe_bench.h")).read()
+    declared = set(re.findall(r"\b(rbbench_[a-z_0-9]+)\s*\(", header))
+    assert declared == set(L.BENCH_SIGNATURES), (declared ^ set(L.BENCH_SIGNATURES))
+    lib = L.load_bench()
+    for name in sorted(declared):
+        assert hasattr(lib, name), f"{name} is declared in rbmoe_bench.h but not exported"
+    # ... and the layer's library holds none of it
+    main = L.load()
+    assert not [n for n in declared if hasattr(main, n)]
+    assert not hasattr(main, "rbmoe_calibrate_mfma")
