@@ -147,7 +147,8 @@ typedef enum rbmoe_option {
     RBMOE_OPT_FUSED_ROUTER = 5,    /* 0: router logits and the routing behind them in separate launches */
     RBMOE_OPT_SIDE_STREAM = 6,     /* 0: everything on the context's one stream */
     RBMOE_OPT_WGRAD_MODE = 7,      /* cut experts' weight gradients: 0 fixed order (default), 1 f32 atomics, 2 never cut */
-    RBMOE_OPT_WGRAD_GENERIC = 8    /* 1: the plain kernel for the weight gradients */
+    RBMOE_OPT_WGRAD_GENERIC = 8,   /* 1: the plain kernel for the weight gradients */
+    RBMOE_OPT_DECODE_COMBINE_FOLD = 9 /* 0: decode-shaped calls combine in a launch of their own */
 } rbmoe_option;
 int rbmoe_layer_set_option(rbmoe_layer* layer, int32_t option, int32_t value);
 

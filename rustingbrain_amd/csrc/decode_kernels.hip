@@ -545,6 +545,10 @@ struct DecodeSide {
     int N, K, row0, rows;
     int a_row0;    // added to a row's number in `a` (rows of one expert inside a per-expert array)
     int out_row0;  // first output row is out_row0 + row0
+    // The rows are read again inside this launch by a workgroup that may sit on another XCD (the folded combine): the
+    // XCDs' L2 caches are not coherent with one another, so such rows are stored with device-scope stores, which
+    // go through to memory, and read back with device-scope loads.
+    bool coherent_out = false;
 };
 
 // NW = waves of a workgroup, each with 1 / NW of the reduction steps: 4 for the gate/up product, 8 for the
@@ -553,9 +557,61 @@ struct DecodeSide {
 template <bool SWIGLU, bool I8, int NW, int BATCH>
 __device__ __forceinline__ void decode_gemm_body(const DecodeSide& sd, int fb, float* red_raw);
 
+// The combine of a decode-shaped call, for the 32 output features of block `fb` and every token: what
+// combine_vec_kernel computes, element by element in the same order (the token's expert rows by ascending position,
+// i.e. ascending expert; gate * row as a rounded multiply, then a rounded add; then the shared expert's row; then
+// the residual).  Run by the last workgroup of the block's column to finish; the rows were stored with device-scope
+// stores and are read with device-scope loads (see DecodeSide::coherent_out).
+template <typename XT>
+__device__ __forceinline__ void decode_combine_block(const DecodeGemmArgs& g, int fb, int nthreads) {
+    const bf16_t* const y = static_cast<const bf16_t*>(g.out);
+    const bf16_t* const ys = g.a_shared ? static_cast<const bf16_t*>(g.out_shared) : nullptr;
+    const XT* const res = static_cast<const XT*>(g.cmb_residual);
+    XT* const out = static_cast<XT*>(g.cmb_out);
+    const int d = g.N, k = g.cmb_k;
+    for (int idx = threadIdx.x; idx < g.cmb_T * 16; idx += nthreads) {
+        const int t = idx >> 4;
+        const int c = fb * 32 + 2 * (idx & 15);
+        const int* const ip = g.cmb_inv_pos + (size_t)t * k;
+        const float* const gp = g.cmb_gate_of + (size_t)t * k;
+        float a0 = 0.0f, a1 = 0.0f;
+        int last = -1;
+        for (int r = 0; r < k; ++r) {
+            int best = 0x7fffffff, bi = -1;  // next smallest position greater than `last`
+            for (int q = 0; q < k; ++q) {
+                const int p = ip[q];
+                if (p > last && p < best) {
+                    best = p;
+                    bi = q;
+                }
+            }
+            if (bi < 0) break;
+            last = best;
+            const uint32_t v = __hip_atomic_load(reinterpret_cast<const uint32_t*>(y + (size_t)best * d + c),
+                                                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const float gt = gp[bi];
+            a0 = __fadd_rn(a0, __fmul_rn(gt, __uint_as_float(v << 16)));
+            a1 = __fadd_rn(a1, __fmul_rn(gt, __uint_as_float(v & 0xffff0000u)));
+        }
+        if (ys) {
+            const uint32_t v = __hip_atomic_load(reinterpret_cast<const uint32_t*>(ys + (size_t)t * d + c),
+                                                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            a0 = __fadd_rn(a0, __uint_as_float(v << 16));
+            a1 = __fadd_rn(a1, __uint_as_float(v & 0xffff0000u));
+        }
+        if (res) {
+            a0 = __fadd_rn(a0, to_f32(res[(size_t)t * d + c]));
+            a1 = __fadd_rn(a1, to_f32(res[(size_t)t * d + c + 1]));
+        }
+        out[(size_t)t * d + c] = from_f32<XT>(a0);
+        out[(size_t)t * d + c + 1] = from_f32<XT>(a1);
+    }
+}
+
 template <bool SWIGLU, bool I8, int NW>
 __global__ __launch_bounds__(NW * 64) void decode_gemm_kernel(DecodeGemmArgs g) {
     __shared__ float red[NW * (SWIGLU ? 2 : 1) * 16 * 64];
+    __shared__ int last_of_block;
     const int fb = blockIdx.x;
     const int ty = blockIdx.y;
     DecodeSide sd;
@@ -569,8 +625,11 @@ __global__ __launch_bounds__(NW * 64) void decode_gemm_kernel(DecodeGemmArgs g) 
     const int live_tiles = *g.ntiles;
     const int t_expert = g.tile_expert[tix], t_row0 = g.tile_row0[tix], t_rows = g.tile_rows[tix];
     asm volatile("" ::"s"(live_tiles), "s"(t_expert), "s"(t_row0), "s"(t_rows));  // all four here, not sunk into the branches
+    // workgroups that write rows of this feature block's columns: the live routed tiles and the shared expert's
+    const int writers = live_tiles + (g.a_shared ? (g.T_shared + 31) / 32 : 0);
+    bool works = true;
     if (routed) {
-        if (ty >= live_tiles) return;
+        if (ty >= live_tiles) works = false;
         const int expert = t_expert;
         sd.a = static_cast<const bf16_t*>(g.a);
         sd.row_index = g.row_index;
@@ -595,6 +654,35 @@ __global__ __launch_bounds__(NW * 64) void decode_gemm_kernel(DecodeGemmArgs g) 
         sd.rows = min(32, g.T_shared - sd.row0);
     }
     if (fb * 32 >= sd.N) return;
+    if constexpr (!SWIGLU) {
+        if (g.cmb_out != nullptr) {  // uniform over the launch
+            if (!works) {
+                // nothing to multiply here; with no writer at all (every row is padding and there is no shared
+                // expert) the first of these workgroups still owes the block its combine
+                if (writers != 0 || ty != 0) return;
+            } else {
+                sd.coherent_out = true;
+                decode_gemm_body<SWIGLU, I8, NW, kBatch>(sd, fb, red);
+                // every wave's row stores have completed (at device scope: they are device-scope stores) before
+                // the workgroup's arrival is counted.  No device-scope fence: that would write back this XCD's
+                // whole L2, once per workgroup.
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                __syncthreads();
+                if (threadIdx.x == 0) {
+                    const int before = atomicAdd(&g.cmb_counter[fb], 1);
+                    last_of_block = before == writers - 1;
+                    if (before == writers - 1) atomicExch(&g.cmb_counter[fb], 0);  // every writer has arrived: ready for the next launch
+                }
+                __syncthreads();
+                if (!last_of_block) return;
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+            }
+            if (g.cmb_f32) decode_combine_block<float>(g, fb, NW * 64);
+            else decode_combine_block<bf16_t>(g, fb, NW * 64);
+            return;
+        }
+    }
+    if (!works) return;
     decode_gemm_body<SWIGLU, I8, NW, kBatch>(sd, fb, red);
 }
 
@@ -686,7 +774,14 @@ __device__ __forceinline__ void decode_gemm_body(const DecodeSide& sd, int fb, f
             if constexpr (I8) u *= sd.scales[sd.N + fb * 32 + f];
             y = silu_bf16_grade(y) * u;
         }
-        if (token < sd.rows) sd.out[(size_t)(sd.out_row0 + sd.row0 + token) * sd.N + fb * 32 + f] = from_f32<bf16_t>(y);
+        if (token < sd.rows) {
+            bf16_t* const where = sd.out + (size_t)(sd.out_row0 + sd.row0 + token) * sd.N + fb * 32 + f;
+            if (sd.coherent_out)
+                __hip_atomic_store(reinterpret_cast<unsigned short*>(where), (unsigned short)f32_to_bf16_bits(y),
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            else
+                *where = from_f32<bf16_t>(y);
+        }
     }
 }
 
@@ -742,7 +837,7 @@ __global__ __launch_bounds__(kSmallThreads, 2) void decode_front_kernel(SmallRou
         sd.out_row0 = 0;
     }
     if (fb * 32 >= sd.N) return;
-    decode_gemm_body<true, I8, kSmallThreads / 64, kBatch / 2>(sd, fb, reinterpret_cast<float*>(smem));
+    decode_gemm_body<true, I8, kSmallThreads / 64, kBatch>(sd, fb, reinterpret_cast<float*>(smem));
 }
 
 bool decode_front_ok(const void* x, const float* wr, int T, int d, int E, int k) {
@@ -776,6 +871,11 @@ hipError_t launch_decode_gemm(const DecodeGemmArgs& g, WeightKind wk, hipStream_
     const int tiles = g.max_tiles + shared_tiles;
     if (tiles <= 0) return hipSuccess;
     const int widest = g.a_shared ? (g.N > g.N_shared ? g.N : g.N_shared) : g.N;
+    if (g.cmb_out != nullptr) {  // the combine rides on a down-shaped launch whose two sides have the same width
+        if (g.swiglu || !g.cmb_counter || !g.cmb_inv_pos || !g.cmb_gate_of || (g.a_shared && g.N_shared != g.N) ||
+            g.N / 32 > kDecodeCombineMaxBlocks || g.N % 2 != 0)
+            return hipErrorInvalidValue;
+    }
     const dim3 grid(widest / 32, tiles);
     if (wk == WeightKind::BF16) {
         if (g.swiglu) RB_LAUNCH((decode_gemm_kernel<true, false, 4>), grid, dim3(256), 0, s, g);

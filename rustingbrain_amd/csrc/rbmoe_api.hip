@@ -171,6 +171,7 @@ struct Work {
     void* ys = nullptr;
     void* hall = nullptr;  // hidden rows of every expert over every row, [E][T, F] (decode_front launches), or null
     void* x16 = nullptr;   // bf16 copy of f32 rows [T, d] (layers with cast_rows), or null
+    int* cmb_counter = nullptr;  // arrival counters of a combine folded into the decode-shaped down launch (all zero between launches)
 };
 
 struct rbmoe_layer {
@@ -193,6 +194,7 @@ struct rbmoe_layer {
     bool decode_front = true;  // ... three, with the routing beside the gate/up products, when most experts are touched
     bool shared_beside = true; // large batches: the shared expert's products on the side stream, beside the routing
     bool fused_router = true;  // logits and everything behind them in one launch where the shapes allow
+    bool decode_fold = true;   // decode-shaped calls: the combine inside the down launch
     bool last_front = false;   // the last forward's hidden rows are per expert over all rows (Work::hall)
     int group_m = 0;
     const char* kernel_name = "none";
@@ -212,6 +214,7 @@ struct rbmoe_layer {
     Buf xg, h, y, hs, ys;
     Buf x16;               // [max_T, d] bf16 copy of f32 rows (cast_rows)
     Buf hall;              // [E][min(max_T, 32), F] hidden rows of decode_front launches
+    Buf cmbcnt;            // [kDecodeCombineMaxBlocks] arrival counters of the folded decode combine
     // feed-forward norm in front of the layer (allocated by rbmoe_set_feed_forward_norm)
     Buf xn, norm_w;  // [max_T, d] activation dtype, [d] f32
     float norm_eps = 0.0f;
@@ -333,6 +336,7 @@ Plan make_plan(rbmoe_layer* L) {
     if (L->cast_rows) p.add(&L->x16, T * d * 2);
     // decode_front launches need most experts touched (tokens * k >= 2 E, at most 32 tokens): none when E > 16 k
     if (L->use_stream && E <= 16 * k) p.add(&L->hall, E * std::min<size_t>(T, kSmallRouteMaxTokens) * F * 2);
+    p.add(&L->cmbcnt, (size_t)kDecodeCombineMaxBlocks * 4);
     p.add(&L->xg, S * d * as);
     p.add(&L->h, S * F * as);
     p.add(&L->y, S * d * as);
@@ -795,6 +799,7 @@ Work work_of_layer(const rbmoe_layer* L) {
     w.h = L->h.p; w.y = L->y.p; w.hs = L->hs.p; w.ys = L->ys.p;
     w.hall = L->hall.p;
     w.x16 = L->x16.p;
+    w.cmb_counter = (int*)L->cmbcnt.p;
     return w;
 }
 
@@ -812,6 +817,9 @@ size_t carve_decode_work(const rbmoe_layer* L, int T, unsigned char* base, Work*
         return p;
     };
     Work v;
+    // first, at the same place for every call and every layer: the arrival counters of the folded combine, which are
+    // zero whenever no call is running (the array starts as zeros and every launch leaves them as it found them)
+    v.cmb_counter = (int*)take((size_t)kDecodeCombineMaxBlocks * 4);
     v.P = (float*)take((size_t)T * E * 4); v.lse = (float*)take((size_t)T * 4);
     v.expert_of = (int*)take(S * 4); v.gate_of = (float*)take(S * 4);
     v.counts = (int*)take(E * 4); v.offsets = (int*)take((E + 1) * 4);
@@ -999,14 +1007,25 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
             d2.scales_shared = wk == WeightKind::I8 ? (const float*)L->ssd.p : nullptr;
             d2.N_shared = d; d2.K_shared = Fs; d2.out_shared = wk_.ys;
         }
+        // the combine inside the same launch: the last workgroup of every block of 32 output columns to finish
+        // sums that block (same order, same roundings as combine_vec_kernel)
+        const bool fold = L->decode_fold && d / 32 <= kDecodeCombineMaxBlocks && wk_.cmb_counter != nullptr;
+        if (fold) {
+            d2.cmb_counter = wk_.cmb_counter;
+            d2.cmb_inv_pos = wk_.inv_pos; d2.cmb_gate_of = wk_.gate_of;
+            d2.cmb_residual = residual; d2.cmb_out = out;
+            d2.cmb_T = T; d2.cmb_k = k; d2.cmb_f32 = abf ? 0 : 1;
+        }
         HIP_TRY(ctx, launch_decode_gemm(d2, wk, s));
         L->replay[RBMOE_STAGE_DOWN] = [=](hipStream_t st) { return launch_decode_gemm(d2, wk, st); };
         HIP_TRY(ctx, mark(5));
         HIP_TRY(ctx, mark(6));
-        CombineArgs cd{wk_.y, c.shared_expert ? wk_.ys : nullptr, residual, wk_.inv_pos, wk_.gate_of, T, d, k, out};
-        cd.rows_bf16 = cast;
-        HIP_TRY(ctx, launch_combine(cd, abf, s));
-        L->replay[RBMOE_STAGE_COMBINE] = [=](hipStream_t st) { return launch_combine(cd, abf, st); };
+        if (!fold) {
+            CombineArgs cd{wk_.y, c.shared_expert ? wk_.ys : nullptr, residual, wk_.inv_pos, wk_.gate_of, T, d, k, out};
+            cd.rows_bf16 = cast;
+            HIP_TRY(ctx, launch_combine(cd, abf, s));
+            L->replay[RBMOE_STAGE_COMBINE] = [=](hipStream_t st) { return launch_combine(cd, abf, st); };
+        }
         HIP_TRY(ctx, mark(7));
         L->last_T = T;
         L->last = wk_;
@@ -1534,6 +1553,7 @@ int rbmoe_layer_set_option(rbmoe_layer* L, int32_t option, int32_t value) {
         case RBMOE_OPT_DECODE_PATH: L->decode_path = value != 0; return RBMOE_OK;
         case RBMOE_OPT_DECODE_FRONT: L->decode_front = value != 0; return RBMOE_OK;
         case RBMOE_OPT_FUSED_ROUTER: L->fused_router = value != 0; return RBMOE_OK;
+        case RBMOE_OPT_DECODE_COMBINE_FOLD: L->decode_fold = value != 0; return RBMOE_OK;
         case RBMOE_OPT_SIDE_STREAM:
             if (value != 0 && L->training)
                 if (const int rc = ensure_side_stream(ctx)) return rc;

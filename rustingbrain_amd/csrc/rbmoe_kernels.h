@@ -272,7 +272,20 @@ struct DecodeGemmArgs {
     int N_shared, K_shared, T_shared;
     void* out_shared;
     int swiglu;
+    // Down-shaped launches only, all null / zero otherwise: the combine folded into the launch.  The last workgroup
+    // of a feature block to finish (one counter per block of 32 output features: zero before the launch, zero
+    // again after it) sums that block's columns for every token - the token's expert rows in ascending expert order,
+    // a rounded multiply by the gate and a rounded add each, then the shared expert's row, then the residual - and
+    // writes them to cmb_out.  Nobody waits for anybody: whoever arrives last does the work.
+    int* cmb_counter = nullptr;           // [N / 32]
+    const int* cmb_inv_pos = nullptr;     // [T * k]
+    const float* cmb_gate_of = nullptr;   // [T * k]
+    const void* cmb_residual = nullptr;   // [T, N] bf16, or f32 when cmb_f32, or null
+    void* cmb_out = nullptr;              // [T, N] bf16, or f32 when cmb_f32; null: no combine in this launch
+    int cmb_T = 0, cmb_k = 0;
+    int cmb_f32 = 0;
 };
+constexpr int kDecodeCombineMaxBlocks = 1024;  // feature blocks a folded combine has counters for
 bool decode_shape_ok(int N, int K);
 hipError_t launch_decode_gemm(const DecodeGemmArgs& g, WeightKind wk, hipStream_t s);
 // Routing and gate/up products in one launch (bf16 rows, no norm): every expert's gate/up product over all T rows,

@@ -84,7 +84,7 @@ _ENV_SWITCHES = {
     "RBMOE_NO_DECODE_PATH": (L.OPT_DECODE_PATH, 0), "RBMOE_NO_DECODE_FRONT": (L.OPT_DECODE_FRONT, 0),
     "RBMOE_NO_FUSED_ROUTER": (L.OPT_FUSED_ROUTER, 0), "RBMOE_NO_SIDE_STREAM": (L.OPT_SIDE_STREAM, 0),
     "RBMOE_ATOMIC_WGRAD": (L.OPT_WGRAD_MODE, 1), "RBMOE_DETERMINISTIC": (L.OPT_WGRAD_MODE, 2),
-    "RBMOE_WGRAD_GENERIC": (L.OPT_WGRAD_GENERIC, 1),
+    "RBMOE_WGRAD_GENERIC": (L.OPT_WGRAD_GENERIC, 1), "RBMOE_NO_DECODE_COMBINE_FOLD": (L.OPT_DECODE_COMBINE_FOLD, 0),
 }
 
 

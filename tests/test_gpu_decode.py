@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 
 @pytest.fixture
 def env():
-    keys = ("RBMOE_NO_DECODE_PATH", "RBMOE_NO_DECODE_FRONT")
+    keys = ("RBMOE_NO_DECODE_PATH", "RBMOE_NO_DECODE_FRONT", "RBMOE_NO_DECODE_COMBINE_FOLD")
     saved = {k: os.environ.get(k) for k in keys}
     yield os.environ
     for k, v in saved.items():
@@ -153,3 +153,39 @@ def test_routing_beside_the_products_changes_nothing_but_the_launch_count(device
     env.pop("RBMOE_NO_DECODE_FRONT", None)
     name, _, _ = run(device, t)
     assert name.startswith("mfma_bf16_decode") and "front" not in name
+
+
+@pytest.mark.parametrize("case", [
+    dict(act="bf16", wt="bf16", shared=True, T=13, k=2, pad="some", residual=True),
+    dict(act="bf16", wt="int8", shared=False, T=32, k=3, pad="none", residual=False),
+    dict(act="bf16", wt="bf16", shared=False, T=6, k=2, pad="all", residual=True),    # no workgroup writes a row
+    dict(act="bf16", wt="bf16", shared=True, T=6, k=2, pad="all", residual=False),    # only the shared expert does
+    dict(act="f32", wt="bf16", shared=True, T=9, k=4, pad="some", residual=True),     # f32 rows over bf16 weights
+], ids=lambda c: "{act}_{wt}_T{T}_k{k}_pad-{pad}".format(**c))
+def test_the_combine_inside_the_down_launch_gives_the_bits_of_the_combine_launch(device, env, case):
+    """The last workgroup of a column block to finish sums the block: same order and roundings as the combine
+    kernel, so the outputs agree in every bit - twice in a row (the arrival counters must be back at zero), with
+    padding rows, with nothing routed at all, with a residual, with f32 rows."""
+    T, k = case["T"], case["k"]
+    t = synth.make(small_workload(d=128, E=8, k=k, F=192, T=T, seed=83, act=case["act"], wt=case["wt"],
+                                  shared=case["shared"], shared_d_ff=128))
+    valid = {"none": None, "some": (np.arange(T) % 3 != 1).astype(np.uint8), "all": np.zeros(T, np.uint8)}[case["pad"]]
+    residual = synth.round_bf16(synth.normal((T, 128), 1.0, 83, 7)) if case["residual"] else None
+    layout = rb.Layout(valid=None if valid is None else [bool(v) for v in valid])
+    outs = {}
+    for fold in (True, False):
+        if fold:
+            env.pop("RBMOE_NO_DECODE_COMBINE_FOLD", None)
+        else:
+            env["RBMOE_NO_DECODE_COMBINE_FOLD"] = "1"
+        layer = gpu_layer(device, t)
+        a, _ = layer.forward_train(t.x, layout, residual=residual)
+        b, _ = layer.forward_train(t.x, layout, residual=residual)
+        assert layer.kernel_name().startswith("mfma_bf16_decode")
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+        outs[fold] = a
+        layer.close()
+    assert np.array_equal(outs[True].view(np.uint32), outs[False].view(np.uint32))
+    ref = oracle_layer(t).forward(t.x, valid=valid, threads=4)
+    want = ref.out if residual is None else ref.out + residual
+    assert rel_l2(outs[True], want) <= 2e-2 if np.any(want) else not np.any(outs[True])

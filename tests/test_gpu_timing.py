@@ -37,7 +37,8 @@ def test_measuring_entry_points_leave_the_results_alone(device, shape):
     ob.upload(np.zeros_like(x))
     kt = layer.forward_kernel_times(xb.ptr, T, ob.ptr)
     assert same(snapshot(), plain)
-    assert kt["gate_up"] > 0 and kt["down"] > 0 and kt["combine"] > 0 and kt["empty"] == 0
+    decode = "decode" in layer.kernel_name()   # decode-shaped: the combine rides in the down launch
+    assert kt["gate_up"] > 0 and kt["down"] > 0 and (kt["combine"] > 0) != decode and kt["empty"] == 0
     assert abs(kt["total"] - sum(v for k, v in kt.items() if k != "total")) <= 1e-6
     assert kt["total"] < 5.0          # milliseconds: these are kernel durations, not garbage
     if shape["shared"] if "shared" in shape else False:
@@ -50,6 +51,9 @@ def test_measuring_entry_points_leave_the_results_alone(device, shape):
         ob.upload(np.zeros_like(x))
         layer.forward_device(xb.ptr, T, ob.ptr)
         ms = layer.replay_stage(stage, 5)
+        if stage == "combine" and decode:
+            assert ms is None
+            continue
         assert ms is not None and 0 < ms < 5.0
         assert layer.enqueue_stage(stage, 2)
         assert same(snapshot(), plain), stage
