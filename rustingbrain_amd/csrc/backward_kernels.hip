@@ -570,6 +570,29 @@ hipError_t launch_rmsnorm_backward(const void* x, const void* up, const float* w
     return hipGetLastError();
 }
 
+// out[i] = bf16(in[i]) (nearest even), 8 elements per thread; n a multiple of 8
+__global__ __launch_bounds__(256) void cast_rows_bf16_kernel(const float* __restrict__ in, bf16_t* __restrict__ out,
+                                                             long long n8) {
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n8) return;
+    const float4 a = reinterpret_cast<const float4*>(in)[2 * i], b = reinterpret_cast<const float4*>(in)[2 * i + 1];
+    uint4 o;
+    o.x = f32_to_bf16_bits(a.x) | ((uint32_t)f32_to_bf16_bits(a.y) << 16);
+    o.y = f32_to_bf16_bits(a.z) | ((uint32_t)f32_to_bf16_bits(a.w) << 16);
+    o.z = f32_to_bf16_bits(b.x) | ((uint32_t)f32_to_bf16_bits(b.y) << 16);
+    o.w = f32_to_bf16_bits(b.z) | ((uint32_t)f32_to_bf16_bits(b.w) << 16);
+    reinterpret_cast<uint4*>(out)[i] = o;
+}
+
+hipError_t launch_cast_rows_bf16(const float* in, void* out, long long n, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    if (n % 8 != 0) return hipErrorInvalidValue;
+    const long long n8 = n / 8;
+    hipLaunchKernelGGL(cast_rows_bf16_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, s, in,
+                       static_cast<bf16_t*>(out), n8);
+    return hipGetLastError();
+}
+
 hipError_t launch_fill_f32(float* p, float v, long long n, hipStream_t s) {
     if (n <= 0) return hipSuccess;
     hipLaunchKernelGGL(fill_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, v, n);

@@ -228,6 +228,7 @@ struct rbmoe_layer {
     Buf xc;                               // copy of the last input [T, d]
     Buf gu, gus;                          // pre-activations (gate | up): [S, 2F], shared [T, 2Fs]
     Buf dy, dgu, dxg;                     // [S, d], [S, 2F], [S, d]
+    Buf g16;                              // [T, d] bf16 copy of an f32 upstream gradient (cast_rows)
     Buf dgus, dxs;                        // shared: [T, 2Fs], [T, d]
     Buf grad_gates, ones, dlogits, dxr, rpartial;
     Buf g_router, g_gu, g_down, g_sgu, g_sdown;   // f32 weight gradients, accumulated
@@ -1454,12 +1455,10 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
         return fail(ctx, RBMOE_UNSUPPORTED, "the backward pass is not defined for int8 weights");
     if (L->weights_set)
         return fail(ctx, RBMOE_INVALID_CONFIG, "enable training before the weights are set");
-    if (L->cast_rows) {
-        // f32 rows with bf16 weights differentiate on the plain kernels, in both directions, on the f32 rows
-        // themselves (no weight has been set yet, so none has been packed for the matrix cores)
-        L->cast_rows = false;
-        L->use_stream = false;
-    }
+    // (f32 rows over bf16 weights - the reference's own mixed-precision shape, src/gpu_model.rs:2146-2153 - stay on
+    // the matrix cores in both directions: the products read the bf16 copy of the rows that the forward writes
+    // anyway and a bf16 copy of the upstream gradient that the backward pass writes first; the router's branch,
+    // the norm and the sums that end in the caller's buffers stay f32)
     const bool bf16_layer = L->use_stream && c.weight_dtype == RBMOE_BF16;
     if (L->max_T > router_grad_max_tokens()) {  // found here, not in the middle of a backward pass
         char buf[160];
@@ -1481,12 +1480,14 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
     // (any other layer - odd widths, mixed dtypes - takes the any-shape kernels in both directions)
     const size_t ws = dtype_size(c.weight_dtype);  // bytes per element of the transposed weight copies
     const size_t as = dtype_size(c.act_dtype);
+    const size_t ps = L->cast_rows ? 2 : as;       // bytes per element of the rows the products read and write
     Plan p;
     p.add(&L->xc, T * d * as);
-    p.add(&L->gu, S * 2 * F * as);
-    p.add(&L->dy, S * d * as);
-    p.add(&L->dgu, S * 2 * F * as);
-    p.add(&L->dxg, S * d * as);
+    if (L->cast_rows) p.add(&L->g16, T * d * 2);
+    p.add(&L->gu, S * 2 * F * ps);
+    p.add(&L->dy, S * d * ps);
+    p.add(&L->dgu, S * 2 * F * ps);
+    p.add(&L->dxg, S * d * ps);
     p.add(&L->grad_gates, S * 4);
     p.add(&L->ones, S * 4);
     p.add(&L->dlogits, T * E * 4);
@@ -1501,7 +1502,7 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
     // How the weight gradients treat an expert far above the average share (and the shared expert, whose one
     // group of rows is always cut): in a fixed order by default (RBMOE_OPT_WGRAD_MODE for f32 atomics or no cut).
     if (L->wgrad_split == WgradSplit::Ordered) {
-        const bool wbf = c.act_dtype == RBMOE_BF16;
+        const bool wbf = c.act_dtype == RBMOE_BF16 || L->cast_rows;
         // sized for every token count up to max_tokens: a smaller batch can need more partial matrices than the
         // largest one, because the cut limit follows the row count with a floor and a rounding
         const int k = c.experts_per_token;
@@ -1515,20 +1516,21 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
     p.add(&L->st_gout, T * d * as);
     p.add(&L->st_gin, T * d * as);
     if (c.shared_expert) {
-        p.add(&L->gus, T * 2 * Fs * as);
-        p.add(&L->dgus, T * 2 * Fs * as);
-        p.add(&L->dxs, T * d * as);
+        p.add(&L->gus, T * 2 * Fs * ps);
+        p.add(&L->dgus, T * 2 * Fs * ps);
+        p.add(&L->dxs, T * d * ps);
         p.add(&L->g_sgu, 2 * Fs * d * 4);
         p.add(&L->g_sdown, d * Fs * 4);
         p.add(&L->swdT, Fs * d * ws);
         p.add(&L->swguT, d * 2 * Fs * ws);
     }
+    // (the second stream first: a failure there must not leave buffers behind that a second attempt would allocate again)
+    if (L->shared_beside)
+        if (const int rc = ensure_side_stream(ctx)) return rc;
     if (const int rc = allocate_plan(L, p, "the training buffers")) return rc;
     HIP_TRY(ctx, launch_fill_f32((float*)L->ones.p, 1.0f, (long long)S, ctx->stream));
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
     L->side_branch = L->shared_beside;
-    if (L->side_branch)
-        if (const int rc = ensure_side_stream(ctx)) return rc;
     L->training = true;
     L->grads_clear = true;
     return ensure_block_training_buffers(L);
@@ -1613,14 +1615,22 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, int32_t tokens, int3
     if (!grad_output || !grad_input) return fail(ctx, RBMOE_NULL_POINTER, "grad_output or grad_input is NULL");
     HIP_TRY(ctx, hipSetDevice(ctx->device));
     hipStream_t s = ctx->stream;
-    const bool abf = c.act_dtype == RBMOE_BF16;
+    const bool xbf = c.act_dtype == RBMOE_BF16;       // the caller's rows and gradients
+    const bool cast = L->cast_rows;                   // ... are f32, the products' rows bf16
+    const bool abf = xbf || cast;                     // the rows of the expert products
     const int S = T * k;
     const int* offsets = (const int*)L->offsets.p;
     const int* counts = (const int*)L->counts.p;
+    // what the expert branch reads of the upstream gradient: the caller's rows, or their bf16 copy
+    const void* gout = grad_output;
+    if (cast) {
+        HIP_TRY(ctx, launch_cast_rows_bf16((const float*)grad_output, L->g16.p, (long long)T * d, s));
+        gout = L->g16.p;
+    }
 
     // upstream of every expert: gate * dOut[token]; gate gradient: dOut[token] . Y[row]
     // (grad_gates of unrouted slots stays unwritten: the only reader skips padding rows)
-    HIP_TRY(ctx, launch_scale_rows(grad_output, L->y.p, (const int*)L->perm_slot.p, (const int*)L->perm_token.p,
+    HIP_TRY(ctx, launch_scale_rows(gout, L->y.p, (const int*)L->perm_slot.p, (const int*)L->perm_token.p,
                                    (const float*)L->gate_of.p, offsets, E, d, S, L->dy.p, (float*)L->grad_gates.p, abf,
                                    s));
     // The router's branch needs nothing but the gate gradients from here on and is a handful of small launches
@@ -1640,7 +1650,7 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, int32_t tokens, int3
                                        (const float*)L->grad_gates.p, counts, offsets, T, E, k, c.aux_loss_weight,
                                        c.router_z_loss_weight, (float*)L->dlogits.p, rs));
     HIP_TRY(ctx, launch_router_grad((const float*)L->dlogits.p, L->xc.p, (const float*)L->router.p, T, d, E,
-                                    (float*)L->rpartial.p, (float*)L->g_router.p, L->dxr.p, abf, rs));
+                                    (float*)L->rpartial.p, (float*)L->g_router.p, L->dxr.p, xbf, rs));
 
     // SwiGlu::backward over the routed rows (src/ffn.rs:87-120)
     GroupedArgs g{};
@@ -1694,15 +1704,15 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, int32_t tokens, int3
     if (c.shared_expert) {
         GroupedArgs sh = g;
         sh.dense_rows = T;
-        sh.a = grad_output; sh.w = L->swdT.p; sh.w_expert_stride = 0; sh.N = Fs; sh.K = d;
+        sh.a = gout; sh.w = L->swdT.p; sh.w_expert_stride = 0; sh.N = Fs; sh.K = d;
         sh.swiglu_grad_gu = L->gus.p; sh.gu_out = L->dgus.p;
         HIP_TRY(ctx, prod(sh));
         GroupedArgs sx = g;
         sx.dense_rows = T; sx.w_expert_stride = 0;
         sx.a = L->dgus.p; sx.w = L->swguT.p; sx.N = d; sx.K = 2 * Fs; sx.out = L->dxs.p;
         HIP_TRY(ctx, prod(sx));
-        HIP_TRY(ctx, wgrad(grad_output, d, L->hs.p, nullptr, Fs, 1, T, T, (float*)L->g_sdown.p, 0));
-        HIP_TRY(ctx, wgrad(L->dgus.p, 2 * Fs, L->xc.p, nullptr, d, 1, T, T, (float*)L->g_sgu.p, 0));
+        HIP_TRY(ctx, wgrad(gout, d, L->hs.p, nullptr, Fs, 1, T, T, (float*)L->g_sdown.p, 0));
+        HIP_TRY(ctx, wgrad(L->dgus.p, 2 * Fs, cast ? L->x16.p : L->xc.p, nullptr, d, 1, T, T, (float*)L->g_sgu.p, 0));
     }
     // grad_input = sum over a token's slots of its expert rows + shared + router
     if (side) HIP_TRY(ctx, hipStreamWaitEvent(s, ctx->ev_join, 0));
@@ -1718,7 +1728,8 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, int32_t tokens, int3
     }
     CombineArgs ca{L->dxg.p, c.shared_expert ? L->dxs.p : nullptr, L->dxr.p, (const int*)L->inv_pos.p,
                    (const float*)L->ones.p, T, d, k, grad_input};
-    HIP_TRY(ctx, launch_combine(ca, abf, s));
+    ca.rows_bf16 = cast;
+    HIP_TRY(ctx, launch_combine(ca, xbf, s));
     L->grads_clear = false;
     return RBMOE_OK;
 }

@@ -206,6 +206,8 @@ int rmsnorm_grad_tiles(int max_tokens);
 hipError_t launch_rmsnorm_backward(const void* x, const void* up, const float* weight, float eps,
                                    const void* residual_grad, int T, int d, void* grad_input, float* inv_rms,
                                    float* partial, float* grad_weight, bool bf16, hipStream_t s);
+// out[i] = bf16(in[i]), nearest even; n a multiple of 8
+hipError_t launch_cast_rows_bf16(const float* in, void* out, long long n, hipStream_t s);
 hipError_t launch_fill_f32(float* p, float v, long long n, hipStream_t s);
 
 // ---- decode-shaped path (a few tokens) -------------------------------------------

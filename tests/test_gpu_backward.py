@@ -24,8 +24,8 @@ def grad_output_for(t, seed):
 
 def check_backward(device, t, valid=None, bias=None, aux_w=0.01, z_w=1e-3, seed=1, tol=None, max_tokens=None):
     w = t.workload
-    if tol is None:
-        tol = 1e-5 if w.act_dtype == "f32" else TOL
+    if tol is None:  # f32 rows over bf16 weights multiply on the bf16 matrix cores where the widths allow
+        tol = 1e-5 if (w.act_dtype == "f32" and w.weight_dtype == "f32") else TOL
     E = w.num_experts
     gout = grad_output_for(t, seed)
     ref_layer = oracle_layer(t, aux_w=aux_w, z_w=z_w)
@@ -338,4 +338,21 @@ def test_backward_of_a_batch_smaller_than_max_tokens_with_two_skewed_experts(dev
     layer.zero_grads()
     layer.backward(gout)
     assert np.array_equal(layer.weight_grad(L.W_DOWN, 3).view(np.uint32), once.view(np.uint32))
+    layer.close()
+
+
+@pytest.mark.parametrize("shape", [dict(d=128, E=8, k=2, F=192, T=300, shared=True, shared_d_ff=128),
+                                   dict(d=768, E=16, k=2, F=1408, T=1024)],
+                         ids=lambda s: "d{d}_E{E}_k{k}_F{F}_T{T}".format(**s))
+def test_f32_rows_over_bf16_weights_train_on_the_matrix_cores(device, shape):
+    """The reference's mixed-precision shape (f32 activations, bf16 expert weights, src/gpu_model.rs:2146-2153): the
+    products of both directions run on the bf16 matrix cores over bf16 copies of the rows and of the upstream
+    gradient; routing, losses and the router's gradient are those of the f32 rows."""
+    t = synth.make(small_workload(seed=33, act="f32", wt="bf16", **shape))
+    valid = (np.arange(shape["T"]) % 11 != 5).astype(np.uint8)
+    layer, ref, gout = check_backward(device, t, valid=valid, tol=TOL)
+    assert layer.kernel_name() == "mfma_bf16_stream"
+    once = layer.weight_grad(L.W_GATE, 1)
+    layer.backward(gout)
+    assert rel_l2(layer.weight_grad(L.W_GATE, 1), 2.0 * once) <= 1e-6
     layer.close()

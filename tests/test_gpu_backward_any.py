@@ -118,7 +118,7 @@ ODD_SHAPES = [
     dict(d=7, E=9, k=3, F=11, T=130, act="f32", wt="f32"),
     dict(d=40, E=4, k=2, F=24, T=200, shared=True, act="bf16", wt="bf16"),
     dict(d=33, E=5, k=2, F=50, T=70, shared=True, shared_d_ff=27, act="bf16", wt="bf16"),
-    dict(d=64, E=4, k=2, F=64, T=90, shared=True, act="f32", wt="bf16"),   # mixed: f32 rows, bf16 weights
+    dict(d=72, E=4, k=2, F=56, T=90, shared=True, act="f32", wt="bf16"),   # mixed: f32 rows, bf16 weights, off the tiles
     dict(d=24, E=20, k=4, F=10, T=300, act="f32", wt="bf16"),
 ]
 
