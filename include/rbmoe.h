@@ -148,7 +148,14 @@ typedef enum rbmoe_option {
     RBMOE_OPT_SIDE_STREAM = 6,     /* 0: everything on the context's one stream */
     RBMOE_OPT_WGRAD_MODE = 7,      /* cut experts' weight gradients: 0 fixed order (default), 1 f32 atomics, 2 never cut */
     RBMOE_OPT_WGRAD_GENERIC = 8,   /* 1: the plain kernel for the weight gradients */
-    RBMOE_OPT_DECODE_COMBINE_FOLD = 9 /* 0: decode-shaped calls combine in a launch of their own */
+    RBMOE_OPT_DECODE_COMBINE_FOLD = 9, /* 0: decode-shaped calls combine in a launch of their own */
+    /* (not switches of a kernel choice, but of what rbmoe_set_weight does with f32 data) */
+    RBMOE_OPT_QUANT_RULE = 10,     /* f32 -> int8 per row, scale = absmax / 127: 0 q = round(w / scale), the checkpoint
+                                      writer's rule (src/transformer.rs:512-519); 1 q = round(w * (1 / scale)), the
+                                      in-memory rule of Quantized::from_matrix (src/quantized.rs:29-51) */
+    RBMOE_OPT_QUANTIZE_ROUTER = 11 /* 1: an f32 router is quantized at upload as well, as TransformerLm::quantize does
+                                      (src/transformer.rs:899-910 via src/moe.rs:491-500), and the layer routes with the
+                                      quantized product (sum x * q in 32 lanes) * scale (src/quantized.rs:55-62, :154-177) */
 } rbmoe_option;
 int rbmoe_layer_set_option(rbmoe_layer* layer, int32_t option, int32_t value);
 
@@ -156,8 +163,11 @@ int rbmoe_layer_set_option(rbmoe_layer* layer, int32_t option, int32_t value);
  * from HOST memory to the device (the caller keeps its buffer).  `dtype` is the
  * dtype of `data`; f32 data is converted to the layer's weight dtype (bf16 by
  * RNE; int8 by the checkpoint rule scale = absmax/127, q = round(w/scale),
- * src/transformer.rs:512-519).  For RBMOE_I8 data, `scales` holds one f32 per
- * row.  `expert` is ignored for the router and the shared expert. */
+ * src/transformer.rs:512-519, or the in-memory rule with RBMOE_OPT_QUANT_RULE).  For
+ * RBMOE_I8 data, `scales` holds one f32 per row.  `expert` is ignored for the router and
+ * the shared expert.  The router is kept in f32 whatever the experts' dtype, unless it is given
+ * as RBMOE_I8 data or RBMOE_OPT_QUANTIZE_ROUTER is set: the layer then routes with the
+ * quantized product of src/quantized.rs:55-62 (inference only). */
 int rbmoe_set_weight(rbmoe_layer* layer, int32_t which, int32_t expert, const void* data,
                      int32_t dtype, const float* scales, int32_t rows, int32_t cols);
 

@@ -202,6 +202,44 @@ void rbo_router_logits(const float* x, const float* w, const float* bias, int T,
         }
 }
 
+// The router after `TransformerLm::quantize()` (src/transformer.rs:899-910 reaches it through
+// MoeLayer::linears_mut, src/moe.rs:491-500): Linear::forward takes Quantized::matmul_rhs_transposed
+// (src/param.rs:778-780, src/quantized.rs:55-99), i.e. per (token, row)
+//     dot(activations, weights) * scale                       (:61)
+// with `dot` = dot_lanes::<32> on every x86-64 machine with AVX2 and FMA (:179-196; the target feature
+// only widens the vectors: Rust never contracts `x * w` and `+=` into one operation), and dot_lanes
+// (:154-177): lanes[c % 32] += x[c] * f32(q[c]) over the whole chunks of 32, a scalar `rest` over the
+// tail, then lanes.iter().sum() - a fold from 0.0 in lane order - plus rest.  (The 8-lane fallback of
+// machines without AVX2 is a different summation order; this restatement follows the 32-lane one.)
+float rbo_dot_q8(const float* x, const int8_t* q, int n) {
+    float lanes[32];
+    for (int l = 0; l < 32; ++l) lanes[l] = 0.0f;
+    const int tail = n - n % 32;
+    for (int c = 0; c < tail; c += 32)
+        for (int l = 0; l < 32; ++l) {
+            const float prod = x[c + l] * (float)q[c + l];
+            lanes[l] = lanes[l] + prod;
+        }
+    float rest = 0.0f;
+    for (int c = tail; c < n; ++c) {
+        const float prod = x[c] * (float)q[c];
+        rest = rest + prod;
+    }
+    float sum = 0.0f;
+    for (int l = 0; l < 32; ++l) sum = sum + lanes[l];
+    return sum + rest;
+}
+
+void rbo_router_logits_q8(const float* x, const int8_t* q, const float* scales, const float* bias, int T, int d,
+                          int E, float* logits) {
+    for (int t = 0; t < T; ++t)
+        for (int e = 0; e < E; ++e) {
+            float v = rbo_dot_q8(x + (int64_t)t * d, q + (int64_t)e * d, d) * scales[e];
+            if (bias) v = v + bias[e];
+            logits[(int64_t)t * E + e] = v;
+        }
+}
+
 // Same product accumulated in f64 in plain index order; used only to count
 // tokens whose routing is sensitive to the f32 summation order.
 void rbo_router_logits_f64(const float* x, const float* w, const float* bias, int T, int d, int E,
@@ -556,6 +594,8 @@ struct rbo_layer {
     const float* router;                // [E, d]
     const rbo_expert_weights* experts;  // [E]
     const rbo_expert_weights* shared;   // or NULL
+    const int8_t* router_q;             // [E, d] quantized router (then `router` is not read by the forward), or NULL
+    const float* router_s;              // [E] its scales
 };
 
 struct rbo_outputs {
@@ -584,7 +624,8 @@ int rbo_moe_forward(const rbo_layer* L, const float* x, int T, int cols, const u
     const int S = T * k;
 
     std::vector<float> logits((size_t)T * E), P((size_t)T * E), lse((size_t)T);
-    rbo_router_logits(x, L->router, router_bias, T, d, E, logits.data());
+    if (L->router_q) rbo_router_logits_q8(x, L->router_q, L->router_s, router_bias, T, d, E, logits.data());
+    else rbo_router_logits(x, L->router, router_bias, T, d, E, logits.data());
     rbo_softmax_rows(logits.data(), T, E, P.data(), lse.data());
 
     std::vector<int32_t> expert_of((size_t)S), counts((size_t)E), offsets((size_t)E + 1),

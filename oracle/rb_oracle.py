@@ -137,6 +137,29 @@ def router_logits(x: np.ndarray, w: np.ndarray, bias: Optional[np.ndarray] = Non
     return out
 
 
+def dot_q8(x: np.ndarray, q: np.ndarray) -> float:
+    """f32 activations against int8 weights in the reference's 32-lane order (src/quantized.rs:154-177)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    q = np.ascontiguousarray(q, dtype=np.int8)
+    assert x.shape == q.shape and x.ndim == 1
+    _lib.rbo_dot_q8.restype = C.c_float
+    return float(_lib.rbo_dot_q8(_fp(x), _qp(q), x.shape[0]))
+
+
+def router_logits_q8(x: np.ndarray, q: np.ndarray, scales: np.ndarray, bias: Optional[np.ndarray] = None) -> np.ndarray:
+    """Logits of a quantized router: dot_q8(x[t], q[e]) * scales[e] (+ bias[e])."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    q = np.ascontiguousarray(q, dtype=np.int8)
+    scales = np.ascontiguousarray(scales, dtype=np.float32)
+    T, d = x.shape
+    E = q.shape[0]
+    out = np.empty((T, E), np.float32)
+    if bias is not None:
+        bias = np.ascontiguousarray(bias, dtype=np.float32)
+    _lib.rbo_router_logits_q8(_fp(x), _qp(q), _fp(scales), _fp(bias), T, d, E, _fp(out))
+    return out
+
+
 def router_logits_f64(x: np.ndarray, w: np.ndarray, bias: Optional[np.ndarray] = None) -> np.ndarray:
     T, d = x.shape
     E = w.shape[0]
@@ -222,7 +245,8 @@ class _Layer(C.Structure):
     _fields_ = [("d_model", C.c_int32), ("num_experts", C.c_int32), ("experts_per_token", C.c_int32),
                 ("d_ff", C.c_int32), ("shared_expert", C.c_int32), ("shared_d_ff", C.c_int32),
                 ("aux_loss_weight", C.c_float), ("router_z_loss_weight", C.c_float),
-                ("router", _f32p), ("experts", C.POINTER(_ExpertWeights)), ("shared", C.POINTER(_ExpertWeights))]
+                ("router", _f32p), ("experts", C.POINTER(_ExpertWeights)), ("shared", C.POINTER(_ExpertWeights)),
+                ("router_q", C.POINTER(C.c_int8)), ("router_s", _f32p)]
 
 
 class _Outputs(C.Structure):
@@ -351,6 +375,10 @@ class OracleLayer:
     aux_loss_weight: float = 0.01
     router_z_loss_weight: float = 1e-3
     _keep: list = field(default_factory=list, repr=False)
+    # the router after TransformerLm::quantize(): int8 rows [E, d] and one scale per row; the forward then routes
+    # with the quantized product (src/quantized.rs:55-62) and does not read `router`
+    router_q: Optional[np.ndarray] = None
+    router_s: Optional[np.ndarray] = None
 
     def swiglu(self, w: ExpertWeights, x: np.ndarray, d_ff: int):
         M, d = x.shape
@@ -370,10 +398,15 @@ class OracleLayer:
         S = T * k
         arr = (_ExpertWeights * E)(*[w._c() for w in self.experts])
         shared_c = self.shared._c() if self.shared is not None else None
+        rq = rs = None
+        if self.router_q is not None:
+            rq = np.ascontiguousarray(self.router_q, dtype=np.int8)
+            rs = np.ascontiguousarray(self.router_s, dtype=np.float32)
         layer = _Layer(d, E, k, F, 1 if self.shared is not None else 0, self.shared_d_ff,
                        self.aux_loss_weight, self.router_z_loss_weight, _fp(self.router),
                        C.cast(arr, C.POINTER(_ExpertWeights)),
-                       C.pointer(shared_c) if shared_c is not None else None)
+                       C.pointer(shared_c) if shared_c is not None else None,
+                       _qp(rq) if rq is not None else None, _fp(rs))
         res = dict(out=np.zeros((T, max(cols, 1)), np.float32), logits=np.zeros((T, E), np.float32),
                    probabilities=np.zeros((T, E), np.float32), lse=np.zeros((T,), np.float32),
                    expert_of=np.zeros((S,), np.int32), gate_of=np.zeros((S,), np.float32),
@@ -439,7 +472,7 @@ class OracleLayer:
         layer = _Layer(d, E, k, F, 1 if self.shared is not None else 0, self.shared_d_ff,
                        self.aux_loss_weight, self.router_z_loss_weight, _fp(self.router),
                        C.cast(arr, C.POINTER(_ExpertWeights)),
-                       C.pointer(shared_c) if shared_c is not None else None)
+                       C.pointer(shared_c) if shared_c is not None else None, None, None)
         gi = np.zeros((T, d), np.float32)
         gr = np.zeros((E, d), np.float32)
         gg = np.zeros((E, F, d), np.float32)

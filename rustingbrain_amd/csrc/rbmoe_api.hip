@@ -203,6 +203,10 @@ struct rbmoe_layer {
 
     // weights
     Buf router;            // f32 [E, d]
+    Buf router_q, router_s; // a quantized router: int8 [E, d], f32 scales [E]
+    bool router_q8 = false; // the layer routes with the quantized product (src/quantized.rs:55-62)
+    bool quantize_router = false;  // f32 router data is quantized at upload (TransformerLm::quantize reaches the router too)
+    int quant_rule = 0;     // f32 -> int8 at upload: 0 the checkpoint writer's rule, 1 the in-memory rule
     Buf wgu, wd;           // [E, 2F, d], [E, d, F] weight dtype
     Buf sgu, sd;           // int8 scales [E, 2F], [E, d]
     Buf swgu, swd;         // shared [2Fs, d], [d, Fs]
@@ -300,6 +304,8 @@ Plan make_plan(rbmoe_layer* L) {
     const size_t ws = dtype_size(c.weight_dtype), as = dtype_size(c.act_dtype);
     Plan p;
     p.add(&L->router, E * d * 4);
+    p.add(&L->router_q, E * d);
+    p.add(&L->router_s, E * 4);
     p.add(&L->wgu, E * 2 * F * d * ws);
     p.add(&L->wd, E * d * F * ws);
     if (c.weight_dtype == RBMOE_I8) {
@@ -633,7 +639,13 @@ int rbmoe_set_weight(rbmoe_layer* L, int32_t which, int32_t expert, const void* 
         return fail(ctx, RBMOE_INVALID_INPUT, buf);
     }
     const size_t n = (size_t)rows * cols;
-    const int target = is_router ? RBMOE_F32 : c.weight_dtype;
+    // The router is f32 whatever the experts' dtype - unless it is given as int8 rows with scales, or the layer
+    // was told to quantize it like every other Linear (TransformerLm::quantize, src/transformer.rs:899-910, reaches
+    // it through MoeLayer::linears_mut, src/moe.rs:491-500): the layer then routes with the quantized product.
+    const bool router_to_i8 = is_router && (dtype == RBMOE_I8 || (L->quantize_router && dtype == RBMOE_F32));
+    const int target = is_router ? (router_to_i8 ? RBMOE_I8 : RBMOE_F32) : c.weight_dtype;
+    if (router_to_i8 && L->training)
+        return fail(ctx, RBMOE_UNSUPPORTED, "the backward pass is not defined for a quantized router");
     HIP_TRY(ctx, hipSetDevice(ctx->device));
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));  // no forward may still read the old weights
 
@@ -657,8 +669,13 @@ int rbmoe_set_weight(rbmoe_layer* L, int32_t which, int32_t expert, const void* 
         for (size_t i = 0; i < n; ++i) o[i] = host_bf16_to_f32(h[i]);
         src = staged.data();
     } else if (dtype == RBMOE_F32 && target == RBMOE_I8) {
-        // The checkpoint writer's rule (reference src/transformer.rs:512-519,
-        // :1839-1847): scale = absmax / 127, q = clamp(round(w / scale)).
+        // Per row: scale = absmax / 127, then
+        //   rule 0, the checkpoint writer's (reference src/transformer.rs:512-519, :1839-1847):
+        //           q = clamp(round(w / scale)), a zero row stays zero;
+        //   rule 1, the in-memory one of Quantized::from_matrix (src/quantized.rs:29-51), which
+        //           TransformerLm::quantize applies: q = clamp(round(w * (1 / scale))).
+        // `round` is f32::round: halves away from zero.  The two differ where the reciprocal's rounding moves a
+        // quotient across a half.
         staged.resize(n);
         staged_scales.resize(rows);
         const float* f = static_cast<const float*>(data);
@@ -668,8 +685,10 @@ int rbmoe_set_weight(rbmoe_layer* L, int32_t which, int32_t expert, const void* 
             for (int cc = 0; cc < cols; ++cc) absmax = std::fmax(absmax, std::fabs(f[(size_t)r * cols + cc]));
             const float scale = absmax / 127.0f;
             staged_scales[r] = scale;
+            const float inverse = scale > 0.0f ? 1.0f / scale : 0.0f;
             for (int cc = 0; cc < cols; ++cc) {
-                float v = scale == 0.0f ? 0.0f : std::round(f[(size_t)r * cols + cc] / scale);
+                const float w = f[(size_t)r * cols + cc];
+                float v = L->quant_rule == 1 ? std::round(w * inverse) : (scale == 0.0f ? 0.0f : std::round(w / scale));
                 v = std::fmin(127.0f, std::fmax(-127.0f, v));
                 q[(size_t)r * cols + cc] = (int8_t)v;
             }
@@ -678,6 +697,17 @@ int rbmoe_set_weight(rbmoe_layer* L, int32_t which, int32_t expert, const void* 
         scales = staged_scales.data();
     } else {
         return fail(ctx, RBMOE_UNSUPPORTED, "this conversion between weight dtypes is not supported");
+    }
+    if (is_router) {
+        if (router_to_i8) {
+            HIP_TRY(ctx, hipMemcpy(L->router_q.p, src, n, hipMemcpyHostToDevice));
+            HIP_TRY(ctx, hipMemcpy(L->router_s.p, scales, (size_t)rows * 4, hipMemcpyHostToDevice));
+        } else {
+            HIP_TRY(ctx, hipMemcpy(L->router.p, src, n * 4, hipMemcpyHostToDevice));
+        }
+        L->router_q8 = router_to_i8;
+        L->weights_set = true;
+        return RBMOE_OK;
     }
     const size_t es = dtype_size(target);
     std::vector<unsigned char> packed;
@@ -905,7 +935,9 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     // norm and write the bf16 copy of f32 rows
     const bool stages_rows = small_route_stages_rows(x, (const float*)L->router.p, T, d, E, abf) &&
                              (!norm_src || small_route_stages_rows(norm_src, (const float*)L->router.p, T, d, E, abf));
-    const bool decode_ok = mfma && L->decode_path && !L->training && small_route_ok(T, E, k) && decode_shape_ok(F, d) &&
+    // (a quantized router has one kernel for its logits, on the large-batch sequence)
+    const bool decode_ok = mfma && L->decode_path && !L->training && !L->router_q8 && small_route_ok(T, E, k) &&
+                           decode_shape_ok(F, d) &&
                            decode_shape_ok(d, F) &&
                            (!c.shared_expert || (decode_shape_ok(Fs, d) && decode_shape_ok(d, Fs))) &&
                            (!cast || stages_rows);
@@ -1101,6 +1133,14 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
                   (int*)L->rank_in_block.p, (int*)L->blockcnt.p, (float*)L->partial.p};
     if (cast) ra.rows16 = L->x16.p;
     ra.allow_fused = L->fused_router;
+    if (L->router_q8) {
+        ra.wq = (const int8_t*)L->router_q.p;
+        ra.wscale = (const float*)L->router_s.p;
+        if (cast) {  // the quantized router's kernel does not write the bf16 copy of f32 rows on its way
+            ra.rows16 = nullptr;
+            HIP_TRY(ctx, launch_cast_rows_bf16((const float*)x, L->x16.p, (long long)T * d, s));
+        }
+    }
     HIP_TRY(ctx, launch_router(ra, abf, s));
     L->replay[RBMOE_STAGE_ROUTER] = [=](hipStream_t st) { return launch_router(ra, abf, st); };
     HIP_TRY(ctx, mark(1));
@@ -1455,6 +1495,8 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
         return fail(ctx, RBMOE_UNSUPPORTED, "the backward pass is not defined for int8 weights");
     if (L->weights_set)
         return fail(ctx, RBMOE_INVALID_CONFIG, "enable training before the weights are set");
+    if (L->quantize_router)
+        return fail(ctx, RBMOE_UNSUPPORTED, "the backward pass is not defined for a quantized router");
     // (f32 rows over bf16 weights - the reference's own mixed-precision shape, src/gpu_model.rs:2146-2153 - stay on
     // the matrix cores in both directions: the products read the bf16 copy of the rows that the forward writes
     // anyway and a bf16 copy of the upstream gradient that the backward pass writes first; the router's branch,
@@ -1567,6 +1609,15 @@ int rbmoe_layer_set_option(rbmoe_layer* L, int32_t option, int32_t value) {
             L->wgrad_split = value == 0 ? WgradSplit::Ordered : value == 1 ? WgradSplit::Atomic : WgradSplit::None;
             return RBMOE_OK;
         case RBMOE_OPT_WGRAD_GENERIC: L->wgrad_generic = value != 0; return RBMOE_OK;
+        case RBMOE_OPT_QUANT_RULE:
+            if (value != 0 && value != 1) return fail(ctx, RBMOE_INVALID_CONFIG, "the quantisation rule is 0 or 1");
+            L->quant_rule = value;
+            return RBMOE_OK;
+        case RBMOE_OPT_QUANTIZE_ROUTER:
+            if (value != 0 && L->training)
+                return fail(ctx, RBMOE_UNSUPPORTED, "the backward pass is not defined for a quantized router");
+            L->quantize_router = value != 0;
+            return RBMOE_OK;
     }
     return fail(ctx, RBMOE_INVALID_CONFIG, "unknown option");
 }

@@ -61,6 +61,10 @@ struct RouterArgs {
     float* partial;      // [nb, E+1]
     void* rows16 = nullptr;  // f32 rows only: [T, d] bf16 copy of x written on the way (d a multiple of 8), or null
     bool allow_fused = true; // logits and everything behind them in one launch where the shapes allow
+    // a quantized router (Quantized::matmul_rhs_transposed, src/quantized.rs:55-62): int8 rows and one scale per row;
+    // `wr` is then not read and the logits are (sum_c x[c] * f32(q[c]), in the reference's 32 lanes) * scale
+    const int8_t* wq = nullptr;      // [E, d]
+    const float* wscale = nullptr;   // [E]
 };
 hipError_t launch_router(const RouterArgs& a, bool bf16, hipStream_t s);
 

@@ -446,6 +446,41 @@ __device__ __forceinline__ void router_tail(
 }
 
 // ---------------------------------------------------------------------------
+// logits_q8_kernel: the logits of a quantized router, one thread per (token, expert).  The reference's order
+// (dot_lanes::<32>, src/quantized.rs:154-177, taken on machines with AVX2, :179-196): lanes[c % 32] += x[c] * f32(q[c])
+// over the whole chunks of 32 columns, a scalar rest over the tail, the lanes folded from 0.0 in lane order, plus the
+// rest, times the row's scale (:61); every product and every sum rounded by itself.  Any width; not tuned (a
+// quantized layer's router is a few hundred kilobytes and this kernel a few percent of its forward).
+// ---------------------------------------------------------------------------
+template <typename XT>
+__global__ __launch_bounds__(256) void logits_q8_kernel(const XT* __restrict__ x, const int8_t* __restrict__ q,
+                                                        const float* __restrict__ scale, const float* __restrict__ bias,
+                                                        int T, int d, int E, float* __restrict__ P) {
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (long long)T * E) return;
+    const int t = (int)(idx / E), e = (int)(idx - (long long)t * E);
+    const XT* const xr = x + (size_t)t * d;
+    const int8_t* const qr = q + (size_t)e * d;
+    float lanes[32];
+#pragma unroll
+    for (int l = 0; l < 32; ++l) lanes[l] = 0.0f;
+    const int tail = d - d % 32;
+    for (int c = 0; c < tail; c += 32) {
+#pragma unroll
+        for (int l = 0; l < 32; ++l)
+            lanes[l] = __fadd_rn(lanes[l], __fmul_rn(to_f32(xr[c + l]), (float)qr[c + l]));
+    }
+    float rest = 0.0f;
+    for (int c = tail; c < d; ++c) rest = __fadd_rn(rest, __fmul_rn(to_f32(xr[c]), (float)qr[c]));
+    float sum = 0.0f;
+#pragma unroll
+    for (int l = 0; l < 32; ++l) sum = __fadd_rn(sum, lanes[l]);
+    float v = __fmul_rn(__fadd_rn(sum, rest), scale[e]);
+    if (bias) v = __fadd_rn(v, bias[e]);
+    P[idx] = v;
+}
+
+// ---------------------------------------------------------------------------
 // route_fused_kernel: the logits AND everything behind them for the 32 tokens of a router block, in one workgroup
 // - one launch and one trip of the logits through memory less than logits_kernel + router_kernel.  A workgroup
 // must then hold every expert of its tokens, and with 32 tokens a wave's 64 lanes are two experts side by side:
@@ -1218,7 +1253,7 @@ static int fused_cols(const RouterArgs& a, size_t xsize) {
 template <typename XT>
 static hipError_t launch_router_t(const RouterArgs& a, hipStream_t s) {
     const int nb = (a.T + kRouterTokens - 1) / kRouterTokens;
-    if (const int cols = fused_cols(a, sizeof(XT))) {
+    if (const int cols = a.wq ? 0 : fused_cols(a, sizeof(XT))) {
         const size_t lds = fused_lds_bytes(a.E, a.k, cols, sizeof(XT));
         auto go = [&](auto ni) {
             RB_LAUNCH((route_fused_kernel<XT, decltype(ni)::value>), dim3(nb), dim3(kRouterThreads), lds, s,
@@ -1247,7 +1282,12 @@ static hipError_t launch_router_t(const RouterArgs& a, hipStream_t s) {
     constexpr int NE = 8;
     const int tiles_t = (a.T + kLogitTokens - 1) / kLogitTokens;
     const dim3 lgrid(tiles_t, (a.E + NE - 1) / NE);
-    if ((long long)lgrid.x * lgrid.y <= 512)  // at most two workgroups on a compute unit
+    if (a.wq) {
+        if (a.rows16 || !a.wscale) return hipErrorInvalidValue;  // (the caller casts f32 rows itself on this path)
+        const long long pairs = (long long)a.T * a.E;
+        RB_LAUNCH(logits_q8_kernel<XT>, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, s,
+                  static_cast<const XT*>(a.x), a.wq, a.wscale, a.bias, a.T, a.d, a.E, a.P);
+    } else if ((long long)lgrid.x * lgrid.y <= 512)  // at most two workgroups on a compute unit
         RB_LAUNCH((logits_kernel<XT, NE, true>), lgrid, dim3(NE * 64), 0, s, static_cast<const XT*>(a.x),
                            a.wr, a.bias, a.T, a.d, a.E, a.P, static_cast<bf16_t*>(a.rows16));
     else

@@ -297,6 +297,19 @@ class MoeLayer:
     def set_router(self, weight: np.ndarray) -> None:
         self._set(L.W_ROUTER, 0, np.asarray(weight, dtype=np.float32))
 
+    def set_router_q8(self, q: np.ndarray, scales: np.ndarray) -> None:
+        """A quantized router as it is: int8 rows ``[num_experts, d_model]`` and one scale per row.  The layer then
+        routes with the quantized product (reference src/quantized.rs:55-62)."""
+        self._set(L.W_ROUTER, 0, np.asarray(q, dtype=np.int8), scales)
+
+    def quantize_on_upload(self, rule: str = "in_memory", router: bool = True) -> None:
+        """What ``TransformerLm::quantize()`` (reference src/transformer.rs:899-910) does to this layer's Linears,
+        applied to f32 weights as they are set from here on: ``rule`` "in_memory" is ``Quantized::from_matrix``
+        (src/quantized.rs:29-51), "checkpoint" the .rbw writer's (src/transformer.rs:512-519); ``router``: the router
+        is quantized too (src/moe.rs:491-500).  The layer's weight dtype must be int8 for the experts to follow."""
+        self.set_option(L.OPT_QUANT_RULE, {"checkpoint": 0, "in_memory": 1}[rule])
+        self.set_option(L.OPT_QUANTIZE_ROUTER, 1 if router else 0)
+
     def set_expert(self, expert: int, gate: np.ndarray, up: np.ndarray, down: np.ndarray) -> None:
         for which, m in ((L.W_GATE, gate), (L.W_UP, up), (L.W_DOWN, down)):
             self._set(which, expert, np.asarray(m, dtype=np.float32))

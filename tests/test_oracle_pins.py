@@ -275,6 +275,73 @@ def test_q8_rounds_half_away_from_zero():
     assert np.array_equal(q, q2) and np.array_equal(s, s2)
 
 
+def test_quantized_router_product_on_the_reference_vectors_and_in_the_32_lane_order():
+    """The router after quantize(): dot(activations, weights) * scale (reference src/quantized.rs:55-62) with the
+    32 lanes of dot_avx2 (:154-183).  Pinned by the reference's own vectors (:202-217), by a vector that only the
+    32-lane order sums to the right value (an 8-lane or a plain index order lose the ones), by one whose products
+    round before they are added (a fused multiply-add gives another value), and by float64."""
+    # the reference's test: within 0.05 of the float product
+    w = np.array([v * 0.37 - 2.0 for v in range(12)], np.float32).reshape(3, 4)
+    x = np.array([0.5, -1.5, 2.0, 0.25, 1.0, 1.0, -1.0, 0.0], np.float32).reshape(2, 4)
+    q, s = orc.q8_quantize(w, 1)
+    got = orc.router_logits_q8(x, q, s)
+    assert np.all(np.abs(got - orc.linear(x, w, plain=True)) < 0.05)
+    # a zero row has scale zero and gives zero (:219-225)
+    q0, s0 = orc.q8_quantize(np.zeros((1, 4), np.float32), 1)
+    assert not orc.router_logits_q8(x, q0, s0).any()
+    # lane order: x[0] = 2^24 sits in lane 0; the ones at columns 8 and 40 share lane 8 in the 32-lane order
+    # (1 + 1 = 2, then 2^24 + 2 is exact) but fall on lane 0 in an 8-lane order and behind 2^24 in index order
+    # (2^24 + 1 = 2^24 twice)
+    xv = np.zeros(64, np.float32)
+    xv[0], xv[8], xv[40] = 2.0 ** 24, 1.0, 1.0
+    ones = np.ones(64, np.int8)
+    assert orc.dot_q8(xv, ones) == 2.0 ** 24 + 2.0
+    lanes8 = np.zeros(8, np.float32)
+    for c in range(64):
+        lanes8[c % 8] = np.float32(lanes8[c % 8] + xv[c])
+    assert float(np.sum(lanes8, dtype=np.float32)) == 2.0 ** 24      # what the other order would give
+    # the tail (columns past the last whole 32) is a scalar sum added after the lanes
+    xt = np.zeros(35, np.float32)
+    xt[0], xt[32], xt[33], xt[34] = 2.0 ** 24, 1.0, 1.0, 1.0       # rest = 3, then 2^24 + 3 -> 2^24 + 4 (nearest even)
+    assert orc.dot_q8(xt, np.ones(35, np.int8)) == 2.0 ** 24 + 4.0
+    # multiply, round, then add: (1 + 2^-23) * 3 = 3 + 3 * 2^-23 rounds to 3 + 2^-21 (a tie, to even) before
+    # the add of -3 leaves 2^-21; a fused multiply-add would leave 1.5 * 2^-22
+    xq = np.zeros(64, np.float32)
+    xq[0], xq[32] = np.float32(1.0 + 2.0 ** -23), 1.0
+    qq = np.zeros(64, np.int8)
+    qq[0], qq[32] = 3, -3
+    assert orc.dot_q8(xq, qq) == float(np.float32(np.float32(xq[0] * np.float32(3.0)) - np.float32(3.0)))
+    assert orc.dot_q8(xq, qq) != float(np.float64(xq[0]) * 3.0 - 3.0)
+    # random rows against float64, and the scale is applied after the sum (one rounding)
+    rng = np.random.default_rng(5)
+    xr = rng.standard_normal((7, 96)).astype(np.float32)
+    qr = rng.integers(-127, 128, (5, 96)).astype(np.int8)
+    sr = rng.uniform(0.001, 0.01, 5).astype(np.float32)
+    got = orc.router_logits_q8(xr, qr, sr)
+    want = (xr.astype(np.float64) @ qr.astype(np.float64).T) * sr.astype(np.float64)
+    assert np.allclose(got, want, rtol=2e-6, atol=1e-6)
+    for t in range(7):
+        for e in range(5):
+            assert got[t, e] == np.float32(np.float32(orc.dot_q8(xr[t], qr[e])) * sr[e])
+    # the bias, a benchmark hook that the reference does not have, is added last
+    b = rng.standard_normal(5).astype(np.float32)
+    assert np.array_equal(orc.router_logits_q8(xr, qr, sr, b), (got + b).astype(np.float32))
+
+
+def test_a_layer_with_a_quantized_router_routes_on_the_quantized_logits():
+    t = synth.make(small_workload(d=64, E=6, k=2, F=32, T=40, seed=6))
+    q, s = orc.q8_quantize(t.router, 1)
+    plain = oracle_layer(t)
+    quant = oracle_layer(t)
+    quant.router_q, quant.router_s = q, s
+    a, b = plain.forward(t.x), quant.forward(t.x)
+    assert np.array_equal(b.logits, orc.router_logits_q8(t.x, q, s))
+    assert not np.array_equal(a.logits, b.logits)
+    # ... and everything behind the logits is the same code: softmax of those logits, top-k, bucket
+    P, lse = orc.softmax_rows(b.logits)
+    assert np.array_equal(P.view(np.uint32), b.probabilities.view(np.uint32))
+
+
 # ------------------------------------------------------------------ silu / swiglu
 def test_silu_known_points():
     # reference src/ffn.rs:346-352
