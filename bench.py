@@ -315,7 +315,8 @@ def weight_bytes(w: synth.Workload) -> int:
     return w.num_experts * 3 * w.d_model * w.d_ff * sw + 3 * w.d_model * Fs * sw + w.num_experts * w.d_model * 4
 
 
-def measure(dev, tools, name: str, steps: int, warmup: int, repeats: int, act_override: str = None) -> dict:
+def measure(dev, tools, name: str, steps: int, warmup: int, repeats: int, act_override: str = None,
+            plain: bool = False) -> dict:
     """One workload.
     * `repeats` loops of `steps` forwards of one layer back to back (median loop -> ms_per_step): weights that fit
       the 256 MiB Infinity Cache stay there;
@@ -325,7 +326,10 @@ def measure(dev, tools, name: str, steps: int, warmup: int, repeats: int, act_ov
       Cache holds in all), forwards and stage launches issued in rotation: every launch finds its weights in HBM;
     * forwards with L2 and Infinity Cache flushed by a read-only sweep before each one, each forward timed by an
       event pair of its own (raw interval);
-    * per-stage event intervals inside one forward (rbmoe_forward_timed), kept for comparison."""
+    * per-stage event intervals inside one forward (rbmoe_forward_timed), kept for comparison.
+    With `plain` only the first measurement and the kernels' own durations inside those forwards are taken (the
+    program then issues nothing but plain forwards: what a kernel trace or a counter run of it sees is the layer
+    as a model runs it)."""
     w = synth.WORKLOADS[name]
     t = synth.make(w)
     if act_override:
@@ -368,7 +372,7 @@ def measure(dev, tools, name: str, steps: int, warmup: int, repeats: int, act_ov
 
     decode = "decode" in layer.kernel_name()   # the library takes the decode-shaped kernels up to 32 tokens
     graph = None
-    if decode:
+    if decode and not plain:
         # A decode step is three short launches: issued one by one from this interpreter, the host's launch calls
         # are part of the step.  The same forward replayed from a HIP graph, timed the same way:
         g = ForwardGraph(dev, tools, fwd)
@@ -384,7 +388,7 @@ def measure(dev, tools, name: str, steps: int, warmup: int, repeats: int, act_ov
     dev.synchronize()
     launch_ms = {}
     for st in REPLAY_STAGES:
-        v = [layer.replay_stage(st, 20) for _ in range(3)]
+        v = [None] if plain else [layer.replay_stage(st, 20) for _ in range(3)]
         launch_ms[st] = None if v[0] is None else float(np.median(v))
 
     # ---- kernel durations inside a forward: every launch carries its own start / stop events, which receive the
@@ -403,20 +407,22 @@ def measure(dev, tools, name: str, steps: int, warmup: int, repeats: int, act_ov
     kernel_ms, kernel_ms_min = kernel_times(False)
     # ---- event intervals between the stages of one forward (each carries the cost of an event pair: `empty`)
     acc = {}
-    for _ in range(nprof):
+    for _ in range(0 if plain else nprof):
         for nm, v in layer.forward_timed(x.ptr, T, out.ptr, bias_ptr=bp).items():
             acc.setdefault(nm, []).append(v)
-    raw_ms = {nm: float(np.mean(v)) for nm, v in acc.items()}
+    raw_ms = {nm: float(np.mean(v)) for nm, v in acc.items()} if acc else {"empty": 0.0}
     over = raw_ms["empty"]
 
     # ---- caches flushed (a read-only sweep of 512 MiB) before every forward
-    cold_kernel_ms, _ = kernel_times(True)
-    flushed = []
-    for _ in range(max(10, min(30, steps))):
+    cold_kernel_ms = kernel_ms if plain else kernel_times(True)[0]
+    flushed = [0.0]
+    for _ in range(0 if plain else max(10, min(30, steps))):
         tools.flush()
         tools.start()
         fwd()
         flushed.append(tools.stop())
+    if len(flushed) > 1:
+        flushed = flushed[1:]
     cold_flush = {"kernel_ms": cold_kernel_ms, "ms_per_step_raw_interval": float(np.median(flushed)),
                   "event_interval_overhead_ms": over,
                   "note": "a read-only sweep of 512 MiB before every forward.  kernel_ms: the dispatches' own time "
@@ -425,13 +431,14 @@ def measure(dev, tools, name: str, steps: int, warmup: int, repeats: int, act_ov
 
     # ---- several layers with their own copies of the weights, in rotation
     wb = weight_bytes(w)
-    nlayers = int(max(4, min(16, -(-(512 << 20) // wb))))
+    nlayers = 1 if plain else int(max(4, min(16, -(-(512 << 20) // wb))))
     layers = [layer] + [new_layer() for _ in range(nlayers - 1)]
     for lay in layers:
         fwd(lay)
     dev.synchronize()
     rr_steps = max(nlayers * 2, (max(20, steps // 2) // nlayers) * nlayers)
-    rr_loops = wall_loops(lambda i: fwd(layers[i % nlayers]), rr_steps, max(3, min(repeats, 5)), dev.synchronize)
+    rr_loops = [ms_per_step] if plain else wall_loops(lambda i: fwd(layers[i % nlayers]), rr_steps,
+                                                      max(3, min(repeats, 5)), dev.synchronize)
     rr_ms = float(np.median(rr_loops))
     rr_launch = {}
     rounds = max(1, 20 // nlayers)
@@ -533,6 +540,10 @@ def measure(dev, tools, name: str, steps: int, warmup: int, repeats: int, act_ov
               "experts_per_token": w.experts_per_token, "d_ff": w.d_ff, "tokens": T,
               "shared_expert": w.shared_expert, "weight_dtype": w.weight_dtype, "act_dtype": w.act_dtype,
               "seed": w.seed, "expert0_share": float(cache.load_fractions()[0]), "routed_slots": routed}
+    if plain:
+        roofline["note"] = stages["note_plain"] = ("--plain: only back-to-back forwards and the kernels' own durations "
+                                                   "inside them were measured; every cold / rotation / replay figure "
+                                                   "repeats those")
     return {"w": w, "t": t, "layer": layer, "x": x, "out": out, "bias": bias, "bp": bp, "alg": alg,
             "ms_per_step": ms_per_step, "loops_ms": loops, "roofline": roofline, "stages": stages, "config": config,
             "bf16": bf16, "decode": decode, "graph": graph, "cold_flush": cold_flush, "round_robin": round_robin}
@@ -631,6 +642,9 @@ def main() -> int:
                     help="the workload of the top-level figures (the metric is quoted on the default)")
     ap.add_argument("--only", action="store_true", help="skip the `workloads` object (the other four workloads)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--plain", action="store_true",
+                    help="issue nothing but plain forwards of the chosen workload (timed loops, then forwards whose "
+                         "launches carry their own events): the command to run under a kernel trace or a counter pass")
     ap.add_argument("--no-backward", action="store_true",
                     help="skip the training-step figures (the `backward` object: forward in training mode, backward "
                          "pass, both; bf16 layers and all-f32 layers)")
@@ -652,7 +666,9 @@ def main() -> int:
 
     dev = rb.Device.open(0)
     tools = Tools(dev)
-    m = measure(dev, tools, args.workload, args.steps, args.warmup, args.repeats)
+    if args.plain:
+        args.only = args.no_cpu = args.no_backward = True
+    m = measure(dev, tools, args.workload, args.steps, args.warmup, args.repeats, plain=args.plain)
     w, T = m["w"], m["w"].tokens
     result = {
         "metric": "MoE-layer fwd tokens/sec at d768 E16 k2; grouped-GEMM % of bf16 MFMA peak",
@@ -697,7 +713,7 @@ def main() -> int:
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(m["t"])
     release(m)
-    if not m["decode"]:
+    if not m["decode"] and not args.plain:
         tools.close()
         result["two_batches_in_flight"] = two_in_flight(w, m["t"], args.steps, args.warmup, max(3, min(args.repeats, 5)))
         tools = Tools(dev)

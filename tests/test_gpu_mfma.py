@@ -131,3 +131,24 @@ def test_f32_rows_block_step_on_the_matrix_cores(device):
         assert_routing_identical(cache, ref)
         assert rel_l2(out, ref.out + t.x) <= 2e-2
         layer.close()
+
+
+def test_shared_expert_beside_the_routing_gives_the_bits_of_one_stream(device):
+    """From 1024 tokens on the shared expert's two products run on the context's second stream, beside the routing
+    kernels.  Same kernels, same operands: the output must not differ in a single bit from the one-stream order,
+    and both stay within the bar of the oracle."""
+    from rustingbrain_amd import _lib as L
+    t = synth.make(small_workload(d=128, E=8, k=2, F=192, T=1500, seed=43, act="bf16", wt="bf16", shared=True,
+                                  shared_d_ff=256))
+    ref = oracle_layer(t).forward(t.x, threads=8)
+    outs = []
+    for side in (1, 0):
+        layer = gpu_layer(device, t)
+        layer.set_option(L.OPT_SIDE_STREAM, side)
+        for _ in range(3):   # repeated: a missing join would show as a stale row sooner or later
+            out, cache = layer.forward_train(t.x)
+        assert_routing_identical(cache, ref)
+        assert rel_l2(out, ref.out) <= 2e-2
+        outs.append(out)
+        layer.close()
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
