@@ -199,6 +199,7 @@ struct rbmoe_layer {
     int group_m = 0;
     const char* kernel_name = "none";
     int last_T = -1;
+    int last_tile_m = kGenericTileM;  // rows per tile of the last forward's tile table
     Work last;  // tables of the last forward
 
     // weights
@@ -925,7 +926,8 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
 
     const bool mfma = L->use_stream;
     const bool f32mc = L->use_f32_mc;
-    const int tile_m0 = mfma ? stream_tile_m() : (f32mc ? f32_tile_m() : kGenericTileM);
+    const int tile_m0 = mfma ? stream_tile_m() : (f32mc ? f32_tile_m(T * k, E, std::min(F, d)) : kGenericTileM);
+    L->last_tile_m = tile_m0;
     L->kernel_name = mfma ? (wk == WeightKind::I8 ? "mfma_bf16_stream_int8w" : "mfma_bf16_stream")
                           : (f32mc ? "mfma_f32" : "generic");
     // a training layer keeps the gathered rows: the weight gradients of gate and up multiply by them
@@ -1183,6 +1185,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
     g1.tile_rows = (const int*)L->tile_rows.p;
     g1.ntiles = (const int*)L->ntiles.p;
     g1.max_tiles = T > 0 ? (T * k) / tile_m0 + E : 0;
+    g1.tile_m = tile_m0;
     g1.dense_rows = -1;
     g1.out = L->h.p;
     g1.swiglu = true;
@@ -1709,7 +1712,8 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, int32_t tokens, int3
     g.tile_row0 = (const int*)L->tile_row0.p;
     g.tile_rows = (const int*)L->tile_rows.p;
     g.ntiles = (const int*)L->ntiles.p;
-    g.max_tiles = S / (L->use_stream ? stream_tile_m() : (L->use_f32_mc ? f32_tile_m() : kGenericTileM)) + E;
+    g.max_tiles = S / L->last_tile_m + E;  // the tile table of the last forward
+    g.tile_m = L->last_tile_m;
     g.dense_rows = -1;
     g.swiglu = false;
     g.group_m = L->group_m;

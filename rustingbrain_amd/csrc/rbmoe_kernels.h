@@ -143,6 +143,7 @@ struct GroupedArgs {
     const void* swiglu_grad_gu = nullptr;
     bool swiglu;
     int group_m;            // MFMA path: M-tiles per scheduling group (0 = default)
+    int tile_m = 0;         // f32 matrix-core path: rows per tile of the tile table (64 or 32)
 };
 hipError_t launch_grouped_generic(const GroupedArgs& a, bool act_bf16, WeightKind wk, int tile_m,
                                   hipStream_t s);
@@ -158,7 +159,7 @@ void pack_weight_bf16(const uint16_t* src, int rows, int cols, uint16_t* dst);
 void pack_weight_i8(const int8_t* src, int rows, int cols, int8_t* dst);
 
 // f32 matrix cores (all-f32 layers): 64-row tiles, plain row-major weights.
-int f32_tile_m();
+int f32_tile_m(int rows, int groups, int n_min);  // tile height (64 or 32) for a batch of `rows` routed rows in `groups` groups; n_min: the narrower product's width
 bool f32_shape_ok(int N, int K);
 hipError_t launch_grouped_f32(const GroupedArgs& a, hipStream_t s);
 
