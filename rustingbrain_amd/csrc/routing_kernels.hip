@@ -496,6 +496,20 @@ __host__ __device__ static size_t fused_lds_bytes(int E, int k, int cols, size_t
     return router_fixed_bytes(E, k) + (size_t)kRouterTokens * (cols * xsize + 16) + (size_t)E * (cols * 4 + 16);
 }
 
+// LDS reads of 16 bytes each that stay where they are written.
+template <typename V>
+__device__ __forceinline__ V lds_load_ahead(const unsigned char* p) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    static_assert(sizeof(V) % 16 == 0, "16-byte pieces");
+    struct Raw {
+        u32x4 v[sizeof(V) / 16];
+    } raw;
+#pragma unroll
+    for (size_t i = 0; i < sizeof(V) / 16; ++i)
+        raw.v[i] = *(const volatile __attribute__((address_space(3))) u32x4*)(const __attribute__((address_space(3))) void*)(p + 16 * i);
+    return __builtin_bit_cast(V, raw);
+}
+
 template <typename XT, int NI>
 __global__ __launch_bounds__(kRouterThreads) void route_fused_kernel(
     const XT* __restrict__ x, const float* __restrict__ wr, const float* __restrict__ bias,
@@ -591,26 +605,50 @@ __global__ __launch_bounds__(kRouterThreads) void route_fused_kernel(
         stage(c0);
         __syncthreads();
         if (c0 + cols < d) fetch(c0 + cols);
+        // The LDS reads of piece q + 1 are issued before the arithmetic of piece q, so that their latency is covered
+        // by it (two waves on a SIMD do not cover it by themselves).  An expert index past E is clamped: its sums
+        // are computed and dropped, which keeps branches out of the loop.
         const unsigned char* const xrow = xs + (size_t)t * xpitch;
-        for (int q = 0; q < np; ++q) {
-            float xv[8];
-            XPiece<XT>::widen(*reinterpret_cast<const piece_t*>(xrow + (size_t)q * sizeof(piece_t)), xv);
+        const unsigned char* wrow[NI];
+#pragma unroll
+        for (int i = 0; i < NI; ++i) wrow[i] = ws + (size_t)min(2 * wave + half + 16 * i, E - 1) * wpitch;
+        struct Operands {
+            piece_t x;
+            float4 wa[NI], wb[NI];
+        };
+        auto read = [&](Operands& o, int q) {
+            o.x = lds_load_ahead<piece_t>(xrow + (size_t)q * sizeof(piece_t));
 #pragma unroll
             for (int i = 0; i < NI; ++i) {
-                const int e = 2 * wave + half + 16 * i;
-                if (e < E) {
-                    const float4 wa = *reinterpret_cast<const float4*>(ws + (size_t)e * wpitch + 32 * q);
-                    const float4 wb = *reinterpret_cast<const float4*>(ws + (size_t)e * wpitch + 32 * q + 16);
-                    la[i][0] = __fadd_rn(la[i][0], __fmul_rn(xv[0], wa.x));
-                    la[i][1] = __fadd_rn(la[i][1], __fmul_rn(xv[1], wa.y));
-                    la[i][2] = __fadd_rn(la[i][2], __fmul_rn(xv[2], wa.z));
-                    la[i][3] = __fadd_rn(la[i][3], __fmul_rn(xv[3], wa.w));
-                    la[i][4] = __fadd_rn(la[i][4], __fmul_rn(xv[4], wb.x));
-                    la[i][5] = __fadd_rn(la[i][5], __fmul_rn(xv[5], wb.y));
-                    la[i][6] = __fadd_rn(la[i][6], __fmul_rn(xv[6], wb.z));
-                    la[i][7] = __fadd_rn(la[i][7], __fmul_rn(xv[7], wb.w));
-                }
+                o.wa[i] = lds_load_ahead<float4>(wrow[i] + 32 * q);
+                o.wb[i] = lds_load_ahead<float4>(wrow[i] + 32 * q + 16);
             }
+            __builtin_amdgcn_sched_barrier(0);  // the reads stay in front of the arithmetic that follows
+        };
+        auto multiply = [&](const Operands& o) {
+            float xv[8];
+            XPiece<XT>::widen(o.x, xv);
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                la[i][0] = __fadd_rn(la[i][0], __fmul_rn(xv[0], o.wa[i].x));
+                la[i][1] = __fadd_rn(la[i][1], __fmul_rn(xv[1], o.wa[i].y));
+                la[i][2] = __fadd_rn(la[i][2], __fmul_rn(xv[2], o.wa[i].z));
+                la[i][3] = __fadd_rn(la[i][3], __fmul_rn(xv[3], o.wa[i].w));
+                la[i][4] = __fadd_rn(la[i][4], __fmul_rn(xv[4], o.wb[i].x));
+                la[i][5] = __fadd_rn(la[i][5], __fmul_rn(xv[5], o.wb[i].y));
+                la[i][6] = __fadd_rn(la[i][6], __fmul_rn(xv[6], o.wb[i].z));
+                la[i][7] = __fadd_rn(la[i][7], __fmul_rn(xv[7], o.wb[i].w));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        // two sets of operand registers take turns, so that nothing is copied between the trips
+        Operands oa, ob;
+        read(oa, 0);
+        for (int q = 0; q < np; q += 2) {
+            read(ob, min(q + 1, np - 1));
+            multiply(oa);
+            read(oa, min(q + 2, np - 1));
+            if (q + 1 < np) multiply(ob);
         }
     }
 #pragma unroll
