@@ -98,13 +98,23 @@ __device__ __forceinline__ void add_tiles(const floatx16 (&acc)[NI][NJ], float* 
     }
 }
 
+// The tile [m0, m0 + tm) x [n0, n0 + tn) of an expert without rows, in a launch that overwrites: zeros.
+__device__ __forceinline__ void zero_tile(float* __restrict__ o, int M, int N, int m0, int n0, int tm, int tn, int tid,
+                                          int threads) {
+    const int w4 = tn / 4;  // N is a multiple of 4
+    for (int i = tid; i < tm * w4; i += threads) {
+        const int m = m0 + i / w4, n = n0 + 4 * (i % w4);
+        if (m < M && n < N) *reinterpret_cast<float4*>(o + (size_t)m * N + n) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+}
+
 // chunk table: expert e with c rows gets ceil(c / limit) chunks of equal size (a multiple of 32)
 // chunk_split[c]: 0 = the expert's only or first chunk (adds in place), 1 = adds with atomics (`ordered` off),
 // 2 + s = stores into partial matrix s; slot_first[e] / slot_count[e]: the partial matrices of expert e, in chunk order
 __global__ __launch_bounds__(256) void chunk_table_kernel(const int* __restrict__ counts,
                                                           const int* __restrict__ offsets, int groups,
                                                           int dense_rows, int limit, int max_chunks, int ordered,
-                                                          int max_slots,
+                                                          int max_slots, int zero_empty,
                                                           int* __restrict__ chunk_expert, int* __restrict__ chunk_row0,
                                                           int* __restrict__ chunk_rows, int* __restrict__ chunk_split,
                                                           int* __restrict__ nchunks, int* __restrict__ slot_first,
@@ -122,7 +132,9 @@ __global__ __launch_bounds__(256) void chunk_table_kernel(const int* __restrict_
             rows = dense_rows >= 0 ? dense_rows : counts[e];
             row0 = dense_rows >= 0 ? 0 : offsets[e];
         }
-        const int n = rows > 0 ? (rows + limit - 1) / limit : 0;
+        // zero_empty: an expert without rows gets one chunk without rows, marked -1: its tiles store zeros
+        const bool empty = zero_empty && e < groups && rows <= 0;
+        const int n = rows > 0 ? (rows + limit - 1) / limit : (empty ? 1 : 0);
         const int nx = n > 1 ? n - 1 : 0;  // chunks beyond the first
         scan[tid] = n;
         scan_x[tid] = nx;
@@ -154,7 +166,7 @@ __global__ __launch_bounds__(256) void chunk_table_kernel(const int* __restrict_
                 chunk_expert[first + c] = e;
                 chunk_row0[first + c] = r > 0 ? row0 + r0 : row0;
                 chunk_rows[first + c] = r;
-                chunk_split[first + c] = !cut ? 0 : (!ordered ? 1 : (c == 0 ? 0 : 2 + first_x + c - 1));
+                chunk_split[first + c] = empty ? -1 : !cut ? 0 : (!ordered ? 1 : (c == 0 ? 0 : 2 + first_x + c - 1));
             }
         }
         __syncthreads();
@@ -203,9 +215,13 @@ __global__ __launch_bounds__(GT) void weight_grad_kernel(
     const int tile = (unit - ch * tiles_m) * tiles_n + idx % tiles_n;
     const int m0 = (tile / tiles_n) * GM, n0 = (tile % tiles_n) * GN;
     const int rows = chunk_rows[ch];
-    if (rows <= 0) return;
-    const int row0 = chunk_row0[ch];
     const int cs = chunk_split[ch];
+    if (rows <= 0) {
+        if (cs == -1 && overwrite)
+            zero_tile(out + (size_t)chunk_expert[ch] * out_expert_stride, M, N, m0, n0, GM, GN, threadIdx.x, GT);
+        return;
+    }
+    const int row0 = chunk_row0[ch];
     const int mode = cs >= 2 ? 2 : cs;
     float* const o = cs >= 2 ? partial + (size_t)(cs - 2) * M * N : out + (size_t)chunk_expert[ch] * out_expert_stride;
 
@@ -320,11 +336,12 @@ __global__ __launch_bounds__(GT) void weight_grad_kernel(
 // s + 1 is complete and nobody reads stage s - 1 any more, whose LDS the DMA of stage s + 3 then takes.  The rows of
 // the last stage past the chunk's end are fetched from the chunk's last row and then zeroed in LDS by the wave that
 // fetched them.  Byte offsets are 32 bits (the launcher checks; larger operands take the kernel above).
-// On C3 this is 3 % faster than the kernel above (113 against 117 us for the gate/up gradient with its side
-// launches): removing, one at a time, the LDS stores, the load latency (a deeper pipeline), the re-reads from L2
-// (every workgroup reading the same rows) and the wait for the fragment reads each moves the time by a few percent
-// only; the product's time is the matrix cores' (38 us), the final stores' (26 us, 138 MB of f32) and the rounds'
-// (594 workgroups of 24 or 52 stages on 256 compute units, one at a time) side by side.
+// On C3 this is 7 % faster than the kernel above (110 against 119 us for the gate/up gradient with its side
+// launches, ordered chunks, overwriting).  Taking out of the kernel above, one at a time, the LDS stores, the load
+// latency (a deeper pipeline), the re-reads from L2 (every workgroup reading the same rows) or the wait for the
+// fragment reads moves the time by a few percent only: the product's time is the matrix cores' (38 us alone), the
+// final stores' (26 us, 138 MB of f32) and the rounds' (594 workgroups of 24 or 52 stages on 256 compute units,
+// one at a time) side by side.
 constexpr int DSTAGE = GR * (GM + GN) * 2;  // 32 KB
 constexpr int DSTAGES = 4;
 
@@ -350,9 +367,13 @@ __global__ __launch_bounds__(GT) void weight_grad_dma_kernel(
     const int tile = (unit - ch * tiles_m) * tiles_n + idx % tiles_n;
     const int m0 = (tile / tiles_n) * GM, n0 = (tile % tiles_n) * GN;
     const int rows = chunk_rows[ch];
-    if (rows <= 0) return;
-    const int row0 = chunk_row0[ch];
     const int cs = chunk_split[ch];
+    if (rows <= 0) {
+        if (cs == -1 && overwrite)
+            zero_tile(out + (size_t)chunk_expert[ch] * out_expert_stride, M, N, m0, n0, GM, GN, threadIdx.x, GT);
+        return;
+    }
+    const int row0 = chunk_row0[ch];
     const int mode = cs >= 2 ? 2 : cs;
     float* const o = cs >= 2 ? partial + (size_t)(cs - 2) * M * N : out + (size_t)chunk_expert[ch] * out_expert_stride;
 
@@ -486,9 +507,13 @@ __global__ __launch_bounds__(FT, 2) void weight_grad_f32_kernel(
     if (ch >= *nchunks) return;
     const int m0 = (unit - ch * tiles_m) * FM, n0 = (idx % tiles_n) * FN;
     const int rows = chunk_rows[ch];
-    if (rows <= 0) return;
-    const int row0 = chunk_row0[ch];
     const int cs = chunk_split[ch];
+    if (rows <= 0) {
+        if (cs == -1 && overwrite)
+            zero_tile(out + (size_t)chunk_expert[ch] * out_expert_stride, M, N, m0, n0, FM, FN, threadIdx.x, FT);
+        return;
+    }
+    const int row0 = chunk_row0[ch];
     const int mode = cs >= 2 ? 2 : cs;
     float* const o = cs >= 2 ? partial + (size_t)(cs - 2) * M * N : out + (size_t)chunk_expert[ch] * out_expert_stride;
 
@@ -667,10 +692,14 @@ hipError_t launch_weight_grad(const void* a, int M, const void* b, int N, const 
     int* const nchunks = chunks + 4 * max_chunks;
     int* const slot_first = nchunks + 1;
     int* const slot_count = slot_first + groups;
+    // Overwriting: with atomic chunks the cut experts and those without rows are cleared by a launch in front; in
+    // the other modes every expert with rows has a chunk that stores, and one without rows gets a chunk that
+    // stores zeros.
+    const bool clear_first = overwrite && split_mode == WgradSplit::Atomic;
     hipLaunchKernelGGL(chunk_table_kernel, dim3(1), dim3(256), 0, s, counts, offsets, groups, dense_rows, limit,
-                       max_chunks, ordered ? 1 : 0, max_slots, chunk_expert, chunk_row0, chunk_rows, chunk_split, nchunks,
-                       slot_first, slot_count);
-    if (overwrite)
+                       max_chunks, ordered ? 1 : 0, max_slots, (overwrite && !clear_first) ? 1 : 0, chunk_expert,
+                       chunk_row0, chunk_rows, chunk_split, nchunks, slot_first, slot_count);
+    if (clear_first)
         hipLaunchKernelGGL(clear_other_experts_kernel, dim3(64, groups), dim3(256), 0, s, counts, dense_rows, limit,
                            ordered ? 1 : 0, out, out_expert_stride, (size_t)M * N);
     const int grid = ((max_chunks * tiles_m + 7) / 8) * 8 * tiles_n;
