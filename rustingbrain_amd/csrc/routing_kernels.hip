@@ -1280,8 +1280,13 @@ __global__ __launch_bounds__(256) void combine_any_kernel(
 // ---------------------------------------------------------------------------
 // Whether route_fused_kernel takes the call: every expert of a token in one workgroup (at most 64, four per lane),
 // rows of whole 8-element pieces on 16-byte boundaries, and a slice of columns that fits LDS.
+// Large launches take the two-launch sequence: logits_kernel fetches the router rows with scalar loads and keeps six
+// waves on a SIMD, which per (token, expert) pair is the faster arithmetic once the launch fills the chip several
+// times over (16 384 tokens x 64 experts: 126 us for both launches against 153 us fused); up to 256 K pairs the
+// saved launch and the saved trip of the logits through memory weigh more (8192 x 16: 22 against 25 us).
 static int fused_cols(const RouterArgs& a, size_t xsize) {
     if (!a.allow_fused || a.E > 64 || a.d % 8 != 0 || a.d < 8) return 0;
+    if ((long long)a.T * a.E > 256 * 1024) return 0;
     if ((reinterpret_cast<uintptr_t>(a.x) & 15) || (reinterpret_cast<uintptr_t>(a.wr) & 15)) return 0;
     if (((size_t)a.d * xsize) % 16 != 0) return 0;
     const int cols = a.E <= 32 ? 256 : 128;
