@@ -697,7 +697,7 @@ __global__ __launch_bounds__(kRouterThreads) void router_kernel(
 // dispatch_fused_kernel: for a modest number of router blocks the layout scan is folded into the
 // dispatch launch: every block re-derives counts, offsets and its own base from all the block
 // histograms (O(blocks^2 x experts) reads in total, but one launch less on the critical path);
-// block 0 also writes counts, offsets, the tile table and the losses.
+// block 0 also writes counts, offsets and the tile table, the last block the losses.
 size_t dispatch_fused_lds_bytes(int E, int k) {
     const int parts = 256 / E;
     return ((size_t)2 * parts * E + (size_t)parts * (E + 1) + 4 * (size_t)(E + 1) + (size_t)kRouterTokens * k) * 4;
@@ -730,6 +730,10 @@ __global__ __launch_bounds__(256) void dispatch_fused_kernel(
     const int p = tid / E;
     const int e = tid - p * E;
     const bool active = p < parts;
+    // Block 0 writes counts, offsets and the tile table; the two losses are the work of another block (the last
+    // one), so that neither of the two is the launch's long pole.  That block fetches the partial sums in the same
+    // batch of loads as the histograms.
+    const bool loss_blk = blk == nb - 1;
     // this thread's first slot does not depend on the scan: fetch it before anything else
     const int t0 = blk * TB;
     const int nt = min(TB, T - t0);
@@ -744,27 +748,25 @@ __global__ __launch_bounds__(256) void dispatch_fused_kernel(
         // Loads in batches of 16 that do not depend on one another: one round trip to L2 per
         // batch instead of one per block.
         int s_all = 0, s_before = 0;
+        float m = 0.0f, zs = 0.0f;
         for (int b = b0; b < b1; b += 16) {
             int c[16];
+            float v[16], z[16];
 #pragma unroll
             for (int u = 0; u < 16; ++u) c[u] = b + u < b1 ? blockcnt[(size_t)(b + u) * E + e] : 0;
-#pragma unroll
-            for (int u = 0; u < 16; ++u) {
-                s_all += c[u];
-                s_before += b + u < blk ? c[u] : 0;
-            }
-        }
-        part_all[p * E + e] = s_all;
-        part_before[p * E + e] = s_before;
-        if (blk == 0) {
-            float m = 0.0f, zs = 0.0f;
-            for (int b = b0; b < b1; b += 16) {
-                float v[16], z[16];
+            if (loss_blk) {
 #pragma unroll
                 for (int u = 0; u < 16; ++u) {
                     v[u] = b + u < b1 ? partial[(size_t)(b + u) * (E + 1) + e] : 0.0f;
                     z[u] = (e == 0 && b + u < b1) ? partial[(size_t)(b + u) * (E + 1) + E] : 0.0f;
                 }
+            }
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                s_all += c[u];
+                s_before += b + u < blk ? c[u] : 0;
+            }
+            if (loss_blk) {
 #pragma unroll
                 for (int u = 0; u < 16; ++u) {
                     if (b + u < b1) {
@@ -773,6 +775,10 @@ __global__ __launch_bounds__(256) void dispatch_fused_kernel(
                     }
                 }
             }
+        }
+        part_all[p * E + e] = s_all;
+        part_before[p * E + e] = s_before;
+        if (loss_blk) {
             part_mass[p * (E + 1) + e] = m;
             if (e == 0) part_mass[p * (E + 1) + E] = zs;
         }
@@ -784,7 +790,7 @@ __global__ __launch_bounds__(256) void dispatch_fused_kernel(
         for (int q = 0; q < parts; ++q) {
             ca += part_all[q * E + tid];
             cb += part_before[q * E + tid];
-            if (blk == 0) m += part_mass[q * (E + 1) + tid];
+            if (loss_blk) m += part_mass[q * (E + 1) + tid];
         }
         cnt[tid] = ca;
         base[tid] = cb;
@@ -792,7 +798,7 @@ __global__ __launch_bounds__(256) void dispatch_fused_kernel(
     }
     // the sum of lse^2 over the parts: by the last thread of the workgroup, which exists for every expert count
     // (a thread numbered E does not when E is the workgroup size) and owns no expert column unless E is 256
-    if (blk == 0 && tid == 255) {
+    if (loss_blk && tid == 255) {
         float zs = 0.0f;
         for (int q = 0; q < parts; ++q) zs += part_mass[q * (E + 1) + E];
         mass[E] = zs;
@@ -834,8 +840,10 @@ __global__ __launch_bounds__(256) void dispatch_fused_kernel(
             }
             if (tid == E - 1) ntiles[0] = first + n;
         }
+        if (tid == 0) offsets[E] = off[E];
+    }
+    if (loss_blk) {
         if (tid == 0) {
-            offsets[E] = off[E];
             // every valid token routes exactly k slots, so the valid-token count is routed / k
             const int V = off[E] / k;
             float aux = 0.0f, z = 0.0f;
