@@ -393,8 +393,11 @@ __device__ __forceinline__ void router_tail(
         gate_of[(size_t)t0 * k + ls] = gates[ls];
     }
 
-    // ---- partial sums for the auxiliary losses (fixed order) --------------
-    for (int e = tid; e <= E; e += kRouterThreads) {
+    // ---- partial sums for the auxiliary losses (fixed order): the waves behind the first, which ranks the slots
+    // at the same time -----------------------------------------------------------
+    const bool one_wave_ranks = nls <= 64;
+    const int pfirst = one_wave_ranks ? 64 : 0;  // first thread that takes partial sums
+    for (int e = tid - pfirst; e >= 0 && e <= E; e += kRouterThreads - pfirst) {
         float s = 0.0f;
         for (int i0 = 0; i0 < nt; i0 += 8) {
             float pvv[8];
@@ -417,6 +420,28 @@ __device__ __forceinline__ void router_tail(
     const int wave = tid >> 6;
     int ebits = 0;
     while ((1 << ebits) < E) ++ebits;
+    if (one_wave_ranks) {
+        // every slot of the block in one wave: a slot's rank is the number of lower lanes with its expert, an
+        // expert's count the size of its group - no barrier, no second pass
+        if (wave == 0) {
+            const int e = (lane < nls) ? lexp[lane] : -1;
+            unsigned long long mask = __ballot(e >= 0);
+            for (int b = 0; b < ebits; ++b) {
+                const bool bit = (e >> b) & 1;
+                const unsigned long long bb = __ballot(bit);
+                mask &= bit ? bb : ~bb;
+            }
+            const int rank_w = __popcll(mask & ((1ull << lane) - 1ull));
+            if (e >= 0) {
+                rank_in_block[(size_t)t0 * k + lane] = rank_w;
+                if (rank_w == 0) running[e] = __popcll(mask);  // zero so far (cleared at the top)
+            }
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's LDS writes have landed
+            __builtin_amdgcn_wave_barrier();
+            for (int idx = lane; idx < E; idx += 64) blockcnt[(size_t)blk * E + idx] = running[idx];
+        }
+        return;
+    }
     const int rounds = (nls + kRouterThreads - 1) / kRouterThreads;
     for (int rd = 0; rd < rounds; ++rd) {
         for (int idx = tid; idx < kRouterWaves * E; idx += kRouterThreads) wcount[idx] = 0;
