@@ -3,12 +3,29 @@
 
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
+
+#include <atomic>
 #include <stddef.h>
 #include <stdint.h>
 
 #include "rbmoe_device.h"
 
 namespace rbmoe {
+
+// A kernel attribute is set once per device.  `done` has one bit per device; setting an attribute twice is
+// harmless, so two threads that race here only repeat the call.  Devices past the 64th set it on every launch.
+template <typename F>
+inline hipError_t once_per_device(std::atomic<unsigned long long>& done, F&& set) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const unsigned long long bit = dev < 64 ? 1ull << dev : 0ull;
+    if (bit && (done.load(std::memory_order_acquire) & bit)) return hipSuccess;
+    e = set();
+    if (e == hipSuccess && bit) done.fetch_or(bit, std::memory_order_release);
+    return e;
+}
+
 
 // Kernel durations the way a kernel trace reports them: while a KernelTimer is installed on the calling thread,
 // every forward-path launch below carries its own start and stop events (hipExtLaunchKernelGGL), which receive the

@@ -664,8 +664,11 @@ hipError_t launch_weight_grad(const void* a, int M, const void* b, int N, const 
     if (groups <= 0 || total_rows <= 0) return hipSuccess;
     if (!weight_grad_shape_ok(M, N, bf16)) return hipErrorInvalidValue;
     if (bf16) {
-        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(weight_grad_kernel),
-                                                           hipFuncAttributeMaxDynamicSharedMemorySize, 2 * GSTAGE);
+        static std::atomic<unsigned long long> attr_set{0};
+        const hipError_t attr = once_per_device(attr_set, [] {
+            return hipFuncSetAttribute(reinterpret_cast<const void*>(weight_grad_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 2 * GSTAGE);
+        });
         if (attr != hipSuccess) return attr;
     }
     const int tile_m = bf16 ? GM : FM, tile_n = bf16 ? GN : FN;
@@ -706,8 +709,11 @@ hipError_t launch_weight_grad(const void* a, int M, const void* b, int N, const 
     // byte offsets inside the operands fit 32 bits: tiles by LDS-DMA
     const bool dma = bf16 && (size_t)total_rows * (size_t)std::max(M, N) * 2 < ((size_t)1 << 32) && GM == GN;
     if (dma) {
-        static const hipError_t attr2 = hipFuncSetAttribute(reinterpret_cast<const void*>(weight_grad_dma_kernel),
-                                                            hipFuncAttributeMaxDynamicSharedMemorySize, DSTAGES * DSTAGE);
+        static std::atomic<unsigned long long> attr2_set{0};
+        const hipError_t attr2 = once_per_device(attr2_set, [] {
+            return hipFuncSetAttribute(reinterpret_cast<const void*>(weight_grad_dma_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, DSTAGES * DSTAGE);
+        });
         if (attr2 != hipSuccess) return attr2;
         hipLaunchKernelGGL(weight_grad_dma_kernel, dim3(grid), dim3(GT), DSTAGES * DSTAGE, s, static_cast<const bf16_t*>(a), M,
                            static_cast<const bf16_t*>(b), N, tiles_m, tiles_n, chunk_expert, chunk_row0, chunk_rows,
