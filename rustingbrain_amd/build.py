@@ -26,6 +26,12 @@ FLAGS = [
 ]
 
 
+# Extra compiler flags for experiments with the kernels' compile-time shapes, e.g.
+#   RBMOE_HIPCC_EXTRA="-DRBMOE_STREAM_NW=8 -DRBMOE_STREAM_OCC=1" python -m rustingbrain_amd.build
+# (eight waves share one activation slice); read here, never by the library.
+FLAGS += os.environ.get("RBMOE_HIPCC_EXTRA", "").split()
+
+
 def sources():
     return sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
 

@@ -55,7 +55,10 @@ namespace {
 #endif
 constexpr int BM = RBMOE_STREAM_BM;   // token rows per workgroup
 constexpr int BK = 64;    // reduction slice held in one LDS stage
-constexpr int NW = 4;     // waves per workgroup
+#ifndef RBMOE_STREAM_NW
+#define RBMOE_STREAM_NW 4
+#endif
+constexpr int NW = RBMOE_STREAM_NW;     // waves per workgroup (4, or 8: one activation slice for twice the features)
 constexpr int NT = NW * 64;
 constexpr int CPR = BK / 8;            // 16-byte pieces per LDS row
 constexpr int TT = BM / 32;            // token blocks per wave
@@ -196,13 +199,17 @@ __device__ __forceinline__ void write_tile(const TileOut& o, floatx16 (&acc)[2][
     // hidden rows, then (only when the caller keeps them for a backward pass) the gate and the
     // up pre-activations, which go to `gu_out` [rows, 2N] with the gate half in columns [0, N).
     constexpr int PASSES = SWIGLU ? 3 : 2;
+    constexpr int WH = NW < 4 ? NW : 4;  // waves that fill the staging tile at a time (32 features each)
+    constexpr int SUB = NW / WH;         // ... in this many turns per block index
+    constexpr int PW = WH * 4;           // 16-byte pieces of a staged row in use
 #pragma unroll
-    for (int b = 0; b < PASSES; ++b) {
+    for (int bh = 0; bh < PASSES * SUB; ++bh) {
+        const int b = bh / SUB, h = bh % SUB;
         if constexpr (SWIGLU) {
             if (b > 0 && gu_out == nullptr) break;  // uniform over the launch
         }
-        if (b) __syncthreads();  // the previous pass has been read out
-        if (SWIGLU ? act0 : (b ? act1 : act0)) {
+        if (bh) __syncthreads();  // the previous pass has been read out
+        if ((wave / WH) == h && (SWIGLU ? act0 : (b ? act1 : act0))) {
             const int rb = b ? r1 : r0;
 #pragma unroll
             for (int t = 0; t < TT; ++t) {
@@ -226,23 +233,23 @@ __device__ __forceinline__ void write_tile(const TileOut& o, floatx16 (&acc)[2][
                             if constexpr (I8) y[i] *= sc[rb + f + i];
                         }
                     }
-                    const int piece = (wave * 4 + q) ^ (m & 15);
+                    const int piece = ((wave % WH) * 4 + q) ^ (m & 15);
                     *reinterpret_cast<uint2*>(stage + m * 256 + piece * 16 + lhalf * 8) =
                         make_uint2(pack2(y[0], y[1]), pack2(y[2], y[3]));
                 }
             }
         }
         __syncthreads();
-        if (b == 0) before_stores();
+        if (bh == 0) before_stores();
         // where this pass goes: hidden rows and down rows into `out` (row stride N), the
         // pre-activations into `gu_out` (row stride 2 N)
-        const int col0 = tn_idx * BN + (SWIGLU ? 0 : b * (NW * 32));
+        const int col0 = tn_idx * BN + (SWIGLU ? 0 : b * (NW * 32)) + h * (WH * 32);
         bf16_t* const dst = (SWIGLU && b > 0) ? gu_out + (b == 2 ? N : 0) : out;
         const size_t dstride = (SWIGLU && b > 0) ? (size_t)2 * N : (size_t)N;
 #pragma unroll
-        for (int i = 0; i < BM * 16 / NT; ++i) {
+        for (int i = 0; i < BM * PW / NT; ++i) {
             const int idx = i * NT + tid;
-            const int r = idx >> 4, p = idx & 15;
+            const int r = idx / PW, p = idx % PW;
             if (r < rows && col0 + 8 * p < N) {
                 const uint4 v = *reinterpret_cast<const uint4*>(stage + r * 256 + ((p ^ (r & 15)) * 16));
                 if constexpr (!SWIGLU) {
