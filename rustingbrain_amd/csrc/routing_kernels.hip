@@ -209,6 +209,213 @@ __global__ __launch_bounds__(NE * 64, (!AHEAD && sizeof(XT) == 2) ? 6 : 2) void 
     }
 }
 
+// Reductions over the G neighbouring lanes of a group (G a power of two up to 64, the same for the whole wave)
+// without LDS: inside a row of 16 lanes through the lane-permuting operand of the instruction itself (every lane of
+// the row ends with the result), across rows through four scalar reads.
+template <int CTRL>
+__device__ __forceinline__ uint32_t lanes_from(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, true);
+}
+template <typename Op>
+__device__ __forceinline__ uint32_t group_reduce(uint32_t v, int G, Op op) {
+    if (G >= 2) v = op(v, lanes_from<0xB1>(v));   // quad_perm [1,0,3,2]
+    if (G >= 4) v = op(v, lanes_from<0x4E>(v));   // quad_perm [2,3,0,1]
+    if (G >= 8) v = op(v, lanes_from<0x141>(v));  // row_half_mirror
+    if (G >= 16) v = op(v, lanes_from<0x140>(v)); // row_mirror
+    if (G >= 32) {
+        const uint32_t r0 = __builtin_amdgcn_readlane(v, 0), r1 = __builtin_amdgcn_readlane(v, 16);
+        const uint32_t r2 = __builtin_amdgcn_readlane(v, 32), r3 = __builtin_amdgcn_readlane(v, 48);
+        const uint32_t lo = op(r0, r1), hi = op(r2, r3);
+        v = G == 64 ? op(lo, hi) : ((threadIdx.x & 32) ? hi : lo);
+    }
+    return v;
+}
+__device__ __forceinline__ uint32_t group_umax(uint32_t v, int G) {
+    return group_reduce(v, G, [](uint32_t a, uint32_t b) { return a > b ? a : b; });
+}
+__device__ __forceinline__ uint32_t group_umin(uint32_t v, int G) {
+    return group_reduce(v, G, [](uint32_t a, uint32_t b) { return a < b ? a : b; });
+}
+// (no NaN among the operands; which zero wins among zeros of both signs does not matter to the callers)
+__device__ __forceinline__ float group_fmax(float v, int G) {
+    return __uint_as_float(group_reduce(__float_as_uint(v), G, [](uint32_t a, uint32_t b) {
+        return __float_as_uint(fmaxf(__uint_as_float(a), __uint_as_float(b)));
+    }));
+}
+
+// softmax, log-sum-exp and the k argmax rounds for the tokens of one wave of a router block (see router_tail).
+// Everything order-sensitive keeps the reference's order: the maximum ignores NaN (f32::max), exp(v - max) is
+// summed one expert after the other in index order, the k argmax rounds prefer the lower index on equal
+// probabilities, and the gates are summed in rank order.
+// The sum: lane l of a group ends with ((ex_0 + ex_1) + ... ) + ex_l after l steps of "take the lane below's sum,
+// add your own value" (a shift of the whole wave by one lane inside the add; a group's first lane keeps the sum
+// carried over from the experts of the slices before) - the reference's chain, one rounded add per expert, with
+// no trip through LDS; lanes past the last expert add zeros.  An argmax round is two reductions of 32 bits: the
+// greatest probability bits (probabilities are never negative, so the bits order like the values), then the
+// lowest expert index among the lanes that hold them.
+// NQ = turns a wave needs for its tokens (64 / G tokens a turn); the NQ turns share no data and run interleaved.
+template <int MAXJ, int NQ>
+__device__ __forceinline__ void softmax_topk(float* __restrict__ prob, float* __restrict__ lsev,
+                                             float* __restrict__ gates, int* __restrict__ lexp, int G, int t0, int nt,
+                                             int ES, const uint8_t* __restrict__ valid, int E, int k) {
+    constexpr int TB = kRouterTokens;
+    constexpr int TW = TB / kRouterWaves;  // tokens of a wave
+    const int lane_ = threadIdx.x & 63, wave_ = threadIdx.x >> 6;
+    const int lig = lane_ & (G - 1);          // lane in group
+    const int gbase = lane_ & ~(G - 1);       // first lane of the group
+    const int tpw = 64 / G;                   // tokens a wave handles in one turn
+    const unsigned long long gmask = (G == 64 ? ~0ull : ((1ull << G) - 1ull)) << gbase;
+    const float neg_inf = __uint_as_float(0xff800000u);
+    int tok[NQ];
+    bool live[NQ], ok[NQ];
+    float* row[NQ];
+    float pv[NQ][MAXJ], mx[NQ], sum[NQ], total[NQ];
+    unsigned taken_bits[NQ];  // bit j: expert lig + G j is taken
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+        tok[q] = wave_ * TW + q * tpw + lane_ / G;  // token of this group in turn q
+        live[q] = tok[q] < nt && tok[q] < (wave_ + 1) * TW && q * tpw < TW;
+        row[q] = prob + (live[q] ? tok[q] : 0) * ES;
+        mx[q] = neg_inf;
+#pragma unroll
+        for (int j = 0; j < MAXJ; ++j) {
+            const int e = lig + G * j;
+            pv[q][j] = (live[q] && e < E) ? row[q][e] : neg_inf;
+            const float vv = (pv[q][j] == pv[q][j]) ? pv[q][j] : neg_inf;  // a NaN never becomes the maximum
+            mx[q] = vv > mx[q] ? vv : mx[q];
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) mx[q] = group_fmax(mx[q], G);
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+#pragma unroll
+        for (int j = 0; j < MAXJ; ++j) {
+            const int e = lig + G * j;
+            // lanes without an expert carry +0 through the sums below
+            pv[q][j] = (live[q] && e < E) ? rb_expf(__fadd_rn(pv[q][j], -mx[q])) : 0.0f;
+        }
+    }
+    // the sums: one chain of adds per token in index order, slice after slice
+    {
+        float carry[NQ];
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) carry[q] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < MAXJ; ++j) {
+            if (G * j >= E) break;  // uniform
+            float acc[NQ], seed[NQ];
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+                seed[q] = __fadd_rn(carry[q], pv[q][j]);  // what a group's first lane holds: 0 + ex_0 = ex_0 in the first slice
+                acc[q] = lig == 0 ? seed[q] : pv[q][j];
+            }
+            for (int st = 1; st < G; ++st) {
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) {
+                    const float below = __uint_as_float(lanes_from<0x138>(__float_as_uint(acc[q])));  // wave_shr:1
+                    const float next = __fadd_rn(below, pv[q][j]);
+                    acc[q] = lig == 0 ? seed[q] : next;
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) carry[q] = __shfl(acc[q], gbase + G - 1);
+        }
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) sum[q] = carry[q];
+    }
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+        if (live[q] && lig == 0) lsev[tok[q]] = __fadd_rn(mx[q], rb_logf(sum[q]));
+#pragma unroll
+        for (int j = 0; j < MAXJ; ++j) {
+            const int e = lig + G * j;
+            if (live[q] && e < E) {
+                if (sum[q] > 0.0f) pv[q][j] = __fdiv_rn(pv[q][j], sum[q]);
+                row[q][e] = pv[q][j];
+            }
+        }
+        ok[q] = live[q] && ((valid == nullptr) || (valid[t0 + tok[q]] != 0));
+        taken_bits[q] = 0;
+        total[q] = 0.0f;
+    }
+    // ---- k rounds of argmax over the experts not yet taken ----
+    for (int r = 0; r < k; ++r) {
+        int first[NQ];
+        uint32_t lbits[NQ], le[NQ];  // this lane's best candidate: probability bits and expert index
+        bool has[NQ];
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            // First expert not yet taken: the lowest set bit of a ballot over the group, taking
+            // the expert slices j in increasing order (slice j holds experts G j .. G j + G - 1).
+            first[q] = 0x7fffffff;
+#pragma unroll
+            for (int j = MAXJ - 1; j >= 0; --j) {
+                const int e = lig + G * j;
+                const unsigned long long m = __ballot(e < E && !((taken_bits[q] >> j) & 1u)) & gmask;
+                if (m != 0ull) first[q] = (__ffsll((long long)m) - 1 - gbase) + G * j;
+            }
+            // best candidate of this lane: not taken, not NaN; greater probability, then lower index
+            has[q] = false;
+            lbits[q] = 0;
+            le[q] = 0x7fffffffu;
+#pragma unroll
+            for (int j = 0; j < MAXJ; ++j) {
+                const int e = lig + G * j;
+                if (live[q] && e < E && !((taken_bits[q] >> j) & 1u) && pv[q][j] == pv[q][j]) {
+                    const uint32_t bits = __float_as_uint(pv[q][j]);
+                    if (!has[q] || bits > lbits[q]) {  // slices in increasing index order: a tie keeps the lower index
+                        lbits[q] = bits;
+                        le[q] = (uint32_t)e;
+                    }
+                    has[q] = true;
+                }
+            }
+        }
+        uint32_t mbits[NQ], ci[NQ];
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) mbits[q] = group_umax(has[q] ? lbits[q] : 0u, G);
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) ci[q] = group_umin((has[q] && lbits[q] == mbits[q]) ? le[q] : 0x7fffffffu, G);
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            // the reference starts from the first untaken expert and replaces it only on a
+            // strictly greater probability: if that first one is NaN nothing replaces it
+            bool first_nan = false;
+#pragma unroll
+            for (int j = 0; j < MAXJ; ++j)
+                if (lig + G * j == first[q] && pv[q][j] != pv[q][j]) first_nan = true;
+            const bool nan_wins = (__ballot(first_nan) & gmask) != 0ull;
+            const bool use_first = nan_wins || ci[q] == 0x7fffffffu;
+            const int best = use_first ? first[q] : (int)ci[q];
+            float mine = 0.0f;
+#pragma unroll
+            for (int j = 0; j < MAXJ; ++j)
+                if (lig + G * j == best) {
+                    mine = pv[q][j];
+                    taken_bits[q] |= 1u << j;
+                }
+            // the winner's probability is the greatest bits themselves; only a NaN first expert has to be fetched
+            float bestv = __uint_as_float(mbits[q]);
+            if (__ballot(use_first) != 0ull) {  // uniform over the wave
+                const float fv = __shfl(mine, gbase + (best & (G - 1)));
+                if (use_first) bestv = fv;
+            }
+            total[q] = __fadd_rn(total[q], bestv);
+            if (live[q] && lig == 0) {
+                lexp[tok[q] * k + r] = ok[q] ? best : -1;
+                gates[tok[q] * k + r] = ok[q] ? bestv : 0.0f;
+            }
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int q = 0; q < NQ; ++q)
+        if (ok[q] && total[q] > 0.0f)
+            for (int r = lig; r < k; r += G) gates[tok[q] * k + r] = __fdiv_rn(gates[tok[q] * k + r], total[q]);
+}
+
 // router_tail: everything behind the logits for the 32 tokens of router block `blk` - softmax, log-sum-exp, top-k,
 // gates, ranks, block histogram, partial sums of the losses.  LOADED = false: the logits are read from P;
 // true: the caller has put them into the `prob` array of `lds_raw` (row pitch E | 1) and met at a barrier.
@@ -242,128 +449,14 @@ __device__ __forceinline__ void router_tail(
     __syncthreads();
 
     // ---- softmax + top-k: G lanes per token, lane j of a group owns experts j, j + G, ... ----
-    // Everything order-sensitive keeps the reference's order: the maximum ignores NaN
-    // (f32::max), exp(v - max) is summed one expert after the other in index order (every
-    // lane of the group walks the same chain from LDS), the k argmax rounds prefer the
-    // lower index on equal probabilities, and the gates are summed in rank order.
     {
         int G = 1;
         while (G < E && G < 64) G <<= 1;
-        const int lane_ = tid & 63, wave_ = tid >> 6;
-        const int lig = lane_ & (G - 1);          // lane in group
-        const int gbase = lane_ & ~(G - 1);       // first lane of the group
-        const int tpw = 64 / G;                   // tokens a wave handles at once
-        const unsigned long long gmask = (G == 64 ? ~0ull : ((1ull << G) - 1ull)) << gbase;
-        const float neg_inf = __uint_as_float(0xff800000u);
-        for (int i0 = wave_ * (TB / kRouterWaves); i0 < (wave_ + 1) * (TB / kRouterWaves); i0 += tpw) {
-            const int i = i0 + lane_ / G;         // token of this group
-            const bool live = i < nt && i < (wave_ + 1) * (TB / kRouterWaves);
-            float* row = prob + (live ? i : 0) * ES;
-            float pv[MAXJ];
-            float mx = neg_inf;
-#pragma unroll
-            for (int j = 0; j < MAXJ; ++j) {
-                const int e = lig + G * j;
-                pv[j] = (live && e < E) ? row[e] : neg_inf;
-                const float vv = (pv[j] == pv[j]) ? pv[j] : neg_inf;  // a NaN never becomes the maximum
-                mx = vv > mx ? vv : mx;
-            }
-            for (int o = 1; o < G; o <<= 1) {
-                const float other = __shfl_xor(mx, o);
-                mx = other > mx ? other : mx;
-            }
-#pragma unroll
-            for (int j = 0; j < MAXJ; ++j) {
-                const int e = lig + G * j;
-                if (live && e < E) {
-                    pv[j] = rb_expf(__fadd_rn(pv[j], -mx));
-                    row[e] = pv[j];
-                }
-            }
-            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the group's LDS writes have landed
-            __builtin_amdgcn_wave_barrier();
-            // the sum stays one chain of adds in index order; the LDS reads feeding it are issued
-            // eight at a time
-            float sum = 0.0f;
-            if (live) {
-                for (int e0 = 0; e0 < E; e0 += 8) {
-                    float ev[8];
-#pragma unroll
-                    for (int u = 0; u < 8; ++u) ev[u] = row[min(e0 + u, E - 1)];
-#pragma unroll
-                    for (int u = 0; u < 8; ++u)
-                        if (e0 + u < E) sum = __fadd_rn(sum, ev[u]);
-                }
-            }
-            __builtin_amdgcn_wave_barrier();
-            if (live && lig == 0) lsev[i] = __fadd_rn(mx, rb_logf(sum));
-#pragma unroll
-            for (int j = 0; j < MAXJ; ++j) {
-                const int e = lig + G * j;
-                if (live && e < E) {
-                    if (sum > 0.0f) pv[j] = __fdiv_rn(pv[j], sum);
-                    row[e] = pv[j];
-                }
-            }
-            // ---- k rounds of argmax over the experts not yet taken ----
-            const bool ok = live && ((valid == nullptr) || (valid[t0 + i] != 0));
-            unsigned taken_bits = 0;  // bit j: expert lig + G j is taken
-            float total = 0.0f;
-            for (int r = 0; r < k; ++r) {
-                // First expert not yet taken: the lowest set bit of a ballot over the group, taking
-                // the expert slices j in increasing order (slice j holds experts G j .. G j + G - 1).
-                int first = 0x7fffffff;
-#pragma unroll
-                for (int j = MAXJ - 1; j >= 0; --j) {
-                    const int e = lig + G * j;
-                    const unsigned long long m = __ballot(e < E && !((taken_bits >> j) & 1u)) & gmask;
-                    if (m != 0ull) first = (__ffsll((long long)m) - 1 - gbase) + G * j;
-                }
-                // Best non-NaN candidate: probabilities are never negative, so their bit patterns
-                // order like the values; with the inverted index below them, one 64-bit maximum over
-                // the group yields the greatest probability and, among equals, the lowest index.
-                unsigned long long key = 0ull;  // no candidate
-#pragma unroll
-                for (int j = 0; j < MAXJ; ++j) {
-                    const int e = lig + G * j;
-                    if (e < E && !((taken_bits >> j) & 1u) && pv[j] == pv[j]) {
-                        const unsigned long long kj =
-                            ((unsigned long long)__float_as_uint(pv[j]) << 32) | (unsigned long long)(0xffffffffu - (unsigned)e);
-                        key = kj > key ? kj : key;
-                    }
-                }
-                for (int o = 1; o < G; o <<= 1) {
-                    const unsigned long long other = __shfl_xor(key, o);
-                    key = other > key ? other : key;
-                }
-                const int ci = key != 0ull ? (int)(0xffffffffu - (unsigned)(key & 0xffffffffull)) : 0x7fffffff;
-                // the reference starts from the first untaken expert and replaces it only on a
-                // strictly greater probability: if that first one is NaN nothing replaces it
-                bool first_nan = false;
-#pragma unroll
-                for (int j = 0; j < MAXJ; ++j)
-                    if (lig + G * j == first && pv[j] != pv[j]) first_nan = true;
-                const bool nan_wins = (__ballot(first_nan) & gmask) != 0ull;
-                const int best = (nan_wins || ci == 0x7fffffff) ? first : ci;
-                float mine = 0.0f;
-#pragma unroll
-                for (int j = 0; j < MAXJ; ++j)
-                    if (lig + G * j == best) {
-                        mine = pv[j];
-                        taken_bits |= 1u << j;
-                    }
-                const float bestv = __shfl(mine, gbase + (best & (G - 1)));
-                total = __fadd_rn(total, bestv);
-                if (live && lig == 0) {
-                    lexp[i * k + r] = ok ? best : -1;
-                    gates[i * k + r] = ok ? bestv : 0.0f;
-                }
-            }
-            __builtin_amdgcn_s_waitcnt(0xc07f);
-            __builtin_amdgcn_wave_barrier();
-            if (ok && total > 0.0f)
-                for (int r = lig; r < k; r += G) gates[i * k + r] = __fdiv_rn(gates[i * k + r], total);
-        }
+        // a wave's four tokens: all at once with up to 16 lanes per token, in two or four turns with 32 or 64 - the
+        // turns are worked on side by side (one instruction stream), because each is a chain of dependent steps
+        if (G == 64) softmax_topk<MAXJ, 4>(prob, lsev, gates, lexp, G, t0, nt, ES, valid, E, k);
+        else if (G == 32) softmax_topk<MAXJ, 2>(prob, lsev, gates, lexp, G, t0, nt, ES, valid, E, k);
+        else softmax_topk<MAXJ, 1>(prob, lsev, gates, lexp, G, t0, nt, ES, valid, E, k);
     }
     __syncthreads();
 
