@@ -94,6 +94,9 @@ __device__ __forceinline__ void token_phase_serial(float* row, int t, int E, int
 // probabilities are >= +0, so their bit patterns order like their values, and among equal ones the lower
 // index wins, as the reference's strict `>` scan does); a taken expert's key is 0, and so is a NaN's, which the
 // scan never prefers to anything and never replaces once it is the candidate.
+// softmax_rows and route of one token by a group of G lanes (16 or 64), lane j owning expert j: the reductions
+// run through lane-permuting operands and the ordered sum as a lane-shift chain (see softmax_topk in
+// routing_kernels.hip for both), so the phase makes two trips to LDS instead of dozens.
 template <int G>
 __device__ __forceinline__ void token_phase_lanes(float* row_lds, int t, int j, int E, int k, const uint8_t* valid,
                                                   float* P, float* lse, float* lsev, int* sexp, int* expert_of,
@@ -103,15 +106,16 @@ __device__ __forceinline__ void token_phase_lanes(float* row_lds, int t, int j, 
     const bool mine = j < E;
     const float neg_inf = __uint_as_float(0xff800000u);
     const float v = mine ? row_lds[j] : neg_inf;
-    float mx = (v == v) ? v : neg_inf;  // a NaN never replaces the maximum
-#pragma unroll
-    for (int o = G / 2; o > 0; o >>= 1) {
-        const float other = __shfl_xor(mx, o);
-        mx = other > mx ? other : mx;
+    const float mx = group_fmax((v == v) ? v : neg_inf, G);  // a NaN never replaces the maximum
+    const float ex = mine ? rb_expf(__fadd_rn(v, -mx)) : 0.0f;   // lanes without an expert carry +0 through the sum
+    // ((ex_0 + ex_1) + ex_2) + ...: lane l holds the sum through expert l after l steps
+    float acc = ex;
+    for (int st = 1; st < G; ++st) {
+        const float below = __uint_as_float(lanes_from<0x138>(__float_as_uint(acc)));  // wave_shr:1
+        const float next = __fadd_rn(below, ex);
+        acc = j == 0 ? ex : next;
     }
-    const float ex = mine ? rb_expf(__fadd_rn(v, -mx)) : 0.0f;
-    float sum = 0.0f;
-    for (int e = 0; e < E; ++e) sum = __fadd_rn(sum, __shfl(ex, base + e));
+    const float sum = __shfl(acc, base + G - 1);
     const float l = __fadd_rn(mx, rb_logf(sum));
     const float p = sum > 0.0f ? __fdiv_rn(ex, sum) : ex;
     if (mine) {
@@ -135,31 +139,30 @@ __device__ __forceinline__ void token_phase_lanes(float* row_lds, int t, int j, 
     // part in no comparison - it is selected only when it is the first expert not yet taken, and then nothing
     // replaces it.
     const bool is_nan = p != p;
-    unsigned long long key =
-        (mine && !is_nan) ? (((unsigned long long)__float_as_uint(p) << 32) | (0xffffffffu - (unsigned)j)) : 0ull;
     bool taken = !mine;
     const unsigned long long gmask = G == 64 ? ~0ull : ((1ull << G) - 1ull);
     float total = 0.0f;
     float my_p = 0.0f;  // lane r keeps round r's probability
     int my_e = -1;
     for (int r = 0; r < k; ++r) {
-        unsigned long long best = key;
-#pragma unroll
-        for (int o = G / 2; o > 0; o >>= 1) {
-            const unsigned long long other = __shfl_xor(best, o);
-            best = other > best ? other : best;
-        }
+        // greatest probability bits among the experts not yet taken (probabilities are never negative), then the
+        // lowest index among the lanes that hold them
+        const bool cand = !taken && !is_nan;
+        const uint32_t mbits = group_umax(cand ? __float_as_uint(p) : 0u, G);
+        const uint32_t ci = group_umin((cand && __float_as_uint(p) == mbits) ? (uint32_t)j : 0x7fffffffu, G);
         const unsigned long long untaken = (__ballot(!taken) >> base) & gmask;
         const unsigned long long nans = (__ballot(!taken && is_nan) >> base) & gmask;
         const int first = __ffsll((long long)untaken) - 1;  // k <= E: some expert is always left
         const bool first_nan = ((nans >> first) & 1ull) != 0ull;
-        const int be = (first_nan || best == 0ull) ? first : (int)(0xffffffffu - (unsigned)(best & 0xffffffffull));
-        const float bv = __shfl(p, base + be);
-        total = __fadd_rn(total, bv);
-        if (j == be) {
-            key = 0ull;
-            taken = true;
+        const bool use_first = first_nan || ci == 0x7fffffffu;
+        const int be = use_first ? first : (int)ci;
+        float bv = __uint_as_float(mbits);  // the winner's probability is the greatest bits themselves
+        if (__ballot(use_first) != 0ull) {  // uniform over the wave: only a NaN first expert has to be fetched
+            const float fv = __shfl(p, base + be);
+            if (use_first) bv = fv;
         }
+        total = __fadd_rn(total, bv);
+        if (j == be) taken = true;
         if (j == r) {
             my_p = bv;
             my_e = be;

@@ -209,40 +209,6 @@ __global__ __launch_bounds__(NE * 64, (!AHEAD && sizeof(XT) == 2) ? 6 : 2) void 
     }
 }
 
-// Reductions over the G neighbouring lanes of a group (G a power of two up to 64, the same for the whole wave)
-// without LDS: inside a row of 16 lanes through the lane-permuting operand of the instruction itself (every lane of
-// the row ends with the result), across rows through four scalar reads.
-template <int CTRL>
-__device__ __forceinline__ uint32_t lanes_from(uint32_t v) {
-    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, true);
-}
-template <typename Op>
-__device__ __forceinline__ uint32_t group_reduce(uint32_t v, int G, Op op) {
-    if (G >= 2) v = op(v, lanes_from<0xB1>(v));   // quad_perm [1,0,3,2]
-    if (G >= 4) v = op(v, lanes_from<0x4E>(v));   // quad_perm [2,3,0,1]
-    if (G >= 8) v = op(v, lanes_from<0x141>(v));  // row_half_mirror
-    if (G >= 16) v = op(v, lanes_from<0x140>(v)); // row_mirror
-    if (G >= 32) {
-        const uint32_t r0 = __builtin_amdgcn_readlane(v, 0), r1 = __builtin_amdgcn_readlane(v, 16);
-        const uint32_t r2 = __builtin_amdgcn_readlane(v, 32), r3 = __builtin_amdgcn_readlane(v, 48);
-        const uint32_t lo = op(r0, r1), hi = op(r2, r3);
-        v = G == 64 ? op(lo, hi) : ((threadIdx.x & 32) ? hi : lo);
-    }
-    return v;
-}
-__device__ __forceinline__ uint32_t group_umax(uint32_t v, int G) {
-    return group_reduce(v, G, [](uint32_t a, uint32_t b) { return a > b ? a : b; });
-}
-__device__ __forceinline__ uint32_t group_umin(uint32_t v, int G) {
-    return group_reduce(v, G, [](uint32_t a, uint32_t b) { return a < b ? a : b; });
-}
-// (no NaN among the operands; which zero wins among zeros of both signs does not matter to the callers)
-__device__ __forceinline__ float group_fmax(float v, int G) {
-    return __uint_as_float(group_reduce(__float_as_uint(v), G, [](uint32_t a, uint32_t b) {
-        return __float_as_uint(fmaxf(__uint_as_float(a), __uint_as_float(b)));
-    }));
-}
-
 // softmax, log-sum-exp and the k argmax rounds for the tokens of one wave of a router block (see router_tail).
 // Everything order-sensitive keeps the reference's order: the maximum ignores NaN (f32::max), exp(v - max) is
 // summed one expert after the other in index order, the k argmax rounds prefer the lower index on equal
