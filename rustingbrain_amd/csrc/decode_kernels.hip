@@ -214,15 +214,17 @@ __device__ __forceinline__ void route_small_body(
         const int nw = E * wp, nx = T * xp;
         const uint4* wsrc = reinterpret_cast<const uint4*>(wr);
         const uint4* xsrc = reinterpret_cast<const uint4*>(x);
-        for (int i0 = 0; i0 < nw + nx; i0 += 4 * kSmallThreads) {
-            uint4 v[4];
+        // eight pieces a thread are requested before the first is stored: 64 KB a round trip (C2's 36 KB: one)
+        constexpr int kPieces = 8;
+        for (int i0 = 0; i0 < nw + nx; i0 += kPieces * kSmallThreads) {
+            uint4 v[kPieces];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < kPieces; ++u) {
                 const int i = min(i0 + u * kSmallThreads + tid, nw + nx - 1);
                 v[u] = i < nw ? wsrc[i] : xsrc[i - nw];
             }
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < kPieces; ++u) {
                 const int i = i0 + u * kSmallThreads + tid;
                 if (i < nw) {
                     const int r = i / wp, c = i - r * wp;
@@ -372,6 +374,48 @@ __device__ __forceinline__ void route_small_body(
     __syncthreads();
 
     // ---- bucket loop: a stable counting sort of the slots by expert ----------------
+    // With at most 64 slots and 64 experts the first wave sorts and the second wave works out the two losses beside
+    // it (same formulas and orders as the general code at the end; the per-expert counts it needs are ballots of
+    // its own), and nothing is left to wait for.
+    const bool side_losses = S <= 64 && E <= 64;
+    if (side_losses && tid >= 64 && tid < 128) {
+        const int ln = tid - 64;
+        const int my = ln < S ? sexp[ln] : -1;
+        int c_mine = 0;  // lane e: slots of expert e
+        for (int e = 0; e < E; ++e) {
+            const int c = __popcll(__ballot(my == e));
+            if (ln == e) c_mine = c;
+        }
+        int V = 0;
+        for (int t = 0; t < T; ++t) V += ((valid == nullptr) || valid[t]) ? 1 : 0;
+        if (ln < E) {
+            float term = 0.0f;
+            if (V > 0) {
+                const float load = (float)c_mine / ((float)V * (float)k);
+                float mass = 0.0f;
+                for (int t = 0; t < T; ++t)
+                    if ((valid == nullptr) || valid[t]) mass = mass + prob[t * E + ln];
+                mass = mass / (float)V;
+                term = load * mass;
+            }
+            aux_term[ln] = term;
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's LDS writes have landed
+        __builtin_amdgcn_wave_barrier();
+        if (ln == 0) {
+            float aux = 0.0f, z = 0.0f;
+            if (V > 0) {
+                for (int e = 0; e < E; ++e) aux = aux + aux_term[e];
+                aux = aux * ((float)E * w_aux);
+                float zs = 0.0f;
+                for (int t = 0; t < T; ++t)
+                    if ((valid == nullptr) || valid[t]) zs = zs + lsev[t] * lsev[t];
+                z = w_z * zs / (float)V;
+            }
+            losses[0] = aux;
+            losses[1] = z;
+        }
+    }
     if (S <= 64) {
         // one wave, slot = lane: a ballot per expert gives its count and every slot's rank
         if (tid < 64) {
@@ -445,6 +489,7 @@ __device__ __forceinline__ void route_small_body(
                 }
         }
     }
+    if (side_losses) return;
     __syncthreads();
 
     // ---- auxiliary losses (src/moe.rs:325-337): per expert in token order ---------
@@ -557,7 +602,7 @@ struct DecodeSide {
 // NW = waves of a workgroup, each with 1 / NW of the reduction steps: 4 for the gate/up product, 8 for the
 // down product (a third of the workgroups and twice the reduction length: with 8 waves every weight byte of
 // the launch is requested before the first multiply there as well).
-template <bool SWIGLU, bool I8, int NW, int BATCH>
+template <bool SWIGLU, bool I8, int NW, int BATCH, int TEAMS = 1>
 __device__ __forceinline__ void decode_gemm_body(const DecodeSide& sd, int fb, float* red_raw);
 
 // The combine of a decode-shaped call, for the 32 output features of block `fb` and every token: what
@@ -689,11 +734,16 @@ __global__ __launch_bounds__(NW * 64) void decode_gemm_kernel(DecodeGemmArgs g) 
     decode_gemm_body<SWIGLU, I8, NW, kBatch>(sd, fb, red);
 }
 
-// red_raw: NW * (SWIGLU ? 2 : 1) * 1024 floats of LDS; BATCH: reduction steps whose loads a wave issues together
-template <bool SWIGLU, bool I8, int NW, int BATCH>
+// red_raw: TEAMS * NW * (SWIGLU ? 2 : 1) * 1024 floats of LDS; BATCH: reduction steps whose loads a wave issues together.
+// TEAMS > 1: the workgroup is TEAMS teams of NW waves, each with a feature block `fb` of its own (the caller hands
+// every team its block; a team without one has left the kernel before: the barrier below counts the waves that
+// are still there).
+template <bool SWIGLU, bool I8, int NW, int BATCH, int TEAMS>
 __device__ __forceinline__ void decode_gemm_body(const DecodeSide& sd, int fb, float* red_raw) {
-    float (*red)[SWIGLU ? 2 : 1][16][64] = reinterpret_cast<float (*)[SWIGLU ? 2 : 1][16][64]>(red_raw);
-    const int tid = threadIdx.x;
+    const int team = TEAMS > 1 ? (int)threadIdx.x / (NW * 64) : 0;
+    float (*red)[SWIGLU ? 2 : 1][16][64] =
+        reinterpret_cast<float (*)[SWIGLU ? 2 : 1][16][64]>(red_raw + (size_t)team * NW * (SWIGLU ? 2 : 1) * 1024);
+    const int tid = (int)threadIdx.x - team * (NW * 64);
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int K = sd.K;
@@ -810,10 +860,12 @@ __global__ __launch_bounds__(kSmallThreads, 2) void decode_front_kernel(SmallRou
             r.perm_slot, r.perm_token, r.inv_pos, nullptr, 0.0f, nullptr, nullptr);
         return;
     }
+    // a product workgroup is two teams of four waves, each with a block of 32 features of its own: the reduction is
+    // split four ways as in the launch without the routing, and a compute unit has twice the weight bytes in flight
     const int widest = g.a_shared ? max(g.N, g.N_shared) : g.N;
-    const int nfb = widest / 32;
+    const int nfb = widest / 32, npair = (nfb + 1) / 2;
     const int idx = blockIdx.x - 1;
-    const int fb = idx % nfb, side = idx / nfb;
+    const int fb = 2 * (idx % npair) + (int)threadIdx.x / (kSmallThreads / 2), side = idx / npair;
     DecodeSide sd;
     sd.row_index = nullptr;
     sd.row0 = 0;
@@ -840,7 +892,7 @@ __global__ __launch_bounds__(kSmallThreads, 2) void decode_front_kernel(SmallRou
         sd.out_row0 = 0;
     }
     if (fb * 32 >= sd.N) return;
-    decode_gemm_body<true, I8, kSmallThreads / 64, kBatch>(sd, fb, reinterpret_cast<float*>(smem));
+    decode_gemm_body<true, I8, kSmallThreads / 128, kBatch, 2>(sd, fb, reinterpret_cast<float*>(smem));
 }
 
 bool decode_front_ok(const void* x, const float* wr, int T, int d, int E, int k) {
@@ -857,7 +909,7 @@ hipError_t launch_decode_front(const SmallRouteArgs& r, const DecodeGemmArgs& g,
     if (!small_route_ok(r.T, r.E, r.k) || r.norm_w || r.rows16 || !g.swiglu) return hipErrorInvalidValue;
     const int shared_tiles = g.a_shared ? (g.T_shared + 31) / 32 : 0;
     const int widest = g.a_shared ? (g.N > g.N_shared ? g.N : g.N_shared) : g.N;
-    const int grid = 1 + (r.E + shared_tiles) * (widest / 32);
+    const int grid = 1 + (r.E + shared_tiles) * ((widest / 32 + 1) / 2);
     if (wk == WeightKind::BF16)
         RB_LAUNCH(decode_front_kernel<false>, dim3(grid), dim3(kSmallThreads), 0, s, r, g, r.E, r.T);
     else if (wk == WeightKind::I8)
