@@ -809,31 +809,37 @@ __device__ __forceinline__ void decode_gemm_body(const DecodeSide& sd, int fb, f
     }
     __syncthreads();
     // accumulator element v of lane l: feature 8 (v / 4) + 4 (l / 32) + v % 4, token l % 32;
-    // the partial sums of the waves are added in wave order
+    // the partial sums of the waves are added in wave order.  A thread takes two neighbouring elements - two
+    // neighbouring features of one token - and writes them with one four-byte store.
 #pragma unroll
-    for (int i = 0; i < 1024 / (NW * 64); ++i) {
+    for (int i = 0; i < 512 / (NW * 64); ++i) {
         const int idx = i * (NW * 64) + tid;
-        const int v = idx >> 6, l = idx & 63;
+        const int v = (idx >> 6) * 2, l = idx & 63;
         const int token = l & 31;
-        const int f = 8 * (v >> 2) + 4 * (l >> 5) + (v & 3);
-        float y = red[0][0][v][l];
+        const int f = 8 * (v >> 2) + 4 * (l >> 5) + (v & 3);  // even
+        float y2[2];
 #pragma unroll
-        for (int w = 1; w < NW; ++w) y += red[w][0][v][l];
-        if constexpr (I8) y *= sd.scales[fb * 32 + f];
-        if constexpr (SWIGLU) {
-            float u = red[0][1][v][l];
+        for (int h = 0; h < 2; ++h) {
+            float y = red[0][0][v + h][l];
 #pragma unroll
-            for (int w = 1; w < NW; ++w) u += red[w][1][v][l];
-            if constexpr (I8) u *= sd.scales[sd.N + fb * 32 + f];
-            y = silu_bf16_grade(y) * u;
+            for (int w = 1; w < NW; ++w) y += red[w][0][v + h][l];
+            if constexpr (I8) y *= sd.scales[fb * 32 + f + h];
+            if constexpr (SWIGLU) {
+                float u = red[0][1][v + h][l];
+#pragma unroll
+                for (int w = 1; w < NW; ++w) u += red[w][1][v + h][l];
+                if constexpr (I8) u *= sd.scales[sd.N + fb * 32 + f + h];
+                y = silu_bf16_grade(y) * u;
+            }
+            y2[h] = y;
         }
         if (token < sd.rows) {
             bf16_t* const where = sd.out + (size_t)(sd.out_row0 + sd.row0 + token) * sd.N + fb * 32 + f;
+            const uint32_t two = (uint32_t)f32_to_bf16_bits(y2[0]) | ((uint32_t)f32_to_bf16_bits(y2[1]) << 16);
             if (sd.coherent_out)
-                __hip_atomic_store(reinterpret_cast<unsigned short*>(where), (unsigned short)f32_to_bf16_bits(y),
-                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(reinterpret_cast<uint32_t*>(where), two, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             else
-                *where = from_f32<bf16_t>(y);
+                *reinterpret_cast<uint32_t*>(where) = two;
         }
     }
 }
