@@ -914,18 +914,18 @@ __global__ __launch_bounds__(256) void dispatch_fused_kernel(
         if (tid == 0) offsets[E] = off[E];
     }
     if (loss_blk) {
+        // every valid token routes exactly k slots, so the valid-token count is routed / k.  The experts' terms
+        // (two divisions and a product each) side by side, then their sum in expert order by one thread.
+        const int V = off[E] / k;
+        const float tokens = (float)V;
+        const float slots = (float)V * (float)k;
+        float* const term = part_mass;  // [E]: the parts' sums are used up
+        if (tid < E && V > 0) term[tid] = ((float)cnt[tid] / slots) * (mass[tid] / tokens);
+        __syncthreads();
         if (tid == 0) {
-            // every valid token routes exactly k slots, so the valid-token count is routed / k
-            const int V = off[E] / k;
             float aux = 0.0f, z = 0.0f;
             if (V > 0) {
-                const float tokens = (float)V;
-                const float slots = (float)V * (float)k;
-                for (int q = 0; q < E; ++q) {
-                    const float load = (float)cnt[q] / slots;
-                    const float ms = mass[q] / tokens;
-                    aux = aux + load * ms;
-                }
+                for (int q = 0; q < E; ++q) aux = aux + term[q];
                 aux = aux * ((float)E * w_aux);
                 z = w_z * mass[E] / tokens;
             }
@@ -1128,19 +1128,19 @@ __global__ __launch_bounds__(kScanThreads) void layout_scan_kernel(
         }
         if (tid == E - 1) ntiles[0] = first + n;
     }
+    // every valid token routes exactly k slots, so the valid-token count is routed / k.  The experts' terms (two
+    // divisions and a product each) side by side, then their sum in expert order by one thread.
+    const int V = off[E] / k;
+    const float tokens = (float)V;
+    const float slots = (float)V * (float)k;
+    float* const term = part_mass;  // [E]: the parts' sums are used up
+    if (tid < E && V > 0) term[tid] = ((float)cnt[tid] / slots) * (mass[tid] / tokens);
+    __syncthreads();
     if (tid == 0) {
         offsets[E] = off[E];
-        // every valid token routes exactly k slots, so the valid-token count is routed / k
-        const int V = off[E] / k;
         float aux = 0.0f, z = 0.0f;
         if (V > 0) {
-            const float tokens = (float)V;
-            const float slots = (float)V * (float)k;
-            for (int q = 0; q < E; ++q) {
-                const float load = (float)cnt[q] / slots;
-                const float ms = mass[q] / tokens;
-                aux = aux + load * ms;
-            }
+            for (int q = 0; q < E; ++q) aux = aux + term[q];
             aux = aux * ((float)E * w_aux);
             z = w_z * mass[E] / tokens;
         }
