@@ -153,9 +153,11 @@ typedef enum rbmoe_option {
     RBMOE_OPT_QUANT_RULE = 10,     /* f32 -> int8 per row, scale = absmax / 127: 0 q = round(w / scale), the checkpoint
                                       writer's rule (src/transformer.rs:512-519); 1 q = round(w * (1 / scale)), the
                                       in-memory rule of Quantized::from_matrix (src/quantized.rs:29-51) */
-    RBMOE_OPT_QUANTIZE_ROUTER = 11 /* 1: an f32 router is quantized at upload as well, as TransformerLm::quantize does
+    RBMOE_OPT_QUANTIZE_ROUTER = 11,/* 1: an f32 router is quantized at upload as well, as TransformerLm::quantize does
                                       (src/transformer.rs:899-910 via src/moe.rs:491-500), and the layer routes with the
                                       quantized product (sum x * q in 32 lanes) * scale (src/quantized.rs:55-62, :154-177) */
+    RBMOE_OPT_DECODE_DOWN_BY_EXPERT = 12 /* (a kernel choice again) 0: the down launch of a decode-shaped call always
+                                      finds its experts through the tile table, also behind RBMOE_OPT_DECODE_FRONT */
 } rbmoe_option;
 int rbmoe_layer_set_option(rbmoe_layer* layer, int32_t option, int32_t value);
 

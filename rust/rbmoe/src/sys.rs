@@ -38,6 +38,7 @@ pub const RBMOE_OPT_WGRAD_GENERIC: i32 = 8;
 pub const RBMOE_OPT_DECODE_COMBINE_FOLD: i32 = 9;
 pub const RBMOE_OPT_QUANT_RULE: i32 = 10;
 pub const RBMOE_OPT_QUANTIZE_ROUTER: i32 = 11;
+pub const RBMOE_OPT_DECODE_DOWN_BY_EXPERT: i32 = 12;
 
 pub const RBMOE_NUM_STAGES: usize = 8;
 

@@ -22,7 +22,7 @@ W_ROUTER, W_GATE, W_UP, W_DOWN, W_SHARED_GATE, W_SHARED_UP, W_SHARED_DOWN, W_NOR
 # rbmoe_option
 (OPT_FORCE_GENERIC, OPT_EXPLICIT_GATHER, OPT_GROUP_M, OPT_DECODE_PATH, OPT_DECODE_FRONT, OPT_FUSED_ROUTER,
  OPT_SIDE_STREAM, OPT_WGRAD_MODE, OPT_WGRAD_GENERIC, OPT_DECODE_COMBINE_FOLD, OPT_QUANT_RULE,
- OPT_QUANTIZE_ROUTER) = range(12)
+ OPT_QUANTIZE_ROUTER, OPT_DECODE_DOWN_BY_EXPERT) = range(13)
 NUM_STAGES = 8
 STATIC_SCRATCH_BYTES = 8 << 20
 STAGE_NAMES = ("router", "empty", "dispatch", "gate_up", "down", "shared", "combine", "total")

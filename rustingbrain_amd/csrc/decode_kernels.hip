@@ -11,6 +11,8 @@
 // and the products are spread over (tile, 32-feature block) workgroups whose four waves
 // split the reduction dimension, so that a few hundred kilobytes of weight fragments are in
 // flight per CU and every byte of a touched expert is fetched exactly once per 32-row tile.
+#include <type_traits>
+
 #include "rbmoe_kernels.h"
 
 namespace rbmoe {
@@ -186,7 +188,7 @@ __device__ __forceinline__ void route_small_body(
     int* __restrict__ tile_row0, int* __restrict__ tile_rows, int* __restrict__ ntiles,
     float* __restrict__ losses, int* __restrict__ perm_slot, int* __restrict__ perm_token,
     int* __restrict__ inv_pos, const float* __restrict__ norm_w, float norm_eps, XT* __restrict__ xn_out,
-    bf16_t* __restrict__ rows16) {
+    bf16_t* __restrict__ rows16, unsigned int* __restrict__ expert_tokens = nullptr) {
     static_assert(STAGE % 16 == 0, "the arrays behind the staging area stay aligned");
     unsigned char* const stage = smem;
     float* const prob = reinterpret_cast<float*>(smem + STAGE);                 // [kSmallRouteMaxPairs]
@@ -421,6 +423,17 @@ __device__ __forceinline__ void route_small_body(
         if (tid < 64) {
             const int my = tid < S ? sexp[tid] : -1;
             int run = 0, tiles = 0;
+            if (expert_tokens != nullptr) {
+                // the tokens of every expert, one bit a token (its rows are these tokens in ascending order: the sort
+                // is stable and a token names an expert at most once), gathered in LDS (`off` is free on this path)
+                for (int e = tid; e < E; e += 64) off[e] = 0;
+                __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+                __builtin_amdgcn_wave_barrier();
+                if (my >= 0) atomicOr(reinterpret_cast<unsigned int*>(&off[my]), 1u << (tid / k));
+                __builtin_amdgcn_s_waitcnt(0xc07f);
+                __builtin_amdgcn_wave_barrier();
+                for (int e = tid; e < E; e += 64) expert_tokens[e] = (unsigned int)off[e];
+            }
             for (int e = 0; e < E; ++e) {
                 const unsigned long long mask = __ballot(my == e);
                 const int c = __popcll(mask);
@@ -480,13 +493,16 @@ __device__ __forceinline__ void route_small_body(
         __syncthreads();
         for (int e = tid; e < E; e += kSmallThreads) {
             int pos = off[e];
+            unsigned int tokens = 0u;
             for (int s = 0; s < S; ++s)
                 if (sexp[s] == e) {
                     perm_slot[pos] = s;
                     perm_token[pos] = s / k;
                     inv_pos[s] = pos;
+                    tokens |= 1u << (s / k);
                     ++pos;
                 }
+            if (expert_tokens != nullptr) expert_tokens[e] = tokens;
         }
     }
     if (side_losses) return;
@@ -602,8 +618,19 @@ struct DecodeSide {
 // NW = waves of a workgroup, each with 1 / NW of the reduction steps: 4 for the gate/up product, 8 for the
 // down product (a third of the workgroups and twice the reduction length: with 8 waves every weight byte of
 // the launch is requested before the first multiply there as well).
-template <bool SWIGLU, bool I8, int NW, int BATCH, int TEAMS = 1>
-__device__ __forceinline__ void decode_gemm_body(const DecodeSide& sd, int fb, float* red_raw);
+// The rows of a routed expert as the routing leaves them for a launch with one workgroup row per expert
+// (decode_down_by_expert_kernel): the tokens the expert takes, one bit a token, and the position of its first row.
+// The words are fetched behind the first weight loads (LATE_ROWS): nothing the weights' addresses need waits for them.
+struct LateRows {
+    const unsigned int* tokens;  // the expert's word
+    const int* first;            // the expert's word
+    const int* with_rows;        // experts with rows (one word for the launch)
+    bool routed;  // false: the side's rows are sd.row0 / sd.rows as they stand (the shared expert)
+    int with_rows_out = 0;
+};
+
+template <bool SWIGLU, bool I8, int NW, int BATCH, int TEAMS = 1, bool LATE_ROWS = false>
+__device__ __forceinline__ void decode_gemm_body(DecodeSide& sd, int fb, float* red_raw, LateRows* late = nullptr);
 
 // The combine of a decode-shaped call, for the 32 output features of block `fb` and every token: what
 // combine_vec_kernel computes, element by element in the same order (the token's expert rows by ascending position,
@@ -711,10 +738,11 @@ __global__ __launch_bounds__(NW * 64) void decode_gemm_kernel(DecodeGemmArgs g) 
             } else {
                 sd.coherent_out = true;
                 decode_gemm_body<SWIGLU, I8, NW, kBatch>(sd, fb, red);
-                // every wave's row stores have completed (at device scope: they are device-scope stores) before
-                // the workgroup's arrival is counted.  No device-scope fence: that would write back this XCD's
-                // whole L2, once per workgroup.
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                // every wave waits until its row stores have been acknowledged (they are device-scope stores: they
+                // go through to memory) before the workgroup's arrival is counted behind the barrier - a barrier
+                // alone does not wait for stores.  No device-scope fence: that would write back this XCD's whole
+                // L2, once per workgroup.
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 __syncthreads();
                 if (threadIdx.x == 0) {
                     const int before = atomicAdd(&g.cmb_counter[fb], 1);
@@ -734,12 +762,170 @@ __global__ __launch_bounds__(NW * 64) void decode_gemm_kernel(DecodeGemmArgs g) 
     decode_gemm_body<SWIGLU, I8, NW, kBatch>(sd, fb, red);
 }
 
+// What a thread of the folded combine can fetch before its workgroup has multiplied anything: the positions of its
+// token's expert rows in ascending order with their gates (at most four slots a token), and the residual.
+constexpr int kCombineEarlySlots = 4;
+struct CombineEarly {
+    int pos[kCombineEarlySlots];  // as the routing wrote them; slots past k repeat the last one
+    float gate[kCombineEarlySlots];
+    uint32_t res[2];  // the residual's two elements as they lie in memory: one word of two bf16, or two f32
+};
+
+__device__ __forceinline__ void decode_combine_fetch(const DecodeGemmArgs& g, int fb, CombineEarly& ce) {
+    // loads only, none of them looked at here and no branch between them: they return while the weights stream in
+    const int t = min((int)threadIdx.x >> 4, g.cmb_T - 1), c = fb * 32 + 2 * ((int)threadIdx.x & 15), k = g.cmb_k;
+    const int* const ip = g.cmb_inv_pos + (size_t)t * k;
+    const float* const gp = g.cmb_gate_of + (size_t)t * k;
+#pragma unroll
+    for (int q = 0; q < kCombineEarlySlots; ++q) {
+        ce.pos[q] = ip[min(q, k - 1)];
+        ce.gate[q] = gp[min(q, k - 1)];
+    }
+    // (without a residual the words of the output's own place are fetched and never used; bf16: the second word is
+    // the first again)
+    const int es = g.cmb_f32 ? 4 : 2;
+    const char* const base = static_cast<const char*>(g.cmb_residual ? g.cmb_residual : g.cmb_out);
+    const char* const at = base + ((size_t)t * g.N + c) * es;
+    ce.res[0] = *reinterpret_cast<const uint32_t*>(at);
+    ce.res[1] = *reinterpret_cast<const uint32_t*>(at + (g.cmb_f32 ? 4 : 0));
+}
+
+// decode_combine_block for a workgroup of 512 threads (one element pair a thread) that fetched `ce` beforehand: the
+// expert rows' loads go out side by side, the sums are taken in the same order.
+template <typename XT>
+__device__ __forceinline__ void decode_combine_block_early(const DecodeGemmArgs& g, int fb, CombineEarly ce) {
+    const int t = (int)threadIdx.x >> 4, c = fb * 32 + 2 * ((int)threadIdx.x & 15);
+    if (t >= g.cmb_T) return;
+    // ascending positions (they are distinct; a padding token's slots and the slots past k have no row): five
+    // exchanges sort four
+#pragma unroll
+    for (int q = 0; q < kCombineEarlySlots; ++q)
+        if (q >= g.cmb_k || ce.pos[q] < 0) ce.pos[q] = 0x7fffffff;
+    auto order = [&](int a, int b) {
+        if (ce.pos[b] < ce.pos[a]) {
+            const int p = ce.pos[a]; ce.pos[a] = ce.pos[b]; ce.pos[b] = p;
+            const float w = ce.gate[a]; ce.gate[a] = ce.gate[b]; ce.gate[b] = w;
+        }
+    };
+    order(0, 1); order(2, 3); order(0, 2); order(1, 3); order(1, 2);
+    const bf16_t* const y = static_cast<const bf16_t*>(g.out);
+    const int d = g.N;
+    uint32_t v[kCombineEarlySlots], vs = 0u;
+#pragma unroll
+    for (int q = 0; q < kCombineEarlySlots; ++q)
+        v[q] = ce.pos[q] != 0x7fffffff
+                   ? __hip_atomic_load(reinterpret_cast<const uint32_t*>(y + (size_t)ce.pos[q] * d + c), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT)
+                   : 0u;
+    if (g.a_shared)
+        vs = __hip_atomic_load(reinterpret_cast<const uint32_t*>(static_cast<const bf16_t*>(g.out_shared) + (size_t)t * d + c),
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+    for (int q = 0; q < kCombineEarlySlots; ++q)
+        if (ce.pos[q] != 0x7fffffff) {
+            a0 = __fadd_rn(a0, __fmul_rn(ce.gate[q], __uint_as_float(v[q] << 16)));
+            a1 = __fadd_rn(a1, __fmul_rn(ce.gate[q], __uint_as_float(v[q] & 0xffff0000u)));
+        }
+    if (g.a_shared) {
+        a0 = __fadd_rn(a0, __uint_as_float(vs << 16));
+        a1 = __fadd_rn(a1, __uint_as_float(vs & 0xffff0000u));
+    }
+    if (g.cmb_residual) {
+        if constexpr (sizeof(XT) == 4) {
+            a0 = __fadd_rn(a0, __uint_as_float(ce.res[0]));
+            a1 = __fadd_rn(a1, __uint_as_float(ce.res[1]));
+        } else {
+            a0 = __fadd_rn(a0, __uint_as_float(ce.res[0] << 16));
+            a1 = __fadd_rn(a1, __uint_as_float(ce.res[0] & 0xffff0000u));
+        }
+    }
+    XT* const out = static_cast<XT*>(g.cmb_out);
+    out[(size_t)t * d + c] = from_f32<XT>(a0);
+    out[(size_t)t * d + c + 1] = from_f32<XT>(a1);
+}
+
+// ---------------------------------------------------------------------------
+// decode_down_by_expert_kernel: the down product and the folded combine behind decode_front_kernel, blockIdx.y =
+// expert (then the shared expert's 32-row blocks).  decode_gemm_kernel learns its expert from the tile table and
+// its rows from the row index - two dependent trips to memory in front of the weight loads and the token loads;
+// here the weights' address follows from the grid, and the three words that say which rows the expert has (its
+// token bits, its first position, the number of experts with rows) are requested before the weights and looked at
+// behind them.  Every thread also fetches what the combine will need of the routing (positions, gates, residual)
+// before the product, so that the last workgroup of a block has only the expert rows left to load.
+// Same products, same order of sums: the outputs are decode_gemm_kernel's bit for bit.
+// ---------------------------------------------------------------------------
+template <bool I8>
+__global__ __launch_bounds__(512) void decode_down_by_expert_kernel(DecodeGemmArgs g, const unsigned int* __restrict__ expert_tokens,
+                                                                    const int* __restrict__ offsets, int E) {
+    __shared__ float red[8 * 16 * 64];
+    __shared__ int last_of_block;
+    const int fb = blockIdx.x, side = blockIdx.y;
+    const bool routed = side < E;
+    LateRows late;
+    late.routed = routed;
+    late.tokens = expert_tokens + (routed ? side : 0);
+    late.first = offsets + (routed ? side : 0);
+    late.with_rows = g.ntiles;  // one tile an expert: the experts with rows
+    const int shared_tiles = g.a_shared ? (g.T_shared + 31) / 32 : 0;
+    DecodeSide sd;
+    sd.row_index = nullptr;
+    sd.a_row0 = 0;
+    sd.out_row0 = 0;
+    sd.row0 = 0;
+    sd.rows = 0;
+    sd.coherent_out = true;
+    if (routed) {
+        sd.a = static_cast<const bf16_t*>(g.a);
+        sd.a_row0 = side * g.a_expert_rows;
+        sd.w = static_cast<const char*>(g.w) + (size_t)side * g.w_expert_stride * (I8 ? 1 : 2);
+        sd.scales = I8 ? g.scales + (size_t)side * g.s_expert_stride : nullptr;
+        sd.out = static_cast<bf16_t*>(g.out);
+        sd.N = g.N;
+        sd.K = g.K;
+    } else {
+        const int st = side - E;
+        sd.a = static_cast<const bf16_t*>(g.a_shared);
+        sd.w = static_cast<const char*>(g.w_shared);
+        sd.scales = I8 ? g.scales_shared : nullptr;
+        sd.out = static_cast<bf16_t*>(g.out_shared);
+        sd.N = g.N_shared;
+        sd.K = g.K_shared;
+        sd.row0 = st * 32;
+        sd.rows = min(32, g.T_shared - sd.row0);
+    }
+    CombineEarly ce;
+    decode_combine_fetch(g, fb, ce);
+    decode_gemm_body<false, I8, 8, kBatch, 1, true>(sd, fb, red, &late);
+    const bool works = sd.rows > 0;
+    const int writers = late.with_rows_out + shared_tiles;
+    if (!works) {
+        // nothing to multiply here; with no writer at all (every row is padding and there is no shared expert) the
+        // first side's workgroups still owe their blocks the combine
+        if (writers != 0 || side != 0) return;
+    } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the row stores have been acknowledged
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            const int before = atomicAdd(&g.cmb_counter[fb], 1);
+            last_of_block = before == writers - 1;
+            if (before == writers - 1) atomicExch(&g.cmb_counter[fb], 0);  // every writer has arrived: ready for the next launch
+        }
+        __syncthreads();
+        if (!last_of_block) return;
+    }
+    if (g.cmb_f32) decode_combine_block_early<float>(g, fb, ce);
+    else decode_combine_block_early<bf16_t>(g, fb, ce);
+}
+
 // red_raw: TEAMS * NW * (SWIGLU ? 2 : 1) * 1024 floats of LDS; BATCH: reduction steps whose loads a wave issues together.
 // TEAMS > 1: the workgroup is TEAMS teams of NW waves, each with a feature block `fb` of its own (the caller hands
 // every team its block; a team without one has left the kernel before: the barrier below counts the waves that
 // are still there).
-template <bool SWIGLU, bool I8, int NW, int BATCH, int TEAMS>
-__device__ __forceinline__ void decode_gemm_body(const DecodeSide& sd, int fb, float* red_raw) {
+// LATE_ROWS: which rows the side has is looked at behind the first weight loads (`late`); a side without rows leaves
+// with sd.rows == 0 and nothing stored.
+template <bool SWIGLU, bool I8, int NW, int BATCH, int TEAMS, bool LATE_ROWS>
+__device__ __forceinline__ void decode_gemm_body(DecodeSide& sd, int fb, float* red_raw, LateRows* late) {
     const int team = TEAMS > 1 ? (int)threadIdx.x / (NW * 64) : 0;
     float (*red)[SWIGLU ? 2 : 1][16][64] =
         reinterpret_cast<float (*)[SWIGLU ? 2 : 1][16][64]>(red_raw + (size_t)team * NW * (SWIGLU ? 2 : 1) * 1024);
@@ -766,14 +952,21 @@ __device__ __forceinline__ void decode_gemm_body(const DecodeSide& sd, int fb, f
         }
     };
     // token fragment: lane -> token lane % 32, columns 16 s + 8 (lane / 32) .. + 7
-    const int trow = (lane & 31) < sd.rows ? (lane & 31) : 0;
-    int grow = (sd.row_index ? sd.row_index[sd.row0 + trow] : sd.row0 + trow) + sd.a_row0;  // awaited after the weight loads
+    int grow = 0;
+    if constexpr (!LATE_ROWS) {
+        const int trow = (lane & 31) < sd.rows ? (lane & 31) : 0;
+        grow = (sd.row_index ? sd.row_index[sd.row0 + trow] : sd.row0 + trow) + sd.a_row0;  // awaited after the weight loads
+    }
 
     floatx16 acc0, acc1;
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc0[v] = acc1[v] = 0.0f;
 
-    for (int s0 = g0; s0 < g1; s0 += BATCH) {
+    // One batch of reduction steps.  The first batch stands in front of the loop over the others, as straight
+    // code: at the head of a loop the compiler waits for every load still under way - the row index, what the
+    // combine fetched early - before the first weight load could go out.  Returns true when the side has no rows.
+    auto batch = [&](const int s0, auto first_tag) -> bool {
+        constexpr bool kFirst = decltype(first_tag)::value;
         bf16x8 wa[BATCH], wb[BATCH], tf[BATCH];
         // the weights first: the address of a token row depends on a load of its own (the row index), and
         // loads are issued in order - nothing of the stream may queue up behind that wait
@@ -784,6 +977,36 @@ __device__ __forceinline__ void decode_gemm_body(const DecodeSide& sd, int fb, f
             if constexpr (SWIGLU) wb[u] = wfrag(w1, s);
         }
         __builtin_amdgcn_sched_barrier(0);
+        if constexpr (LATE_ROWS && kFirst) {
+            {
+                // the three words, by scalar loads issued here and nowhere earlier (the compiler would fetch them
+                // in front of the weights, or with vector loads that queue up behind them)
+                unsigned int tokens;
+                int first, with_rows;
+                asm volatile(
+                    "s_load_dword %0, %3, 0x0\n\t"
+                    "s_load_dword %1, %4, 0x0\n\t"
+                    "s_load_dword %2, %5, 0x0\n\t"
+                    "s_waitcnt lgkmcnt(0)"
+                    : "=&s"(tokens), "=&s"(first), "=&s"(with_rows)
+                    : "s"(late->tokens), "s"(late->first), "s"(late->with_rows)
+                    : "memory");
+                late->with_rows_out = with_rows;
+                if (late->routed) {
+                    sd.rows = __popc(tokens);
+                    sd.row0 = first;
+                }
+                if (sd.rows <= 0) return true;  // the whole workgroup
+                const int trow = (lane & 31) < sd.rows ? (lane & 31) : 0;
+                int token = sd.row0 + trow;
+                if (late->routed) {  // row `trow` of the expert: the token of its set bit number `trow`
+                    unsigned int rest = tokens;
+                    for (int i = 0; i < trow; ++i) rest &= rest - 1u;
+                    token = __ffs(rest) - 1;
+                }
+                grow = token + sd.a_row0;
+            }
+        }
         // (the empty statement pins the first use of the row index, and with it the wait for it, below the
         // weight loads; the barriers keep every load of the batch ahead of the first multiply)
         asm volatile("" : "+v"(grow));
@@ -801,7 +1024,14 @@ __device__ __forceinline__ void decode_gemm_body(const DecodeSide& sd, int fb, f
                 if constexpr (SWIGLU) acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[u], tf[u], acc1, 0, 0, 0);
             }
         }
+        return false;
+    };
+    // (LATE_ROWS: every wave takes the first batch, also one without a reduction step of its own, so that all of
+    // them learn the rows and leave together when there are none)
+    if (LATE_ROWS || g0 < g1) {
+        if (batch(g0, std::true_type{})) return;
     }
+    for (int s0 = g0 + BATCH; s0 < g1; s0 += BATCH) batch(s0, std::false_type{});
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
         red[wave][0][v][lane] = acc0[v];
@@ -809,37 +1039,38 @@ __device__ __forceinline__ void decode_gemm_body(const DecodeSide& sd, int fb, f
     }
     __syncthreads();
     // accumulator element v of lane l: feature 8 (v / 4) + 4 (l / 32) + v % 4, token l % 32;
-    // the partial sums of the waves are added in wave order.  A thread takes two neighbouring elements - two
-    // neighbouring features of one token - and writes them with one four-byte store.
-#pragma unroll
-    for (int i = 0; i < 512 / (NW * 64); ++i) {
-        const int idx = i * (NW * 64) + tid;
-        const int v = (idx >> 6) * 2, l = idx & 63;
-        const int token = l & 31;
-        const int f = 8 * (v >> 2) + 4 * (l >> 5) + (v & 3);  // even
-        float y2[2];
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            float y = red[0][0][v + h][l];
-#pragma unroll
-            for (int w = 1; w < NW; ++w) y += red[w][0][v + h][l];
-            if constexpr (I8) y *= sd.scales[fb * 32 + f + h];
-            if constexpr (SWIGLU) {
-                float u = red[0][1][v + h][l];
-#pragma unroll
-                for (int w = 1; w < NW; ++w) u += red[w][1][v + h][l];
-                if constexpr (I8) u *= sd.scales[sd.N + fb * 32 + f + h];
-                y = silu_bf16_grade(y) * u;
-            }
-            y2[h] = y;
-        }
+    // the partial sums of the waves are added in wave order.  A thread takes four neighbouring features of one token
+    // and eight neighbouring threads one token's 32 features of the block: a row segment of 64 bytes leaves as one
+    // piece (rows that another workgroup of the launch reads go through to memory, where a write of a few bytes
+    // costs what a whole segment does).
+    if (tid < 256) {
+        const int token = tid >> 3, q = tid & 7;
+        const int v = 4 * (q >> 1), l = token + 32 * (q & 1), f = 4 * q;
         if (token < sd.rows) {
+            float y4[4];
+#pragma unroll
+            for (int h = 0; h < 4; ++h) {
+                float y = red[0][0][v + h][l];
+#pragma unroll
+                for (int w = 1; w < NW; ++w) y += red[w][0][v + h][l];
+                if constexpr (I8) y *= sd.scales[fb * 32 + f + h];
+                if constexpr (SWIGLU) {
+                    float u = red[0][1][v + h][l];
+#pragma unroll
+                    for (int w = 1; w < NW; ++w) u += red[w][1][v + h][l];
+                    if constexpr (I8) u *= sd.scales[sd.N + fb * 32 + f + h];
+                    y = silu_bf16_grade(y) * u;
+                }
+                y4[h] = y;
+            }
             bf16_t* const where = sd.out + (size_t)(sd.out_row0 + sd.row0 + token) * sd.N + fb * 32 + f;
-            const uint32_t two = (uint32_t)f32_to_bf16_bits(y2[0]) | ((uint32_t)f32_to_bf16_bits(y2[1]) << 16);
+            const unsigned long long four =
+                (unsigned long long)((uint32_t)f32_to_bf16_bits(y4[0]) | ((uint32_t)f32_to_bf16_bits(y4[1]) << 16)) |
+                ((unsigned long long)((uint32_t)f32_to_bf16_bits(y4[2]) | ((uint32_t)f32_to_bf16_bits(y4[3]) << 16)) << 32);
             if (sd.coherent_out)
-                __hip_atomic_store(reinterpret_cast<uint32_t*>(where), two, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(reinterpret_cast<unsigned long long*>(where), four, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             else
-                *reinterpret_cast<uint32_t*>(where) = two;
+                *reinterpret_cast<unsigned long long*>(where) = four;
         }
     }
 }
@@ -863,7 +1094,7 @@ __global__ __launch_bounds__(kSmallThreads, 2) void decode_front_kernel(SmallRou
         route_small_body<bf16_t, kFrontStageBytes>(
             smem, static_cast<const bf16_t*>(r.x), r.wr, r.bias, r.valid, r.T, r.d, r.E, r.k, r.w_aux, r.w_z, r.tile_m, r.P,
             r.lse, r.expert_of, r.gate_of, r.counts, r.offsets, r.tile_expert, r.tile_row0, r.tile_rows, r.ntiles, r.losses,
-            r.perm_slot, r.perm_token, r.inv_pos, nullptr, 0.0f, nullptr, nullptr);
+            r.perm_slot, r.perm_token, r.inv_pos, nullptr, 0.0f, nullptr, nullptr, r.expert_tokens);
         return;
     }
     // a product workgroup is two teams of four waves, each with a block of 32 features of its own: the reduction is
@@ -920,6 +1151,27 @@ hipError_t launch_decode_front(const SmallRouteArgs& r, const DecodeGemmArgs& g,
         RB_LAUNCH(decode_front_kernel<false>, dim3(grid), dim3(kSmallThreads), 0, s, r, g, r.E, r.T);
     else if (wk == WeightKind::I8)
         RB_LAUNCH(decode_front_kernel<true>, dim3(grid), dim3(kSmallThreads), 0, s, r, g, r.E, r.T);
+    else
+        return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+bool decode_down_by_expert_ok(const DecodeGemmArgs& g, int E, int T, int k) {
+    return !g.swiglu && g.cmb_out != nullptr && g.cmb_counter != nullptr && g.cmb_inv_pos != nullptr &&
+           g.cmb_gate_of != nullptr && g.a_expert_rows == T && T >= 1 && T <= 32 && k <= kCombineEarlySlots &&
+           g.cmb_T == T && g.cmb_k == k && (!g.a_shared || g.N_shared == g.N) && g.N / 32 <= kDecodeCombineMaxBlocks &&
+           g.N % 32 == 0 && E >= 1;
+}
+
+hipError_t launch_decode_down_by_expert(const DecodeGemmArgs& g, const unsigned int* expert_tokens, const int* offsets,
+                                        int E, WeightKind wk, hipStream_t s) {
+    if (!expert_tokens || !offsets || !decode_down_by_expert_ok(g, E, g.cmb_T, g.cmb_k)) return hipErrorInvalidValue;
+    const int shared_tiles = g.a_shared ? (g.T_shared + 31) / 32 : 0;
+    const dim3 grid(g.N / 32, E + shared_tiles);
+    if (wk == WeightKind::BF16)
+        RB_LAUNCH(decode_down_by_expert_kernel<false>, grid, dim3(512), 0, s, g, expert_tokens, offsets, E);
+    else if (wk == WeightKind::I8)
+        RB_LAUNCH(decode_down_by_expert_kernel<true>, grid, dim3(512), 0, s, g, expert_tokens, offsets, E);
     else
         return hipErrorInvalidValue;
     return hipGetLastError();

@@ -172,6 +172,7 @@ struct Work {
     void* hall = nullptr;  // hidden rows of every expert over every row, [E][T, F] (decode_front launches), or null
     void* x16 = nullptr;   // bf16 copy of f32 rows [T, d] (layers with cast_rows), or null
     int* cmb_counter = nullptr;  // arrival counters of a combine folded into the decode-shaped down launch (all zero between launches)
+    unsigned int* expert_tokens = nullptr;  // [E] the tokens of every expert, one bit a token (decode_front launches), or null
 };
 
 struct rbmoe_layer {
@@ -195,6 +196,7 @@ struct rbmoe_layer {
     bool shared_beside = true; // large batches: the shared expert's products on the side stream, beside the routing
     bool fused_router = true;  // logits and everything behind them in one launch where the shapes allow
     bool decode_fold = true;   // decode-shaped calls: the combine inside the down launch
+    bool decode_down_by_expert = true;  // behind a decode_front launch: the down launch's workgroup rows are experts, not tile-table entries
     bool last_front = false;   // the last forward's hidden rows are per expert over all rows (Work::hall)
     int group_m = 0;
     const char* kernel_name = "none";
@@ -219,6 +221,7 @@ struct rbmoe_layer {
     Buf xg, h, y, hs, ys;
     Buf x16;               // [max_T, d] bf16 copy of f32 rows (cast_rows)
     Buf hall;              // [E][min(max_T, 32), F] hidden rows of decode_front launches
+    Buf etok;              // [E] token bits of every expert (decode_front launches)
     Buf cmbcnt;            // [kDecodeCombineMaxBlocks] arrival counters of the folded decode combine
     // feed-forward norm in front of the layer (allocated by rbmoe_set_feed_forward_norm)
     Buf xn, norm_w;  // [max_T, d] activation dtype, [d] f32
@@ -343,7 +346,10 @@ Plan make_plan(rbmoe_layer* L) {
     p.add(&L->inv_pos, S * 4);
     if (L->cast_rows) p.add(&L->x16, T * d * 2);
     // decode_front launches need most experts touched (tokens * k >= 2 E, at most 32 tokens): none when E > 16 k
-    if (L->use_stream && E <= 16 * k) p.add(&L->hall, E * std::min<size_t>(T, kSmallRouteMaxTokens) * F * 2);
+    if (L->use_stream && E <= 16 * k) {
+        p.add(&L->hall, E * std::min<size_t>(T, kSmallRouteMaxTokens) * F * 2);
+        p.add(&L->etok, E * 4);
+    }
     p.add(&L->cmbcnt, (size_t)kDecodeCombineMaxBlocks * 4);
     p.add(&L->xg, S * d * as);
     p.add(&L->h, S * F * as);
@@ -830,6 +836,7 @@ Work work_of_layer(const rbmoe_layer* L) {
     w.perm_slot = (int*)L->perm_slot.p; w.perm_token = (int*)L->perm_token.p; w.inv_pos = (int*)L->inv_pos.p;
     w.h = L->h.p; w.y = L->y.p; w.hs = L->hs.p; w.ys = L->ys.p;
     w.hall = L->hall.p;
+    w.expert_tokens = (unsigned int*)L->etok.p;
     w.x16 = L->x16.p;
     w.cmb_counter = (int*)L->cmbcnt.p;
     return w;
@@ -859,7 +866,10 @@ size_t carve_decode_work(const rbmoe_layer* L, int T, unsigned char* base, Work*
     v.ntiles = (int*)take(8); v.losses = (float*)take(8);
     v.perm_slot = (int*)take(S * 4); v.perm_token = (int*)take(S * 4); v.inv_pos = (int*)take(S * 4);
     v.h = take(S * F * as); v.y = take(S * d * as);
-    if ((size_t)T * k >= 2 * E) v.hall = take(E * (size_t)T * F * 2);  // (the condition of decode_front_ok)
+    if ((size_t)T * k >= 2 * E) {  // (the condition of decode_front_ok)
+        v.hall = take(E * (size_t)T * F * 2);
+        v.expert_tokens = (unsigned int*)take(E * 4);
+    }
     if (c.shared_expert) {
         v.hs = take((size_t)T * Fs * as);
         v.ys = take((size_t)T * d * as);
@@ -1019,6 +1029,7 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
         if (front) {
             d1.row_index = nullptr;
             d1.out = wk_.hall;
+            sr.expert_tokens = wk_.expert_tokens;
             HIP_TRY(ctx, launch_decode_front(sr, d1, wk, s));
             L->replay[RBMOE_STAGE_GATE_UP] = [=](hipStream_t st) { return launch_decode_front(sr, d1, wk, st); };
         } else {
@@ -1051,8 +1062,17 @@ int forward_impl(rbmoe_layer* L, const void* x, int T, int cols, const uint8_t* 
             d2.cmb_residual = residual; d2.cmb_out = out;
             d2.cmb_T = T; d2.cmb_k = k; d2.cmb_f32 = abf ? 0 : 1;
         }
-        HIP_TRY(ctx, launch_decode_gemm(d2, wk, s));
-        L->replay[RBMOE_STAGE_DOWN] = [=](hipStream_t st) { return launch_decode_gemm(d2, wk, st); };
+        // behind the routing-beside-the-products launch every expert's rows are known by its token bits: the down
+        // launch then has one row of workgroups per expert, whose weights go out before anything of the routing is read
+        if (front && fold && L->decode_down_by_expert && wk_.expert_tokens != nullptr && decode_down_by_expert_ok(d2, E, T, k)) {
+            const unsigned int* const etok = wk_.expert_tokens;
+            const int* const offs = wk_.offsets;
+            HIP_TRY(ctx, launch_decode_down_by_expert(d2, etok, offs, E, wk, s));
+            L->replay[RBMOE_STAGE_DOWN] = [=](hipStream_t st) { return launch_decode_down_by_expert(d2, etok, offs, E, wk, st); };
+        } else {
+            HIP_TRY(ctx, launch_decode_gemm(d2, wk, s));
+            L->replay[RBMOE_STAGE_DOWN] = [=](hipStream_t st) { return launch_decode_gemm(d2, wk, st); };
+        }
         HIP_TRY(ctx, mark(5));
         HIP_TRY(ctx, mark(6));
         if (!fold) {
@@ -1601,6 +1621,7 @@ int rbmoe_layer_set_option(rbmoe_layer* L, int32_t option, int32_t value) {
         case RBMOE_OPT_DECODE_FRONT: L->decode_front = value != 0; return RBMOE_OK;
         case RBMOE_OPT_FUSED_ROUTER: L->fused_router = value != 0; return RBMOE_OK;
         case RBMOE_OPT_DECODE_COMBINE_FOLD: L->decode_fold = value != 0; return RBMOE_OK;
+        case RBMOE_OPT_DECODE_DOWN_BY_EXPERT: L->decode_down_by_expert = value != 0; return RBMOE_OK;
         case RBMOE_OPT_SIDE_STREAM:
             if (value != 0 && L->training)
                 if (const int rc = ensure_side_stream(ctx)) return rc;

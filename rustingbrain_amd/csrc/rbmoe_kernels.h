@@ -268,6 +268,9 @@ struct SmallRouteArgs {
     // f32 rows only: a bf16 copy [T, d] of the rows the routing is decided on (after the norm, if any), for the
     // matrix-core products; only for calls whose rows are staged in LDS (small_route_stages_rows)
     void* rows16 = nullptr;
+    // launch_decode_front only, or null: [E] the tokens every expert takes, one bit a token (at most 32 tokens); the
+    // expert's rows are these tokens in ascending order
+    unsigned int* expert_tokens = nullptr;
 };
 bool small_route_stages_rows(const void* x, const float* wr, int T, int d, int E, bool bf16);
 bool small_route_ok(int T, int E, int k);
@@ -316,5 +319,12 @@ hipError_t launch_decode_gemm(const DecodeGemmArgs& g, WeightKind wk, hipStream_
 // hidden rows to g.out as [E][T, N]; the shared expert as in launch_decode_gemm.  g.a / g.a_shared: the T rows.
 bool decode_front_ok(const void* x, const float* wr, int T, int d, int E, int k);
 hipError_t launch_decode_front(const SmallRouteArgs& r, const DecodeGemmArgs& g, WeightKind wk, hipStream_t s);
+// The down product behind launch_decode_front with the combine folded in (g as for launch_decode_gemm: cmb_* set,
+// a_expert_rows = tokens of the call), one row of workgroups per EXPERT instead of per entry of the tile table: a
+// workgroup knows its weights from its place in the grid and requests them at once, and learns its rows from
+// expert_tokens / offsets / g.ntiles behind them.  An expert without rows costs its weights' bytes.
+bool decode_down_by_expert_ok(const DecodeGemmArgs& g, int E, int T, int k);
+hipError_t launch_decode_down_by_expert(const DecodeGemmArgs& g, const unsigned int* expert_tokens, const int* offsets,
+                                        int E, WeightKind wk, hipStream_t s);
 
 }  // namespace rbmoe

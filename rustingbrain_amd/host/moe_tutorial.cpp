@@ -221,6 +221,41 @@ static void gpu_checks() {
         // no backward pass for a layer that is not in training mode
         EXPECT(throws<InvalidConfig>([&] { layer.backward(Matrix(ROWS, D)); }));
     }
+    // TransformerLm::quantize on the layer (reference src/transformer.rs:899-910): a router quantized at upload by
+    // the in-memory rule routes exactly as the same int8 rows and scales handed over as they are
+    {
+        const size_t QD = 64, QE = 8, QF = 32, QR = 96;
+        MoeLayer at_upload(QD, MoeConfig(QE, 2, QF), device, QR, RBMOE_F32, RBMOE_I8);
+        MoeLayer as_stored(QD, MoeConfig(QE, 2, QF), device, QR, RBMOE_F32, RBMOE_I8);
+        at_upload.quantize_on_upload(true, true);
+        as_stored.quantize_on_upload(true, false);
+        const Matrix router = random_matrix(QE, QD, 0.5f, 31);
+        std::vector<int8_t> q(QE * QD);
+        std::vector<float> scales(QE);
+        for (size_t e = 0; e < QE; ++e) {   // Quantized::from_matrix, reference src/quantized.rs:29-51
+            float absmax = 0.0f;
+            for (size_t c = 0; c < QD; ++c) absmax = std::fmax(absmax, std::fabs(router.row(e)[c]));
+            const float scale = absmax / 127.0f, inv = scale > 0.0f ? 1.0f / scale : 0.0f;
+            scales[e] = scale;
+            for (size_t c = 0; c < QD; ++c)
+                q[e * QD + c] = (int8_t)std::fmin(127.0f, std::fmax(-127.0f, std::round(router.row(e)[c] * inv)));
+        }
+        at_upload.set_router(router);
+        as_stored.set_router_q8(q.data(), scales.data());
+        const float qb = std::sqrt(6.0f / (float)(QD + QF));
+        for (size_t e = 0; e < QE; ++e) {
+            const Matrix g = random_matrix(QF, QD, qb, 300 + 3 * e), u = random_matrix(QF, QD, qb, 301 + 3 * e),
+                         d = random_matrix(QD, QF, qb, 302 + 3 * e);
+            at_upload.set_expert(e, g, u, d);
+            as_stored.set_expert(e, g, u, d);
+        }
+        const Matrix x = random_matrix(QR, QD, 1.0f, 33);
+        auto a = at_upload.forward_train(x, Layout{});
+        auto b = as_stored.forward_train(x, Layout{});
+        EXPECT(a.second.assignments == b.second.assignments);
+        EXPECT(a.second.probabilities.data == b.second.probabilities.data);
+        EXPECT(a.first.data == b.first.data);
+    }
     // a budget that cannot hold the layer is refused before anything is allocated
     EXPECT(throws<MemoryBudget>([&] {
         auto small = Device::open(0, 1);

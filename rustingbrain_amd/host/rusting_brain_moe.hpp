@@ -202,6 +202,22 @@ class MoeLayer {
         check(rbmoe_set_weight(layer_, which, expert, q, RBMOE_I8, scales, (int32_t)rows, (int32_t)cols), device_->raw());
     }
 
+    // A quantized router as it is stored: int8 rows [num_experts, d_model] and one scale per row; the layer then
+    // routes with the quantized product (src/quantized.rs:55-62).
+    void set_router_q8(const int8_t* q, const float* scales) {
+        set_weight_q8(RBMOE_W_ROUTER, 0, q, scales, config.num_experts, d_model_);
+    }
+
+    // What TransformerLm::quantize() (src/transformer.rs:899-910) does to this layer's Linears, applied to f32
+    // weights as they are set from here on.  in_memory_rule: q = round(w * (1 / scale)) as Quantized::from_matrix
+    // (src/quantized.rs:29-51), otherwise the .rbw writer's q = round(w / scale) (src/transformer.rs:512-519);
+    // router: the router is quantized as well (src/moe.rs:491-500).  The experts follow only on a layer whose weight
+    // dtype is RBMOE_I8.
+    void quantize_on_upload(bool in_memory_rule = true, bool router = true) {
+        set_option(RBMOE_OPT_QUANT_RULE, in_memory_rule ? 1 : 0);
+        set_option(RBMOE_OPT_QUANTIZE_ROUTER, router ? 1 : 0);
+    }
+
     Matrix forward(const Matrix& input) { return forward_train(input, Layout{}).first; }
 
     std::pair<Matrix, MoeCache> forward_train(const Matrix& input, const Layout& layout) {

@@ -85,6 +85,7 @@ _ENV_SWITCHES = {
     "RBMOE_NO_FUSED_ROUTER": (L.OPT_FUSED_ROUTER, 0), "RBMOE_NO_SIDE_STREAM": (L.OPT_SIDE_STREAM, 0),
     "RBMOE_ATOMIC_WGRAD": (L.OPT_WGRAD_MODE, 1), "RBMOE_DETERMINISTIC": (L.OPT_WGRAD_MODE, 2),
     "RBMOE_WGRAD_GENERIC": (L.OPT_WGRAD_GENERIC, 1), "RBMOE_NO_DECODE_COMBINE_FOLD": (L.OPT_DECODE_COMBINE_FOLD, 0),
+    "RBMOE_NO_DECODE_DOWN_BY_EXPERT": (L.OPT_DECODE_DOWN_BY_EXPERT, 0),
 }
 
 

@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 
 @pytest.fixture
 def env():
-    keys = ("RBMOE_NO_DECODE_PATH", "RBMOE_NO_DECODE_FRONT", "RBMOE_NO_DECODE_COMBINE_FOLD")
+    keys = ("RBMOE_NO_DECODE_PATH", "RBMOE_NO_DECODE_FRONT", "RBMOE_NO_DECODE_COMBINE_FOLD", "RBMOE_NO_DECODE_DOWN_BY_EXPERT")
     saved = {k: os.environ.get(k) for k in keys}
     yield os.environ
     for k, v in saved.items():
@@ -189,3 +189,67 @@ def test_the_combine_inside_the_down_launch_gives_the_bits_of_the_combine_launch
     ref = oracle_layer(t).forward(t.x, valid=valid, threads=4)
     want = ref.out if residual is None else ref.out + residual
     assert rel_l2(outs[True], want) <= 2e-2 if np.any(want) else not np.any(outs[True])
+
+
+BY_EXPERT_CASES = [
+    dict(act="bf16", wt="bf16", shared=True, d=256, E=8, k=2, F=192, T=11, pad="some", bias=True, residual=True),
+    dict(act="bf16", wt="int8", shared=False, d=128, E=8, k=3, F=192, T=21, pad="none", bias=False, residual=False),
+    dict(act="bf16", wt="bf16", shared=False, d=768, E=8, k=2, F=1408, T=8, pad="none", bias=False, residual=False),  # the decode workload of the benchmark
+    dict(act="bf16", wt="bf16", shared=False, d=128, E=8, k=4, F=64, T=32, pad="none", bias=False, residual=True),   # 128 slots, full tiles
+    dict(act="bf16", wt="bf16", shared=False, d=128, E=4, k=2, F=192, T=6, pad="all", bias=False, residual=True),   # no workgroup writes a row
+    dict(act="bf16", wt="bf16", shared=True, d=128, E=4, k=2, F=192, T=6, pad="all", bias=False, residual=False),   # only the shared expert does
+    dict(act="bf16", wt="bf16", shared=True, d=64, E=2, k=1, F=64, T=5, pad="some", bias=True, residual=False,
+         shared_d_ff=192),                                                                                         # a shared expert wider than the routed ones
+    dict(act="bf16", wt="bf16", shared=False, d=64, E=16, k=4, F=64, T=8, pad="none", bias=True, residual=False,
+         lopsided=True),                                                                                           # most experts without a row
+]
+
+
+@pytest.mark.parametrize("case", BY_EXPERT_CASES,
+                         ids=lambda c: "{wt}_d{d}_E{E}_k{k}_F{F}_T{T}_pad-{pad}".format(**c))
+def test_down_launch_by_expert_gives_the_bits_of_the_tile_table_launch(device, env, case):
+    """Behind the launch that routes beside the gate/up products, the down launch has one row of workgroups per
+    expert (weights requested at once, the expert's rows read off its token bits behind them, the combine's
+    positions and gates fetched early): routing tables, losses and outputs are those of the launch that walks the
+    tile table, in every bit - three calls in a row, the last one with fewer tokens."""
+    T, k, E, d = case["T"], case["k"], case["E"], case["d"]
+    t = synth.make(small_workload(d=d, E=E, k=k, F=case["F"], T=T, seed=59, act=case["act"], wt=case["wt"],
+                                  shared=case["shared"], shared_d_ff=case.get("shared_d_ff", 128)))
+    valid = {"none": None, "some": (np.arange(T) % 4 != 2).astype(np.uint8), "all": np.zeros(T, np.uint8)}[case["pad"]]
+    bias = synth.normal((E,), 0.5, 59, 98) if case["bias"] else None
+    if case.get("lopsided"):
+        bias = np.where(np.arange(E) < 5, 30.0, -30.0).astype(np.float32)
+    residual = synth.round_bf16(synth.normal((T, d), 1.0, 59, 7)) if case["residual"] else None
+    layout = rb.Layout(valid=None if valid is None else [bool(v) for v in valid])
+    T2 = max(1, T // 2)
+    while T2 * k < 2 * E and T2 < T:   # the shorter call takes the same kernels
+        T2 += 1
+    layout2 = rb.Layout(valid=None if valid is None else [bool(v) for v in valid[:T2]])
+    got = {}
+    for by_expert in (True, False):
+        if by_expert:
+            env.pop("RBMOE_NO_DECODE_DOWN_BY_EXPERT", None)
+        else:
+            env["RBMOE_NO_DECODE_DOWN_BY_EXPERT"] = "1"
+        layer = gpu_layer(device, t)
+        a, ca = layer.forward_train(t.x, layout, router_bias=bias, residual=residual)
+        assert layer.kernel_name().startswith("mfma_bf16_decode_front")
+        b, _ = layer.forward_train(t.x, layout, router_bias=bias, residual=residual)
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+        c, cc = layer.forward_train(t.x[:T2], layout2, router_bias=bias, residual=None if residual is None else residual[:T2])
+        got[by_expert] = (a, ca, c, cc)
+        layer.close()
+    for i in (0, 2):
+        assert np.array_equal(got[True][i].view(np.uint32), got[False][i].view(np.uint32)), "outputs"
+    for i in (1, 3):
+        cw, cp = got[True][i], got[False][i]
+        for f in ("expert_of", "counts", "offsets", "perm_slot", "perm_token"):
+            assert np.array_equal(getattr(cw, f), getattr(cp, f)), f
+        assert np.array_equal(cw.gate_of.view(np.uint32), cp.gate_of.view(np.uint32))
+        assert cw.aux_loss() == cp.aux_loss() and cw.z_loss() == cp.z_loss()
+    ref = oracle_layer(t).forward(t.x, valid=valid, router_bias=bias, threads=4)
+    assert_routing_identical(got[True][1], ref)
+    if case.get("lopsided"):
+        assert int((ref.counts > 0).sum()) <= 5
+    want = ref.out if residual is None else ref.out + residual
+    assert rel_l2(got[True][0], want) <= 2e-2 if np.any(want) else not np.any(got[True][0])
