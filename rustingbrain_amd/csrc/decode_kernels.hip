@@ -434,6 +434,36 @@ __device__ __forceinline__ void route_small_body(
                 __builtin_amdgcn_wave_barrier();
                 for (int e = tid; e < E; e += 64) expert_tokens[e] = (unsigned int)off[e];
             }
+            if (E <= 64) {
+                // the loop keeps everything in registers - slot `tid` its position, lane e expert e's count, first
+                // position and first tile - and every store follows it, side by side
+                int pos = -1, e_cnt = 0, e_off = 0, e_tile0 = 0;
+                for (int e = 0; e < E; ++e) {
+                    const unsigned long long mask = __ballot(my == e);
+                    const int c = __popcll(mask);
+                    pos = my == e ? run + __popcll(mask & ((1ull << tid) - 1ull)) : pos;
+                    e_cnt = tid == e ? c : e_cnt;
+                    e_off = tid == e ? run : e_off;
+                    e_tile0 = tid == e ? tiles : e_tile0;
+                    run += c;
+                    tiles += c <= tile_m ? (c > 0 ? 1 : 0) : (c + tile_m - 1) / tile_m;
+                }
+                if (my >= 0) {
+                    perm_slot[pos] = tid;
+                    perm_token[pos] = tid / k;
+                    inv_pos[tid] = pos;
+                }
+                if (tid < E) {
+                    cnt[tid] = e_cnt;
+                    counts[tid] = e_cnt;
+                    offsets[tid] = e_off;
+                    for (int r0 = 0, ti = e_tile0; r0 < e_cnt; r0 += tile_m, ++ti) {
+                        tile_expert[ti] = tid;
+                        tile_row0[ti] = e_off + r0;
+                        tile_rows[ti] = min(tile_m, e_cnt - r0);
+                    }
+                }
+            } else
             for (int e = 0; e < E; ++e) {
                 const unsigned long long mask = __ballot(my == e);
                 const int c = __popcll(mask);
