@@ -216,26 +216,32 @@ __device__ __forceinline__ void route_small_body(
         const int nw = E * wp, nx = T * xp;
         const uint4* wsrc = reinterpret_cast<const uint4*>(wr);
         const uint4* xsrc = reinterpret_cast<const uint4*>(x);
-        // eight pieces a thread are requested before the first is stored: 64 KB a round trip (C2's 36 KB: one)
-        constexpr int kPieces = 8;
-        for (int i0 = 0; i0 < nw + nx; i0 += kPieces * kSmallThreads) {
-            uint4 v[kPieces];
-#pragma unroll
-            for (int u = 0; u < kPieces; ++u) {
-                const int i = min(i0 + u * kSmallThreads + tid, nw + nx - 1);
-                v[u] = i < nw ? wsrc[i] : xsrc[i - nw];
+        // One load a piece from a chosen address (not a chosen one of two loads: loads under a branch stay in front
+        // of their own stores, and the round trips follow one another), into variables of their own (an array of
+        // pieces ends up in scratch memory).
+        auto fetch = [&](int i) -> uint4 {
+            i = min(i, nw + nx - 1);
+            const uint4* const from = i < nw ? wsrc + i : xsrc + (i - nw);
+            return *from;
+        };
+        auto put = [&](int i, const uint4& v) {
+            if (i < nw) {
+                const int r = i / wp, c = i - r * wp;
+                *reinterpret_cast<uint4*>(ws + (size_t)r * ds + 4 * c) = v;
+            } else if (i < nw + nx) {
+                const int r = (i - nw) / xp, c = (i - nw) - r * xp;
+                *reinterpret_cast<uint4*>(reinterpret_cast<char*>(xs + (size_t)r * ds) + 16 * c) = v;
             }
-#pragma unroll
-            for (int u = 0; u < kPieces; ++u) {
-                const int i = i0 + u * kSmallThreads + tid;
-                if (i < nw) {
-                    const int r = i / wp, c = i - r * wp;
-                    *reinterpret_cast<uint4*>(ws + (size_t)r * ds + 4 * c) = v[u];
-                } else if (i < nw + nx) {
-                    const int r = (i - nw) / xp, c = (i - nw) - r * xp;
-                    *reinterpret_cast<uint4*>(reinterpret_cast<char*>(xs + (size_t)r * ds) + 16 * c) = v[u];
-                }
-            }
+        };
+        // eight pieces a thread are requested before the first is stored: 64 KB a round trip (36 KB for 8 tokens,
+        // 8 experts and 768 columns: one)
+        constexpr int NT = kSmallThreads;
+        for (int i = tid; i < nw + nx; i += 8 * NT) {
+            const uint4 v0 = fetch(i), v1 = fetch(i + NT), v2 = fetch(i + 2 * NT), v3 = fetch(i + 3 * NT);
+            const uint4 v4 = fetch(i + 4 * NT), v5 = fetch(i + 5 * NT), v6 = fetch(i + 6 * NT), v7 = fetch(i + 7 * NT);
+            __builtin_amdgcn_sched_barrier(0);
+            put(i, v0); put(i + NT, v1); put(i + 2 * NT, v2); put(i + 3 * NT, v3);
+            put(i + 4 * NT, v4); put(i + 5 * NT, v5); put(i + 6 * NT, v6); put(i + 7 * NT, v7);
         }
         __syncthreads();
         if (norm_w != nullptr) {

@@ -524,29 +524,35 @@ __global__ __launch_bounds__(FT, 2) void weight_grad_f32_kernel(
     const int pc = tid & 31, tr = tid >> 5;
     const float* const a_src = a + (size_t)row0 * M + (m0 + 4 * pc < M ? m0 + 4 * pc : 0);
     const float* const b_src = b + (size_t)row0 * N + (n0 + 4 * pc < N ? n0 + 4 * pc : 0);
+    // (three sets of registers by name: an array of sets is placed in scratch memory)
     struct Set {
-        float4 a[2], b[2];
-    } sets[GDEPTH];
+        float4 a0, a1, b0, b1;
+    } set0, set1, set2;
+    static_assert(GDEPTH == 3, "one named set per stage in flight");
     auto fetch = [&](auto kc, int r0) {
         constexpr int k = decltype(kc)::value;
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int r = min(r0 + tr + 8 * i, rows - 1);
-            sets[k].a[i] = *reinterpret_cast<const float4*>(a_src + (size_t)r * M);
-            sets[k].b[i] = *reinterpret_cast<const float4*>(b_src + (size_t)r * N);
-        }
+        Set& st = k == 0 ? set0 : k == 1 ? set1 : set2;
+        const int ra = min(r0 + tr, rows - 1), rb = min(r0 + tr + 8, rows - 1);
+        st.a0 = *reinterpret_cast<const float4*>(a_src + (size_t)ra * M);
+        st.b0 = *reinterpret_cast<const float4*>(b_src + (size_t)ra * N);
+        st.a1 = *reinterpret_cast<const float4*>(a_src + (size_t)rb * M);
+        st.b1 = *reinterpret_cast<const float4*>(b_src + (size_t)rb * N);
     };
     auto stage = [&](auto kc, int buf, int r0) {
         constexpr int k = decltype(kc)::value;
+        const Set& st = k == 0 ? set0 : k == 1 ? set1 : set2;
         float* const A = lds + buf * FSTAGE;
         float* const B = A + FR * FP;
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const bool in = r0 + tr + 8 * i < rows;
-            const float4 z = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-            *reinterpret_cast<float4*>(A + (tr + 8 * i) * FP + pc * 4) = in ? sets[k].a[i] : z;
-            *reinterpret_cast<float4*>(B + (tr + 8 * i) * FP + pc * 4) = in ? sets[k].b[i] : z;
-        }
+        // (rows past the chunk's end are zeros; a choice between two named float4 would be a choice between their
+        // addresses, and the sets would live in scratch memory)
+        const float in0 = r0 + tr < rows ? 1.0f : 0.0f, in1 = r0 + tr + 8 < rows ? 1.0f : 0.0f;
+        auto keep = [](const float4& v, float on) {
+            return make_float4(on != 0.0f ? v.x : 0.0f, on != 0.0f ? v.y : 0.0f, on != 0.0f ? v.z : 0.0f, on != 0.0f ? v.w : 0.0f);
+        };
+        *reinterpret_cast<float4*>(A + tr * FP + pc * 4) = keep(st.a0, in0);
+        *reinterpret_cast<float4*>(B + tr * FP + pc * 4) = keep(st.b0, in0);
+        *reinterpret_cast<float4*>(A + (tr + 8) * FP + pc * 4) = keep(st.a1, in1);
+        *reinterpret_cast<float4*>(B + (tr + 8) * FP + pc * 4) = keep(st.b1, in1);
     };
 
     floatx16 acc[2][2];
