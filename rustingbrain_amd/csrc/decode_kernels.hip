@@ -719,85 +719,6 @@ __device__ __forceinline__ void decode_combine_block(const DecodeGemmArgs& g, in
     }
 }
 
-template <bool SWIGLU, bool I8, int NW>
-__global__ __launch_bounds__(NW * 64) void decode_gemm_kernel(DecodeGemmArgs g) {
-    __shared__ float red[NW * (SWIGLU ? 2 : 1) * 16 * 64];
-    __shared__ int last_of_block;
-    const int fb = blockIdx.x;
-    const int ty = blockIdx.y;
-    DecodeSide sd;
-    sd.a_row0 = 0;
-    sd.out_row0 = 0;
-    // One round trip for the whole tile table: the four entries are fetched side by side (a stale entry past
-    // *ntiles is read and dropped), not one after the other - with cold caches every dependent scalar load in
-    // front of the first weight load is a few hundred nanoseconds of a launch that lasts ten microseconds.
-    const bool routed = ty < g.max_tiles;
-    const int tix = routed ? ty : 0;
-    const int live_tiles = *g.ntiles;
-    const int t_expert = g.tile_expert[tix], t_row0 = g.tile_row0[tix], t_rows = g.tile_rows[tix];
-    asm volatile("" ::"s"(live_tiles), "s"(t_expert), "s"(t_row0), "s"(t_rows));  // all four here, not sunk into the branches
-    // workgroups that write rows of this feature block's columns: the live routed tiles and the shared expert's
-    const int writers = live_tiles + (g.a_shared ? (g.T_shared + 31) / 32 : 0);
-    bool works = true;
-    if (routed) {
-        if (ty >= live_tiles) works = false;
-        const int expert = t_expert;
-        sd.a = static_cast<const bf16_t*>(g.a);
-        sd.row_index = g.row_index;
-        sd.w = static_cast<const char*>(g.w) + (size_t)expert * g.w_expert_stride * (I8 ? 1 : 2);
-        sd.scales = I8 ? g.scales + (size_t)expert * g.s_expert_stride : nullptr;
-        sd.out = static_cast<bf16_t*>(g.out);
-        sd.N = g.N;
-        sd.K = g.K;
-        sd.row0 = t_row0;
-        sd.rows = t_rows;
-        sd.a_row0 = expert * g.a_expert_rows;
-    } else {
-        const int st = ty - g.max_tiles;
-        sd.a = static_cast<const bf16_t*>(g.a_shared);
-        sd.row_index = nullptr;
-        sd.w = static_cast<const char*>(g.w_shared);
-        sd.scales = I8 ? g.scales_shared : nullptr;
-        sd.out = static_cast<bf16_t*>(g.out_shared);
-        sd.N = g.N_shared;
-        sd.K = g.K_shared;
-        sd.row0 = st * 32;
-        sd.rows = min(32, g.T_shared - sd.row0);
-    }
-    if (fb * 32 >= sd.N) return;
-    if constexpr (!SWIGLU) {
-        if (g.cmb_out != nullptr) {  // uniform over the launch
-            if (!works) {
-                // nothing to multiply here; with no writer at all (every row is padding and there is no shared
-                // expert) the first of these workgroups still owes the block its combine
-                if (writers != 0 || ty != 0) return;
-            } else {
-                sd.coherent_out = true;
-                decode_gemm_body<SWIGLU, I8, NW, kBatch>(sd, fb, red);
-                // every wave waits until its row stores have been acknowledged (they are device-scope stores: they
-                // go through to memory) before the workgroup's arrival is counted behind the barrier - a barrier
-                // alone does not wait for stores.  No device-scope fence: that would write back this XCD's whole
-                // L2, once per workgroup.
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                __syncthreads();
-                if (threadIdx.x == 0) {
-                    const int before = atomicAdd(&g.cmb_counter[fb], 1);
-                    last_of_block = before == writers - 1;
-                    if (before == writers - 1) atomicExch(&g.cmb_counter[fb], 0);  // every writer has arrived: ready for the next launch
-                }
-                __syncthreads();
-                if (!last_of_block) return;
-                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-            }
-            if (g.cmb_f32) decode_combine_block<float>(g, fb, NW * 64);
-            else decode_combine_block<bf16_t>(g, fb, NW * 64);
-            return;
-        }
-    }
-    if (!works) return;
-    decode_gemm_body<SWIGLU, I8, NW, kBatch>(sd, fb, red);
-}
-
 // What a thread of the folded combine can fetch before its workgroup has multiplied anything: the positions of its
 // token's expert rows in ascending order with their gates (at most four slots a token), and the residual.
 constexpr int kCombineEarlySlots = 4;
@@ -879,6 +800,94 @@ __device__ __forceinline__ void decode_combine_block_early(const DecodeGemmArgs&
     XT* const out = static_cast<XT*>(g.cmb_out);
     out[(size_t)t * d + c] = from_f32<XT>(a0);
     out[(size_t)t * d + c + 1] = from_f32<XT>(a1);
+}
+
+template <bool SWIGLU, bool I8, int NW>
+__global__ __launch_bounds__(NW * 64) void decode_gemm_kernel(DecodeGemmArgs g) {
+    __shared__ float red[NW * (SWIGLU ? 2 : 1) * 16 * 64];
+    __shared__ int last_of_block;
+    const int fb = blockIdx.x;
+    const int ty = blockIdx.y;
+    DecodeSide sd;
+    sd.a_row0 = 0;
+    sd.out_row0 = 0;
+    // One round trip for the whole tile table: the four entries are fetched side by side (a stale entry past
+    // *ntiles is read and dropped), not one after the other - with cold caches every dependent scalar load in
+    // front of the first weight load is a few hundred nanoseconds of a launch that lasts ten microseconds.
+    const bool routed = ty < g.max_tiles;
+    const int tix = routed ? ty : 0;
+    const int live_tiles = *g.ntiles;
+    const int t_expert = g.tile_expert[tix], t_row0 = g.tile_row0[tix], t_rows = g.tile_rows[tix];
+    asm volatile("" ::"s"(live_tiles), "s"(t_expert), "s"(t_row0), "s"(t_rows));  // all four here, not sunk into the branches
+    // workgroups that write rows of this feature block's columns: the live routed tiles and the shared expert's
+    const int writers = live_tiles + (g.a_shared ? (g.T_shared + 31) / 32 : 0);
+    bool works = true;
+    if (routed) {
+        if (ty >= live_tiles) works = false;
+        const int expert = t_expert;
+        sd.a = static_cast<const bf16_t*>(g.a);
+        sd.row_index = g.row_index;
+        sd.w = static_cast<const char*>(g.w) + (size_t)expert * g.w_expert_stride * (I8 ? 1 : 2);
+        sd.scales = I8 ? g.scales + (size_t)expert * g.s_expert_stride : nullptr;
+        sd.out = static_cast<bf16_t*>(g.out);
+        sd.N = g.N;
+        sd.K = g.K;
+        sd.row0 = t_row0;
+        sd.rows = t_rows;
+        sd.a_row0 = expert * g.a_expert_rows;
+    } else {
+        const int st = ty - g.max_tiles;
+        sd.a = static_cast<const bf16_t*>(g.a_shared);
+        sd.row_index = nullptr;
+        sd.w = static_cast<const char*>(g.w_shared);
+        sd.scales = I8 ? g.scales_shared : nullptr;
+        sd.out = static_cast<bf16_t*>(g.out_shared);
+        sd.N = g.N_shared;
+        sd.K = g.K_shared;
+        sd.row0 = st * 32;
+        sd.rows = min(32, g.T_shared - sd.row0);
+    }
+    if (fb * 32 >= sd.N) return;
+    if constexpr (!SWIGLU) {
+        if (g.cmb_out != nullptr) {  // uniform over the launch
+            // eight waves and at most four slots a token: what the combine needs of the routing is fetched now
+            const bool early = NW == 8 && g.cmb_k <= kCombineEarlySlots;
+            CombineEarly ce;
+            if (early) decode_combine_fetch(g, fb, ce);
+            if (!works) {
+                // nothing to multiply here; with no writer at all (every row is padding and there is no shared
+                // expert) the first of these workgroups still owes the block its combine
+                if (writers != 0 || ty != 0) return;
+            } else {
+                sd.coherent_out = true;
+                decode_gemm_body<SWIGLU, I8, NW, kBatch>(sd, fb, red);
+                // every wave waits until its row stores have been acknowledged (they are device-scope stores: they
+                // go through to memory) before the workgroup's arrival is counted behind the barrier - a barrier
+                // alone does not wait for stores.  No device-scope fence: that would write back this XCD's whole
+                // L2, once per workgroup.
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                if (threadIdx.x == 0) {
+                    const int before = atomicAdd(&g.cmb_counter[fb], 1);
+                    last_of_block = before == writers - 1;
+                    if (before == writers - 1) atomicExch(&g.cmb_counter[fb], 0);  // every writer has arrived: ready for the next launch
+                }
+                __syncthreads();
+                if (!last_of_block) return;
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+            }
+            if (early) {
+                if (g.cmb_f32) decode_combine_block_early<float>(g, fb, ce);
+                else decode_combine_block_early<bf16_t>(g, fb, ce);
+            } else {
+                if (g.cmb_f32) decode_combine_block<float>(g, fb, NW * 64);
+                else decode_combine_block<bf16_t>(g, fb, NW * 64);
+            }
+            return;
+        }
+    }
+    if (!works) return;
+    decode_gemm_body<SWIGLU, I8, NW, kBatch>(sd, fb, red);
 }
 
 // ---------------------------------------------------------------------------

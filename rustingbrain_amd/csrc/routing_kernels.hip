@@ -1265,23 +1265,32 @@ __global__ __launch_bounds__(256) void combine_vec_kernel(
         pos[r] = 0x7fffffff;
         gate[r] = 0.0f;
     }
+    // (all positions and gates are requested before the first is looked at, from addresses that do not depend on
+    // one another - a slot past k repeats the last one: loads under a branch would follow one another, two trips to
+    // memory a slot in front of the rows')
+    int p_in[KMAX];
+    float g_in[KMAX];
 #pragma unroll
     for (int r = 0; r < KMAX; ++r) {
-        if (r < k) {
-            int p = inv_pos[(size_t)t * k + r];
-            float g = gate_of[(size_t)t * k + r];
-            if (p >= 0) {
-                ++n;
+        const int rr = r < k ? r : k - 1;
+        p_in[r] = inv_pos[(size_t)t * k + rr];
+        g_in[r] = gate_of[(size_t)t * k + rr];
+    }
 #pragma unroll
-                for (int q = 0; q < KMAX; ++q) {
-                    if (p < pos[q]) {
-                        const int tp = pos[q];
-                        const float tg = gate[q];
-                        pos[q] = p;
-                        gate[q] = g;
-                        p = tp;
-                        g = tg;
-                    }
+    for (int r = 0; r < KMAX; ++r) {
+        int p = p_in[r];
+        float g = g_in[r];
+        if (r < k && p >= 0) {
+            ++n;
+#pragma unroll
+            for (int q = 0; q < KMAX; ++q) {
+                if (p < pos[q]) {
+                    const int tp = pos[q];
+                    const float tg = gate[q];
+                    pos[q] = p;
+                    gate[q] = g;
+                    p = tp;
+                    g = tg;
                 }
             }
         }
