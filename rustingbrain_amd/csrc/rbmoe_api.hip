@@ -113,7 +113,7 @@ struct rbmoe_ctx {
     // The backward pass runs the router's branch beside the weight gradients: a second stream (default
     // priority, like the first) forked from and joined to `stream` with two events.  Created on first use.
     hipStream_t side_stream = nullptr;
-    hipEvent_t ev_fork = nullptr, ev_fork2 = nullptr, ev_join = nullptr;
+    hipEvent_t ev_fork = nullptr, ev_fork2 = nullptr, ev_join = nullptr, ev_tables = nullptr;
     size_t budget_bytes = 0;
     size_t allocated = 0;
     void* static_scratch = nullptr;  // this device's copy of rbmoe_static_scratch (RBMOE_STATIC_SCRATCH_BYTES)
@@ -469,6 +469,7 @@ static void ctx_release(rbmoe_ctx* ctx) {
     if (ctx->ev_fork) (void)hipEventDestroy(ctx->ev_fork);
     if (ctx->ev_fork2) (void)hipEventDestroy(ctx->ev_fork2);
     if (ctx->ev_join) (void)hipEventDestroy(ctx->ev_join);
+    if (ctx->ev_tables) (void)hipEventDestroy(ctx->ev_tables);
     if (ctx->own_stream) {
         (void)hipStreamSynchronize(ctx->own_stream);
         (void)hipStreamDestroy(ctx->own_stream);
@@ -808,11 +809,11 @@ namespace {
 int ensure_side_stream(rbmoe_ctx* ctx) {
     if (ctx->side_stream) return RBMOE_OK;
     HIP_TRY(ctx, hipSetDevice(ctx->device));
-    // all four or none: a stream without its events would be used as if it were complete
+    // all five or none: a stream without its events would be used as if it were complete
     hipStream_t st = nullptr;
-    hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
+    hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr};
     hipError_t e = hipStreamCreateWithFlags(&st, hipStreamNonBlocking);
-    for (int i = 0; i < 3 && e == hipSuccess; ++i) e = hipEventCreateWithFlags(&ev[i], hipEventDisableTiming);
+    for (int i = 0; i < 4 && e == hipSuccess; ++i) e = hipEventCreateWithFlags(&ev[i], hipEventDisableTiming);
     if (e != hipSuccess) {
         for (hipEvent_t x : ev)
             if (x) (void)hipEventDestroy(x);
@@ -823,7 +824,14 @@ int ensure_side_stream(rbmoe_ctx* ctx) {
     ctx->ev_fork = ev[0];
     ctx->ev_fork2 = ev[1];
     ctx->ev_join = ev[2];
+    ctx->ev_tables = ev[3];
     return RBMOE_OK;
+}
+
+// ints of one chunk table of a training layer's weight-gradient launches (the largest of them)
+static size_t wgrad_table_ints(const rbmoe_layer* L) {
+    const int E = L->cfg.num_experts;
+    return (size_t)std::max(weight_grad_table_ints(E, L->max_S), weight_grad_table_ints(1, L->max_T));
 }
 
 Work work_of_layer(const rbmoe_layer* L) {
@@ -1563,7 +1571,8 @@ int rbmoe_layer_enable_training(rbmoe_layer* L) {
     p.add(&L->g_down, E * d * F * 4);
     p.add(&L->wdT, E * F * d * ws);
     p.add(&L->wguT, E * d * 2 * F * ws);
-    p.add(&L->wg_chunks, (size_t)std::max(weight_grad_table_ints((int)E, (int)S), weight_grad_table_ints(1, (int)T)) * 4);
+    // (four tables: down and gate/up gradients of the routed experts and of the shared one)
+    p.add(&L->wg_chunks, (size_t)4 * wgrad_table_ints(L) * 4);
     // How the weight gradients treat an expert far above the average share (and the shared expert, whose one
     // group of rows is always cut): in a fixed order by default (RBMOE_OPT_WGRAD_MODE for f32 atomics or no cut).
     if (L->wgrad_split == WgradSplit::Ordered) {
@@ -1718,9 +1727,32 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, int32_t tokens, int3
         HIP_TRY(ctx, hipEventRecord(ctx->ev_fork, s));
         HIP_TRY(ctx, hipStreamWaitEvent(rs, ctx->ev_fork, 0));
     }
+    // grad_input = sum over a token's slots of its expert rows + shared + router
+    CombineArgs ca{L->dxg.p, c.shared_expert ? L->dxs.p : nullptr, L->dxr.p, (const int*)L->inv_pos.p,
+                   (const float*)L->ones.p, T, d, k, grad_input};
+    ca.rows_bf16 = cast;
+    const bool combine_on_side = side && !c.shared_expert;
+    const bool tables_early = side && !L->wgrad_generic;
     // From here to the join the side stream hangs off the main one: an error in between must not leave it forked
     // (a stream capture in progress could then never end), so the rest runs as one unit that is always joined.
     auto forked = [&]() -> int {
+    if (tables_early) {
+        // the chunk tables of the weight-gradient launches depend on nothing but the forward's counts and offsets:
+        // they are worked out here, on the side stream, instead of in front of each product on the main one
+        auto table = [&](int which, int M, int N, int groups, int dense_rows, int total_rows) -> hipError_t {
+            if (!weight_grad_shape_ok(M, N, abf)) return hipSuccess;
+            return launch_weight_grad(nullptr, M, nullptr, N, counts, offsets, groups, dense_rows, total_rows, L->wgrad_split,
+                                      L->grads_clear, (int*)L->wg_chunks.p + (size_t)which * wgrad_table_ints(L),
+                                      (float*)L->wg_partial.p, L->wg_partial.bytes, nullptr, 0, abf, rs, WgradPart::TableOnly);
+        };
+        HIP_TRY(ctx, table(0, d, F, E, -1, S));
+        HIP_TRY(ctx, table(1, 2 * F, d, E, -1, S));
+        if (c.shared_expert) {
+            HIP_TRY(ctx, table(2, d, Fs, 1, T, T));
+            HIP_TRY(ctx, table(3, 2 * Fs, d, 1, T, T));
+        }
+        HIP_TRY(ctx, hipEventRecord(ctx->ev_tables, rs));
+    }
     HIP_TRY(ctx, launch_route_backward((const float*)L->P.p, (const float*)L->lse.p, (const int*)L->expert_of.p,
                                        (const float*)L->grad_gates.p, counts, offsets, T, E, k, c.aux_loss_weight,
                                        c.router_z_loss_weight, (float*)L->dlogits.p, rs));
@@ -1757,25 +1789,30 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, int32_t tokens, int3
         HIP_TRY(ctx, hipEventRecord(ctx->ev_fork2, s));
         HIP_TRY(ctx, hipStreamWaitEvent(rs, ctx->ev_fork2, 0));
         HIP_TRY(ctx, prod_on(gx, rs));
+        // without a shared expert everything the final sum reads is written on the side stream: it runs there too,
+        // beside the weight gradients
+        if (combine_on_side) HIP_TRY(ctx, launch_combine(ca, xbf, rs));
         HIP_TRY(ctx, hipEventRecord(ctx->ev_join, rs));
     } else {
         HIP_TRY(ctx, prod(gx));
     }
     // weight gradients (src/param.rs:819-821): down += dY^T . H; (gate | up) += (dG | dU)^T . X[token]
-    auto wgrad = [&](const void* a, int M, const void* b, const int* b_rows, int N, int groups, int dense_rows,
-                     int total_rows, float* out, size_t stride) -> hipError_t {
+    auto wgrad = [&](int table, const void* a, int M, const void* b, const int* b_rows, int N, int groups,
+                     int dense_rows, int total_rows, float* out, size_t stride) -> hipError_t {
         if (!L->wgrad_generic && !b_rows && weight_grad_shape_ok(M, N, abf))
             return launch_weight_grad(a, M, b, N, counts, offsets, groups, dense_rows, total_rows,
-                                      L->wgrad_split, L->grads_clear, (int*)L->wg_chunks.p, (float*)L->wg_partial.p,
-                                      L->wg_partial.bytes, out, stride, abf, s);
+                                      L->wgrad_split, L->grads_clear, (int*)L->wg_chunks.p + (size_t)table * wgrad_table_ints(L),
+                                      (float*)L->wg_partial.p, L->wg_partial.bytes, out, stride, abf, s,
+                                      tables_early ? WgradPart::ProductOnly : WgradPart::Both);
         if (L->grads_clear) {
             const hipError_t e = launch_fill_f32(out, 0.0f, (long long)((size_t)groups * (stride ? stride : (size_t)M * N)), s);
             if (e != hipSuccess) return e;
         }
         return launch_grouped_tn(a, M, b, b_rows, N, counts, offsets, groups, dense_rows, out, stride, abf, s);
     };
-    HIP_TRY(ctx, wgrad(L->dy.p, d, L->h.p, nullptr, F, E, -1, S, (float*)L->g_down.p, (size_t)d * F));
-    HIP_TRY(ctx, wgrad(L->dgu.p, 2 * F, L->xg.p, nullptr, d, E, -1, S, (float*)L->g_gu.p, (size_t)2 * F * d));
+    if (tables_early) HIP_TRY(ctx, hipStreamWaitEvent(s, ctx->ev_tables, 0));
+    HIP_TRY(ctx, wgrad(0, L->dy.p, d, L->h.p, nullptr, F, E, -1, S, (float*)L->g_down.p, (size_t)d * F));
+    HIP_TRY(ctx, wgrad(1, L->dgu.p, 2 * F, L->xg.p, nullptr, d, E, -1, S, (float*)L->g_gu.p, (size_t)2 * F * d));
     // shared expert over every row (src/moe.rs:356-361)
     if (c.shared_expert) {
         GroupedArgs sh = g;
@@ -1787,8 +1824,8 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, int32_t tokens, int3
         sx.dense_rows = T; sx.w_expert_stride = 0;
         sx.a = L->dgus.p; sx.w = L->swguT.p; sx.N = d; sx.K = 2 * Fs; sx.out = L->dxs.p;
         HIP_TRY(ctx, prod(sx));
-        HIP_TRY(ctx, wgrad(gout, d, L->hs.p, nullptr, Fs, 1, T, T, (float*)L->g_sdown.p, 0));
-        HIP_TRY(ctx, wgrad(L->dgus.p, 2 * Fs, cast ? L->x16.p : L->xc.p, nullptr, d, 1, T, T, (float*)L->g_sgu.p, 0));
+        HIP_TRY(ctx, wgrad(2, gout, d, L->hs.p, nullptr, Fs, 1, T, T, (float*)L->g_sdown.p, 0));
+        HIP_TRY(ctx, wgrad(3, L->dgus.p, 2 * Fs, cast ? L->x16.p : L->xc.p, nullptr, d, 1, T, T, (float*)L->g_sgu.p, 0));
     }
     // grad_input = sum over a token's slots of its expert rows + shared + router
     if (side) HIP_TRY(ctx, hipStreamWaitEvent(s, ctx->ev_join, 0));
@@ -1802,10 +1839,7 @@ int rbmoe_backward(rbmoe_layer* L, const void* grad_output, int32_t tokens, int3
         }
         return rc;
     }
-    CombineArgs ca{L->dxg.p, c.shared_expert ? L->dxs.p : nullptr, L->dxr.p, (const int*)L->inv_pos.p,
-                   (const float*)L->ones.p, T, d, k, grad_input};
-    ca.rows_bf16 = cast;
-    HIP_TRY(ctx, launch_combine(ca, xbf, s));
+    if (!combine_on_side) HIP_TRY(ctx, launch_combine(ca, xbf, s));
     L->grads_clear = false;
     return RBMOE_OK;
 }

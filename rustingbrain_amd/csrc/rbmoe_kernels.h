@@ -207,10 +207,14 @@ size_t weight_grad_partial_bytes(int M, int N, int groups, int dense_rows, int t
 // ... for a buffer that serves every launch of 1 .. max_tokens tokens (rows_per_token rows each; dense: rows = tokens)
 size_t weight_grad_partial_bytes_upto(int M, int N, int groups, bool dense, int max_tokens, int rows_per_token,
                                       bool bf16);
+// `part`: the chunk table is a launch of its own in front of the product and depends on nothing but counts and
+// offsets - a caller may have it computed early, on another stream (TableOnly), and later issue the product with
+// the same arguments (ProductOnly) once that launch has completed.
+enum class WgradPart : int { Both = 0, TableOnly = 1, ProductOnly = 2 };
 hipError_t launch_weight_grad(const void* a, int M, const void* b, int N, const int* counts, const int* offsets,
                               int groups, int dense_rows, int total_rows, WgradSplit split_mode, bool overwrite,
                               int* chunks, float* partial, size_t partial_bytes, float* out, size_t out_expert_stride,
-                              bool bf16, hipStream_t s);
+                              bool bf16, hipStream_t s, WgradPart part = WgradPart::Both);
 
 // gates -> probabilities -> logits, with the gradients of the two auxiliary losses
 hipError_t launch_route_backward(const float* P, const float* lse, const int* expert_of, const float* grad_gates,

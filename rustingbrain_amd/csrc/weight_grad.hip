@@ -666,7 +666,7 @@ size_t weight_grad_partial_bytes_upto(int M, int N, int groups, bool dense, int 
 hipError_t launch_weight_grad(const void* a, int M, const void* b, int N, const int* counts, const int* offsets,
                               int groups, int dense_rows, int total_rows, WgradSplit split_mode, bool overwrite,
                               int* chunks, float* partial, size_t partial_bytes, float* out, size_t out_expert_stride,
-                              bool bf16, hipStream_t s) {
+                              bool bf16, hipStream_t s, WgradPart part) {
     if (groups <= 0 || total_rows <= 0) return hipSuccess;
     if (!weight_grad_shape_ok(M, N, bf16)) return hipErrorInvalidValue;
     if (bf16) {
@@ -705,9 +705,11 @@ hipError_t launch_weight_grad(const void* a, int M, const void* b, int N, const 
     // the other modes every expert with rows has a chunk that stores, and one without rows gets a chunk that
     // stores zeros.
     const bool clear_first = overwrite && split_mode == WgradSplit::Atomic;
-    hipLaunchKernelGGL(chunk_table_kernel, dim3(1), dim3(256), 0, s, counts, offsets, groups, dense_rows, limit,
-                       max_chunks, ordered ? 1 : 0, max_slots, (overwrite && !clear_first) ? 1 : 0, chunk_expert,
-                       chunk_row0, chunk_rows, chunk_split, nchunks, slot_first, slot_count);
+    if (part != WgradPart::ProductOnly)
+        hipLaunchKernelGGL(chunk_table_kernel, dim3(1), dim3(256), 0, s, counts, offsets, groups, dense_rows, limit,
+                           max_chunks, ordered ? 1 : 0, max_slots, (overwrite && !clear_first) ? 1 : 0, chunk_expert,
+                           chunk_row0, chunk_rows, chunk_split, nchunks, slot_first, slot_count);
+    if (part == WgradPart::TableOnly) return hipGetLastError();
     if (clear_first)
         hipLaunchKernelGGL(clear_other_experts_kernel, dim3(64, groups), dim3(256), 0, s, counts, dense_rows, limit,
                            ordered ? 1 : 0, out, out_expert_stride, (size_t)M * N);
