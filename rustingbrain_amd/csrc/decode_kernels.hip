@@ -868,9 +868,9 @@ __global__ __launch_bounds__(NW * 64) void decode_gemm_kernel(DecodeGemmArgs g) 
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 __syncthreads();
                 if (threadIdx.x == 0) {
-                    const int before = atomicAdd(&g.cmb_counter[fb], 1);
+                    const int before = atomicAdd(&g.cmb_counter[fb * kDecodeCombineCounterStride], 1);
                     last_of_block = before == writers - 1;
-                    if (before == writers - 1) atomicExch(&g.cmb_counter[fb], 0);  // every writer has arrived: ready for the next launch
+                    if (before == writers - 1) atomicExch(&g.cmb_counter[fb * kDecodeCombineCounterStride], 0);  // every writer has arrived: ready for the next launch
                 }
                 __syncthreads();
                 if (!last_of_block) return;
@@ -952,9 +952,9 @@ __global__ __launch_bounds__(512) void decode_down_by_expert_kernel(DecodeGemmAr
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the row stores have been acknowledged
         __syncthreads();
         if (threadIdx.x == 0) {
-            const int before = atomicAdd(&g.cmb_counter[fb], 1);
+            const int before = atomicAdd(&g.cmb_counter[fb * kDecodeCombineCounterStride], 1);
             last_of_block = before == writers - 1;
-            if (before == writers - 1) atomicExch(&g.cmb_counter[fb], 0);  // every writer has arrived: ready for the next launch
+            if (before == writers - 1) atomicExch(&g.cmb_counter[fb * kDecodeCombineCounterStride], 0);  // every writer has arrived: ready for the next launch
         }
         __syncthreads();
         if (!last_of_block) return;

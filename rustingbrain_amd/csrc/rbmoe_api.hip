@@ -350,7 +350,7 @@ Plan make_plan(rbmoe_layer* L) {
         p.add(&L->hall, E * std::min<size_t>(T, kSmallRouteMaxTokens) * F * 2);
         p.add(&L->etok, E * 4);
     }
-    p.add(&L->cmbcnt, (size_t)kDecodeCombineMaxBlocks * 4);
+    p.add(&L->cmbcnt, kDecodeCombineCounterBytes);
     p.add(&L->xg, S * d * as);
     p.add(&L->h, S * F * as);
     p.add(&L->y, S * d * as);
@@ -866,7 +866,7 @@ size_t carve_decode_work(const rbmoe_layer* L, int T, unsigned char* base, Work*
     Work v;
     // first, at the same place for every call and every layer: the arrival counters of the folded combine, which are
     // zero whenever no call is running (the array starts as zeros and every launch leaves them as it found them)
-    v.cmb_counter = (int*)take((size_t)kDecodeCombineMaxBlocks * 4);
+    v.cmb_counter = (int*)take(kDecodeCombineCounterBytes);
     v.P = (float*)take((size_t)T * E * 4); v.lse = (float*)take((size_t)T * 4);
     v.expert_of = (int*)take(S * 4); v.gate_of = (float*)take(S * 4);
     v.counts = (int*)take(E * 4); v.offsets = (int*)take((E + 1) * 4);

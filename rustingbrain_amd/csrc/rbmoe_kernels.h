@@ -308,7 +308,7 @@ struct DecodeGemmArgs {
     // again after it) sums that block's columns for every token - the token's expert rows in ascending expert order,
     // a rounded multiply by the gate and a rounded add each, then the shared expert's row, then the residual - and
     // writes them to cmb_out.  Nobody waits for anybody: whoever arrives last does the work.
-    int* cmb_counter = nullptr;           // [N / 32]
+    int* cmb_counter = nullptr;           // block b's counter at [b * kDecodeCombineCounterStride]
     const int* cmb_inv_pos = nullptr;     // [T * k]
     const float* cmb_gate_of = nullptr;   // [T * k]
     const void* cmb_residual = nullptr;   // [T, N] bf16, or f32 when cmb_f32, or null
@@ -317,6 +317,10 @@ struct DecodeGemmArgs {
     int cmb_f32 = 0;
 };
 constexpr int kDecodeCombineMaxBlocks = 1024;  // feature blocks a folded combine has counters for
+// ints between two blocks' counters: every block's arrivals go to a cache line - and an L2 channel - of their own
+// (side by side in one line, the atomics of a launch's two hundred workgroups queue up behind one another)
+constexpr int kDecodeCombineCounterStride = 64;
+constexpr size_t kDecodeCombineCounterBytes = (size_t)kDecodeCombineMaxBlocks * kDecodeCombineCounterStride * 4;
 bool decode_shape_ok(int N, int K);
 hipError_t launch_decode_gemm(const DecodeGemmArgs& g, WeightKind wk, hipStream_t s);
 // Routing and gate/up products in one launch (bf16 rows, no norm): every expert's gate/up product over all T rows,
