@@ -581,7 +581,10 @@ __device__ __forceinline__ V lds_load_ahead(const unsigned char* p) {
     return __builtin_bit_cast(V, raw);
 }
 
-template <typename XT, int NI>
+// WIDE (bf16 rows): the token rows are widened to f32 once, on their way into LDS, instead of by each of the 16
+// lanes that read an element (a shift or a mask per element and lane: a fifth of the kernel's vector
+// instructions); the staged slice then takes twice the LDS, so the launcher asks for it only where that fits.
+template <typename XT, int NI, bool WIDE>
 __global__ __launch_bounds__(kRouterThreads) void route_fused_kernel(
     const XT* __restrict__ x, const float* __restrict__ wr, const float* __restrict__ bias,
     const uint8_t* __restrict__ valid, int T, int d, int E, int k, int cols, float* __restrict__ P,
@@ -589,11 +592,13 @@ __global__ __launch_bounds__(kRouterThreads) void route_fused_kernel(
     int* __restrict__ rank_in_block, int* __restrict__ blockcnt, float* __restrict__ partial,
     bf16_t* __restrict__ rows16) {
     typedef typename XPiece<XT>::raw_t piece_t;
+    typedef typename std::conditional<WIDE, float, XT>::type ST;  // the element type of the staged token rows
+    typedef typename XPiece<ST>::raw_t spiece_t;
     extern __shared__ __align__(16) unsigned char lds_raw[];
     constexpr int TB = kRouterTokens;
     const int ES = E | 1;
     float* const prob = reinterpret_cast<float*>(lds_raw);
-    const int xpitch = cols * (int)sizeof(XT) + 16, wpitch = cols * 4 + 16;  // bytes; + 16: rows start in different banks
+    const int xpitch = cols * (int)sizeof(ST) + 16, wpitch = cols * 4 + 16;  // bytes; + 16: rows start in different banks
     unsigned char* const xs = lds_raw + router_fixed_bytes(E, k);
     unsigned char* const ws = xs + (size_t)TB * xpitch;
 
@@ -644,7 +649,15 @@ __global__ __launch_bounds__(kRouterThreads) void route_fused_kernel(
             const int idx = tid + u * kRouterThreads;
             if (idx < TB * np) {
                 const int r = idx / np, q = idx - r * np;
-                *reinterpret_cast<piece_t*>(xs + (size_t)r * xpitch + (size_t)q * sizeof(piece_t)) = pre_x[u];
+                if constexpr (WIDE && sizeof(XT) == 2) {
+                    float f[8];
+                    XPiece<XT>::widen(pre_x[u], f);
+                    float4* const to = reinterpret_cast<float4*>(xs + (size_t)r * xpitch + (size_t)q * sizeof(spiece_t));
+                    to[0] = make_float4(f[0], f[1], f[2], f[3]);
+                    to[1] = make_float4(f[4], f[5], f[6], f[7]);
+                } else {
+                    *reinterpret_cast<piece_t*>(xs + (size_t)r * xpitch + (size_t)q * sizeof(piece_t)) = pre_x[u];
+                }
                 if constexpr (sizeof(XT) == 4) {
                     if (rows16 != nullptr && r < nt) {  // the bf16 copy of f32 rows for the expert products (see logits_kernel)
                         float f[8];
@@ -684,11 +697,11 @@ __global__ __launch_bounds__(kRouterThreads) void route_fused_kernel(
 #pragma unroll
         for (int i = 0; i < NI; ++i) wrow[i] = ws + (size_t)min(2 * wave + half + 16 * i, E - 1) * wpitch;
         struct Operands {
-            piece_t x;
+            spiece_t x;
             float4 wa[NI], wb[NI];
         };
         auto read = [&](Operands& o, int q) {
-            o.x = lds_load_ahead<piece_t>(xrow + (size_t)q * sizeof(piece_t));
+            o.x = lds_load_ahead<spiece_t>(xrow + (size_t)q * sizeof(spiece_t));
 #pragma unroll
             for (int i = 0; i < NI; ++i) {
                 o.wa[i] = lds_load_ahead<float4>(wrow[i] + 32 * q);
@@ -698,7 +711,7 @@ __global__ __launch_bounds__(kRouterThreads) void route_fused_kernel(
         };
         auto multiply = [&](const Operands& o) {
             float xv[8];
-            XPiece<XT>::widen(o.x, xv);
+            XPiece<ST>::widen(o.x, xv);
 #pragma unroll
             for (int i = 0; i < NI; ++i) {
                 la[i][0] = __fadd_rn(la[i][0], __fmul_rn(xv[0], o.wa[i].x));
@@ -1385,16 +1398,27 @@ template <typename XT>
 static hipError_t launch_router_t(const RouterArgs& a, hipStream_t s) {
     const int nb = (a.T + kRouterTokens - 1) / kRouterTokens;
     if (const int cols = a.wq ? 0 : fused_cols(a, sizeof(XT))) {
-        const size_t lds = fused_lds_bytes(a.E, a.k, cols, sizeof(XT));
-        auto go = [&](auto ni) {
-            RB_LAUNCH((route_fused_kernel<XT, decltype(ni)::value>), dim3(nb), dim3(kRouterThreads), lds, s,
+        // bf16 rows staged as f32 where a slice of the same width then still fits
+        const bool wide = sizeof(XT) == 2 && fused_cols(a, 4) == cols;
+        const size_t lds = fused_lds_bytes(a.E, a.k, cols, wide ? 4 : sizeof(XT));
+        auto go = [&](auto ni, auto wide_tag) {
+            RB_LAUNCH((route_fused_kernel<XT, decltype(ni)::value, decltype(wide_tag)::value>), dim3(nb),
+                               dim3(kRouterThreads), lds, s,
                                static_cast<const XT*>(a.x), a.wr, a.bias, a.valid, a.T, a.d, a.E, a.k, cols, a.P, a.lse,
                                a.expert_of, a.gate_of, a.rank_in_block, a.blockcnt, a.partial,
                                static_cast<bf16_t*>(a.rows16));
         };
-        if (a.E <= 16) go(std::integral_constant<int, 1>{});
-        else if (a.E <= 32) go(std::integral_constant<int, 2>{});
-        else go(std::integral_constant<int, 4>{});
+        auto pick = [&](auto wide_tag) {
+            if (a.E <= 16) go(std::integral_constant<int, 1>{}, wide_tag);
+            else if (a.E <= 32) go(std::integral_constant<int, 2>{}, wide_tag);
+            else go(std::integral_constant<int, 4>{}, wide_tag);
+        };
+        if constexpr (sizeof(XT) == 2) {
+            if (wide) pick(std::true_type{});
+            else pick(std::false_type{});
+        } else {
+            pick(std::false_type{});
+        }
         return hipGetLastError();
     }
     static std::atomic<unsigned long long> attr_set{0};
