@@ -83,16 +83,38 @@ struct XPiece<float> {
 // `rows16` (f32 rows only, or null): a bf16 copy of the rows, rounded to nearest even, for the expert products of a
 // layer whose weights are bf16 or int8 - written on the way by the workgroups of the first group of experts, which
 // have every piece of their rows in hand anyway (widths that are multiples of 8).
-template <typename XT, int NE, bool AHEAD>
+// WIDE (bf16 rows): the rows are widened to f32 once, on their way into LDS, instead of by each of the NE waves
+// that read them (one of the three vector instructions per element); a slice is then half as many columns, so
+// that a workgroup takes no more LDS and as many of them fit a compute unit.
+template <typename XT, int NE, bool AHEAD, bool WIDE = false>
 __global__ __launch_bounds__(NE * 64, (!AHEAD && sizeof(XT) == 2) ? 6 : 2) void logits_kernel(const XT* __restrict__ x,
                                                                 const float* __restrict__ wr,
                                                                 const float* __restrict__ bias, int T, int d, int E,
                                                                 float* __restrict__ logits,
                                                                 bf16_t* __restrict__ rows16) {
+    static_assert(!WIDE || sizeof(XT) == 2, "only bf16 rows are widened");
     typedef typename XPiece<XT>::raw_t piece_t;
-    constexpr int PIECES = kLogitChunk / 8;  // pieces per row per slice
-    constexpr int STRIDE = PIECES + 1;       // one piece of padding per row
-    __shared__ piece_t xs[kLogitTokens * STRIDE];
+    typedef typename std::conditional<WIDE, float, XT>::type ST;  // the element type of the staged rows
+    typedef typename XPiece<ST>::raw_t spiece_t;
+    constexpr int kChunk = WIDE ? kLogitChunk / 2 : kLogitChunk;
+    constexpr int PIECES = kChunk / 8;  // pieces per row per slice
+    constexpr int ROWB = PIECES * (int)sizeof(spiece_t) + 16;  // bytes of a staged row: 16 of padding, so that the lanes' rows start in different banks
+    __shared__ __align__(16) unsigned char xs_raw[kLogitTokens * ROWB];
+    auto staged = [&](int r, int q) -> spiece_t* {
+        return reinterpret_cast<spiece_t*>(xs_raw + (size_t)r * ROWB + (size_t)q * sizeof(spiece_t));
+    };
+    auto put = [&](int r, int q, const piece_t& v) {
+        if constexpr (WIDE) {
+            float f[8];
+            XPiece<XT>::widen(v, f);
+            spiece_t o;
+            o.a = make_float4(f[0], f[1], f[2], f[3]);
+            o.b = make_float4(f[4], f[5], f[6], f[7]);
+            *staged(r, q) = o;
+        } else {
+            *staged(r, q) = v;
+        }
+    };
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -151,7 +173,7 @@ __global__ __launch_bounds__(NE * 64, (!AHEAD && sizeof(XT) == 2) ? 6 : 2) void 
         }
     };
     if (AHEAD && tail > 0) fetch(0);
-    for (int c0 = 0; c0 < tail; c0 += kLogitChunk) {
+    for (int c0 = 0; c0 < tail; c0 += kChunk) {
         const int np = min(PIECES, (tail - c0) / 8);  // pieces in this slice
         __syncthreads();
         if (AHEAD) {
@@ -159,16 +181,16 @@ __global__ __launch_bounds__(NE * 64, (!AHEAD && sizeof(XT) == 2) ? 6 : 2) void 
             for (int u = 0; u < MAXP; ++u) {
                 const int idx = tid + u * kLogitThreads;
                 const int r = idx / PIECES, q = idx % PIECES;
-                if (r < kLogitTokens && q < np) xs[r * STRIDE + q] = pre[u];
+                if (r < kLogitTokens && q < np) put(r, q, pre[u]);
             }
         } else {
             for (int idx = tid; idx < kLogitTokens * np; idx += kLogitThreads) {
                 const int r = idx / np, q = idx - r * np;
-                xs[r * STRIDE + q] = load_piece(r, c0 + 8 * q);
+                put(r, q, load_piece(r, c0 + 8 * q));
             }
         }
         __syncthreads();
-        if (AHEAD && c0 + kLogitChunk < tail) fetch(c0 + kLogitChunk);
+        if (AHEAD && c0 + kChunk < tail) fetch(c0 + kChunk);
         if (has) {
             const float* wa = w0 + c0;
             int q = 0;
@@ -177,20 +199,20 @@ __global__ __launch_bounds__(NE * 64, (!AHEAD && sizeof(XT) == 2) ? 6 : 2) void 
                 float wv[8 * kLogitBatch];
 #pragma unroll
                 for (int j = 0; j < 8 * kLogitBatch; ++j) wv[j] = wa[8 * q + j];
-                piece_t xp[kLogitBatch];
+                spiece_t xp[kLogitBatch];
 #pragma unroll
-                for (int b = 0; b < kLogitBatch; ++b) xp[b] = xs[lane * STRIDE + q + b];
+                for (int b = 0; b < kLogitBatch; ++b) xp[b] = *staged(lane, q + b);
 #pragma unroll
                 for (int b = 0; b < kLogitBatch; ++b) {
                     float xv[8];
-                    XPiece<XT>::widen(xp[b], xv);
+                    XPiece<ST>::widen(xp[b], xv);
 #pragma unroll
                     for (int l = 0; l < 8; ++l) la[l] = __fadd_rn(la[l], __fmul_rn(xv[l], wv[8 * b + l]));
                 }
             }
             for (; q < np; ++q) {
                 float xv[8];
-                XPiece<XT>::widen(xs[lane * STRIDE + q], xv);
+                XPiece<ST>::widen(*staged(lane, q), xv);
 #pragma unroll
                 for (int l = 0; l < 8; ++l) la[l] = __fadd_rn(la[l], __fmul_rn(xv[l], wa[8 * q + l]));
             }
@@ -1446,7 +1468,7 @@ static hipError_t launch_router_t(const RouterArgs& a, hipStream_t s) {
         RB_LAUNCH((logits_kernel<XT, NE, true>), lgrid, dim3(NE * 64), 0, s, static_cast<const XT*>(a.x),
                            a.wr, a.bias, a.T, a.d, a.E, a.P, static_cast<bf16_t*>(a.rows16));
     else
-        RB_LAUNCH((logits_kernel<XT, NE, false>), lgrid, dim3(NE * 64), 0, s, static_cast<const XT*>(a.x),
+        RB_LAUNCH((logits_kernel<XT, NE, false, sizeof(XT) == 2>), lgrid, dim3(NE * 64), 0, s, static_cast<const XT*>(a.x),
                            a.wr, a.bias, a.T, a.d, a.E, a.P, static_cast<bf16_t*>(a.rows16));
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
