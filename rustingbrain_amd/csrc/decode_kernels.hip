@@ -1,5 +1,5 @@
 // Decode-shaped forward (a few tokens): the layer is bound by streaming the touched experts'
-// weights once from HBM and by launch latency, so the work is cut into four launches
+// weights once from HBM and by launch latency.  The work is cut into four launches
 //
 //   route_small_kernel   one workgroup: logits, softmax, top-k, counting sort, tile table,
 //                        auxiliary losses (MoeLayer::forward_train, src/moe.rs:243-341, up to
@@ -8,9 +8,12 @@
 //   decode_gemm_kernel   down product of both
 //   combine              (the same kernel as the large path)
 //
-// and the products are spread over (tile, 32-feature block) workgroups whose four waves
-// split the reduction dimension, so that a few hundred kilobytes of weight fragments are in
-// flight per CU and every byte of a touched expert is fetched exactly once per 32-row tile.
+// which the layer folds into fewer where the call allows it: the combine into the down launch (the last
+// workgroup of a block of output columns to finish sums it), and - when most experts are about to be touched -
+// the routing into the gate/up launch (decode_front_kernel), behind which the down launch has one row of
+// workgroups per expert (decode_down_by_expert_kernel): two launches.  The products are spread over (tile,
+// 32-feature block) workgroups whose waves split the reduction dimension, so that a few hundred kilobytes of
+// weight fragments are in flight per CU and every byte of a touched expert is fetched exactly once per 32-row tile.
 #include <type_traits>
 
 #include "rbmoe_kernels.h"
