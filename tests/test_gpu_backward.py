@@ -124,6 +124,41 @@ def test_an_expert_without_tokens_gets_exactly_zero_gradients(device):
     layer.close()
 
 
+def test_router_gradient_of_one_expert_per_token_is_no_further_from_float64_than_the_oracle(device):
+    # With k = 1 the gate is p / p, so the gate's gradient reaches the probabilities as dgate - gate * dgate
+    # (src/moe.rs:404-419): zero in exact arithmetic, one rounding of a number of size |dgate| in f32.  That noise
+    # is larger than what the two losses contribute, and it depends on the last bits of dgate, which differ between
+    # any two orders of summation: the router gradient of such a layer is compared with its float64 value, where
+    # the GPU has to be as close as the oracle is; every other gradient is compared with the oracle as usual.
+    T, E = 2049, 2
+    t = synth.make(small_workload(d=384, E=E, k=1, F=512, T=T, seed=16026, act="f32", wt="f32"))
+    gout = grad_output_for(t, 5)
+    ref_layer = oracle_layer(t)
+    fwd = ref_layer.forward(t.x, threads=8)
+    ref = ref_layer.backward(t.x, gout, threads=8)
+    layer = gpu_layer(device, t, training=True)
+    out, cache = layer.forward_train(t.x)
+    assert_routing_identical(cache, fwd)
+    gin = layer.backward(gout)
+    assert rel_l2(gin, ref.grad_input) <= 1e-5
+    for e in range(E):
+        for which, want in ((L.W_GATE, ref.grad_gate), (L.W_UP, ref.grad_up), (L.W_DOWN, ref.grad_down)):
+            assert rel_l2(layer.weight_grad(which, e), want[e]) <= 1e-5
+    # float64: the gate contributes nothing; balance loss d aux / d p[t, e] = w_aux E load_e / V, z loss
+    # d z / d logit[t, e] = 2 w_z lse_t p[t, e] / V (src/moe.rs:421-478), softmax backward, then dlogits^T X
+    P = fwd.probabilities.astype(np.float64)
+    lse = fwd.lse.astype(np.float64)
+    dp = np.broadcast_to(0.01 * E * (fwd.counts.astype(np.float64) / T) / T, (T, E))
+    dlogits = P * (dp - (P * dp).sum(1, keepdims=True)) + 1e-3 * 2.0 * lse[:, None] * P / T
+    exact = dlogits.T @ t.x.astype(np.float64)
+    oracle_off = np.linalg.norm(ref.grad_router.astype(np.float64) - exact)
+    gpu_off = np.linalg.norm(layer.weight_grad(L.W_ROUTER).astype(np.float64) - exact)
+    print(f"|exact| {np.linalg.norm(exact):.3e}  oracle off by {oracle_off:.3e}  GPU off by {gpu_off:.3e}")
+    assert oracle_off > 0.05 * np.linalg.norm(exact), "the case no longer shows the cancellation it is here for"
+    assert gpu_off <= 2.0 * oracle_off
+    layer.close()
+
+
 def test_large_auxiliary_loss_weights_reach_the_router(device):
     # reference test src/moe.rs:969-1013: the balance and z losses are differentiated inside backward
     t = synth.make(small_workload(d=64, E=8, k=2, F=64, T=256, seed=24, act="bf16", wt="bf16"))
