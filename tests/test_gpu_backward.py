@@ -125,11 +125,12 @@ def test_an_expert_without_tokens_gets_exactly_zero_gradients(device):
 
 
 def test_router_gradient_of_one_expert_per_token_is_no_further_from_float64_than_the_oracle(device):
-    # With k = 1 the gate is p / p, so the gate's gradient reaches the probabilities as dgate - gate * dgate
-    # (src/moe.rs:404-419): zero in exact arithmetic, one rounding of a number of size |dgate| in f32.  That noise
-    # is larger than what the two losses contribute, and it depends on the last bits of dgate, which differ between
-    # any two orders of summation: the router gradient of such a layer is compared with its float64 value, where
-    # the GPU has to be as close as the oracle is; every other gradient is compared with the oracle as usual.
+    # With k = 1 the gate is p / p, and its gradient reaches the probability as g / total - (g p) / (total total)
+    # with total = p (src/moe.rs:427-441): zero in exact arithmetic, the roundings of two quotients of size |g| / p
+    # in f32.  That noise is larger than what the two losses contribute, and it depends on the last bits of g (a dot
+    # product of d terms), which differ between any two orders of summation: the router gradient of such a layer is
+    # compared with its float64 value, where the GPU has to be as close as the oracle is; every other gradient is
+    # compared with the oracle as usual.
     T, E = 2049, 2
     t = synth.make(small_workload(d=384, E=E, k=1, F=512, T=T, seed=16026, act="f32", wt="f32"))
     gout = grad_output_for(t, 5)
