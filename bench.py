@@ -19,6 +19,7 @@ import argparse
 import ctypes as C
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -629,7 +630,49 @@ def summary(m: dict) -> dict:
     return s
 
 
+def library_gemm_child(slots: int, d_ff: int, d_model: int) -> int:
+    """The measuring half of library_gemm: a process of its own (torch brings its own copy of the HIP runtime, which
+    finds no device in a process where this program's library has already opened one).  Prints one JSON object."""
+    import torch
+    out = {"library": f"torch {torch.__version__} matmul (bf16 x bf16 -> bf16)", "runs": "20 launches between one pair "
+           "of events, median of 5 runs, in a process of its own"}
+    for name, (M, N, K) in (("gate_up", (slots, 2 * d_ff, d_model)), ("down", (slots, d_model, d_ff))):
+        a = torch.randn(M, K, device="cuda:0", dtype=torch.bfloat16)
+        b = torch.randn(N, K, device="cuda:0", dtype=torch.bfloat16)
+        for _ in range(5):
+            a @ b.t()
+        torch.cuda.synchronize()
+        runs = []
+        for _ in range(5):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(20):
+                a @ b.t()
+            e1.record()
+            torch.cuda.synchronize()
+            runs.append(e0.elapsed_time(e1) / 20)
+        ms = statistics.median(runs)
+        tf = 2.0 * M * N * K / (ms * 1e-3) / 1e12
+        out[name] = {"M": M, "N": N, "K": K, "avg_launch_ms": ms, "tflops": tf, "frac_of_peak": tf / PEAK_BF16_TFLOPS}
+    print(json.dumps(out))
+    return 0
+
+
+def library_gemm(w) -> dict:
+    """The vendor library's bf16 product on the dense shapes of the two grouped products of workload `w` (all routed
+    rows as one group), measured by a child process (library_gemm_child)."""
+    import subprocess
+    cmd = [sys.executable, os.path.abspath(__file__), "--library-gemm-child", str(w.tokens * w.experts_per_token),
+           str(w.d_ff), str(w.d_model)]
+    res = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+    if res.returncode != 0:
+        return {"error": (res.stderr or "").strip().splitlines()[-1:] or ["child failed"]}
+    return json.loads(res.stdout.strip().splitlines()[-1])
+
+
 def main() -> int:
+    if sys.argv[1:2] == ["--library-gemm-child"]:
+        return library_gemm_child(int(sys.argv[2]), int(sys.argv[3]), int(sys.argv[4]))
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
@@ -657,6 +700,10 @@ def main() -> int:
     ap.add_argument("--calibrate-read", action="store_true",
                     help="also run a plain 39 MiB read with cold and warm caches (`calibration.read`): what a launch "
                          "the size of the decode gate/up product can get out of HBM")
+    ap.add_argument("--calibrate-library-gemm", action="store_true",
+                    help="also time the vendor library's bf16 matrix product (torch.matmul, i.e. hipBLASLt) on the dense "
+                         "shapes of the workload's two grouped products (`calibration.library_gemm`): what a plain "
+                         "product of these shapes - no gather, no ragged groups, no SwiGLU - gets out of the matrix cores")
     args = ap.parse_args()
     if args.repeats <= 0:
         args.repeats = max(5, min(25, 300 // max(args.steps, 1)))
@@ -705,6 +752,8 @@ def main() -> int:
         rd["note"] = ("warm: 20 launches of read_only_kernel between one pair of events; cold: a read-only sweep of "
                       "512 MiB before every launch, each launch in an event pair of its own, raw interval")
         calibration["read"] = rd
+    if args.calibrate_library_gemm:
+        calibration["library_gemm"] = library_gemm(w)
     if calibration:
         result["calibration"] = calibration
     if not args.no_backward:
